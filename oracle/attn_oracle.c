@@ -1,0 +1,621 @@
+/*
+ * attn_oracle.c -- CPU restatement of rustorch's attention hot path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the checker the HIP kernels are
+ * compared against (tests, the smoke check and the CPU-baseline leg of the
+ * benchmark).  Nothing in the shipped library calls, links or falls back to
+ * it.
+ *
+ * Every function restates one function of the reference and cites it
+ * (paths relative to the reference checkout):
+ *
+ *   ro_flash_forward_masked   crates/rustorch-attention/src/cpu_forward.rs:193-425
+ *   ro_flash_forward_scalar   crates/rustorch-attention/src/cpu_forward.rs:594-686
+ *   ro_naive_forward_masked   crates/rustorch-attention/src/cpu_forward.rs:702-763
+ *   ro_mask_is_masked         crates/rustorch-attention/src/mask.rs:40-46
+ *   ro_osm_*                  crates/rustorch-attention/src/online_softmax.rs:44-151
+ *   ro_gqa_forward_f32        crates/rustorch-nn/src/gqa.rs:94-270
+ *   ro_kv_cache_append        crates/rustorch-nn/src/kv_cache.rs:77-112
+ *   ro_kv_trim                crates/rustorch-llm/src/model.rs:638-650
+ *   ro_gqa_decode_online_bf16 crates/rustorch-cuda/src/llm_kernels.rs:396-457
+ *   ro_kv_append_bf16         crates/rustorch-cuda/src/llm_kernels.rs:353-372
+ *   ro_f32_to_bf16            half 2.7.1 bf16::from_f32 (round to nearest even),
+ *                             the rule crates/rustorch-amp/src/bf16_kernels.rs:266-267 uses
+ *
+ * The tile products of the native forward live in the third-party crate
+ * `gemm` 0.18.2 (Cargo.lock:1359-1362), which is not vendored.  Its result
+ * is restated here as the mathematical product accumulated in f32 in
+ * ascending contraction order; agreement with that crate's summation order
+ * at the last-bit level is therefore "parity unpinned".  What is pinned: the
+ * reference's own flash-vs-naive tolerance (1e-4), the closed forms and the
+ * edge/NaN rules (see tests/test_oracle_*.py).
+ *
+ * Built with -ffp-contract=off so that mul and add stay separate roundings,
+ * as in the reference's scalar Rust loops.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define RO_EXPORT __attribute__((visibility("default")))
+
+/* ---- status codes (same numbering as include/rt_attn.h) ----------------- */
+enum {
+    RO_OK = 0,
+    RO_ERR_ZERO_DIM = 1,
+    RO_ERR_BUFFER_SHAPE_MISMATCH = 2,
+    RO_ERR_OUTPUT_SHAPE_MISMATCH = 3,
+    RO_ERR_PADDING_LENGTH_MISMATCH = 4,
+    RO_ERR_HEAD_COUNT_MISMATCH = 5,
+    RO_ERR_WRONG_INPUT_LEN = 6,
+    RO_ERR_KV_OVERFLOW = 7,
+    RO_ERR_KV_WRONG_INPUT_LEN = 8,
+};
+
+enum { RO_MASK_NONE = 0, RO_MASK_CAUSAL = 1, RO_MASK_PADDING = 2 };
+enum { RO_WHICH_Q = 0, RO_WHICH_K = 1, RO_WHICH_V = 2, RO_WHICH_OUT = 3, RO_WHICH_FLASH = 4 };
+
+typedef struct {
+    uint64_t batch, heads, seq, dim, br, bc;
+} ro_shape;
+
+typedef struct {
+    int32_t which;
+    uint64_t expected;
+    uint64_t got;
+    uint64_t got2;
+} ro_err;
+
+static void set_err(ro_err *e, int which, uint64_t expected, uint64_t got) {
+    if (e) {
+        e->which = which;
+        e->expected = expected;
+        e->got = got;
+        e->got2 = 0;
+    }
+}
+
+/* ---- mask.rs:40-46 ------------------------------------------------------ */
+RO_EXPORT int ro_mask_is_masked(int kind, const uint8_t *keep, size_t keep_n, size_t qi, size_t kj) {
+    switch (kind) {
+    case RO_MASK_CAUSAL:
+        return kj > qi;
+    case RO_MASK_PADDING:
+        return kj < keep_n && !keep[kj];
+    default:
+        return 0;
+    }
+}
+
+/* ---- cpu_forward.rs:142-169 (validate) + mask.rs:51-65 ------------------ */
+static int validate(const ro_shape *s, size_t qn, size_t kn, size_t vn, size_t on, int kind, size_t keep_n,
+                    ro_err *err) {
+    if (s->dim == 0) return RO_ERR_ZERO_DIM;
+    uint64_t expected = s->batch * s->heads * s->seq * s->dim;
+    size_t lens[3] = {qn, kn, vn};
+    for (int i = 0; i < 3; i++) {
+        if (lens[i] != expected) {
+            set_err(err, i, expected, lens[i]);
+            return RO_ERR_BUFFER_SHAPE_MISMATCH;
+        }
+    }
+    if (on != expected) {
+        set_err(err, RO_WHICH_OUT, expected, on);
+        return RO_ERR_OUTPUT_SHAPE_MISMATCH;
+    }
+    if (kind == RO_MASK_PADDING && keep_n != s->seq) {
+        set_err(err, -1, s->seq, keep_n);
+        return RO_ERR_PADDING_LENGTH_MISMATCH;
+    }
+    return RO_OK;
+}
+
+/* ---- cpu_forward.rs:268-425, one (b,h) slab ----------------------------- */
+static void flash_bh_tiles(const float *q, const float *k, const float *v, float *out_slab, int kind,
+                           const uint8_t *keep, size_t keep_n, float scale, size_t seq, size_t dim, size_t br,
+                           size_t bc) {
+    float *s_buf = (float *)malloc(sizeof(float) * br * bc);
+    float *p_buf = (float *)malloc(sizeof(float) * br * bc);
+    float *o_buf = (float *)malloc(sizeof(float) * br * dim);
+    float *m_buf = (float *)malloc(sizeof(float) * br);
+    float *l_buf = (float *)malloc(sizeof(float) * br);
+    float *kt = (float *)malloc(sizeof(float) * bc * dim); /* K tile, transposed, for a vectorisable product */
+
+    for (size_t qi = 0; qi < seq; qi += br) {
+        size_t qi_end = qi + br < seq ? qi + br : seq;
+        size_t br_used = qi_end - qi;
+        for (size_t r = 0; r < br_used; r++) {
+            m_buf[r] = -INFINITY;
+            l_buf[r] = 0.0f;
+            for (size_t d = 0; d < dim; d++) o_buf[r * dim + d] = 0.0f;
+        }
+        /* every kv tile is visited, also those a causal mask empties (:311-313) */
+        for (size_t kj = 0; kj < seq; kj += bc) {
+            size_t kj_end = kj + bc < seq ? kj + bc : seq;
+            size_t bc_used = kj_end - kj;
+
+            /* S = scale * (Q_tile . K_tile^T): dot product first, scale applied to the
+             * finished sum (gemm alpha=0, beta=scale; :487-507). */
+            for (size_t d = 0; d < dim; d++)
+                for (size_t c = 0; c < bc_used; c++) kt[d * bc_used + c] = k[(kj + c) * dim + d];
+            for (size_t r = 0; r < br_used; r++) {
+                float *s_row = s_buf + r * bc_used;
+                const float *q_row = q + (qi + r) * dim;
+                for (size_t c = 0; c < bc_used; c++) s_row[c] = 0.0f;
+                for (size_t d = 0; d < dim; d++) {
+                    float qd = q_row[d];
+                    const float *kt_row = kt + d * bc_used;
+                    for (size_t c = 0; c < bc_used; c++) s_row[c] += qd * kt_row[c];
+                }
+                for (size_t c = 0; c < bc_used; c++) s_row[c] *= scale;
+            }
+            /* mask -> -inf (:342-352) */
+            if (kind != RO_MASK_NONE) {
+                for (size_t r = 0; r < br_used; r++)
+                    for (size_t c = 0; c < bc_used; c++)
+                        if (ro_mask_is_masked(kind, keep, keep_n, qi + r, kj + c)) s_buf[r * bc_used + c] = -INFINITY;
+            }
+            /* per-row online softmax (:355-386) */
+            for (size_t r = 0; r < br_used; r++) {
+                const float *s_row = s_buf + r * bc_used;
+                float m_tile = -INFINITY;
+                for (size_t c = 0; c < bc_used; c++)
+                    if (s_row[c] > m_tile) m_tile = s_row[c];
+                float m_prev = m_buf[r];
+                float m_new = m_tile > m_prev ? m_tile : m_prev;
+                float alpha = (m_prev == -INFINITY) ? 0.0f : expf(m_prev - m_new);
+                if (alpha != 1.0f) {
+                    l_buf[r] *= alpha;
+                    for (size_t d = 0; d < dim; d++) o_buf[r * dim + d] *= alpha;
+                }
+                float *p_row = p_buf + r * bc_used;
+                float tile_l = 0.0f;
+                for (size_t c = 0; c < bc_used; c++) {
+                    float p = expf(s_row[c] - m_new);
+                    p_row[c] = p;
+                    tile_l += p;
+                }
+                l_buf[r] += tile_l;
+                m_buf[r] = m_new;
+            }
+            /* O += P . V_tile (gemm alpha=1, beta=1; :564-584) */
+            for (size_t r = 0; r < br_used; r++) {
+                float *o_row = o_buf + r * dim;
+                const float *p_row = p_buf + r * bc_used;
+                for (size_t c = 0; c < bc_used; c++) {
+                    float p = p_row[c];
+                    const float *v_row = v + (kj + c) * dim;
+                    for (size_t d = 0; d < dim; d++) o_row[d] += p * v_row[d];
+                }
+            }
+        }
+        /* normalise or NaN (:405-421) */
+        for (size_t r = 0; r < br_used; r++) {
+            float *dst = out_slab + (qi + r) * dim;
+            float l = l_buf[r];
+            if (l > 0.0f && isfinite(l)) {
+                float inv_l = 1.0f / l;
+                for (size_t d = 0; d < dim; d++) dst[d] = o_buf[r * dim + d] * inv_l;
+            } else {
+                for (size_t d = 0; d < dim; d++) dst[d] = NAN;
+            }
+        }
+    }
+    free(s_buf);
+    free(p_buf);
+    free(o_buf);
+    free(m_buf);
+    free(l_buf);
+    free(kt);
+}
+
+/* ---- cpu_forward.rs:193-242 --------------------------------------------- */
+RO_EXPORT int ro_flash_forward_masked(const ro_shape *s, const float *q, size_t qn, const float *k, size_t kn,
+                                      const float *v, size_t vn, int mask_kind, const uint8_t *keep, size_t keep_n,
+                                      float *out, size_t on, ro_err *err, int threads) {
+    int rc = validate(s, qn, kn, vn, on, mask_kind, keep_n, err);
+    if (rc) return rc;
+    if (s->seq == 0) return RO_OK;
+    float scale = 1.0f / sqrtf((float)s->dim);
+    size_t s_h = s->seq * s->dim;
+    long n_slabs = (long)(s->batch * s->heads);
+    if (threads < 1) threads = 1;
+    /* one task per (b,h) slab, as rayon's par_chunks_mut(s_h) (:219) */
+#pragma omp parallel for schedule(dynamic, 1) num_threads(threads)
+    for (long bh = 0; bh < n_slabs; bh++) {
+        size_t base = (size_t)bh * s_h;
+        flash_bh_tiles(q + base, k + base, v + base, out + base, mask_kind, keep, keep_n, scale, s->seq, s->dim,
+                       s->br, s->bc);
+    }
+    return RO_OK;
+}
+
+/* ---- online_softmax.rs:44-151 ------------------------------------------- */
+typedef struct {
+    float m, l;
+} ro_osm_state;
+
+RO_EXPORT void ro_osm_empty(ro_osm_state *st) {
+    st->m = -INFINITY;
+    st->l = 0.0f;
+}
+RO_EXPORT void ro_osm_from_scalar(ro_osm_state *st, float x) {
+    st->m = x;
+    st->l = 1.0f;
+}
+RO_EXPORT void ro_osm_absorb(ro_osm_state *st, float x) {
+    if (x > st->m) {
+        st->l = st->l * expf(st->m - x) + 1.0f;
+        st->m = x;
+    } else {
+        st->l += expf(x - st->m);
+    }
+}
+RO_EXPORT int ro_osm_is_empty(const ro_osm_state *st) { return st->m == -INFINITY && st->l == 0.0f; }
+RO_EXPORT void ro_osm_combine(const ro_osm_state *a, const ro_osm_state *b, ro_osm_state *r) {
+    if (ro_osm_is_empty(a)) {
+        *r = *b;
+        return;
+    }
+    if (ro_osm_is_empty(b)) {
+        *r = *a;
+        return;
+    }
+    float m_new = a->m > b->m ? a->m : b->m;
+    ro_osm_state o;
+    o.m = m_new;
+    if (a->m == m_new && b->m == m_new)
+        o.l = a->l + b->l;
+    else if (a->m == m_new)
+        o.l = a->l + b->l * expf(b->m - m_new);
+    else
+        o.l = a->l * expf(a->m - m_new) + b->l;
+    *r = o;
+}
+RO_EXPORT void ro_osm_full(const float *xs, size_t n, ro_osm_state *st) {
+    ro_osm_empty(st);
+    for (size_t i = 0; i < n; i++) ro_osm_absorb(st, xs[i]);
+}
+
+/* ---- cpu_forward.rs:594-686: the row-by-row statement of the same recurrence */
+RO_EXPORT int ro_flash_forward_scalar(const ro_shape *s, const float *q, size_t qn, const float *k, size_t kn,
+                                      const float *v, size_t vn, int mask_kind, const uint8_t *keep, size_t keep_n,
+                                      float *out, size_t on, ro_err *err) {
+    int rc = validate(s, qn, kn, vn, on, mask_kind, keep_n, err);
+    if (rc) return rc;
+    if (s->seq == 0) return RO_OK;
+    float scale = 1.0f / sqrtf((float)s->dim);
+    size_t seq = s->seq, dim = s->dim, bc = s->bc;
+    float *o_row = (float *)malloc(sizeof(float) * dim);
+    float *scores = (float *)malloc(sizeof(float) * bc);
+    for (size_t bh = 0; bh < s->batch * s->heads; bh++) {
+        size_t base = bh * seq * dim;
+        for (size_t qi = 0; qi < seq; qi++) {
+            ro_osm_state st;
+            ro_osm_empty(&st);
+            for (size_t d = 0; d < dim; d++) o_row[d] = 0.0f;
+            const float *q_row = q + base + qi * dim;
+            for (size_t kj = 0; kj < seq; kj += bc) {
+                size_t kj_end = kj + bc < seq ? kj + bc : seq;
+                size_t bc_used = kj_end - kj;
+                for (size_t kk = kj; kk < kj_end; kk++) {
+                    const float *k_row = k + base + kk * dim;
+                    float acc = 0.0f;
+                    for (size_t d = 0; d < dim; d++) acc += q_row[d] * k_row[d];
+                    scores[kk - kj] =
+                        ro_mask_is_masked(mask_kind, keep, keep_n, qi, kk) ? -INFINITY : acc * scale;
+                }
+                float m_tile = -INFINITY;
+                for (size_t c = 0; c < bc_used; c++) m_tile = fmaxf(m_tile, scores[c]);
+                float m_comb = m_tile > st.m ? m_tile : st.m;
+                float alpha = (st.m == -INFINITY) ? 0.0f : expf(st.m - m_comb);
+                if (alpha != 1.0f) {
+                    st.l *= alpha;
+                    for (size_t d = 0; d < dim; d++) o_row[d] *= alpha;
+                }
+                float tile_l = 0.0f;
+                for (size_t c = 0; c < bc_used; c++) {
+                    float p = expf(scores[c] - m_comb);
+                    tile_l += p;
+                    const float *v_row = v + base + (kj + c) * dim;
+                    for (size_t d = 0; d < dim; d++) o_row[d] += p * v_row[d];
+                }
+                st.l += tile_l;
+                st.m = m_comb;
+            }
+            float *dst = out + base + qi * dim;
+            if (st.l > 0.0f && isfinite(st.l)) {
+                for (size_t d = 0; d < dim; d++) dst[d] = o_row[d] / st.l;
+            } else {
+                for (size_t d = 0; d < dim; d++) dst[d] = NAN;
+            }
+        }
+    }
+    free(o_row);
+    free(scores);
+    return RO_OK;
+}
+
+/* ---- cpu_forward.rs:702-763 --------------------------------------------- */
+RO_EXPORT int ro_naive_forward_masked(const ro_shape *s, const float *q, size_t qn, const float *k, size_t kn,
+                                      const float *v, size_t vn, int mask_kind, const uint8_t *keep, size_t keep_n,
+                                      float *out, size_t on, ro_err *err) {
+    int rc = validate(s, qn, kn, vn, on, mask_kind, keep_n, err);
+    if (rc) return rc;
+    float scale = 1.0f / sqrtf((float)s->dim);
+    size_t seq = s->seq, dim = s->dim;
+    float *scores = (float *)malloc(sizeof(float) * (seq * seq + 1));
+    for (size_t bh = 0; bh < s->batch * s->heads; bh++) {
+        size_t base = bh * seq * dim;
+        for (size_t i = 0; i < seq; i++)
+            for (size_t j = 0; j < seq; j++) {
+                if (ro_mask_is_masked(mask_kind, keep, keep_n, i, j)) {
+                    scores[i * seq + j] = -INFINITY;
+                    continue;
+                }
+                float acc = 0.0f;
+                for (size_t d = 0; d < dim; d++) acc += q[base + i * dim + d] * k[base + j * dim + d];
+                scores[i * seq + j] = acc * scale;
+            }
+        for (size_t i = 0; i < seq; i++) {
+            float *row = scores + i * seq;
+            float m = -INFINITY;
+            for (size_t j = 0; j < seq; j++) m = fmaxf(m, row[j]);
+            float sum = 0.0f;
+            for (size_t j = 0; j < seq; j++) {
+                row[j] = expf(row[j] - m);
+                sum += row[j];
+            }
+            float *dst = out + base + i * dim;
+            if (sum > 0.0f && isfinite(sum)) {
+                for (size_t j = 0; j < seq; j++) row[j] /= sum;
+                for (size_t d = 0; d < dim; d++) {
+                    float o = 0.0f;
+                    for (size_t j = 0; j < seq; j++) o += row[j] * v[base + j * dim + d];
+                    dst[d] = o;
+                }
+            } else {
+                for (size_t d = 0; d < dim; d++) dst[d] = NAN;
+            }
+        }
+    }
+    free(scores);
+    return RO_OK;
+}
+
+/* ---- gqa.rs:216-270 ----------------------------------------------------- */
+static void decode_attn_row(size_t bh_idx, const float *q, const float *k, const float *v, float *out_block,
+                            size_t n_heads, size_t n_kv_heads, size_t seq_q, size_t seq_kv, size_t head_dim,
+                            float scale, size_t group_size) {
+    size_t b = bh_idx / n_heads, h = bh_idx % n_heads, kv_h = h / group_size;
+    const float *q_block = q + b * n_heads * seq_q * head_dim + h * seq_q * head_dim;
+    size_t kv_off = b * n_kv_heads * seq_kv * head_dim + kv_h * seq_kv * head_dim;
+    const float *k_block = k + kv_off, *v_block = v + kv_off;
+    float *scores = (float *)malloc(sizeof(float) * (seq_kv + 1));
+    for (size_t q_pos = 0; q_pos < seq_q; q_pos++) {
+        const float *q_row = q_block + q_pos * head_dim;
+        for (size_t k_pos = 0; k_pos < seq_kv; k_pos++) {
+            const float *k_row = k_block + k_pos * head_dim;
+            float acc = 0.0f;
+            for (size_t d = 0; d < head_dim; d++) acc += q_row[d] * k_row[d];
+            scores[k_pos] = acc * scale;
+        }
+        float max_s = -INFINITY;
+        for (size_t t = 0; t < seq_kv; t++) max_s = fmaxf(max_s, scores[t]);
+        float sum_exp = 0.0f;
+        for (size_t t = 0; t < seq_kv; t++) {
+            scores[t] = expf(scores[t] - max_s);
+            sum_exp += scores[t];
+        }
+        float inv_sum = 1.0f / sum_exp;
+        for (size_t t = 0; t < seq_kv; t++) scores[t] *= inv_sum;
+        float *out_row = out_block + q_pos * head_dim;
+        for (size_t d = 0; d < head_dim; d++) out_row[d] = 0.0f;
+        for (size_t t = 0; t < seq_kv; t++) {
+            const float *v_row = v_block + t * head_dim;
+            float w = scores[t];
+            for (size_t d = 0; d < head_dim; d++) out_row[d] += w * v_row[d];
+        }
+    }
+    free(scores);
+}
+
+/* ---- gqa.rs:94-210 ------------------------------------------------------ */
+RO_EXPORT int ro_gqa_forward_f32(const float *q, size_t qn, const float *k, size_t kn, const float *v, size_t vn,
+                                 float *out, size_t on, size_t batch, size_t n_heads, size_t n_kv_heads,
+                                 size_t seq_q, size_t seq_kv, size_t head_dim, ro_err *err, int threads) {
+    if (n_kv_heads == 0 || n_heads % n_kv_heads != 0) {
+        set_err(err, -1, n_heads, n_kv_heads);
+        return RO_ERR_HEAD_COUNT_MISMATCH;
+    }
+    size_t q_len = batch * n_heads * seq_q * head_dim;
+    size_t kv_len = batch * n_kv_heads * seq_kv * head_dim;
+    if (qn != q_len) return set_err(err, RO_WHICH_Q, q_len, qn), RO_ERR_WRONG_INPUT_LEN;
+    if (kn != kv_len) return set_err(err, RO_WHICH_K, kv_len, kn), RO_ERR_WRONG_INPUT_LEN;
+    if (vn != kv_len) return set_err(err, RO_WHICH_V, kv_len, vn), RO_ERR_WRONG_INPUT_LEN;
+    if (on != q_len) return set_err(err, RO_WHICH_OUT, q_len, on), RO_ERR_WRONG_INPUT_LEN;
+    size_t group_size = n_heads / n_kv_heads;
+
+    if (seq_q == seq_kv) {
+        /* prefill: replicate K/V to n_heads, then unmasked flash (:151-177) */
+        size_t kv_h_size = seq_kv * head_dim, kv_block = batch * n_heads * kv_h_size;
+        float *k_rep = (float *)malloc(sizeof(float) * (kv_block + 1));
+        float *v_rep = (float *)malloc(sizeof(float) * (kv_block + 1));
+        for (size_t b = 0; b < batch; b++)
+            for (size_t h = 0; h < n_heads; h++) {
+                size_t kv_h = h / group_size;
+                size_t src = b * n_kv_heads * kv_h_size + kv_h * kv_h_size;
+                size_t dst = b * n_heads * kv_h_size + h * kv_h_size;
+                memcpy(k_rep + dst, k + src, sizeof(float) * kv_h_size);
+                memcpy(v_rep + dst, v + src, sizeof(float) * kv_h_size);
+            }
+        ro_shape s = {batch, n_heads, seq_q, head_dim, 64, 64};
+        int rc = ro_flash_forward_masked(&s, q, qn, k_rep, kv_block, v_rep, kv_block, RO_MASK_NONE, NULL, 0, out, on,
+                                         NULL, threads);
+        free(k_rep);
+        free(v_rep);
+        if (rc) {
+            /* any flash error is reported as WrongInputLen{which:"flash_forward",0,0} (:171-175) */
+            set_err(err, RO_WHICH_FLASH, 0, 0);
+            return RO_ERR_WRONG_INPUT_LEN;
+        }
+        return RO_OK;
+    }
+    float scale = 1.0f / sqrtf((float)head_dim);
+    long n = (long)(batch * n_heads);
+    if (seq_q == 1 || threads <= 1) {
+        /* single-thread loop for seq_q == 1 (:190-198) */
+        for (long i = 0; i < n; i++)
+            decode_attn_row((size_t)i, q, k, v, out + (size_t)i * seq_q * head_dim, n_heads, n_kv_heads, seq_q,
+                            seq_kv, head_dim, scale, group_size);
+        return RO_OK;
+    }
+#pragma omp parallel for schedule(dynamic, 1) num_threads(threads)
+    for (long i = 0; i < n; i++)
+        decode_attn_row((size_t)i, q, k, v, out + (size_t)i * seq_q * head_dim, n_heads, n_kv_heads, seq_q, seq_kv,
+                        head_dim, scale, group_size);
+    return RO_OK;
+}
+
+/* ---- kv_cache.rs:77-112: append [B,H,s_new,D] at current_len into [B,H,max_seq,D] */
+RO_EXPORT int ro_kv_cache_append(float *k_cache, float *v_cache, size_t batch, size_t n_heads, size_t max_seq,
+                                 size_t head_dim, size_t current_len, size_t seq_added, const float *new_k,
+                                 size_t nk, const float *new_v, size_t nv, ro_err *err) {
+    if (current_len + seq_added > max_seq) {
+        set_err(err, -1, max_seq, current_len + seq_added);
+        return RO_ERR_KV_OVERFLOW;
+    }
+    size_t bhsd = batch * n_heads * seq_added * head_dim;
+    if (nk != bhsd || nv != bhsd) {
+        set_err(err, -1, bhsd, nk);
+        if (err) err->got2 = nv;
+        return RO_ERR_KV_WRONG_INPUT_LEN;
+    }
+    for (size_t b = 0; b < batch; b++)
+        for (size_t h = 0; h < n_heads; h++) {
+            size_t src = b * n_heads * seq_added * head_dim + h * seq_added * head_dim;
+            size_t dst = b * n_heads * max_seq * head_dim + h * max_seq * head_dim + current_len * head_dim;
+            memcpy(k_cache + dst, new_k + src, sizeof(float) * seq_added * head_dim);
+            memcpy(v_cache + dst, new_v + src, sizeof(float) * seq_added * head_dim);
+        }
+    return RO_OK;
+}
+
+/* ---- model.rs:638-650: copy the valid prefix [..kv_len] of every head out of the
+ * [H,max_seq,D] slab into a contiguous [H,kv_len,D] buffer */
+RO_EXPORT void ro_kv_trim(const float *cache, float *trimmed, size_t n_kv_heads, size_t max_seq, size_t kv_len,
+                          size_t head_dim) {
+    for (size_t h = 0; h < n_kv_heads; h++)
+        memcpy(trimmed + h * kv_len * head_dim, cache + h * max_seq * head_dim, sizeof(float) * kv_len * head_dim);
+}
+
+/* ---- bf16 <-> f32, round to nearest even (half 2.7.1 bf16::from_f32) ------ */
+RO_EXPORT uint16_t ro_f32_to_bf16(float x) {
+    uint32_t u;
+    memcpy(&u, &x, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u); /* NaN stays NaN (quiet) */
+    uint32_t round_bit = 0x00008000u;
+    if ((u & round_bit) != 0 && (u & (3 * round_bit - 1)) != 0) return (uint16_t)((u >> 16) + 1);
+    return (uint16_t)(u >> 16);
+}
+RO_EXPORT float ro_bf16_to_f32(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+RO_EXPORT void ro_f32_to_bf16_array(const float *x, uint16_t *y, size_t n) {
+    for (size_t i = 0; i < n; i++) y[i] = ro_f32_to_bf16(x[i]);
+}
+RO_EXPORT void ro_bf16_to_f32_array(const uint16_t *x, float *y, size_t n) {
+    for (size_t i = 0; i < n; i++) y[i] = ro_bf16_to_f32(x[i]);
+}
+
+/* ---- llm_kernels.rs:353-372 --------------------------------------------- */
+RO_EXPORT void ro_kv_append_bf16(uint16_t *k_cache, uint16_t *v_cache, const uint16_t *k_in, const uint16_t *v_in,
+                                 int pos, int n_kv, int head_dim, int max_seq) {
+    for (int kv_h = 0; kv_h < n_kv; kv_h++)
+        for (int i = 0; i < head_dim; i++) {
+            size_t cache_off = (size_t)kv_h * max_seq * head_dim + (size_t)pos * head_dim + i;
+            size_t in_off = (size_t)kv_h * head_dim + i;
+            k_cache[cache_off] = k_in[in_off];
+            v_cache[cache_off] = v_in[in_off];
+        }
+}
+
+/* ---- llm_kernels.rs:396-457: one pass, f32 state (m=-1e30, l, o), bf16 in/out.
+ * The block-wide tree reduction of the dot product is restated as an
+ * ascending f32 sum. */
+RO_EXPORT void ro_gqa_decode_online_bf16(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache,
+                                         uint16_t *out, int n_heads, int n_kv, int kv_len, int head_dim,
+                                         int max_seq) {
+    float scale = 1.0f / sqrtf((float)head_dim);
+    float *o = (float *)malloc(sizeof(float) * head_dim);
+    for (int h = 0; h < n_heads; h++) {
+        int kv_h = h * n_kv / n_heads;
+        float m = -1e30f, l = 0.0f;
+        for (int i = 0; i < head_dim; i++) o[i] = 0.0f;
+        for (int t = 0; t < kv_len; t++) {
+            size_t row = ((size_t)kv_h * max_seq + t) * head_dim;
+            float dot = 0.0f;
+            for (int i = 0; i < head_dim; i++)
+                dot += ro_bf16_to_f32(q[(size_t)h * head_dim + i]) * ro_bf16_to_f32(k_cache[row + i]);
+            float s_t = dot * scale;
+            float new_m = fmaxf(m, s_t);
+            float correction = expf(m - new_m);
+            float p = expf(s_t - new_m);
+            for (int i = 0; i < head_dim; i++) o[i] = o[i] * correction + p * ro_bf16_to_f32(v_cache[row + i]);
+            l = l * correction + p;
+            m = new_m;
+        }
+        for (int i = 0; i < head_dim; i++) out[(size_t)h * head_dim + i] = ro_f32_to_bf16(o[i] / fmaxf(l, 1e-12f));
+    }
+    free(o);
+}
+
+/* ---- Batched, ragged decode: the CPU path (model.rs:638-668 trim + gqa.rs
+ * decode_attn_row) applied per sequence b with its own kv_len, in f32 on
+ * bf16-rounded inputs.  q [B,Hq,D] bf16, caches [B,Hkv,max_seq,D] bf16,
+ * out [B,Hq,D] f32.  kv_len == 0 leaves the row as 0/0 = NaN, as gqa.rs:256 would. */
+RO_EXPORT void ro_gqa_decode_batched_bf16(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache,
+                                          const int32_t *kv_lens, float *out, int batch, int n_heads, int n_kv,
+                                          int head_dim, int max_seq, int threads) {
+    size_t group = (size_t)n_heads / n_kv;
+    float scale = 1.0f / sqrtf((float)head_dim);
+    if (threads < 1) threads = 1;
+    long n_tasks = (long)batch * n_kv;
+#pragma omp parallel for schedule(dynamic, 1) num_threads(threads)
+    for (long task = 0; task < n_tasks; task++) {
+        size_t b = (size_t)task / n_kv, kv_h = (size_t)task % n_kv;
+        size_t kv_len = (size_t)kv_lens[b];
+        size_t D = (size_t)head_dim;
+        float *kf = (float *)malloc(sizeof(float) * (kv_len * D + 1));
+        float *vf = (float *)malloc(sizeof(float) * (kv_len * D + 1));
+        float *qf = (float *)malloc(sizeof(float) * D);
+        size_t base = (b * n_kv + kv_h) * (size_t)max_seq * D;
+        ro_bf16_to_f32_array(k_cache + base, kf, kv_len * D);
+        ro_bf16_to_f32_array(v_cache + base, vf, kv_len * D);
+        for (size_t g = 0; g < group; g++) {
+            size_t h = kv_h * group + g;
+            ro_bf16_to_f32_array(q + (b * n_heads + h) * D, qf, D);
+            /* a 1-batch, 1-head, 1-kv-head call of the row kernel on the trimmed prefix */
+            decode_attn_row(0, qf, kf, vf, out + (b * n_heads + h) * D, 1, 1, 1, kv_len, D, scale, 1);
+        }
+        free(kf);
+        free(vf);
+        free(qf);
+    }
+}
+
+RO_EXPORT int ro_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}

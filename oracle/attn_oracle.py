@@ -1,0 +1,355 @@
+"""ctypes binding of the CPU oracle (``libattn_oracle.so``, built from ``attn_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by ``__graft_entry__.smoke()``
+and by the ``cpu_baseline`` leg of ``bench.py`` as the checker.  The shipped
+package (``rustorch_amd``) never imports it.
+
+Each wrapper keeps the name of the reference function it restates
+(``crates/rustorch-attention/src/cpu_forward.rs``, ``mask.rs``,
+``online_softmax.rs``; ``crates/rustorch-nn/src/gqa.rs``, ``kv_cache.rs``;
+``crates/rustorch-cuda/src/llm_kernels.rs``); the C file cites the lines.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+from dataclasses import dataclass
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libattn_oracle.so")
+
+MASK_NONE, MASK_CAUSAL, MASK_PADDING = 0, 1, 2
+
+OK = 0
+ERR_ZERO_DIM = 1
+ERR_BUFFER_SHAPE_MISMATCH = 2
+ERR_OUTPUT_SHAPE_MISMATCH = 3
+ERR_PADDING_LENGTH_MISMATCH = 4
+ERR_HEAD_COUNT_MISMATCH = 5
+ERR_WRONG_INPUT_LEN = 6
+ERR_KV_OVERFLOW = 7
+ERR_KV_WRONG_INPUT_LEN = 8
+
+WHICH = {0: "q", 1: "k", 2: "v", 3: "out", 4: "flash_forward", -1: ""}
+
+
+class _Shape(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in ("batch", "heads", "seq", "dim", "br", "bc")]
+
+
+class _Err(C.Structure):
+    _fields_ = [("which", C.c_int32), ("expected", C.c_uint64), ("got", C.c_uint64), ("got2", C.c_uint64)]
+
+
+class _Osm(C.Structure):
+    _fields_ = [("m", C.c_float), ("l", C.c_float)]
+
+
+@dataclass
+class OracleError(Exception):
+    code: int
+    which: str = ""
+    expected: int = 0
+    got: int = 0
+    got2: int = 0
+
+    def __str__(self):
+        return f"oracle error code={self.code} which={self.which!r} expected={self.expected} got={self.got}"
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with its Makefile (gcc); returns the library path."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE] + (["-B"] if force else []), stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = C.CDLL(_LIB_PATH)
+        fp, u8p, u16p, i32p = (C.POINTER(C.c_float), C.POINTER(C.c_uint8), C.POINTER(C.c_uint16),
+                               C.POINTER(C.c_int32))
+        sz = C.c_size_t
+        fwd_args = [C.POINTER(_Shape), fp, sz, fp, sz, fp, sz, C.c_int, u8p, sz, fp, sz, C.POINTER(_Err)]
+        L.ro_flash_forward_masked.argtypes = fwd_args + [C.c_int]
+        L.ro_flash_forward_scalar.argtypes = fwd_args
+        L.ro_naive_forward_masked.argtypes = fwd_args
+        L.ro_mask_is_masked.argtypes = [C.c_int, u8p, sz, sz, sz]
+        L.ro_gqa_forward_f32.argtypes = [fp, sz, fp, sz, fp, sz, fp, sz, sz, sz, sz, sz, sz, sz, C.POINTER(_Err),
+                                         C.c_int]
+        L.ro_kv_cache_append.argtypes = [fp, fp, sz, sz, sz, sz, sz, sz, fp, sz, fp, sz, C.POINTER(_Err)]
+        L.ro_kv_trim.argtypes = [fp, fp, sz, sz, sz, sz]
+        L.ro_kv_trim.restype = None
+        L.ro_f32_to_bf16_array.argtypes = [fp, u16p, sz]
+        L.ro_f32_to_bf16_array.restype = None
+        L.ro_bf16_to_f32_array.argtypes = [u16p, fp, sz]
+        L.ro_bf16_to_f32_array.restype = None
+        L.ro_kv_append_bf16.argtypes = [u16p, u16p, u16p, u16p, C.c_int, C.c_int, C.c_int, C.c_int]
+        L.ro_kv_append_bf16.restype = None
+        L.ro_gqa_decode_online_bf16.argtypes = [u16p, u16p, u16p, u16p] + [C.c_int] * 5
+        L.ro_gqa_decode_online_bf16.restype = None
+        L.ro_gqa_decode_batched_bf16.argtypes = [u16p, u16p, u16p, i32p, fp] + [C.c_int] * 6
+        L.ro_gqa_decode_batched_bf16.restype = None
+        for name in ("ro_osm_empty",):
+            getattr(L, name).argtypes = [C.POINTER(_Osm)]
+            getattr(L, name).restype = None
+        L.ro_osm_from_scalar.argtypes = [C.POINTER(_Osm), C.c_float]
+        L.ro_osm_from_scalar.restype = None
+        L.ro_osm_absorb.argtypes = [C.POINTER(_Osm), C.c_float]
+        L.ro_osm_absorb.restype = None
+        L.ro_osm_is_empty.argtypes = [C.POINTER(_Osm)]
+        L.ro_osm_combine.argtypes = [C.POINTER(_Osm)] * 3
+        L.ro_osm_combine.restype = None
+        L.ro_osm_full.argtypes = [fp, sz, C.POINTER(_Osm)]
+        L.ro_osm_full.restype = None
+        L.ro_max_threads.restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def _f32(a):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return a, a.ctypes.data_as(C.POINTER(C.c_float))
+
+
+def _raise(code, err):
+    if code != OK:
+        raise OracleError(code, WHICH.get(err.which, ""), err.expected, err.got, err.got2)
+
+
+@dataclass
+class AttentionShape:
+    """``AttentionShape`` of cpu_forward.rs:49-89 (``new`` => br = bc = 64)."""
+    batch: int
+    heads: int
+    seq: int
+    dim: int
+    br: int = 64
+    bc: int = 64
+
+    def buffer_len(self) -> int:
+        return self.batch * self.heads * self.seq * self.dim
+
+    def _c(self):
+        return _Shape(self.batch, self.heads, self.seq, self.dim, self.br, self.bc)
+
+
+def _mask_args(mask):
+    """mask: None | "causal" | ("padding", keep-array)."""
+    if mask is None or mask == "none":
+        return MASK_NONE, None, 0, None
+    if mask == "causal":
+        return MASK_CAUSAL, None, 0, None
+    kind, keep = mask
+    assert kind == "padding"
+    keep = np.ascontiguousarray(np.asarray(keep, dtype=np.uint8))
+    return MASK_PADDING, keep.ctypes.data_as(C.POINTER(C.c_uint8)), keep.size, keep
+
+
+def _forward(fn, shape, q, k, v, mask, out_len, extra):
+    q, qp = _f32(np.ravel(q))
+    k, kp = _f32(np.ravel(k))
+    v, vp = _f32(np.ravel(v))
+    n_out = shape.buffer_len() if out_len is None else out_len
+    out = np.zeros(n_out, dtype=np.float32)
+    kind, keep_p, keep_n, _keep = _mask_args(mask)
+    err = _Err()
+    s = shape._c()
+    code = fn(C.byref(s), qp, q.size, kp, k.size, vp, v.size, kind, keep_p, keep_n,
+              out.ctypes.data_as(C.POINTER(C.c_float)), out.size, C.byref(err), *extra)
+    _raise(code, err)
+    return out
+
+
+def flash_forward_masked(shape, q, k, v, mask=None, threads=None, out_len=None):
+    """cpu_forward.rs:193-425 (tiled forward).  Returns the flat ``out`` array."""
+    t = lib().ro_max_threads() if threads is None else threads
+    return _forward(lib().ro_flash_forward_masked, shape, q, k, v, mask, out_len, (t,))
+
+
+def flash_forward(shape, q, k, v, threads=None, out_len=None):
+    """cpu_forward.rs:175-183."""
+    return flash_forward_masked(shape, q, k, v, None, threads, out_len)
+
+
+def flash_forward_scalar(shape, q, k, v, mask=None):
+    """cpu_forward.rs:594-686 (row-by-row statement of the same recurrence)."""
+    return _forward(lib().ro_flash_forward_scalar, shape, q, k, v, mask, None, ())
+
+
+def naive_forward_masked(shape, q, k, v, mask=None):
+    """cpu_forward.rs:702-763."""
+    return _forward(lib().ro_naive_forward_masked, shape, q, k, v, mask, None, ())
+
+
+def naive_forward(shape, q, k, v):
+    return naive_forward_masked(shape, q, k, v, None)
+
+
+def mask_is_masked(mask, qi, kj) -> bool:
+    kind, keep_p, keep_n, _keep = _mask_args(mask)
+    return bool(lib().ro_mask_is_masked(kind, keep_p, keep_n, qi, kj))
+
+
+def gqa_forward_f32(q, k, v, batch, n_heads, n_kv_heads, seq_q, seq_kv, head_dim, threads=None, out_len=None):
+    """gqa.rs:94-270.  Returns flat out [batch, n_heads, seq_q, head_dim]."""
+    q, qp = _f32(np.ravel(q))
+    k, kp = _f32(np.ravel(k))
+    v, vp = _f32(np.ravel(v))
+    n_out = batch * n_heads * seq_q * head_dim if out_len is None else out_len
+    out = np.zeros(n_out, dtype=np.float32)
+    err = _Err()
+    t = lib().ro_max_threads() if threads is None else threads
+    code = lib().ro_gqa_forward_f32(qp, q.size, kp, k.size, vp, v.size, out.ctypes.data_as(C.POINTER(C.c_float)),
+                                    out.size, batch, n_heads, n_kv_heads, seq_q, seq_kv, head_dim, C.byref(err), t)
+    _raise(code, err)
+    return out
+
+
+def kv_cache_append(k_cache, v_cache, batch, n_heads, max_seq, head_dim, current_len, seq_added, new_k, new_v):
+    """kv_cache.rs:77-112, in place on the two float32 cache arrays."""
+    assert k_cache.dtype == np.float32 and v_cache.dtype == np.float32
+    nk, nkp = _f32(np.ravel(new_k))
+    nv, nvp = _f32(np.ravel(new_v))
+    err = _Err()
+    code = lib().ro_kv_cache_append(k_cache.ctypes.data_as(C.POINTER(C.c_float)),
+                                    v_cache.ctypes.data_as(C.POINTER(C.c_float)), batch, n_heads, max_seq,
+                                    head_dim, current_len, seq_added, nkp, nk.size, nvp, nv.size, C.byref(err))
+    _raise(code, err)
+
+
+def kv_trim(cache, n_kv_heads, max_seq, kv_len, head_dim):
+    """model.rs:638-650."""
+    cache, cp = _f32(np.ravel(cache))
+    out = np.zeros(n_kv_heads * kv_len * head_dim, dtype=np.float32)
+    lib().ro_kv_trim(cp, out.ctypes.data_as(C.POINTER(C.c_float)), n_kv_heads, max_seq, kv_len, head_dim)
+    return out
+
+
+def f32_to_bf16(x):
+    """Round-to-nearest-even f32 -> bf16 bit patterns (uint16)."""
+    x, xp = _f32(np.ravel(x))
+    y = np.empty(x.size, dtype=np.uint16)
+    lib().ro_f32_to_bf16_array(xp, y.ctypes.data_as(C.POINTER(C.c_uint16)), x.size)
+    return y
+
+
+def bf16_to_f32(y):
+    y = np.ascontiguousarray(np.ravel(y), dtype=np.uint16)
+    x = np.empty(y.size, dtype=np.float32)
+    lib().ro_bf16_to_f32_array(y.ctypes.data_as(C.POINTER(C.c_uint16)), x.ctypes.data_as(C.POINTER(C.c_float)),
+                               y.size)
+    return x
+
+
+def _u16(a):
+    a = np.ascontiguousarray(np.ravel(a), dtype=np.uint16)
+    return a, a.ctypes.data_as(C.POINTER(C.c_uint16))
+
+
+def kv_append_bf16(k_cache, v_cache, k_in, v_in, pos, n_kv, head_dim, max_seq):
+    """llm_kernels.rs:353-372, in place on the uint16 cache arrays."""
+    assert k_cache.dtype == np.uint16 and v_cache.dtype == np.uint16
+    ki, kip = _u16(k_in)
+    vi, vip = _u16(v_in)
+    lib().ro_kv_append_bf16(k_cache.ctypes.data_as(C.POINTER(C.c_uint16)),
+                            v_cache.ctypes.data_as(C.POINTER(C.c_uint16)), kip, vip, pos, n_kv, head_dim, max_seq)
+
+
+def gqa_decode_online_bf16(q, k_cache, v_cache, n_heads, n_kv, kv_len, head_dim, max_seq):
+    """llm_kernels.rs:396-457.  bf16 bit patterns in, bf16 bit patterns out [n_heads*head_dim]."""
+    q, qp = _u16(q)
+    kc, kp = _u16(k_cache)
+    vc, vp = _u16(v_cache)
+    out = np.zeros(n_heads * head_dim, dtype=np.uint16)
+    lib().ro_gqa_decode_online_bf16(qp, kp, vp, out.ctypes.data_as(C.POINTER(C.c_uint16)), n_heads, n_kv, kv_len,
+                                    head_dim, max_seq)
+    return out
+
+
+def gqa_decode_batched_bf16(q, k_cache, v_cache, kv_lens, batch, n_heads, n_kv, head_dim, max_seq, threads=None):
+    """The CPU decode path (trim + decode_attn_row) per sequence with its own length, f32 on
+    bf16-rounded inputs.  Returns float32 [batch*n_heads*head_dim]."""
+    q, qp = _u16(q)
+    kc, kp = _u16(k_cache)
+    vc, vp = _u16(v_cache)
+    lens = np.ascontiguousarray(kv_lens, dtype=np.int32)
+    out = np.zeros(batch * n_heads * head_dim, dtype=np.float32)
+    t = lib().ro_max_threads() if threads is None else threads
+    lib().ro_gqa_decode_batched_bf16(qp, kp, vp, lens.ctypes.data_as(C.POINTER(C.c_int32)),
+                                     out.ctypes.data_as(C.POINTER(C.c_float)), batch, n_heads, n_kv, head_dim,
+                                     max_seq, t)
+    return out
+
+
+def varlen_causal_forward(q, k, v, seq_lens, batch, heads, max_seq, dim, zero_padded_rows=True, threads=None):
+    """Padded-batch causal prefill: for sequence b the valid rows [0, len_b) equal the
+    reference's ``flash_forward_masked(Mask::Causal)`` on the truncated (1,H,len_b,D)
+    problem (causal already hides keys >= len_b from valid queries); rows >= len_b are
+    0.0 (or NaN when ``zero_padded_rows`` is False, the reference's no-visible-key rule,
+    cpu_forward.rs:411-420)."""
+    q = np.asarray(q, dtype=np.float32).reshape(batch, heads, max_seq, dim)
+    k = np.asarray(k, dtype=np.float32).reshape(batch, heads, max_seq, dim)
+    v = np.asarray(v, dtype=np.float32).reshape(batch, heads, max_seq, dim)
+    fill = 0.0 if zero_padded_rows else np.nan
+    out = np.full((batch, heads, max_seq, dim), fill, dtype=np.float32)
+    for b in range(batch):
+        n = int(seq_lens[b])
+        if n == 0:
+            continue
+        sh = AttentionShape(1, heads, n, dim)
+        o = flash_forward_masked(sh, q[b, :, :n], k[b, :, :n], v[b, :, :n], "causal", threads)
+        out[b, :, :n] = o.reshape(heads, n, dim)
+    return out.ravel()
+
+
+class OnlineSoftmaxState:
+    """online_softmax.rs:44-151."""
+
+    def __init__(self, m=-np.inf, l=0.0):
+        self._s = _Osm(m, l)
+
+    @property
+    def m(self):
+        return self._s.m
+
+    @property
+    def l(self):
+        return self._s.l
+
+    @classmethod
+    def from_scalar(cls, x):
+        st = cls()
+        lib().ro_osm_from_scalar(C.byref(st._s), x)
+        return st
+
+    def absorb(self, x):
+        lib().ro_osm_absorb(C.byref(self._s), x)
+
+    def is_empty(self):
+        return bool(lib().ro_osm_is_empty(C.byref(self._s)))
+
+
+def combine_tiles(a: OnlineSoftmaxState, b: OnlineSoftmaxState) -> OnlineSoftmaxState:
+    r = OnlineSoftmaxState()
+    lib().ro_osm_combine(C.byref(a._s), C.byref(b._s), C.byref(r._s))
+    return r
+
+
+def online_softmax_full(xs) -> OnlineSoftmaxState:
+    xs, xp = _f32(np.ravel(xs))
+    r = OnlineSoftmaxState()
+    lib().ro_osm_full(xp, xs.size, C.byref(r._s))
+    return r
+
+
+def max_threads() -> int:
+    return lib().ro_max_threads()
