@@ -1,0 +1,175 @@
+/*
+ * rt_attn.h -- C ABI of librt_attn_hip.so, the MI355X (gfx950) attention engine that stands
+ * in for rustorch's attention hot path.
+ *
+ * Every entry point replaces one call surface of the reference (paths relative to the
+ * reference checkout) and keeps its argument meaning and its error order.  Plain pointers and
+ * sizes only; `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *
+ * Host-slice entry points (rt_flash_forward*_f32, rt_gqa_forward_f32) are synchronous, like
+ * the Rust functions they replace: they stage the slices to HBM, run the kernels and copy the
+ * result back before returning.  Device entry points (*_dev, rt_gqa_decode_*, rt_kv_append_*)
+ * take device addresses, enqueue on `stream` and return without synchronising, like the
+ * reference's `LlmKernels` launchers.
+ *
+ * There is no CPU fallback: with no usable gfx950 device every compute entry point returns
+ * RT_ERR_NO_DEVICE / RT_ERR_HIP.
+ */
+#ifndef RT_ATTN_H
+#define RT_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* AttentionShape -- crates/rustorch-attention/src/cpu_forward.rs:49-89.  Row-major
+ * [batch, heads, seq, dim].  br/bc are the reference's CPU tile sizes (64 by default); the
+ * GPU kernels choose their own tiling and use bc only to reproduce the reference's result for
+ * a padding mask whose first bc keys are all masked (every row NaN, see rt_flash_forward_masked_f32). */
+typedef struct rt_attention_shape {
+    uint64_t batch;
+    uint64_t heads;
+    uint64_t seq;
+    uint64_t dim;
+    uint64_t br;
+    uint64_t bc;
+} rt_attention_shape;
+
+/* Return codes.  1-4 mirror AttentionError / MaskError (cpu_forward.rs:93-114, mask.rs:70-78),
+ * 5-6 GQAError (crates/rustorch-nn/src/gqa.rs:37-55), 7-8 KVCacheError
+ * (crates/rustorch-nn/src/kv_cache.rs:229-256); the rest are this library's own. */
+enum rt_status {
+    RT_OK = 0,
+    RT_ERR_ZERO_DIM = 1,                /* AttentionError::ZeroDim */
+    RT_ERR_BUFFER_SHAPE_MISMATCH = 2,   /* AttentionError::BufferShapeMismatch{which,expected,got} */
+    RT_ERR_OUTPUT_SHAPE_MISMATCH = 3,   /* AttentionError::OutputShapeMismatch{expected,got} */
+    RT_ERR_PADDING_LENGTH_MISMATCH = 4, /* AttentionError::Mask(PaddingLengthMismatch{expected,got}) */
+    RT_ERR_HEAD_COUNT_MISMATCH = 5,     /* GQAError::HeadCountMismatch{n_heads=expected,n_kv_heads=got} */
+    RT_ERR_WRONG_INPUT_LEN = 6,         /* GQAError::WrongInputLen{which,expected,got} */
+    RT_ERR_KV_OVERFLOW = 7,             /* KVCacheError::Overflow{requested=got,max=expected} */
+    RT_ERR_KV_WRONG_INPUT_LEN = 8,      /* KVCacheError::WrongInputLen{expected,got_k=got,got_v=got2} */
+    RT_ERR_NULL_POINTER = 20,
+    RT_ERR_UNSUPPORTED = 21,            /* shape outside what the kernels cover; message says which */
+    RT_ERR_WORKSPACE_TOO_SMALL = 22,    /* expected = bytes needed, got = bytes given */
+    RT_ERR_NO_DEVICE = 30,              /* no HIP device, or the device is not gfx950 */
+    RT_ERR_HIP = 31                     /* a HIP call failed; hip_error holds its code */
+};
+
+/* Mask -- crates/rustorch-attention/src/mask.rs:26-46. */
+enum rt_mask_kind {
+    RT_MASK_NONE = 0,
+    RT_MASK_CAUSAL = 1, /* masked iff kj > qi */
+    RT_MASK_PADDING = 2 /* masked iff !keep[kj]; one keep vector of length seq for all batches/heads */
+};
+
+/* `which` of BufferShapeMismatch / WrongInputLen. */
+enum rt_which { RT_WHICH_Q = 0, RT_WHICH_K = 1, RT_WHICH_V = 2, RT_WHICH_OUT = 3, RT_WHICH_FLASH = 4 };
+
+/* Payload of the error enums above.  May be NULL. */
+typedef struct rt_err_detail {
+    int32_t which; /* rt_which, or -1 */
+    uint64_t expected;
+    uint64_t got;
+    uint64_t got2;
+    int32_t hip_error; /* hipError_t when the status is RT_ERR_HIP */
+    char message[160];
+} rt_err_detail;
+
+/* ---- library ------------------------------------------------------------------------------ */
+
+/* Selects `device`, checks that it is gfx950 and warms the kernels' module.  Optional: every
+ * compute entry point does the same lazily on first use (the reference compiles its kernels
+ * lazily behind a OnceLock, crates/rustorch-cuda/src/llm_kernels.rs:578-641). */
+int rt_init(int device, rt_err_detail *err);
+const char *rt_version(void);
+const char *rt_status_name(int status);
+
+/* ---- prefill, host slices ------------------------------------------------------------------- */
+
+/* rustorch_attention::flash_forward -- cpu_forward.rs:175-183. */
+int rt_flash_forward_f32(const rt_attention_shape *shape, const float *q, size_t q_len, const float *k,
+                         size_t k_len, const float *v, size_t v_len, float *out, size_t out_len,
+                         rt_err_detail *err);
+
+/* rustorch_attention::flash_forward_masked -- cpu_forward.rs:193-242.  Check order: ZeroDim,
+ * q, k, v lengths, out length, padding length; seq == 0 returns RT_OK without touching `out`.
+ * A row with no visible key is NaN (cpu_forward.rs:411-420); with RT_MASK_PADDING, when none of
+ * keep[0 .. min(bc, seq)) is set every row is NaN, as the reference's tiled recurrence gives. */
+int rt_flash_forward_masked_f32(const rt_attention_shape *shape, const float *q, size_t q_len, const float *k,
+                                size_t k_len, const float *v, size_t v_len, int mask_kind, const uint8_t *keep,
+                                size_t keep_len, float *out, size_t out_len, rt_err_detail *err);
+
+/* rustorch_nn::gqa::gqa_forward_f32 -- crates/rustorch-nn/src/gqa.rs:94-210.  q/out
+ * [batch,n_heads,seq_q,head_dim], k/v [batch,n_kv_heads,seq_kv,head_dim]; query head h reads kv
+ * head h / (n_heads / n_kv_heads).  seq_q == seq_kv runs the unmasked flash forward (without
+ * materialising the replicated K/V); otherwise unmasked attention of every query row over all
+ * seq_kv keys (the decode branch).  Check order: head counts, then q, k, v, out lengths. */
+int rt_gqa_forward_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len,
+                       float *out, size_t out_len, size_t batch, size_t n_heads, size_t n_kv_heads, size_t seq_q,
+                       size_t seq_kv, size_t head_dim, rt_err_detail *err);
+
+/* ---- prefill, device pointers ---------------------------------------------------------------- */
+
+/* flash_forward_masked on device-resident f32 tensors (same semantics; keep is a device
+ * pointer to `seq` bytes).  n_kv_heads = 0 means n_kv_heads = heads. */
+int rt_flash_forward_f32_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const float *q,
+                             const float *k, const float *v, int mask_kind, const uint8_t *keep, float *out,
+                             rt_err_detail *err);
+
+/* The bf16 counterpart (bf16 in, f32 accumulate, bf16 out rounded once, to nearest even):
+ * q/out [batch,heads,seq,dim], k/v [batch,n_kv_heads,seq,dim].  MFMA kernels cover dim 64 and
+ * 128; other dims return RT_ERR_UNSUPPORTED. */
+int rt_flash_forward_bf16_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const void *q,
+                              const void *k, const void *v, int mask_kind, const uint8_t *keep, void *out,
+                              rt_err_detail *err);
+
+/* Padded-batch causal prefill: sequence b has seq_lens[b] <= seq valid positions (device
+ * int32[batch]); key j of sequence b is masked iff j > i or j >= seq_lens[b].  Valid rows equal
+ * flash_forward_masked(Mask::Causal) on the truncated problem; rows i >= seq_lens[b] are written
+ * as 0 when zero_padded_rows != 0, as NaN (the reference's no-visible-key rule) otherwise.
+ * No counterpart in the reference, whose padding mask is one per-key vector for the whole batch. */
+int rt_flash_forward_varlen_bf16_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads,
+                                     const void *q, const void *k, const void *v, const int32_t *seq_lens,
+                                     int zero_padded_rows, void *out, rt_err_detail *err);
+
+/* ---- decode, device pointers ------------------------------------------------------------------ */
+
+/* LlmKernels::kv_append_bf16 -- crates/rustorch-cuda/src/llm_kernels.rs:353-372, :874-910.
+ * cache[kv_h*max_seq*head_dim + pos*head_dim + i] = in[kv_h*head_dim + i] for K and V. */
+int rt_kv_append_bf16(void *stream, void *k_cache, void *v_cache, const void *k_in, const void *v_in, int32_t pos,
+                      int32_t n_kv, int32_t head_dim, int32_t max_seq, rt_err_detail *err);
+
+/* LlmKernels::gqa_decode_online_bf16 -- llm_kernels.rs:396-457, :915-958.  q/out
+ * [n_heads,head_dim] bf16, caches [n_kv,max_seq,head_dim] bf16 of which [..kv_len] is read;
+ * kv head = h*n_kv/n_heads; f32 accumulation, output rounded once. */
+int rt_gqa_decode_online_bf16(void *stream, const void *q, const void *k_cache, const void *v_cache, void *out,
+                              int32_t n_heads, int32_t n_kv, int32_t kv_len, int32_t head_dim, int32_t max_seq,
+                              rt_err_detail *err);
+
+/* The batched, ragged form of the same call: q/out [batch,n_heads,head_dim], caches
+ * [batch,n_kv,max_seq,head_dim], kv_lens device int32[batch] (sequence b reads [..kv_lens[b]]).
+ * Split-K over the context with a second-pass (m, l, o) merge; `workspace` (device, at least
+ * rt_gqa_decode_workspace_bytes(...) bytes, 256-byte aligned) holds the partial results.
+ * batch = 1 with kv_lens = [kv_len] is the reference call.  A sequence with kv_lens[b] == 0
+ * gives NaN rows (0/0, as crates/rustorch-nn/src/gqa.rs:256 would). */
+int rt_gqa_decode_batched_bf16(void *stream, const void *q, const void *k_cache, const void *v_cache, void *out,
+                               const int32_t *kv_lens, int32_t batch, int32_t n_heads, int32_t n_kv,
+                               int32_t head_dim, int32_t max_seq, void *workspace, size_t workspace_bytes,
+                               rt_err_detail *err);
+size_t rt_gqa_decode_workspace_bytes(int32_t batch, int32_t n_heads, int32_t n_kv, int32_t head_dim,
+                                     int32_t max_seq);
+
+/* ---- device buffers (the slot of Storage::Cuda, crates/rustorch-core/src/tensor/storage.rs:776-817) */
+void *rt_buf_alloc(size_t bytes, rt_err_detail *err);
+int rt_buf_free(void *ptr, rt_err_detail *err);
+int rt_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream, rt_err_detail *err);
+int rt_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream, rt_err_detail *err);
+int rt_stream_synchronize(void *stream, rt_err_detail *err);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RT_ATTN_H */

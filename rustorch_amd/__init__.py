@@ -1,0 +1,16 @@
+"""rustorch_amd: MI355X (gfx950) attention engine behind rustorch's attention call surfaces.
+
+Host mirror of the reference interface (`attention`, `gqa`, `llm_kernels`) over the C ABI of
+librt_attn_hip.so (include/rt_attn.h).  All arithmetic runs in hand-written HIP kernels; there is
+no CPU fallback.
+"""
+from . import _lib
+from .attention import (AttentionShape, Mask, flash_forward, flash_forward_bf16_dev, flash_forward_f32_dev,
+                        flash_forward_masked, flash_forward_varlen_bf16_dev)
+from .device import HipStorage, init, synchronize
+from .errors import (AttentionError, BufferShapeMismatch, DeviceError, GQAError, HeadCountMismatch, KVCacheError,
+                     MaskError, OutputShapeMismatch, Overflow, PaddingLengthMismatch, WrongInputLen, ZeroDim)
+from .gqa import gqa_forward_f32
+from .llm_kernels import LlmKernels
+
+__all__ = [n for n in dir() if not n.startswith("_")]

@@ -1,0 +1,132 @@
+"""Host-side mirror of `rustorch_attention` (crates/rustorch-attention/src/{cpu_forward,mask}.rs)
+over the HIP library: same names, argument meaning and errors; the arithmetic runs on the GPU.
+
+    shape = AttentionShape.new(B, H, N, D)
+    out = flash_forward_masked(shape, q, k, v, Mask.causal())      # numpy f32 in, numpy f32 out
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import _lib as L
+from .device import dev_ptr
+from .errors import raise_for
+
+
+@dataclass
+class AttentionShape:
+    """cpu_forward.rs:49-89."""
+    batch: int
+    heads: int
+    seq: int
+    dim: int
+    br: int = 64
+    bc: int = 64
+
+    @classmethod
+    def new(cls, batch, heads, seq, dim):
+        return cls(batch, heads, seq, dim, 64, 64)
+
+    def buffer_len(self) -> int:
+        return self.batch * self.heads * self.seq * self.dim
+
+    def strides(self):
+        s_n = self.dim
+        s_h = self.seq * s_n
+        return self.heads * s_h, s_h, s_n
+
+    def _c(self):
+        return L.RtShape(self.batch, self.heads, self.seq, self.dim, self.br, self.bc)
+
+
+class Mask:
+    """mask.rs:26-66: Mask::None | Mask::Causal | Mask::Padding(keep)."""
+
+    def __init__(self, kind: int, keep=None):
+        self.kind = kind
+        self.keep = None if keep is None else np.ascontiguousarray(np.asarray(keep, dtype=np.bool_)).view(np.uint8)
+
+    @classmethod
+    def none(cls):
+        return cls(L.RT_MASK_NONE)
+
+    @classmethod
+    def causal(cls):
+        return cls(L.RT_MASK_CAUSAL)
+
+    @classmethod
+    def padding(cls, keep):
+        return cls(L.RT_MASK_PADDING, keep)
+
+    def is_masked(self, qi: int, kj: int) -> bool:
+        if self.kind == L.RT_MASK_CAUSAL:
+            return kj > qi
+        if self.kind == L.RT_MASK_PADDING:
+            return kj < self.keep.size and not self.keep[kj]
+        return False
+
+
+def _f32(a):
+    a = np.ascontiguousarray(np.ravel(a), dtype=np.float32)
+    return a, a.ctypes.data_as(C.POINTER(C.c_float))
+
+
+def flash_forward_masked(shape: AttentionShape, q, k, v, mask: Mask, out=None):
+    """cpu_forward.rs:193-242.  q, k, v: flat f32 [B,H,N,D]; returns (and fills) flat f32 `out`."""
+    q, qp = _f32(q)
+    k, kp = _f32(k)
+    v, vp = _f32(v)
+    if out is None:
+        out = np.zeros(shape.buffer_len(), dtype=np.float32)
+    assert out.dtype == np.float32 and out.flags.c_contiguous
+    keep_p, keep_n = None, 0
+    if mask.kind == L.RT_MASK_PADDING:
+        keep_p, keep_n = mask.keep.ctypes.data_as(C.POINTER(C.c_uint8)), mask.keep.size
+    err = L.RtErr()
+    s = shape._c()
+    rc = L.lib().rt_flash_forward_masked_f32(C.byref(s), qp, q.size, kp, k.size, vp, v.size, mask.kind, keep_p,
+                                             keep_n, out.ctypes.data_as(C.POINTER(C.c_float)), out.size,
+                                             C.byref(err))
+    raise_for(rc, err)
+    return out
+
+
+def flash_forward(shape: AttentionShape, q, k, v, out=None):
+    """cpu_forward.rs:175-183."""
+    return flash_forward_masked(shape, q, k, v, Mask.none(), out)
+
+
+# ---- device-resident tensors (torch GPU tensors, HipStorage, or raw addresses) ---------------------------
+
+
+def flash_forward_f32_dev(shape, q, k, v, out, mask: Mask = None, keep_dev=None, n_kv_heads=0, stream=None):
+    mask = mask or Mask.none()
+    err = L.RtErr()
+    s = shape._c()
+    rc = L.lib().rt_flash_forward_f32_dev(stream, C.byref(s), n_kv_heads, dev_ptr(q), dev_ptr(k), dev_ptr(v),
+                                          mask.kind, dev_ptr(keep_dev), dev_ptr(out), C.byref(err))
+    raise_for(rc, err)
+
+
+def flash_forward_bf16_dev(shape, q, k, v, out, mask: Mask = None, keep_dev=None, n_kv_heads=0, stream=None):
+    """bf16 [B,H,N,D] device tensors; enqueues on `stream` and returns."""
+    mask = mask or Mask.none()
+    err = L.RtErr()
+    s = shape._c()
+    rc = L.lib().rt_flash_forward_bf16_dev(stream, C.byref(s), n_kv_heads, dev_ptr(q), dev_ptr(k), dev_ptr(v),
+                                           mask.kind, dev_ptr(keep_dev), dev_ptr(out), C.byref(err))
+    raise_for(rc, err)
+
+
+def flash_forward_varlen_bf16_dev(shape, q, k, v, seq_lens_dev, out, zero_padded_rows=True, n_kv_heads=0,
+                                  stream=None):
+    """Padded-batch causal prefill: per-sequence valid lengths (device int32[batch])."""
+    err = L.RtErr()
+    s = shape._c()
+    rc = L.lib().rt_flash_forward_varlen_bf16_dev(stream, C.byref(s), n_kv_heads, dev_ptr(q), dev_ptr(k),
+                                                  dev_ptr(v), dev_ptr(seq_lens_dev), int(bool(zero_padded_rows)),
+                                                  dev_ptr(out), C.byref(err))
+    raise_for(rc, err)

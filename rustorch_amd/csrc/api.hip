@@ -1,0 +1,541 @@
+// C ABI of librt_attn_hip.so (declared in include/rt_attn.h): argument checks in the
+// reference's order, device selection, host staging for the slice entry points, kernel dispatch.
+// There is no CPU path in this library.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <mutex>
+
+#include "../../include/rt_attn.h"
+#include "rt_kernels.hpp"
+
+#define RT_API extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+void clear_err(rt_err_detail* e) {
+    if (e) {
+        e->which = -1;
+        e->expected = e->got = e->got2 = 0;
+        e->hip_error = 0;
+        e->message[0] = 0;
+    }
+}
+
+int fail(rt_err_detail* e, int status, int which, uint64_t expected, uint64_t got, const char* msg, uint64_t got2 = 0) {
+    if (e) {
+        e->which = which;
+        e->expected = expected;
+        e->got = got;
+        e->got2 = got2;
+        e->hip_error = 0;
+        snprintf(e->message, sizeof(e->message), "%s", msg ? msg : "");
+    }
+    return status;
+}
+
+int fail_hip(rt_err_detail* e, hipError_t code, const char* where) {
+    if (e) {
+        e->which = -1;
+        e->expected = e->got = e->got2 = 0;
+        e->hip_error = (int32_t)code;
+        snprintf(e->message, sizeof(e->message), "%s: %s", where, hipGetErrorString(code));
+    }
+    return RT_ERR_HIP;
+}
+
+#define HIP_TRY(expr, where)                                  \
+    do {                                                      \
+        hipError_t _e = (expr);                               \
+        if (_e != hipSuccess) return fail_hip(err, _e, where); \
+    } while (0)
+
+std::mutex g_init_mutex;
+int g_init_status = -1;  // -1: not tried
+char g_init_msg[160];
+
+// Finds a gfx950 device once per process.  Never falls back to anything else.
+int ensure_device(rt_err_detail* err, int device = -1) {
+    std::lock_guard<std::mutex> lock(g_init_mutex);
+    if (g_init_status == RT_OK && device < 0) return RT_OK;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0) {
+        (void)hipGetLastError();
+        snprintf(g_init_msg, sizeof(g_init_msg), "no HIP device visible (%s)",
+                 e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+        g_init_status = RT_ERR_NO_DEVICE;
+        return fail(err, RT_ERR_NO_DEVICE, -1, 0, 0, g_init_msg);
+    }
+    int dev = device >= 0 ? device : 0;
+    if (device < 0) (void)hipGetDevice(&dev);
+    if (dev >= count) {
+        snprintf(g_init_msg, sizeof(g_init_msg), "device %d requested, %d visible", dev, count);
+        return fail(err, RT_ERR_NO_DEVICE, -1, (uint64_t)count, (uint64_t)dev, g_init_msg);
+    }
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return fail_hip(err, e, "hipGetDeviceProperties");
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        snprintf(g_init_msg, sizeof(g_init_msg), "device %d is %s; this library holds gfx950 code only", dev,
+                 prop.gcnArchName);
+        g_init_status = RT_ERR_NO_DEVICE;
+        return fail(err, RT_ERR_NO_DEVICE, -1, 0, 0, g_init_msg);
+    }
+    if (device >= 0) {
+        e = hipSetDevice(dev);
+        if (e != hipSuccess) return fail_hip(err, e, "hipSetDevice");
+    }
+    g_init_status = RT_OK;
+    return RT_OK;
+}
+
+// validate() of cpu_forward.rs:142-169 followed by Mask::validate (mask.rs:51-65)
+int validate_flash(const rt_attention_shape* s, size_t qn, size_t kn, size_t vn, size_t on, int mask_kind,
+                   size_t keep_n, rt_err_detail* err) {
+    if (s->dim == 0) return fail(err, RT_ERR_ZERO_DIM, -1, 0, 0, "dim must be > 0");
+    uint64_t expected = s->batch * s->heads * s->seq * s->dim;
+    const size_t lens[3] = {qn, kn, vn};
+    static const char* names[3] = {"q", "k", "v"};
+    for (int i = 0; i < 3; i++)
+        if (lens[i] != expected) {
+            char msg[96];
+            snprintf(msg, sizeof(msg), "%s buffer has %zu elements, expected %llu", names[i], lens[i],
+                     (unsigned long long)expected);
+            return fail(err, RT_ERR_BUFFER_SHAPE_MISMATCH, i, expected, lens[i], msg);
+        }
+    if (on != expected) return fail(err, RT_ERR_OUTPUT_SHAPE_MISMATCH, RT_WHICH_OUT, expected, on, "output buffer length");
+    if (mask_kind == RT_MASK_PADDING && keep_n != s->seq)
+        return fail(err, RT_ERR_PADDING_LENGTH_MISMATCH, -1, s->seq, keep_n, "padding mask length");
+    if (mask_kind != RT_MASK_NONE && mask_kind != RT_MASK_CAUSAL && mask_kind != RT_MASK_PADDING)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, (uint64_t)mask_kind, "unknown mask kind");
+    return RT_OK;
+}
+
+bool fits_int(uint64_t x) { return x <= 0x7fffffffull; }
+
+int check_flash_dims(const rt_attention_shape* s, uint64_t n_kv_heads, rt_err_detail* err) {
+    if (!fits_int(s->batch) || !fits_int(s->heads) || !fits_int(s->seq) || !fits_int(s->dim) || s->batch > 65535 ||
+        s->heads > 65535)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    if (n_kv_heads == 0 || s->heads % n_kv_heads != 0)
+        return fail(err, RT_ERR_HEAD_COUNT_MISMATCH, -1, s->heads, n_kv_heads, "heads not divisible by n_kv_heads");
+    return RT_OK;
+}
+
+int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n_kv_heads, const float* q,
+                     const float* k, const float* v, int mask_kind, const uint8_t* keep, float* out,
+                     rt_err_detail* err) {
+    if (s->dim > 128) return fail(err, RT_ERR_UNSUPPORTED, -1, 128, s->dim, "f32 flash kernel covers dim <= 128");
+    rt::FlashF32Params p;
+    p.q = q;
+    p.k = k;
+    p.v = v;
+    p.out = out;
+    p.keep = keep;
+    p.batch = (int)s->batch;
+    p.heads = (int)s->heads;
+    p.kv_heads = (int)n_kv_heads;
+    p.group = (int)(s->heads / n_kv_heads);
+    p.seq = (int)s->seq;
+    p.dim = (int)s->dim;
+    p.mask = mask_kind;
+    p.ref_bc = (int)(s->bc == 0 ? 1 : (s->bc > 0x7fffffffull ? 0x7fffffff : s->bc));
+    p.scale = 1.0f / sqrtf((float)s->dim);
+    HIP_TRY(rt::launch_flash_f32(stream, p), "flash_fwd_f32 launch");
+    return RT_OK;
+}
+
+struct DevBuf {
+    void* p = nullptr;
+    ~DevBuf() {
+        if (p) (void)hipFree(p);
+    }
+};
+
+}  // namespace
+
+RT_API const char* rt_version(void) { return "rt_attn_hip 0.1 (gfx950)"; }
+
+RT_API const char* rt_status_name(int status) {
+    switch (status) {
+        case RT_OK: return "Ok";
+        case RT_ERR_ZERO_DIM: return "ZeroDim";
+        case RT_ERR_BUFFER_SHAPE_MISMATCH: return "BufferShapeMismatch";
+        case RT_ERR_OUTPUT_SHAPE_MISMATCH: return "OutputShapeMismatch";
+        case RT_ERR_PADDING_LENGTH_MISMATCH: return "PaddingLengthMismatch";
+        case RT_ERR_HEAD_COUNT_MISMATCH: return "HeadCountMismatch";
+        case RT_ERR_WRONG_INPUT_LEN: return "WrongInputLen";
+        case RT_ERR_KV_OVERFLOW: return "Overflow";
+        case RT_ERR_KV_WRONG_INPUT_LEN: return "KvWrongInputLen";
+        case RT_ERR_NULL_POINTER: return "NullPointer";
+        case RT_ERR_UNSUPPORTED: return "Unsupported";
+        case RT_ERR_WORKSPACE_TOO_SMALL: return "WorkspaceTooSmall";
+        case RT_ERR_NO_DEVICE: return "NoDeviceFound";
+        case RT_ERR_HIP: return "Driver";
+        default: return "Unknown";
+    }
+}
+
+RT_API int rt_init(int device, rt_err_detail* err) {
+    clear_err(err);
+    return ensure_device(err, device < 0 ? 0 : device);
+}
+
+// ---- prefill, host slices -------------------------------------------------------------------------
+
+RT_API int rt_flash_forward_masked_f32(const rt_attention_shape* shape, const float* q, size_t q_len, const float* k,
+                                       size_t k_len, const float* v, size_t v_len, int mask_kind,
+                                       const uint8_t* keep, size_t keep_len, float* out, size_t out_len,
+                                       rt_err_detail* err) {
+    clear_err(err);
+    if (!shape) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "shape is NULL");
+    int rc = validate_flash(shape, q_len, k_len, v_len, out_len, mask_kind, keep_len, err);
+    if (rc) return rc;
+    if (shape->seq == 0) return RT_OK;  // cpu_forward.rs:203-206
+    size_t n = q_len;
+    if (n == 0) return RT_OK;  // batch or heads is 0
+    if (!q || !k || !v || !out || (mask_kind == RT_MASK_PADDING && !keep))
+        return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    rc = check_flash_dims(shape, shape->heads, err);
+    if (rc) return rc;
+    rc = ensure_device(err);
+    if (rc) return rc;
+
+    DevBuf dq, dk, dv, dout, dkeep;
+    size_t bytes = n * sizeof(float);
+    HIP_TRY(hipMalloc(&dq.p, bytes), "hipMalloc q");
+    HIP_TRY(hipMalloc(&dk.p, bytes), "hipMalloc k");
+    HIP_TRY(hipMalloc(&dv.p, bytes), "hipMalloc v");
+    HIP_TRY(hipMalloc(&dout.p, bytes), "hipMalloc out");
+    HIP_TRY(hipMemcpy(dq.p, q, bytes, hipMemcpyHostToDevice), "copy q");
+    HIP_TRY(hipMemcpy(dk.p, k, bytes, hipMemcpyHostToDevice), "copy k");
+    HIP_TRY(hipMemcpy(dv.p, v, bytes, hipMemcpyHostToDevice), "copy v");
+    if (mask_kind == RT_MASK_PADDING) {
+        HIP_TRY(hipMalloc(&dkeep.p, keep_len), "hipMalloc keep");
+        HIP_TRY(hipMemcpy(dkeep.p, keep, keep_len, hipMemcpyHostToDevice), "copy keep");
+    }
+    rc = flash_f32_device(nullptr, shape, shape->heads, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p,
+                          mask_kind, (const uint8_t*)dkeep.p, (float*)dout.p, err);
+    if (rc) return rc;
+    HIP_TRY(hipMemcpy(out, dout.p, bytes, hipMemcpyDeviceToHost), "copy out");
+    return RT_OK;
+}
+
+RT_API int rt_flash_forward_f32(const rt_attention_shape* shape, const float* q, size_t q_len, const float* k,
+                                size_t k_len, const float* v, size_t v_len, float* out, size_t out_len,
+                                rt_err_detail* err) {
+    return rt_flash_forward_masked_f32(shape, q, q_len, k, k_len, v, v_len, RT_MASK_NONE, nullptr, 0, out, out_len,
+                                       err);
+}
+
+RT_API int rt_gqa_forward_f32(const float* q, size_t q_len, const float* k, size_t k_len, const float* v,
+                              size_t v_len, float* out, size_t out_len, size_t batch, size_t n_heads,
+                              size_t n_kv_heads, size_t seq_q, size_t seq_kv, size_t head_dim, rt_err_detail* err) {
+    clear_err(err);
+    // gqa.rs:106-141
+    if (n_kv_heads == 0 || n_heads % n_kv_heads != 0)
+        return fail(err, RT_ERR_HEAD_COUNT_MISMATCH, -1, n_heads, n_kv_heads, "n_heads not divisible by n_kv_heads");
+    size_t q_expected = batch * n_heads * seq_q * head_dim;
+    size_t kv_expected = batch * n_kv_heads * seq_kv * head_dim;
+    if (q_len != q_expected) return fail(err, RT_ERR_WRONG_INPUT_LEN, RT_WHICH_Q, q_expected, q_len, "q length");
+    if (k_len != kv_expected) return fail(err, RT_ERR_WRONG_INPUT_LEN, RT_WHICH_K, kv_expected, k_len, "k length");
+    if (v_len != kv_expected) return fail(err, RT_ERR_WRONG_INPUT_LEN, RT_WHICH_V, kv_expected, v_len, "v length");
+    if (out_len != q_expected) return fail(err, RT_ERR_WRONG_INPUT_LEN, RT_WHICH_OUT, q_expected, out_len, "out length");
+    if (seq_q == seq_kv && head_dim == 0)
+        // the prefill branch's flash_forward fails with ZeroDim, reported as WrongInputLen{"flash_forward",0,0} (gqa.rs:171-175)
+        return fail(err, RT_ERR_WRONG_INPUT_LEN, RT_WHICH_FLASH, 0, 0, "flash_forward");
+    if (q_expected == 0) return RT_OK;
+    if (!q || !out || (kv_expected && (!k || !v))) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    if (!fits_int(batch) || !fits_int(n_heads) || !fits_int(seq_q) || !fits_int(seq_kv) || !fits_int(head_dim) ||
+        batch > 65535 || n_heads > 65535)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    int rc = ensure_device(err);
+    if (rc) return rc;
+
+    DevBuf dq, dk, dv, dout;
+    HIP_TRY(hipMalloc(&dq.p, q_expected * 4), "hipMalloc q");
+    HIP_TRY(hipMalloc(&dout.p, q_expected * 4), "hipMalloc out");
+    HIP_TRY(hipMalloc(&dk.p, kv_expected ? kv_expected * 4 : 4), "hipMalloc k");
+    HIP_TRY(hipMalloc(&dv.p, kv_expected ? kv_expected * 4 : 4), "hipMalloc v");
+    HIP_TRY(hipMemcpy(dq.p, q, q_expected * 4, hipMemcpyHostToDevice), "copy q");
+    if (kv_expected) {
+        HIP_TRY(hipMemcpy(dk.p, k, kv_expected * 4, hipMemcpyHostToDevice), "copy k");
+        HIP_TRY(hipMemcpy(dv.p, v, kv_expected * 4, hipMemcpyHostToDevice), "copy v");
+    }
+    if (seq_q == seq_kv) {
+        // prefill: unmasked flash; the kernel maps query head -> kv head itself (no replicated copy)
+        rt_attention_shape s = {batch, n_heads, seq_q, head_dim, 64, 64};
+        rc = flash_f32_device(nullptr, &s, n_kv_heads, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p,
+                              RT_MASK_NONE, nullptr, (float*)dout.p, err);
+        if (rc) return rc;
+    } else {
+        if (head_dim > 512) return fail(err, RT_ERR_UNSUPPORTED, -1, 512, head_dim, "decode rows kernel covers dim <= 512");
+        if (seq_q > 65535 * 32ull) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, seq_q, "seq_q too large");
+        rt::AttnRowsParams p;
+        p.q = dq.p;
+        p.k = dk.p;
+        p.v = dv.p;
+        p.out = dout.p;
+        p.kv_lens = nullptr;
+        p.batch = (int)batch;
+        p.heads = (int)n_heads;
+        p.kv_heads = (int)n_kv_heads;
+        p.seq_q = (int)seq_q;
+        p.kv_len = (int)seq_kv;
+        p.kv_stride = (int)seq_kv;
+        p.dim = (int)head_dim;
+        p.head_map = 0;
+        p.scale = 1.0f / sqrtf((float)head_dim);
+        HIP_TRY(rt::launch_attn_rows_f32(nullptr, p), "attn_rows_f32 launch");
+    }
+    HIP_TRY(hipMemcpy(out, dout.p, q_expected * 4, hipMemcpyDeviceToHost), "copy out");
+    return RT_OK;
+}
+
+// ---- prefill, device pointers -----------------------------------------------------------------------
+
+RT_API int rt_flash_forward_f32_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,
+                                    const float* q, const float* k, const float* v, int mask_kind,
+                                    const uint8_t* keep, float* out, rt_err_detail* err) {
+    clear_err(err);
+    if (!shape) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "shape is NULL");
+    if (shape->dim == 0) return fail(err, RT_ERR_ZERO_DIM, -1, 0, 0, "dim must be > 0");
+    if (mask_kind < RT_MASK_NONE || mask_kind > RT_MASK_PADDING)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, (uint64_t)mask_kind, "unknown mask kind");
+    if (n_kv_heads == 0) n_kv_heads = shape->heads;
+    if (shape->seq == 0 || shape->batch == 0 || shape->heads == 0) return RT_OK;
+    int rc = check_flash_dims(shape, n_kv_heads, err);
+    if (rc) return rc;
+    if (!q || !k || !v || !out || (mask_kind == RT_MASK_PADDING && !keep))
+        return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    rc = ensure_device(err);
+    if (rc) return rc;
+    return flash_f32_device((hipStream_t)stream, shape, n_kv_heads, q, k, v, mask_kind, keep, out, err);
+}
+
+static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads, const void* q,
+                             const void* k, const void* v, int mask, const uint8_t* keep, const int32_t* seq_lens,
+                             int zero_padded_rows, void* out, rt_err_detail* err) {
+    clear_err(err);
+    if (!shape) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "shape is NULL");
+    if (shape->dim == 0) return fail(err, RT_ERR_ZERO_DIM, -1, 0, 0, "dim must be > 0");
+    if (n_kv_heads == 0) n_kv_heads = shape->heads;
+    if (shape->seq == 0 || shape->batch == 0 || shape->heads == 0) return RT_OK;
+    int rc = check_flash_dims(shape, n_kv_heads, err);
+    if (rc) return rc;
+    if (shape->dim != 64 && shape->dim != 128)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 128, shape->dim, "bf16 flash kernels cover dim 64 and 128");
+    if ((shape->seq + 127) / 128 * shape->batch * shape->heads > 0x7fffffffull)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    if (!q || !k || !v || !out || (mask == rt::kMaskPadding && !keep) || (mask == rt::kMaskVarlenCausal && !seq_lens))
+        return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    rc = ensure_device(err);
+    if (rc) return rc;
+    rt::FlashBf16Params p;
+    p.q = (const uint16_t*)q;
+    p.k = (const uint16_t*)k;
+    p.v = (const uint16_t*)v;
+    p.out = (uint16_t*)out;
+    p.keep = keep;
+    p.seq_lens = seq_lens;
+    p.batch = (int)shape->batch;
+    p.heads = (int)shape->heads;
+    p.kv_heads = (int)n_kv_heads;
+    p.group = (int)(shape->heads / n_kv_heads);
+    p.seq = (int)shape->seq;
+    p.dim = (int)shape->dim;
+    p.mask = mask;
+    p.ref_bc = (int)(shape->bc == 0 ? 1 : (shape->bc > 0x7fffffffull ? 0x7fffffff : shape->bc));
+    p.zero_padded_rows = zero_padded_rows;
+    p.scale_log2e = (1.0f / sqrtf((float)shape->dim)) * rt::kLog2eHost;
+    HIP_TRY(rt::launch_flash_bf16((hipStream_t)stream, p), "flash_fwd_bf16 launch");
+    return RT_OK;
+}
+
+RT_API int rt_flash_forward_bf16_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,
+                                     const void* q, const void* k, const void* v, int mask_kind, const uint8_t* keep,
+                                     void* out, rt_err_detail* err) {
+    if (mask_kind < RT_MASK_NONE || mask_kind > RT_MASK_PADDING) {
+        clear_err(err);
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, (uint64_t)mask_kind, "unknown mask kind");
+    }
+    return flash_bf16_common(stream, shape, n_kv_heads, q, k, v, mask_kind, keep, nullptr, 0, out, err);
+}
+
+RT_API int rt_flash_forward_varlen_bf16_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,
+                                            const void* q, const void* k, const void* v, const int32_t* seq_lens,
+                                            int zero_padded_rows, void* out, rt_err_detail* err) {
+    return flash_bf16_common(stream, shape, n_kv_heads, q, k, v, rt::kMaskVarlenCausal, nullptr, seq_lens,
+                             zero_padded_rows, out, err);
+}
+
+// ---- decode, device pointers -------------------------------------------------------------------------
+
+RT_API int rt_kv_append_bf16(void* stream, void* k_cache, void* v_cache, const void* k_in, const void* v_in,
+                             int32_t pos, int32_t n_kv, int32_t head_dim, int32_t max_seq, rt_err_detail* err) {
+    clear_err(err);
+    if (n_kv < 0 || head_dim < 0 || max_seq < 0) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "negative dimension");
+    if (pos < 0 || pos >= max_seq)
+        return fail(err, RT_ERR_KV_OVERFLOW, -1, (uint64_t)max_seq, (uint64_t)(int64_t)pos + 1, "position outside the cache");
+    if (n_kv == 0 || head_dim == 0) return RT_OK;
+    if (!k_cache || !v_cache || !k_in || !v_in) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    int rc = ensure_device(err);
+    if (rc) return rc;
+    HIP_TRY(rt::launch_kv_append_bf16((hipStream_t)stream, (uint16_t*)k_cache, (uint16_t*)v_cache,
+                                      (const uint16_t*)k_in, (const uint16_t*)v_in, pos, n_kv, head_dim, max_seq),
+            "kv_append_bf16 launch");
+    return RT_OK;
+}
+
+static int check_decode_dims(int32_t batch, int32_t n_heads, int32_t n_kv, int32_t head_dim, int32_t max_seq,
+                             rt_err_detail* err) {
+    if (batch < 0 || n_heads < 0 || n_kv < 0 || head_dim < 0 || max_seq < 0)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "negative dimension");
+    if (n_kv == 0 || n_heads % n_kv != 0)
+        return fail(err, RT_ERR_HEAD_COUNT_MISMATCH, -1, (uint64_t)n_heads, (uint64_t)n_kv,
+                    "n_heads not divisible by n_kv");
+    if (head_dim == 0) return fail(err, RT_ERR_ZERO_DIM, -1, 0, 0, "head_dim must be > 0");
+    if (batch > 65535 || n_heads > 65535) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    return RT_OK;
+}
+
+RT_API int rt_gqa_decode_online_bf16(void* stream, const void* q, const void* k_cache, const void* v_cache,
+                                     void* out, int32_t n_heads, int32_t n_kv, int32_t kv_len, int32_t head_dim,
+                                     int32_t max_seq, rt_err_detail* err) {
+    clear_err(err);
+    int rc = check_decode_dims(1, n_heads, n_kv, head_dim, max_seq, err);
+    if (rc) return rc;
+    if (kv_len < 0 || kv_len > max_seq)
+        return fail(err, RT_ERR_KV_OVERFLOW, -1, (uint64_t)max_seq, (uint64_t)(int64_t)kv_len, "kv_len outside the cache");
+    if (n_heads == 0) return RT_OK;
+    if (head_dim > 512) return fail(err, RT_ERR_UNSUPPORTED, -1, 512, (uint64_t)head_dim, "decode rows kernel covers dim <= 512");
+    if (!q || !out || (kv_len > 0 && (!k_cache || !v_cache))) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    rc = ensure_device(err);
+    if (rc) return rc;
+    rt::AttnRowsParams p;
+    p.q = q;
+    p.k = k_cache;
+    p.v = v_cache;
+    p.out = out;
+    p.kv_lens = nullptr;
+    p.batch = 1;
+    p.heads = n_heads;
+    p.kv_heads = n_kv;
+    p.seq_q = 1;
+    p.kv_len = kv_len;
+    p.kv_stride = max_seq;
+    p.dim = head_dim;
+    p.head_map = 1;
+    p.scale = 1.0f / sqrtf((float)head_dim);
+    HIP_TRY(rt::launch_attn_rows_bf16((hipStream_t)stream, p), "attn_rows_bf16 launch");
+    return RT_OK;
+}
+
+RT_API size_t rt_gqa_decode_workspace_bytes(int32_t batch, int32_t n_heads, int32_t n_kv, int32_t head_dim,
+                                            int32_t max_seq) {
+    if (batch <= 0 || n_heads <= 0 || n_kv <= 0 || head_dim <= 0 || max_seq < 0) return 0;
+    if (!rt::decode_split_supported(n_heads, n_kv, head_dim)) return 0;
+    return rt::decode_split_workspace_bytes(batch, n_heads, head_dim, max_seq);
+}
+
+RT_API int rt_gqa_decode_batched_bf16(void* stream, const void* q, const void* k_cache, const void* v_cache,
+                                      void* out, const int32_t* kv_lens, int32_t batch, int32_t n_heads,
+                                      int32_t n_kv, int32_t head_dim, int32_t max_seq, void* workspace,
+                                      size_t workspace_bytes, rt_err_detail* err) {
+    clear_err(err);
+    int rc = check_decode_dims(batch, n_heads, n_kv, head_dim, max_seq, err);
+    if (rc) return rc;
+    if (batch == 0 || n_heads == 0) return RT_OK;
+    if (!q || !out || !kv_lens || (max_seq > 0 && (!k_cache || !v_cache)))
+        return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    rc = ensure_device(err);
+    if (rc) return rc;
+    if (rt::decode_split_supported(n_heads, n_kv, head_dim)) {
+        size_t need = rt::decode_split_workspace_bytes(batch, n_heads, head_dim, max_seq);
+        if (!workspace || workspace_bytes < need)
+            return fail(err, RT_ERR_WORKSPACE_TOO_SMALL, -1, need, workspace ? workspace_bytes : 0, "workspace too small");
+        rt::DecodeSplitParams p;
+        p.q = (const uint16_t*)q;
+        p.k_cache = (const uint16_t*)k_cache;
+        p.v_cache = (const uint16_t*)v_cache;
+        p.out = (uint16_t*)out;
+        p.kv_lens = kv_lens;
+        p.ws = (float*)workspace;
+        p.batch = batch;
+        p.heads = n_heads;
+        p.kv_heads = n_kv;
+        p.dim = head_dim;
+        p.max_seq = max_seq;
+        p.chunk = rt::decode_split_chunk(max_seq);
+        p.n_chunks = (max_seq + p.chunk - 1) / p.chunk;
+        if (p.n_chunks == 0) p.n_chunks = 1;
+        p.scale_log2e = (1.0f / sqrtf((float)head_dim)) * rt::kLog2eHost;
+        HIP_TRY(rt::launch_decode_split((hipStream_t)stream, p), "decode_split launch");
+        return RT_OK;
+    }
+    // shapes outside the split-K kernel: one workgroup per (sequence, head), no workspace
+    if (head_dim > 512) return fail(err, RT_ERR_UNSUPPORTED, -1, 512, (uint64_t)head_dim, "decode rows kernel covers dim <= 512");
+    rt::AttnRowsParams p;
+    p.q = q;
+    p.k = k_cache;
+    p.v = v_cache;
+    p.out = out;
+    p.kv_lens = kv_lens;
+    p.batch = batch;
+    p.heads = n_heads;
+    p.kv_heads = n_kv;
+    p.seq_q = 1;
+    p.kv_len = 0;
+    p.kv_stride = max_seq;
+    p.dim = head_dim;
+    p.head_map = 1;
+    p.scale = 1.0f / sqrtf((float)head_dim);
+    HIP_TRY(rt::launch_attn_rows_bf16((hipStream_t)stream, p), "attn_rows_bf16 launch");
+    return RT_OK;
+}
+
+// ---- device buffers ------------------------------------------------------------------------------------
+
+RT_API void* rt_buf_alloc(size_t bytes, rt_err_detail* err) {
+    clear_err(err);
+    if (ensure_device(err) != RT_OK) return nullptr;
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+    if (e != hipSuccess) {
+        fail_hip(err, e, "hipMalloc");
+        return nullptr;
+    }
+    return p;
+}
+
+RT_API int rt_buf_free(void* ptr, rt_err_detail* err) {
+    clear_err(err);
+    if (!ptr) return RT_OK;
+    HIP_TRY(hipFree(ptr), "hipFree");
+    return RT_OK;
+}
+
+RT_API int rt_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream, rt_err_detail* err) {
+    clear_err(err);
+    if (bytes == 0) return RT_OK;
+    if (!dst || !src) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream), "hipMemcpyAsync h2d");
+    return RT_OK;
+}
+
+RT_API int rt_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream, rt_err_detail* err) {
+    clear_err(err);
+    if (bytes == 0) return RT_OK;
+    if (!dst || !src) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream), "hipMemcpyAsync d2h");
+    return RT_OK;
+}
+
+RT_API int rt_stream_synchronize(void* stream, rt_err_detail* err) {
+    clear_err(err);
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
+    return RT_OK;
+}

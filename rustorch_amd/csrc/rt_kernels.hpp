@@ -1,0 +1,79 @@
+// Kernel parameter blocks and launchers shared between the kernel files and the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rt {
+
+// 0..2 are rt_mask_kind of the C ABI; 3 is the padded-batch mode (per-sequence length + causal).
+enum MaskKind : int { kMaskNone = 0, kMaskCausal = 1, kMaskPadding = 2, kMaskVarlenCausal = 3 };
+constexpr float kLog2eHost = 1.4426950408889634f;
+
+struct FlashF32Params {
+    const float* q;
+    const float* k;
+    const float* v;
+    float* out;
+    const uint8_t* keep;  // device, `seq` bytes, for kMaskPadding
+    int batch, heads, kv_heads, group;
+    int seq, dim;
+    int mask;
+    int ref_bc;  // the reference's key-tile size, for the leading-masked-tile rule
+    float scale;
+};
+// dim <= 128.  Returns hipErrorInvalidValue for an unsupported dim.
+hipError_t launch_flash_f32(hipStream_t stream, const FlashF32Params& p);
+
+struct FlashBf16Params {
+    const uint16_t* q;
+    const uint16_t* k;
+    const uint16_t* v;
+    uint16_t* out;
+    const uint8_t* keep;      // kMaskPadding
+    const int32_t* seq_lens;  // kMaskVarlenCausal: device int32[batch]
+    int batch, heads, kv_heads, group;
+    int seq, dim;
+    int mask;
+    int ref_bc;
+    int zero_padded_rows;
+    float scale_log2e;  // (1/sqrt(dim)) * log2(e)
+};
+// dim in {64, 128}.
+hipError_t launch_flash_bf16(hipStream_t stream, const FlashBf16Params& p);
+
+// Unmasked attention of every query row over all keys; generic in dim (<= 512), head
+// grouping, kv_len and query count.  T is float or uint16_t (bf16 bits).
+struct AttnRowsParams {
+    const void* q;    // [batch, heads, seq_q, dim]
+    const void* k;    // [batch, kv_heads, kv_stride, dim]
+    const void* v;
+    void* out;        // [batch, heads, seq_q, dim]
+    const int32_t* kv_lens;  // device int32[batch] or nullptr (then kv_len)
+    int batch, heads, kv_heads;
+    int seq_q, kv_len, kv_stride, dim;
+    int head_map;  // 0: kv_h = h / (heads/kv_heads) (gqa.rs:233); 1: kv_h = h*kv_heads/heads (llm_kernels.rs:410)
+    float scale;
+};
+hipError_t launch_attn_rows_f32(hipStream_t stream, const AttnRowsParams& p);
+hipError_t launch_attn_rows_bf16(hipStream_t stream, const AttnRowsParams& p);
+
+struct DecodeSplitParams {
+    const uint16_t* q;        // [batch, heads, dim]
+    const uint16_t* k_cache;  // [batch, kv_heads, max_seq, dim]
+    const uint16_t* v_cache;
+    uint16_t* out;            // [batch, heads, dim]
+    const int32_t* kv_lens;   // device int32[batch]
+    float* ws;                // partial (o, m, l) per (b, head, chunk)
+    int batch, heads, kv_heads, dim, max_seq;
+    int chunk, n_chunks;
+    float scale_log2e;
+};
+bool decode_split_supported(int heads, int kv_heads, int dim);
+int decode_split_chunk(int max_seq);
+size_t decode_split_workspace_bytes(int batch, int heads, int dim, int max_seq);
+hipError_t launch_decode_split(hipStream_t stream, const DecodeSplitParams& p);
+
+hipError_t launch_kv_append_bf16(hipStream_t stream, uint16_t* k_cache, uint16_t* v_cache, const uint16_t* k_in,
+                                 const uint16_t* v_in, int pos, int n_kv, int head_dim, int max_seq);
+
+}  // namespace rt

@@ -1,0 +1,135 @@
+"""GPU parity of the decode path through the C ABI (rt_kv_append_bf16, rt_gqa_decode_online_bf16,
+rt_gqa_decode_batched_bf16) against the CPU oracle.  Bar: max-abs <= 2e-2 vs the f32 CPU path on
+the same bf16-rounded inputs."""
+import numpy as np
+import pytest
+
+import rustorch_amd as ra
+from _gpu import bf16_round, dev, max_abs
+from _util import seeded_normal
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+K = ra.LlmKernels()
+
+
+def test_kv_append_bf16_matches_oracle(oracle):
+    n_kv, d, max_seq = 8, 128, 33
+    kc = np.random.default_rng(1).integers(0, 2 ** 16, n_kv * max_seq * d).astype(np.uint16)
+    vc = np.random.default_rng(2).integers(0, 2 ** 16, n_kv * max_seq * d).astype(np.uint16)
+    dk, dv = dev(kc), dev(vc)
+    for pos in (0, 17, 32):
+        k_in = np.random.default_rng(pos).integers(0, 2 ** 16, n_kv * d).astype(np.uint16)
+        v_in = np.random.default_rng(pos + 100).integers(0, 2 ** 16, n_kv * d).astype(np.uint16)
+        K.kv_append_bf16(None, dk, dv, dev(k_in), dev(v_in), pos, n_kv, d, max_seq)
+        oracle.kv_append_bf16(kc, vc, k_in, v_in, pos, n_kv, d, max_seq)
+    ra.synchronize()
+    assert np.array_equal(dk.download(np.uint16), kc) and np.array_equal(dv.download(np.uint16), vc)
+    with pytest.raises(ra.Overflow):
+        K.kv_append_bf16(None, dk, dv, dk, dv, max_seq, n_kv, d, max_seq)
+
+
+@pytest.mark.parametrize("hq,hkv,d,max_seq,kv_len", [(8, 2, 32, 320, 1), (8, 2, 32, 320, 77), (32, 8, 128, 600, 600),
+                                                     (6, 3, 96, 50, 49), (4, 4, 256, 40, 40), (8, 2, 64, 10, 0)])
+def test_gqa_decode_online_bf16_matches_oracle(oracle, hq, hkv, d, max_seq, kv_len):
+    """The reference call (batch 1): compared with the restated device kernel (bf16 out) and with
+    the CPU path in f32."""
+    qb, qf = bf16_round(seeded_normal((hq, d), 1))
+    kb, kf = bf16_round(seeded_normal((hkv, max_seq, d), 2))
+    vb, vf = bf16_round(seeded_normal((hkv, max_seq, d), 3))
+    dout = ra.HipStorage(hq * d * 2)
+    dout.upload(np.full(hq * d, 0x7B7B, dtype=np.uint16))
+    K.gqa_decode_online_bf16(None, dev(qb), dev(kb), dev(vb), dout, hq, hkv, kv_len, d, max_seq)
+    ra.synchronize()
+    got = oracle.bf16_to_f32(dout.download(np.uint16))
+    want_dev = oracle.bf16_to_f32(oracle.gqa_decode_online_bf16(qb, kb, vb, hq, hkv, kv_len, d, max_seq))
+    assert max_abs(got, want_dev) <= TOL
+    want_cpu = oracle.gqa_decode_batched_bf16(qb, kb, vb, [kv_len], 1, hq, hkv, d, max_seq)
+    assert max_abs(got, want_cpu) <= TOL
+    if kv_len == 1:
+        g = hq // hkv
+        assert np.array_equal(got.reshape(hq, d), np.repeat(vf.reshape(hkv, max_seq, d)[:, 0], g, axis=0))
+    if kv_len == 0:
+        assert (got == 0).all()
+
+
+def run_batched(oracle, qb, kb, vb, lens, b, hq, hkv, d, max_seq):
+    ws_bytes = K.gqa_decode_workspace_bytes(b, hq, hkv, d, max_seq)
+    ws = ra.HipStorage(max(ws_bytes, 256))
+    dout = ra.HipStorage(b * hq * d * 2)
+    dout.upload(np.full(b * hq * d, 0x7B7B, dtype=np.uint16))
+    K.gqa_decode_batched_bf16(None, dev(qb), dev(kb), dev(vb), dout, dev(np.asarray(lens, dtype=np.int32)), b, hq,
+                              hkv, d, max_seq, ws, ws.byte_len)
+    ra.synchronize()
+    return oracle.bf16_to_f32(dout.download(np.uint16))
+
+
+@pytest.mark.parametrize("b,hq,hkv,d,max_seq,lens", [
+    (5, 32, 8, 128, 1100, [1, 511, 512, 513, 1100]),
+    (3, 8, 8, 64, 700, [700, 0, 33]),
+    (2, 8, 1, 128, 1500, [1500, 1023]),
+    (2, 16, 8, 64, 300, [300, 17]),
+    (2, 6, 2, 128, 100, [100, 50]),   # group of 3: outside the split-K kernel, generic path
+    (2, 4, 2, 96, 100, [100, 50]),    # head dim 96: generic path
+])
+def test_gqa_decode_batched_matches_oracle(oracle, b, hq, hkv, d, max_seq, lens):
+    qb, qf = bf16_round(seeded_normal((b, hq, d), 1))
+    kb, kf = bf16_round(seeded_normal((b, hkv, max_seq, d), 2))
+    vb, vf = bf16_round(seeded_normal((b, hkv, max_seq, d), 3))
+    got = run_batched(oracle, qb, kb, vb, lens, b, hq, hkv, d, max_seq)
+    want = oracle.gqa_decode_batched_bf16(qb, kb, vb, lens, b, hq, hkv, d, max_seq)
+    assert np.isfinite(got).all()
+    assert max_abs(got, want) <= TOL
+    g4 = got.reshape(b, hq, d)
+    v4 = vf.reshape(b, hkv, max_seq, d)
+    for i, L in enumerate(lens):
+        if L == 1:  # one key: out == v_0 exactly
+            assert np.array_equal(g4[i], np.repeat(v4[i, :, 0], hq // hkv, axis=0))
+        if L == 0:
+            assert (g4[i] == 0).all()
+
+
+def test_decode_split_equals_unsplit(oracle):
+    """Split-K invariance: the batched (chunked) path and the single-pass reference call agree for
+    lengths on both sides of every chunk boundary."""
+    hq, hkv, d, max_seq = 8, 2, 128, 2100
+    qb, _ = bf16_round(seeded_normal((1, hq, d), 1))
+    kb, _ = bf16_round(seeded_normal((1, hkv, max_seq, d), 2))
+    vb, _ = bf16_round(seeded_normal((1, hkv, max_seq, d), 3))
+    dq, dk, dv = dev(qb), dev(kb), dev(vb)
+    for L in (511, 512, 513, 1024, 1025, 2047, 2100):
+        split = run_batched(oracle, qb, kb, vb, [L], 1, hq, hkv, d, max_seq)
+        dout = ra.HipStorage(hq * d * 2)
+        K.gqa_decode_online_bf16(None, dq, dk, dv, dout, hq, hkv, L, d, max_seq)
+        ra.synchronize()
+        one = oracle.bf16_to_f32(dout.download(np.uint16))
+        assert max_abs(split, one) <= 2 ** -7 * np.abs(one).max() + 1e-6, L
+
+
+def test_decode_workspace_too_small_is_an_error():
+    b, hq, hkv, d, max_seq = 2, 8, 2, 128, 1024
+    z = ra.HipStorage(b * hkv * max_seq * d * 2)
+    lens = dev(np.array([5, 5], dtype=np.int32))
+    with pytest.raises(ra.DeviceError) as ei:
+        K.gqa_decode_batched_bf16(None, z, z, z, z, lens, b, hq, hkv, d, max_seq, z, 16)
+    assert ei.value.status == 22 and ei.value.expected == K.gqa_decode_workspace_bytes(b, hq, hkv, d, max_seq)
+
+
+def test_config_decode_b64_h32_kv8_d128_lmax8192(oracle):
+    """BASELINE configs[3] at full size: lengths uniform in [512, 8192] from a seed, N(0,1) bf16
+    caches in the contiguous (B, Hkv, Lmax, D) layout."""
+    b, hq, hkv, d, max_seq = 64, 32, 8, 128, 8192
+    lens = np.random.default_rng(4).integers(512, 8193, size=b).astype(np.int32)
+    rng = np.random.default_rng(44)
+    n_cache = b * hkv * max_seq * d
+    kb = np.empty(n_cache, dtype=np.uint16)
+    vb = np.empty(n_cache, dtype=np.uint16)
+    step = n_cache // 16
+    for i in range(16):  # generate in slices to bound host memory
+        kb[i * step:(i + 1) * step] = oracle.f32_to_bf16(rng.standard_normal(step, dtype=np.float32))
+        vb[i * step:(i + 1) * step] = oracle.f32_to_bf16(rng.standard_normal(step, dtype=np.float32))
+    qb, _ = bf16_round(seeded_normal((b, hq, d), 1))
+    got = run_batched(oracle, qb, kb, vb, lens, b, hq, hkv, d, max_seq)
+    want = oracle.gqa_decode_batched_bf16(qb, kb, vb, lens, b, hq, hkv, d, max_seq)
+    assert np.isfinite(got).all()
+    assert max_abs(got, want) <= TOL, f"lens={lens.tolist()}"

@@ -1,0 +1,225 @@
+"""GPU parity of the f32 prefill path through the C ABI (rt_flash_forward[_masked]_f32,
+rt_gqa_forward_f32) against the CPU oracle.  Bar: max-abs <= 1e-5, NaN patterns exact.  The cases
+are the reference's own (cpu_forward.rs:804-1087, tests/equivalence.rs, gqa.rs:278-388)."""
+import numpy as np
+import pytest
+
+import rustorch_amd as ra
+from _gpu import assert_close_nan, max_abs
+from _util import hash_buffer, lcg_buffer, seeded_normal
+from test_oracle_forward import FIXTURE_SHAPES
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+def buffers(n, span):
+    return lcg_buffer(n, 0xC0FFEE, span), lcg_buffer(n, 0xBADBEEF, span), lcg_buffer(n, 0xCAFE00, span)
+
+
+def omask(mask):
+    if mask.kind == 0:
+        return None
+    if mask.kind == 1:
+        return "causal"
+    return ("padding", mask.keep)
+
+
+@pytest.mark.parametrize("bhnd", FIXTURE_SHAPES)
+def test_flash_matches_oracle_on_20_fixed_shapes(oracle, bhnd):
+    shape = ra.AttentionShape.new(*bhnd)
+    q, k, v = buffers(shape.buffer_len(), 2.0)
+    rng = np.random.default_rng(bhnd[2])
+    keep = rng.random(bhnd[2]) < 0.7
+    keep[0] = True
+    for mask in (ra.Mask.none(), ra.Mask.causal(), ra.Mask.padding(keep)):
+        got = ra.flash_forward_masked(shape, q, k, v, mask)
+        want = oracle.flash_forward_masked(oracle.AttentionShape(*bhnd), q, k, v, omask(mask))
+        assert_close_nan(got, want, TOL, f"{bhnd} mask={mask.kind}")
+        assert np.isfinite(got).all()
+
+
+@pytest.mark.parametrize("bhnd", [(2, 4, 32, 16), (1, 2, 70, 24), (2, 4, 128, 64), (4, 8, 96, 32), (1, 3, 300, 128),
+                                  (1, 2, 33, 100), (2, 1, 257, 5)])
+def test_flash_matches_oracle_unit_shapes(oracle, bhnd):
+    shape = ra.AttentionShape.new(*bhnd)
+    q, k, v = buffers(shape.buffer_len(), 3.0)
+    for mask in (ra.Mask.none(), ra.Mask.causal()):
+        got = ra.flash_forward_masked(shape, q, k, v, mask)
+        want = oracle.flash_forward_masked(oracle.AttentionShape(*bhnd), q, k, v, omask(mask))
+        assert_close_nan(got, want, TOL, str(bhnd))
+
+
+def test_scaling_factor_is_one_over_sqrt_d():
+    shape = ra.AttentionShape.new(1, 1, 1, 4)
+    e0 = np.array([1.0, 0, 0, 0], dtype=np.float32)
+    v = np.array([5.0, -2.0, 7.0, 1.0], dtype=np.float32)
+    assert max_abs(ra.flash_forward(shape, e0, e0, v), v) <= 1e-6
+
+
+def test_scale_value_two_keys_analytic():
+    D = 16
+    shape = ra.AttentionShape.new(1, 1, 2, D)
+    q = np.zeros((2, D), dtype=np.float32)
+    k = np.zeros((2, D), dtype=np.float32)
+    q[:, 0] = 4.0
+    k[0, 0] = 4.0
+    v = np.zeros((2, D), dtype=np.float32)
+    v[0], v[1] = 1.0, -1.0
+    w0 = 1.0 / (1.0 + np.exp(-4.0))
+    assert np.allclose(ra.flash_forward(shape, q, k, v), 2 * w0 - 1, atol=1e-6)
+
+
+def test_empty_seq_is_no_op():
+    shape = ra.AttentionShape.new(2, 4, 0, 16)
+    assert ra.flash_forward(shape, [], [], []).size == 0
+
+
+def test_errors_in_reference_order():
+    e = np.zeros(0, dtype=np.float32)
+    with pytest.raises(ra.ZeroDim):
+        ra.flash_forward(ra.AttentionShape.new(1, 1, 4, 0), e, e, e)
+    shape = ra.AttentionShape.new(1, 1, 4, 8)
+    good, bad = np.zeros(32, np.float32), np.zeros(16, np.float32)
+    with pytest.raises(ra.BufferShapeMismatch) as ei:
+        ra.flash_forward(shape, good, bad, good)
+    assert (ei.value.which, ei.value.expected, ei.value.got) == ("k", 32, 16)
+    with pytest.raises(ra.OutputShapeMismatch):
+        ra.flash_forward(shape, good, good, good, out=np.zeros(31, np.float32))
+    with pytest.raises(ra.PaddingLengthMismatch) as ei:
+        ra.flash_forward_masked(ra.AttentionShape.new(1, 1, 4, 4), bad, bad, bad, ra.Mask.padding([True] * 3))
+    assert (ei.value.expected, ei.value.got) == (4, 3)
+
+
+def test_nan_input_propagates_to_output(oracle):
+    shape = ra.AttentionShape(1, 1, 4, 8, 4, 4)
+    q = lcg_buffer(32, 1, 3.0)
+    q[0] = np.nan
+    k, v = lcg_buffer(32, 2, 3.0), lcg_buffer(32, 3, 3.0)
+    got = ra.flash_forward(shape, q, k, v)
+    want = oracle.flash_forward(oracle.AttentionShape(1, 1, 4, 8, 4, 4), q, k, v)
+    assert_close_nan(got, want, TOL)
+    assert np.isnan(got[:8]).all() and np.isfinite(got[8:]).all()
+    # a NaN key poisons exactly the rows that can see it
+    q = lcg_buffer(32, 1, 3.0)
+    k[2 * 8 + 3] = np.nan
+    for mask, om in ((ra.Mask.causal(), "causal"), (ra.Mask.none(), None)):
+        got = ra.flash_forward_masked(shape, q, k, v, mask)
+        want = oracle.flash_forward_masked(oracle.AttentionShape(1, 1, 4, 8, 4, 4), q, k, v, om)
+        assert_close_nan(got, want, TOL)
+
+
+def test_causal_first_query_only_attends_to_self():
+    shape = ra.AttentionShape.new(1, 1, 4, 8)
+    ones = np.ones(32, dtype=np.float32)
+    v = np.zeros(32, dtype=np.float32)
+    v[0:8] = 10.0 * np.arange(1, 9)
+    v[8:16], v[16:24] = -99.0, 99.0
+    out = ra.flash_forward_masked(shape, ones, ones, v, ra.Mask.causal())
+    assert max_abs(out[:8], v[:8]) <= 1e-6
+
+
+def test_causal_constant_qk_gives_prefix_means():
+    N, D = 70, 8
+    shape = ra.AttentionShape.new(1, 1, N, D)
+    ones = np.ones(N * D, dtype=np.float32)
+    v = seeded_normal((N, D), 5)
+    expect = np.cumsum(v.astype(np.float64), axis=0) / np.arange(1, N + 1)[:, None]
+    out = ra.flash_forward_masked(shape, ones, ones, v, ra.Mask.causal()).reshape(N, D)
+    assert max_abs(out, expect) < 2e-6
+
+
+def test_padding_mask_excludes_padded_positions_exactly():
+    shape = ra.AttentionShape.new(1, 1, 4, 4)
+    ones = np.ones(16, dtype=np.float32)
+    v = np.array([10, 0, 0, 0, 99, 0, 0, 0, -99, 0, 0, 0, 30, 0, 0, 0], dtype=np.float32)
+    out = ra.flash_forward_masked(shape, ones, ones, v, ra.Mask.padding([True, False, False, True]))
+    assert abs(out[0] - 20.0) <= 1e-5
+
+
+def test_fully_masked_rows_and_leading_masked_tile(oracle):
+    """Rows without a visible key are NaN; a padding mask hiding the reference's whole first key
+    tile [0, bc) makes every row NaN (what the reference's recurrence produces)."""
+    shape = ra.AttentionShape(1, 2, 5, 4)
+    q, k, v = buffers(shape.buffer_len(), 2.0)
+    assert np.isnan(ra.flash_forward_masked(shape, q, k, v, ra.Mask.padding([False] * 5))).all()
+    for bc, keep in ((4, [False] * 4 + [True] * 8), (4, [False] * 3 + [True] * 9), (8, [False] * 7 + [True] * 5),
+                     (8, [False] * 8 + [True] * 4), (64, [False] * 11 + [True]), (4, [True] * 4 + [False] * 4 + [True] * 4)):
+        shape = ra.AttentionShape(1, 1, 12, 4, 4, bc)
+        q, k, v = buffers(shape.buffer_len(), 2.0)
+        got = ra.flash_forward_masked(shape, q, k, v, ra.Mask.padding(keep))
+        want = oracle.flash_forward_masked(oracle.AttentionShape(1, 1, 12, 4, 4, bc), q, k, v, ("padding", keep))
+        assert_close_nan(got, want, TOL, f"bc={bc} keep={keep}")
+
+
+def test_flash_stable_for_large_q_k_magnitudes(oracle):
+    shape = ra.AttentionShape.new(1, 1, 16, 8)
+    i = np.arange(shape.buffer_len(), dtype=np.float32)
+    q = (1e3 + np.sin(i * np.float32(0.01))).astype(np.float32)
+    k = (1e3 + np.cos(i * np.float32(0.013))).astype(np.float32)
+    v = np.sin(i * np.float32(0.07)).astype(np.float32)
+    got = ra.flash_forward(shape, q, k, v)
+    want = oracle.naive_forward(oracle.AttentionShape(1, 1, 16, 8), q, k, v)
+    assert np.isfinite(got).all()
+    # scores ~1e6/sqrt(8): one f32 ulp of a score is ~0.03, so the reference's own bar (1e-3 rel) applies here
+    assert np.all(np.abs(got - want) <= 1e-3 + 1e-3 * np.maximum(np.abs(got), np.abs(want)))
+
+
+def test_flash_matches_oracle_random_shapes(oracle):
+    rng = np.random.default_rng(20260504)
+    cases = [(1, 1, 1, 4)] + [(int(rng.integers(1, 3)), int(rng.integers(1, 4)), int(rng.integers(1, 40)),
+                               int(rng.integers(4, 16))) for _ in range(100)]
+    for bhnd in cases:
+        shape = ra.AttentionShape(*bhnd, 16, 16)
+        n = shape.buffer_len()
+        q, k, v = hash_buffer(n, 1), hash_buffer(n, 13), hash_buffer(n, 29)
+        got = ra.flash_forward(shape, q, k, v)
+        want = oracle.flash_forward(oracle.AttentionShape(*bhnd, 16, 16), q, k, v)
+        assert_close_nan(got, want, TOL, str(bhnd))
+
+
+def test_config_f32_causal_b1_h8_n2048_d64(oracle):
+    """BASELINE configs[0]: the reference's own CPU-runnable case, N(0,1) inputs, causal."""
+    bhnd = (1, 8, 2048, 64)
+    q, k, v = (seeded_normal(bhnd, s) for s in (101, 102, 103))
+    shape = ra.AttentionShape.new(*bhnd)
+    got = ra.flash_forward_masked(shape, q, k, v, ra.Mask.causal())
+    want = oracle.flash_forward_masked(oracle.AttentionShape(*bhnd), q, k, v, "causal")
+    assert_close_nan(got, want, TOL, "cfg f32")
+    assert max_abs(got.reshape(bhnd)[0, :, 0], v[0, :, 0]) <= 1e-6  # causal row 0 == V[0]
+
+
+# ---- gqa_forward_f32 ------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("b,hq,hkv,sq,skv,d", [(1, 4, 4, 3, 3, 4), (1, 8, 2, 4, 4, 8), (2, 6, 3, 1, 37, 16),
+                                              (2, 6, 3, 5, 37, 16), (1, 32, 8, 1, 700, 128), (1, 4, 2, 1, 1, 8),
+                                              (2, 8, 2, 130, 130, 64), (1, 3, 1, 2, 9, 200)])
+def test_gqa_forward_matches_oracle(oracle, b, hq, hkv, sq, skv, d):
+    q = seeded_normal((b, hq, sq, d), 1)
+    k = seeded_normal((b, hkv, skv, d), 2)
+    v = seeded_normal((b, hkv, skv, d), 3)
+    out = np.full(b * hq * sq * d, 7.0, dtype=np.float32)
+    ra.gqa_forward_f32(q, k, v, out, b, hq, hkv, sq, skv, d)
+    want = oracle.gqa_forward_f32(q, k, v, b, hq, hkv, sq, skv, d)
+    assert_close_nan(out, want, TOL)
+    vv = v.reshape(b, hkv, skv * d)
+    o = out.reshape(b, hq, sq * d)
+    g = hq // hkv
+    for h in range(hq):  # outputs inside [min V, max V] of the mapped kv head (gqa.rs:303-317)
+        assert (o[:, h].min(axis=1) >= vv[:, h // g].min(axis=1) - 1e-5).all()
+        assert (o[:, h].max(axis=1) <= vv[:, h // g].max(axis=1) + 1e-5).all()
+
+
+def test_gqa_errors():
+    z = lambda n: np.zeros(n, dtype=np.float32)
+    with pytest.raises(ra.HeadCountMismatch):
+        ra.gqa_forward_f32(z(20), z(8), z(8), z(20), 1, 5, 2, 1, 1, 4)
+    with pytest.raises(ra.HeadCountMismatch):
+        ra.gqa_forward_f32(z(20), z(8), z(8), z(20), 1, 4, 0, 1, 1, 4)
+    with pytest.raises(ra.WrongInputLen) as ei:
+        ra.gqa_forward_f32(z(7), z(8), z(8), z(16), 1, 4, 2, 1, 1, 4)
+    assert (ei.value.which, ei.value.expected, ei.value.got) == ("q", 16, 7)
+    with pytest.raises(ra.WrongInputLen) as ei:
+        ra.gqa_forward_f32(z(16), z(8), z(8), z(15), 1, 4, 2, 1, 1, 4)
+    assert ei.value.which == "out"
