@@ -1,0 +1,243 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+A step is one pass of the bf16 causal prefill kernel over BASELINE's workload
+B=4, H=32, N=4096, D=128 (inputs resident in HBM before the timed region); the same run also
+times the batched GQA decode workload (batch 64, 32 query / 8 kv heads, D=128, context lengths
+uniform in [512, 8192], Lmax 8192) and reports it under "decode".
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+
+Prints ONE JSON line.  `value` is prefill TFLOP/s with causal-counted FLOPs
+(4*B*H*D*N*(N+1)/2: skipped tiles are not credited); `roofline` prices it against the dense bf16
+MFMA peak, `decode.roofline` against the HBM peak with algorithmic bytes (K+V read once per kv
+head, Q in, O out).  Kernel durations are measured with HIP events on the stream the kernels
+are launched on.  `cpu_baseline` times the CPU oracle (a C restatement of the reference's CPU
+path; the reference itself is Rust and cannot be built here) on a bounded sample, on this box's
+host cores.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+
+class Hip:
+    """The few HIP runtime calls the timing needs (stream + events), straight from libamdhip64."""
+
+    def __init__(self):
+        self.lib = C.CDLL("libamdhip64.so")
+        for name, args in (("hipStreamCreate", [C.POINTER(C.c_void_p)]), ("hipEventCreate", [C.POINTER(C.c_void_p)]),
+                           ("hipEventRecord", [C.c_void_p, C.c_void_p]), ("hipEventSynchronize", [C.c_void_p]),
+                           ("hipEventElapsedTime", [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]),
+                           ("hipStreamSynchronize", [C.c_void_p]), ("hipDeviceSynchronize", [])):
+            getattr(self.lib, name).argtypes = args
+
+    def check(self, rc, what):
+        if rc != 0:
+            raise RuntimeError(f"{what} failed with hipError {rc}")
+
+    def stream(self):
+        s = C.c_void_p()
+        self.check(self.lib.hipStreamCreate(C.byref(s)), "hipStreamCreate")
+        return s
+
+    def event(self):
+        e = C.c_void_p()
+        self.check(self.lib.hipEventCreate(C.byref(e)), "hipEventCreate")
+        return e
+
+    def record(self, e, s):
+        self.check(self.lib.hipEventRecord(e, s), "hipEventRecord")
+
+    def elapsed_ms(self, e0, e1):
+        self.check(self.lib.hipEventSynchronize(e1), "hipEventSynchronize")
+        ms = C.c_float()
+        self.check(self.lib.hipEventElapsedTime(C.byref(ms), e0, e1), "hipEventElapsedTime")
+        return ms.value
+
+    def sync(self):
+        self.check(self.lib.hipDeviceSynchronize(), "hipDeviceSynchronize")
+
+
+def time_steps(hip, stream, launch, steps, warmup):
+    """W untimed steps, then K steps: whole-region wall time (sync on both sides) and per-launch
+    durations from one pair of events per step on `stream`."""
+    for i in range(warmup):
+        launch(i)
+    hip.sync()
+    evs = [(hip.event(), hip.event()) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        hip.record(evs[i][0], stream)
+        launch(warmup + i)
+        hip.record(evs[i][1], stream)
+    hip.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    per = np.array([hip.elapsed_ms(a, b) for a, b in evs])
+    return wall_ms, per
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity sample")
+    ap.add_argument("--only", choices=["prefill", "decode"], default=None)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (attention shards over batch/heads "
+              "with no exchange step); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import rustorch_amd as ra
+    from oracle import attn_oracle as oracle  # checker + cpu_baseline leg only
+
+    ra.init(0)
+    hip = Hip()
+    stream = hip.stream()
+    K = ra.LlmKernels()
+    rng = np.random.default_rng(1234)
+    out = {}
+
+    # ------------------------------------------------------------------ prefill (the step)
+    B, H, N, D = 4, 32, 4096, 128
+    prefill = None
+    if args.only in (None, "prefill"):
+        n_el = B * H * N * D
+        qb, kb, vb = (oracle.f32_to_bf16(rng.standard_normal(n_el, dtype=np.float32)) for _ in range(3))
+        dq, dk, dv = (ra.HipStorage.from_numpy(x) for x in (qb, kb, vb))
+        dout = ra.HipStorage(n_el * 2)
+        shape = ra.AttentionShape.new(B, H, N, D)
+        causal = ra.Mask.causal()
+        wall_ms, per = time_steps(hip, stream, lambda i: ra.flash_forward_bf16_dev(shape, dq, dk, dv, dout, causal,
+                                                                                  stream=stream),
+                                  args.steps, args.warmup)
+        flops_causal = 4.0 * B * H * D * (N * (N + 1) / 2.0)
+        flops_full = 4.0 * B * H * D * float(N) * N
+        ms_step = wall_ms / args.steps
+        ms_kernel = float(per.mean())
+        prefill = {"ms_per_step": ms_step, "kernel_ms_mean": ms_kernel, "kernel_ms_median": float(np.median(per)),
+                   "kernel_ms_min": float(per.min()), "tflops": flops_causal / (ms_step * 1e-3) / 1e12,
+                   "tflops_kernel": flops_causal / (ms_kernel * 1e-3) / 1e12,
+                   "tflops_unmasked_convention": flops_full / (ms_kernel * 1e-3) / 1e12}
+        if not args.no_cpu:
+            # parity + CPU baseline on a sample of (b,h) slabs: the oracle computes every tile, like the reference
+            threads = min(oracle.max_threads(), 16)
+            slabs = [(i * 7) % (B * H) for i in range(min(B * H, threads))]
+            got = oracle.bf16_to_f32(dout.download(np.uint16)).reshape(B * H, N * D)
+            qs = np.stack([oracle.bf16_to_f32(qb.reshape(B * H, -1)[s]) for s in slabs])
+            ks = np.stack([oracle.bf16_to_f32(kb.reshape(B * H, -1)[s]) for s in slabs])
+            vs = np.stack([oracle.bf16_to_f32(vb.reshape(B * H, -1)[s]) for s in slabs])
+            t0 = time.perf_counter()
+            want = oracle.flash_forward_masked(oracle.AttentionShape(1, len(slabs), N, D), qs, ks, vs, "causal",
+                                               threads=threads).reshape(len(slabs), N * D)
+            cpu_s = time.perf_counter() - t0
+            err = float(np.abs(got[slabs] - want).max())
+            prefill["parity_max_abs"] = err
+            prefill["cpu"] = {"value": flops_causal * len(slabs) / (B * H) / cpu_s / 1e12, "unit": "TFLOP/s",
+                              "cores": threads, "kind": "port",
+                              "sample": f"{len(slabs)} of {B * H} (b,h) slabs of the same workload, one thread per "
+                                        f"slab as rayon does, {cpu_s:.1f} s; f32 on the bf16-rounded inputs; "
+                                        f"causal-counted FLOPs although every tile is computed, as in the reference"}
+            if err > 2e-2:
+                print(f"PARITY FAILURE: prefill max-abs {err}", file=sys.stderr)
+                sys.exit(1)
+        del dq, dk, dv, dout
+
+    # ------------------------------------------------------------------ decode
+    decode = None
+    if args.only in (None, "decode"):
+        Bd, Hq, Hkv, Dd, Lmax = 64, 32, 8, 128, 8192
+        lens = np.random.default_rng(4).integers(512, 8193, size=Bd).astype(np.int32)
+        n_cache = Bd * Hkv * Lmax * Dd
+        kc = np.empty(n_cache, dtype=np.uint16)
+        vc = np.empty(n_cache, dtype=np.uint16)
+        step = n_cache // 16
+        for i in range(16):
+            kc[i * step:(i + 1) * step] = oracle.f32_to_bf16(rng.standard_normal(step, dtype=np.float32))
+            vc[i * step:(i + 1) * step] = oracle.f32_to_bf16(rng.standard_normal(step, dtype=np.float32))
+        qd = oracle.f32_to_bf16(rng.standard_normal(Bd * Hq * Dd, dtype=np.float32))
+        # rotate over several copies of the cache so that a step never finds its keys in the 256 MB
+        # last-level cache left there by the previous step
+        n_sets = 3
+        sets = [(ra.HipStorage.from_numpy(kc), ra.HipStorage.from_numpy(vc)) for _ in range(n_sets)]
+        d_q = ra.HipStorage.from_numpy(qd)
+        d_lens = ra.HipStorage.from_numpy(lens)
+        d_o = ra.HipStorage(Bd * Hq * Dd * 2)
+        ws_bytes = K.gqa_decode_workspace_bytes(Bd, Hq, Hkv, Dd, Lmax)
+        ws = ra.HipStorage(max(ws_bytes, 256))
+
+        def launch(i):
+            k_, v_ = sets[i % n_sets]
+            K.gqa_decode_batched_bf16(stream, d_q, k_, v_, d_o, d_lens, Bd, Hq, Hkv, Dd, Lmax, ws, ws.byte_len)
+
+        wall_ms, per = time_steps(hip, stream, launch, args.steps, args.warmup)
+        alg_bytes = float(lens.astype(np.int64).sum()) * 2 * Hkv * Dd * 2 + Bd * Hq * Dd * 2 * 2
+        ms_kernel = float(per.mean())
+        decode = {"metric": "decode attn HBM GB/s", "value": alg_bytes / (wall_ms / args.steps * 1e-3) / 1e9,
+                  "unit": "GB/s", "ms_per_step": wall_ms / args.steps, "kernel_ms_mean": ms_kernel,
+                  "kernel_ms_median": float(np.median(per)), "kernel_ms_min": float(per.min()),
+                  "algorithmic_bytes": alg_bytes,
+                  "config": {"workload": "bf16 GQA decode, batch 64, 32 q / 8 kv heads, D=128, ctx U[512,8192] "
+                                         "(seed 4), cache (B,Hkv,Lmax=8192,D)", "sum_len": int(lens.sum()),
+                             "cache_sets_rotated": n_sets},
+                  "roofline": {"bound": "hbm", "achieved": alg_bytes / (ms_kernel * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                               "unit": "GB/s", "frac": alg_bytes / (ms_kernel * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                               "traffic": None, "kernels": "decode_split + decode_merge (one event pair per step)"}}
+        if not args.no_cpu:
+            threads = min(oracle.max_threads(), 16)
+            got = oracle.bf16_to_f32(d_o.download(np.uint16))
+            t0 = time.perf_counter()
+            want = oracle.gqa_decode_batched_bf16(qd, kc, vc, lens, Bd, Hq, Hkv, Dd, Lmax, threads=threads)
+            cpu_s = time.perf_counter() - t0
+            err = float(np.abs(got - want).max())
+            decode["parity_max_abs"] = err
+            decode["cpu_baseline"] = {"value": alg_bytes / cpu_s / 1e9, "unit": "GB/s", "cores": threads,
+                                      "kind": "port",
+                                      "sample": f"the whole decode step once ({cpu_s:.1f} s): trim + decode_attn_row "
+                                                f"per (sequence, kv head) task, f32 on bf16-rounded inputs; the "
+                                                f"reference runs seq_q = 1 on a single thread"}
+            if err > 2e-2:
+                print(f"PARITY FAILURE: decode max-abs {err}", file=sys.stderr)
+                sys.exit(1)
+
+    if prefill is None:  # --only decode: report the decode line as the main one
+        print(json.dumps(dict(decode, n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True,
+                              dtype="bf16", data="synthetic", vs_baseline=None)))
+        return
+    achieved = prefill["tflops_kernel"]
+    out = {
+        "metric": "prefill attn TFLOP/s (% bf16 MFMA peak); decode attn HBM GB/s (% peak)",
+        "value": prefill["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": prefill["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "bf16 causal prefill attention, B=4 H=32 N=4096 D=128, N(0,1) inputs (seed 1234), "
+                               "f32 accumulation", "flop_convention": "4*B*H*D*N*(N+1)/2 (causal-counted)",
+                   "tflops_unmasked_convention_4BHN2D": prefill["tflops_unmasked_convention"]},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "flash_fwd_bf16_kernel<128>",
+                     "kernel_ms_mean": prefill["kernel_ms_mean"], "kernel_ms_median": prefill["kernel_ms_median"],
+                     "kernel_ms_min": prefill["kernel_ms_min"]},
+    }
+    if "cpu" in prefill:
+        out["cpu_baseline"] = prefill["cpu"]
+        out["parity_max_abs"] = prefill["parity_max_abs"]
+    if decode is not None:
+        out["decode"] = decode
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

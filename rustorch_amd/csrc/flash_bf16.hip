@@ -3,17 +3,22 @@
 // tensors: bf16 in, f32 accumulation on the matrix cores, bf16 out rounded once.
 //
 // Workgroup = 4 wavefronts = 128 query rows of one (batch, head); each wave owns 32 rows and
-// the workgroup walks the keys 64 at a time through LDS.  Per wave and step:
+// the workgroup walks the keys 64 at a time through a double-buffered LDS tile.  Per wave and step:
 //
 //   S^T[kv, q]  = K[kv, :] . Q[q, :]      v_mfma_f32_32x32x16_bf16, A = K tile (LDS), B = Q (registers)
 //   online softmax on S^T: lane l holds 32 scores of query row l % 32, so row max / row sum are
 //                          in-lane plus one exchange with lane l ^ 32
-//   O^T[d, q]  += V^T[d, kv] . P^T[kv, q]  A = V tile read transposed from LDS, B = P (registers)
+//   O^T[d, q]  += V^T[d, kv] . P^T[kv, q]  A = V tile, read transposed out of its row-major LDS
+//                                          copy by ds_read_b64_tr_b16; B = P (registers)
 //
 // The C layout of the first product (lane: column q, rows kv = 8j + 4*(l/32) + r) is, read as 8
 // consecutive registers, exactly a B operand of the second product under a fixed permutation of
 // the 16 contraction slots; the V operand is fetched with the same permutation, so P is never
 // written to LDS.
+//
+// The running max is only raised (and O, l rescaled) when some row's tile max exceeds it by more
+// than 2^8 in the exp2 domain: P then stays below 2^8, harmless in f32/bf16, and the rescale of the
+// 64 O registers leaves the steady-state loop.
 #include "rt_common.hpp"
 #include "rt_kernels.hpp"
 
@@ -24,19 +29,39 @@ namespace {
 constexpr int BR = 128;  // query rows per workgroup
 constexpr int BC = 64;   // key rows per step
 constexpr int NTHREADS = 256;
+constexpr float kLazyLog2 = 8.0f;
 
-template <int HD>
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
+    f32x2_t x = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2_t));  // v_cvt_pk_bf16_f32, RNE
+}
+
+// Transposing LDS read.  Within each group of 16 lanes, lane j receives element (j % 4) of the 8
+// bytes addressed by lanes 4e + j/4, e = 0..3.  With lane 4e + c pointing at row k0+e, columns
+// n0+4c.., lane j ends up with column n0+j of rows k0..k0+3: a contraction-major MFMA operand
+// fragment out of a row-major tile.
+__device__ __forceinline__ u32x2_t lds_read_tr16(const uint16_t* p) {
+    s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3)))*)(p));
+    return __builtin_bit_cast(u32x2_t, v);
+}
+
+template <int HD, int MODE>
 __global__ __launch_bounds__(NTHREADS, 2) void flash_fwd_bf16_kernel(FlashBf16Params p) {
-    constexpr int LDK = HD + 8;   // K tile row stride (bf16): +16 B so 16 rows x 16 B cover all banks once
-    constexpr int LDV = BC + 4;   // V^T tile row stride: 34 banks, 32 rows x 8 B cover all banks once
+    constexpr int LDK = HD + 8;   // K row stride (bf16): +16 B, 16 rows x 16 B tile all 64 banks
+    constexpr int LDV = HD + 32;  // V row stride: = 64 B (mod 256 B), 4 rows x 64 B tile all 64 banks
     constexpr int KS = HD / 16;   // contraction steps of the score product
     constexpr int DT = HD / 32;   // 32-row tiles of O^T
     constexpr int CH = HD / 8;    // 16-byte chunks per row
     constexpr int ROWS_PER_PASS = NTHREADS / CH;
     constexpr int PASSES = BC / ROWS_PER_PASS;
+    constexpr bool kCausal = (MODE == kMaskCausal) || (MODE == kMaskVarlenCausal);
 
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[BC * LDK];
-    __shared__ __attribute__((aligned(16))) uint16_t Vt[HD * LDV];
+    __shared__ __attribute__((aligned(16))) uint16_t Ks[2][BC * LDK];
+    __shared__ __attribute__((aligned(16))) uint16_t Vs[2][BC * LDV];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -71,12 +96,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void flash_fwd_bf16_kernel(FlashBf16Pa
     const uint16_t* __restrict__ Vg = p.v + ((size_t)b * p.kv_heads + kvh) * (size_t)N * HD;
     uint16_t* __restrict__ Og = p.out + ((size_t)b * p.heads + h) * (size_t)N * HD;
 
-    const bool causal = (p.mask == kMaskCausal) || (p.mask == kMaskVarlenCausal);
     int n_keys = N;  // keys that exist for this sequence
-    if (p.mask == kMaskVarlenCausal) n_keys = min(N, max(0, p.seq_lens[b]));
+    if (MODE == kMaskVarlenCausal) n_keys = min(N, max(0, p.seq_lens[b]));
 
-    bool poison = false;  // see flash_f32.hip: a padding mask hiding the reference's whole first key tile
-    if (p.mask == kMaskPadding) {
+    bool poison = false;  // a padding mask hiding the reference's whole first key tile: every row NaN
+    if (MODE == kMaskPadding) {
         int lim = p.ref_bc < N ? p.ref_bc : N;
         bool any = false;
         for (int j = lane; j < lim; j += kWave) any |= (p.keep[j] != 0);
@@ -99,12 +123,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void flash_fwd_bf16_kernel(FlashBf16Pa
         for (int i = 0; i < 16; i++) acc_o[t][i] = 0.0f;
     float m_run = neg_inf(), l_run = 0.0f;
     const float c = p.scale_log2e;
+    const float lazy_raw = kLazyLog2 / c;  // the rescale threshold in raw-score units
 
     int kv_end = n_keys;
-    if (causal) kv_end = min(n_keys, q0 + BR);
+    if (kCausal) kv_end = min(n_keys, q0 + BR);
+    if (MODE == kMaskVarlenCausal && q0 >= n_keys) kv_end = 0;  // a tile of padded query rows
     const int n_steps = (kv_end + BC - 1) / BC;
 
-    // ---- global -> register prefetch of one K/V tile
+    // ---- global -> register prefetch of one K/V tile, then register -> LDS
     const int ld_c = tid % CH, ld_r = tid / CH;
     u32x4_t kreg[PASSES], vreg[PASSES];
     auto prefetch = [&](int kv0) {
@@ -120,102 +146,121 @@ __global__ __launch_bounds__(NTHREADS, 2) void flash_fwd_bf16_kernel(FlashBf16Pa
             vreg[i] = zv;
         }
     };
-    if (n_steps > 0) prefetch(0);
-
-    for (int step = 0; step < n_steps; step++) {
-        const int kv0 = step * BC;
-        __syncthreads();  // everyone is done reading the previous tile
+    auto stage = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < PASSES; i++) {
             int r = ld_r + i * ROWS_PER_PASS;
-            *(u32x4_t*)(Ks + r * LDK + 8 * ld_c) = kreg[i];
-#pragma unroll
-            for (int e = 0; e < 4; e++) {  // V goes in transposed: Vt[d][kv]
-                uint32_t w = vreg[i][e];
-                Vt[(8 * ld_c + 2 * e) * LDV + r] = (uint16_t)(w & 0xffffu);
-                Vt[(8 * ld_c + 2 * e + 1) * LDV + r] = (uint16_t)(w >> 16);
-            }
+            *(u32x4_t*)(&Ks[buf][r * LDK + 8 * ld_c]) = kreg[i];
+            *(u32x4_t*)(&Vs[buf][r * LDV + 8 * ld_c]) = vreg[i];
         }
-        __syncthreads();
-        if (step + 1 < n_steps) prefetch(kv0 + BC);
+    };
+    if (n_steps > 0) {
+        prefetch(0);
+        stage(0);
+        if (n_steps > 1) prefetch(BC);
+    }
+    __syncthreads();
 
-        if (causal && kv0 > qw + 31) continue;  // this wave's rows see nothing of the tile (wave-uniform)
+    // per-lane part of the transposing V read: lane -> (row within a group of 4, 4-column chunk)
+    const int tr_row = (lane & 15) >> 2;
+    const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-        // ---- S^T = K . Q^T for the two 32-key halves of the tile
-        f32x16_t s[2];
-#pragma unroll
-        for (int t = 0; t < 2; t++) {
-#pragma unroll
-            for (int i = 0; i < 16; i++) s[t][i] = 0.0f;
-#pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                bf16x8_t a = *(const bf16x8_t*)(Ks + (32 * t + col) * LDK + 16 * ks + 8 * hh);
-                s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[ks], s[t], 0, 0, 0);
-            }
+    for (int step = 0; step < n_steps; step++) {
+        const int kv0 = step * BC;
+        const int buf = step & 1;
+        // tile step+1 goes into the other buffer (last read in step-1, before the barrier that ended it)
+        if (step + 1 < n_steps) {
+            stage(buf ^ 1);
+            if (step + 2 < n_steps) prefetch(kv0 + 2 * BC);
         }
 
-        // ---- mask (only tiles that need it) and row max
-        const bool need_mask = (kv0 + BC > n_keys) || (causal && kv0 + BC - 1 > qw) || (p.mask == kMaskPadding);
-        float m_tile = neg_inf();
-        if (need_mask) {
+        if (!(kCausal && kv0 > qw + 31)) {  // wave-uniform: this wave's rows see something of the tile
+            const uint16_t* Kb = Ks[buf];
+            const uint16_t* Vb = Vs[buf];
+            // ---- S^T = K . Q^T for the two 32-key halves of the tile
+            f32x16_t s[2];
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) s[t][i] = 0.0f;
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) {
+                    bf16x8_t a = *(const bf16x8_t*)(Kb + (32 * t + col) * LDK + 16 * ks + 8 * hh);
+                    s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[ks], s[t], 0, 0, 0);
+                }
+            }
+
+            // ---- mask (only tiles that need it)
+            bool need_mask = (kv0 + BC > n_keys);
+            if (kCausal) need_mask |= (kv0 + BC - 1 > qw);
+            if (MODE == kMaskPadding) need_mask = true;
+            if (need_mask) {
+#pragma unroll
+                for (int t = 0; t < 2; t++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        int kr = kv0 + 32 * t + 8 * (i >> 2) + 4 * hh + (i & 3);
+                        bool masked = kr >= n_keys;
+                        if (kCausal) masked |= kr > q_row;
+                        if (MODE == kMaskPadding) masked |= (kr < N) && (p.keep[kr] == 0);
+                        s[t][i] = masked ? neg_inf() : s[t][i];
+                    }
+            }
+            // ---- row max (in-lane, then the other half of the wave)
+            float m_tile = neg_inf();
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) m_tile = fmaxf(m_tile, s[t][i]);
+            m_tile = fmaxf(m_tile, other_half(m_tile));
+
+            // ---- raise the running max only when it pays (wave-uniform branch; no MFMA inside)
+            if (__any(m_tile > m_run + lazy_raw)) {
+                float m_new = fmaxf(m_run, m_tile);
+                float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+                float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);  // m_run = -inf -> 0
+                m_run = m_new;
+                l_run *= alpha;
+#pragma unroll
+                for (int t = 0; t < DT; t++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) acc_o[t][i] *= alpha;
+            }
+            const float mc = ((m_run == neg_inf()) ? 0.0f : m_run) * c;
+            float tile_l = 0.0f;
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
-                    int kr = kv0 + 32 * t + 8 * (i >> 2) + 4 * hh + (i & 3);
-                    bool masked = kr >= n_keys;
-                    if (causal) masked |= kr > q_row;
-                    if (p.mask == kMaskPadding) masked |= (kr < N) && (p.keep[kr] == 0);
-                    s[t][i] = masked ? neg_inf() : s[t][i];
+                    float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][i], c, -mc));
+                    s[t][i] = e;
+                    tile_l += e;
+                }
+            l_run += tile_l;
+
+            // ---- O^T += V^T . P^T
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    u32x4_t pb;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) pb[e] = cvt_pk_bf16(s[t][8 * u + 2 * e], s[t][8 * u + 2 * e + 1]);
+                    const bf16x8_t pB = __builtin_bit_cast(bf16x8_t, pb);
+                    // contraction slots 0-3 of this lane: keys kv_lo..kv_lo+3; slots 4-7: kv_lo+8..kv_lo+11
+                    const int kv_lo = 32 * t + 16 * u + 4 * hh;
+#pragma unroll
+                    for (int dt = 0; dt < DT; dt++) {
+                        const uint16_t* vp = Vb + (kv_lo + tr_row) * LDV + dt * 32 + tr_col;
+                        u32x2_t lo = lds_read_tr16(vp);
+                        u32x2_t hi = lds_read_tr16(vp + 8 * LDV);
+                        u32x4_t av = {lo[0], lo[1], hi[0], hi[1]};
+                        acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), pB,
+                                                                            acc_o[dt], 0, 0, 0);
+                    }
                 }
         }
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) m_tile = fmaxf(m_tile, s[t][i]);
-        m_tile = fmaxf(m_tile, other_half(m_tile));
-
-        // ---- online softmax in the exp2 domain; branch-free (MFMA ignores the exec mask)
-        float m_new = fmaxf(m_run, m_tile);
-        float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
-        float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
-        float mc = m_use * c;
-        m_run = m_new;
-        float tile_l = 0.0f;
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][i], c, -mc));
-                s[t][i] = e;
-                tile_l += e;
-            }
-        l_run = l_run * alpha + tile_l;
-#pragma unroll
-        for (int t = 0; t < DT; t++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) acc_o[t][i] *= alpha;
-
-        // ---- O^T += V^T . P^T
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int u = 0; u < 2; u++) {
-                u32x4_t pb;
-#pragma unroll
-                for (int e = 0; e < 4; e++) pb[e] = pack_bf16x2(s[t][8 * u + 2 * e], s[t][8 * u + 2 * e + 1]);
-                bf16x8_t pB = __builtin_bit_cast(bf16x8_t, pb);
-                const int kv_lo = 32 * t + 16 * u + 4 * hh;
-#pragma unroll
-                for (int dt = 0; dt < DT; dt++) {
-                    const uint16_t* vrow = Vt + (dt * 32 + col) * LDV + kv_lo;
-                    u32x2_t lo = *(const u32x2_t*)(vrow);
-                    u32x2_t hi = *(const u32x2_t*)(vrow + 8);
-                    u32x4_t av = {lo[0], lo[1], hi[0], hi[1]};
-                    acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), pB,
-                                                                        acc_o[dt], 0, 0, 0);
-                }
-            }
+        __syncthreads();  // tile `buf` is free again; tile buf^1 is complete
     }
 
     // ---- normalise and store.  acc_o[dt][i] = O^T[d = 32dt + 8(i/4) + 4hh + i%4][q_row]
@@ -223,7 +268,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void flash_fwd_bf16_kernel(FlashBf16Pa
     bool good = (l > 0.0f) && (l < __uint_as_float(0x7f800000u)) && !poison;
     float inv_l = 1.0f / l;
     if (q_row < N) {
-        const bool padded_row = (p.mask == kMaskVarlenCausal) && (q_row >= n_keys);
+        const bool padded_row = (MODE == kMaskVarlenCausal) && (q_row >= n_keys);
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
@@ -235,10 +280,24 @@ __global__ __launch_bounds__(NTHREADS, 2) void flash_fwd_bf16_kernel(FlashBf16Pa
                     if (padded_row) x = p.zero_padded_rows ? 0.0f : quiet_nan();
                     o[r] = x;
                 }
-                u32x2_t w = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
+                u32x2_t w = {cvt_pk_bf16(o[0], o[1]), cvt_pk_bf16(o[2], o[3])};
                 *(u32x2_t*)(Og + (size_t)q_row * HD + dt * 32 + 8 * j + 4 * hh) = w;
             }
     }
+}
+
+template <int HD>
+hipError_t launch_hd(hipStream_t stream, const FlashBf16Params& p, dim3 grid, dim3 block) {
+    switch (p.mask) {
+        case kMaskNone: hipLaunchKernelGGL((flash_fwd_bf16_kernel<HD, kMaskNone>), grid, block, 0, stream, p); break;
+        case kMaskCausal: hipLaunchKernelGGL((flash_fwd_bf16_kernel<HD, kMaskCausal>), grid, block, 0, stream, p); break;
+        case kMaskPadding: hipLaunchKernelGGL((flash_fwd_bf16_kernel<HD, kMaskPadding>), grid, block, 0, stream, p); break;
+        case kMaskVarlenCausal:
+            hipLaunchKernelGGL((flash_fwd_bf16_kernel<HD, kMaskVarlenCausal>), grid, block, 0, stream, p);
+            break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
 }
 
 }  // namespace
@@ -248,11 +307,10 @@ hipError_t launch_flash_bf16(hipStream_t stream, const FlashBf16Params& p) {
     int n_qtiles = (p.seq + BR - 1) / BR;
     dim3 grid((unsigned)((size_t)n_qtiles * p.batch * p.heads)), block(NTHREADS);
     switch (p.dim) {
-        case 64: hipLaunchKernelGGL(flash_fwd_bf16_kernel<64>, grid, block, 0, stream, p); break;
-        case 128: hipLaunchKernelGGL(flash_fwd_bf16_kernel<128>, grid, block, 0, stream, p); break;
+        case 64: return launch_hd<64>(stream, p, grid, block);
+        case 128: return launch_hd<128>(stream, p, grid, block);
         default: return hipErrorInvalidValue;
     }
-    return hipGetLastError();
 }
 
 }  // namespace rt
