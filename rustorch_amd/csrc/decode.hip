@@ -30,6 +30,16 @@ __device__ __forceinline__ float load_elem<uint16_t>(const uint16_t* p, size_t i
 __device__ __forceinline__ void store_elem(float* p, size_t i, float x) { p[i] = x; }
 __device__ __forceinline__ void store_elem(uint16_t* p, size_t i, float x) { p[i] = f32_to_bf16_bits(x); }
 
+typedef short s16x4v __attribute__((ext_vector_type(4)));
+typedef float f32x2v __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
+// transposing LDS read (see flash_bf16.hip): lane j of a 16-lane group gets element j%4 of the 8 bytes
+// addressed by lanes 4e + j/4, e = 0..3
+__device__ __forceinline__ u32x2_t lds_read_tr16_b64(const uint16_t* p) {
+    s16x4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4v __attribute__((address_space(3)))*)(p));
+    return __builtin_bit_cast(u32x2_t, v);
+}
+
 __device__ __forceinline__ float wave_sum(float x) {
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off, 64);
@@ -118,159 +128,163 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(AttnRowsParams p) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Split-K GQA decode, bf16 cache, HD in {64, 128}, G = query heads per kv head (<= 8).
-// grid (n_chunks, kv_heads, batch), 256 threads.  A key row (HD bf16) is read by LPR = HD/8 adjacent
-// lanes, 16 bytes each, so a wave load instruction covers 64/LPR whole rows, fully coalesced.
-template <int HD, int G>
-__global__ __launch_bounds__(256) void decode_split_kernel(DecodeSplitParams p) {
-    constexpr int LPR = HD / 8;        // lanes per row
-    constexpr int RPW = 64 / LPR;      // rows per wave load
-    constexpr int RPB = 4 * RPW;       // rows per workgroup pass
-    constexpr int UN = 4;              // passes kept in flight
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int sub = lane % LPR, rsub = lane / LPR;
+// Split-K GQA decode, bf16 cache, HD in {64, 128}, up to 16 query heads per kv head.
+// grid (n_chunks, kv_heads, batch), ONE wavefront per workgroup: a wave streams `chunk` key rows of
+// one (sequence, kv head) and serves every query head of the group from that single read.
+//
+// Per step of 32 rows the wave loads K and V with fully coalesced 16-byte loads (a load instruction
+// covers 4 whole rows), parks them in its private LDS tile, and runs both products on the matrix
+// cores with the group's query heads as the (zero-padded) 16-wide column block:
+//
+//   S^T[kv, h]  = K[kv, :] . Q[h, :]        v_mfma_f32_16x16x32_bf16, A = K tile, B = Q (registers)
+//   O^T[d, h]  += V^T[d, kv] . P^T[kv, h]    A = V tile read transposed (ds_read_b64_tr_b16), B = P
+//
+// Lane l holds column h = l % 16 and the 8 keys 16*rt + 4*(l/16) + i of the step, which as they
+// stand are the 8 contraction slots of its B operand for the second product; the V operand is
+// fetched with the same slot -> key map.  The memory system sees nothing but long coalesced
+// streams; the VALU work per byte is a small fraction of a lane-per-element formulation.
+constexpr int kDecRows = 32;  // key rows per step
+
+template <int HD>
+__global__ __launch_bounds__(64) void decode_split_kernel(DecodeSplitParams p) {
+    constexpr int LDK = HD + 8;    // +16 B: 16 rows x 16 B tile all 64 banks
+    constexpr int LDV = HD + 16;   // +32 B: 8 rows x 32 B tile all 64 banks (transposing reads)
+    constexpr int KS = HD / 32;    // contraction steps of the score product
+    constexpr int DT = HD / 16;    // 16-row tiles of O^T
+    constexpr int CH = HD / 8;     // 16-byte chunks per row
+    constexpr int RPI = 64 / CH;   // rows covered by one wave load instruction
+    constexpr int NLD = kDecRows / RPI;  // load instructions per tile
+    __shared__ __attribute__((aligned(16))) uint16_t Kw[kDecRows * LDK];
+    __shared__ __attribute__((aligned(16))) uint16_t Vw[kDecRows * LDV];
+
+    const int lane = threadIdx.x;
+    const int hcol = lane & 15, g4 = lane >> 4;
     const int chunk = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    const int G = p.heads / p.kv_heads;
     const int kv_len = min(max(p.kv_lens[b], 0), p.max_seq);
     const int r_begin = chunk * p.chunk;
-    if (r_begin >= kv_len) return;  // whole workgroup leaves together; the merge kernel never reads this slot
+    if (r_begin >= kv_len) return;  // the merge kernel never reads this slot
     const int r_end = min(kv_len, r_begin + p.chunk);
 
     const size_t cache_base = ((size_t)b * p.kv_heads + kvh) * (size_t)p.max_seq * HD;
     const uint16_t* __restrict__ K = p.k_cache + cache_base;
     const uint16_t* __restrict__ V = p.v_cache + cache_base;
 
-    // this lane's 8 elements of each query head of the group, pre-multiplied by scale*log2(e)
-    float qf[G][8];
+    // Q as B operand: column h = lane % 16 (zero beyond the group), contraction slots 8*(lane/16)..+8
+    bf16x8_t qreg[KS];
 #pragma unroll
-    for (int g = 0; g < G; g++) {
-        const uint16_t* qp = p.q + ((size_t)b * p.heads + (size_t)kvh * G + g) * HD + 8 * sub;
-        u32x4_t w = *(const u32x4_t*)qp;
+    for (int ks = 0; ks < KS; ks++) {
+        u32x4_t z = {0u, 0u, 0u, 0u};
+        if (hcol < G) z = *(const u32x4_t*)(p.q + ((size_t)b * p.heads + (size_t)kvh * G + hcol) * HD + 32 * ks + 8 * g4);
+        qreg[ks] = __builtin_bit_cast(bf16x8_t, z);
+    }
+    f32x4_t acc_o[DT];
+#pragma unroll
+    for (int t = 0; t < DT; t++) acc_o[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = neg_inf(), l_run = 0.0f;
+    const float c = p.scale_log2e;
+    const float lazy_raw = 8.0f / c;
+
+    const int ld_row = lane / CH, ld_c = lane % CH;
+    const int k_off = hcol * LDK + 8 * g4;
+    const int tr_off = (4 * g4 + (hcol >> 2)) * LDV + 4 * (hcol & 3);
+
+    u32x4_t kreg[NLD], vreg[NLD];
+    auto issue_loads = [&](int r0) {
+#pragma unroll
+        for (int i = 0; i < NLD; i++) {
+            int r = min(r0 + RPI * i + ld_row, r_end - 1);  // rows past the end re-read the last row; masked below
+            kreg[i] = *(const u32x4_t*)(K + (size_t)r * HD + 8 * ld_c);
+            vreg[i] = *(const u32x4_t*)(V + (size_t)r * HD + 8 * ld_c);
+        }
+    };
+    issue_loads(r_begin);
+
+    for (int r0 = r_begin; r0 < r_end; r0 += kDecRows) {
+        // registers -> the wave's LDS tile (the previous step's reads have been consumed by its MFMAs)
+#pragma unroll
+        for (int i = 0; i < NLD; i++) {
+            *(u32x4_t*)(Kw + (RPI * i + ld_row) * LDK + 8 * ld_c) = kreg[i];
+            *(u32x4_t*)(Vw + (RPI * i + ld_row) * LDV + 8 * ld_c) = vreg[i];
+        }
+        if (r0 + kDecRows < r_end) issue_loads(r0 + kDecRows);  // next step's rows fly while this one computes
+
+        // ---- S^T = K . Q^T, two 16-key row tiles
+        f32x4_t s[2];
+#pragma unroll
+        for (int rt = 0; rt < 2; rt++) {
+            s[rt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                bf16x8_t a = *(const bf16x8_t*)(Kw + 16 * rt * LDK + k_off + 32 * ks);
+                s[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[ks], s[rt], 0, 0, 0);
+            }
+        }
+        if (r0 + kDecRows > r_end) {  // ragged last step
+#pragma unroll
+            for (int rt = 0; rt < 2; rt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    if (r0 + 16 * rt + 4 * g4 + i >= r_end) s[rt][i] = neg_inf();
+        }
+        // ---- column max over the 32 keys: in-lane, then across the four 16-lane groups
+        float m_step = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                             fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+        {
+            auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(m_step), __float_as_uint(m_step), false, false);
+            m_step = fmaxf(__uint_as_float(r16[0]), __uint_as_float(r16[1]));
+            auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(m_step), __float_as_uint(m_step), false, false);
+            m_step = fmaxf(__uint_as_float(r32[0]), __uint_as_float(r32[1]));
+        }
+        if (__any(m_step > m_run + lazy_raw)) {  // raise the running max only when it pays (wave-uniform)
+            float m_new = fmaxf(m_run, m_step);
+            float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+            float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int t = 0; t < DT; t++) acc_o[t] *= alpha;
+        }
+        const float mc = ((m_run == neg_inf()) ? 0.0f : m_run) * c;
+        float pe[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) pe[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i >> 2][i & 3], c, -mc));
+        l_run += ((pe[0] + pe[1]) + (pe[2] + pe[3])) + ((pe[4] + pe[5]) + (pe[6] + pe[7]));
+        u32x4_t pb;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            qf[g][2 * e] = bf16_lo(w[e]) * p.scale_log2e;
-            qf[g][2 * e + 1] = bf16_hi(w[e]) * p.scale_log2e;
+            f32x2v x = {pe[2 * e], pe[2 * e + 1]};
+            pb[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2v));
         }
-    }
-    float m[G], l[G], o[G][8];
+        const bf16x8_t pB = __builtin_bit_cast(bf16x8_t, pb);
+        // ---- O^T += V^T . P^T: slots 0-3 of a lane are keys 4g..4g+3, slots 4-7 keys 16+4g..16+4g+3
 #pragma unroll
-    for (int g = 0; g < G; g++) {
-        m[g] = neg_inf();
-        l[g] = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 8; e++) o[g][e] = 0.0f;
-    }
-
-    for (int base = r_begin + wave * RPW; base < r_end; base += UN * RPB) {  // wave-uniform trip count
-        u32x4_t kw[UN], vw[UN];
-        bool ok[UN];
-#pragma unroll
-        for (int u = 0; u < UN; u++) {
-            int r = base + rsub + u * RPB;
-            ok[u] = r < r_end;
-            u32x4_t z = {0u, 0u, 0u, 0u};
-            kw[u] = ok[u] ? *(const u32x4_t*)(K + (size_t)r * HD + 8 * sub) : z;
-            vw[u] = ok[u] ? *(const u32x4_t*)(V + (size_t)r * HD + 8 * sub) : z;
-        }
-        float s[UN][G];
-#pragma unroll
-        for (int u = 0; u < UN; u++) {
-            float kf[8];
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                kf[2 * e] = bf16_lo(kw[u][e]);
-                kf[2 * e + 1] = bf16_hi(kw[u][e]);
-            }
-#pragma unroll
-            for (int g = 0; g < G; g++) {
-                float acc = 0.0f;
-#pragma unroll
-                for (int e = 0; e < 8; e++) acc = __builtin_fmaf(qf[g][e], kf[e], acc);
-#pragma unroll
-                for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
-                s[u][g] = ok[u] ? acc : neg_inf();
-            }
-        }
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            float m_new = m[g];
-#pragma unroll
-            for (int u = 0; u < UN; u++) m_new = fmaxf(m_new, s[u][g]);
-            float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
-            float alpha = __builtin_amdgcn_exp2f(m[g] - m_use);
-            m[g] = m_new;
-            float pe[UN];
-            float lsum = 0.0f;
-#pragma unroll
-            for (int u = 0; u < UN; u++) {
-                pe[u] = __builtin_amdgcn_exp2f(s[u][g] - m_use);
-                lsum += pe[u];
-            }
-            l[g] = l[g] * alpha + lsum;
-#pragma unroll
-            for (int e = 0; e < 8; e++) o[g][e] *= alpha;
-#pragma unroll
-            for (int u = 0; u < UN; u++) {
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    o[g][2 * e] = __builtin_fmaf(pe[u], bf16_lo(vw[u][e]), o[g][2 * e]);
-                    o[g][2 * e + 1] = __builtin_fmaf(pe[u], bf16_hi(vw[u][e]), o[g][2 * e + 1]);
-                }
-            }
+        for (int dt = 0; dt < DT; dt++) {
+            const uint16_t* vp = Vw + tr_off + 16 * dt;
+            u32x2_t lo = lds_read_tr16_b64(vp);
+            u32x2_t hi = lds_read_tr16_b64(vp + 16 * LDV);
+            u32x4_t av = {lo[0], lo[1], hi[0], hi[1]};
+            acc_o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av), pB, acc_o[dt], 0, 0, 0);
         }
     }
 
-    // ---- fold the RPW row groups of the wave (lanes differing in rsub), then the 4 waves through LDS
-#pragma unroll
-    for (int g = 0; g < G; g++) {
-#pragma unroll
-        for (int off = LPR; off < 64; off <<= 1) {
-            float m_o = __shfl_xor(m[g], off, 64);
-            float l_o = __shfl_xor(l[g], off, 64);
-            float m_new = fmaxf(m[g], m_o);
-            float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
-            float ca = __builtin_amdgcn_exp2f(m[g] - m_use), cb = __builtin_amdgcn_exp2f(m_o - m_use);
-            l[g] = l[g] * ca + l_o * cb;
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                float o_o = __shfl_xor(o[g][e], off, 64);
-                o[g][e] = o[g][e] * ca + o_o * cb;
-            }
-            m[g] = m_new;
-        }
+    // ---- row sum across the four lane groups, then the partial (o, m, l) of this chunk
+    {
+        auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
+        l_run = __uint_as_float(r16[0]) + __uint_as_float(r16[1]);
+        auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
+        l_run = __uint_as_float(r32[0]) + __uint_as_float(r32[1]);
     }
-    __shared__ float sm[4][G], sl[4][G];
-    __shared__ float so[4][G][HD];
-    if (rsub == 0) {
+    if (hcol < G) {
+        float* ws_o = p.ws;
+        float* ws_ml = p.ws + (size_t)p.batch * p.heads * p.n_chunks * HD;
+        const size_t slot = ((size_t)b * p.heads + (size_t)kvh * G + hcol) * p.n_chunks + chunk;
+        // acc_o[dt][i] = O^T[d = 16dt + 4g + i][h]
 #pragma unroll
-        for (int g = 0; g < G; g++) {
-            if (sub == 0) {
-                sm[wave][g] = m[g];
-                sl[wave][g] = l[g];
-            }
-#pragma unroll
-            for (int e = 0; e < 8; e++) so[wave][g][8 * sub + e] = o[g][e];
-        }
-    }
-    __syncthreads();
-    // partial layout: ws_o[(b*heads + h)*n_chunks + chunk][HD], then ws_ml[...][2]
-    float* ws_o = p.ws;
-    float* ws_ml = p.ws + (size_t)p.batch * p.heads * p.n_chunks * HD;
-    for (int idx = threadIdx.x; idx < G * HD; idx += 256) {
-        int g = idx / HD, d = idx % HD;
-        float m_all = fmaxf(fmaxf(sm[0][g], sm[1][g]), fmaxf(sm[2][g], sm[3][g]));
-        float m_use = (m_all == neg_inf()) ? 0.0f : m_all;
-        float acc = 0.0f, l_all = 0.0f;
-#pragma unroll
-        for (int w = 0; w < 4; w++) {
-            float cw = __builtin_amdgcn_exp2f(sm[w][g] - m_use);
-            acc += so[w][g][d] * cw;
-            l_all += sl[w][g] * cw;
-        }
-        size_t slot = ((size_t)b * p.heads + (size_t)kvh * G + g) * p.n_chunks + chunk;
-        ws_o[slot * HD + d] = acc;
-        if (d == 0) {
-            ws_ml[slot * 2] = m_all;
-            ws_ml[slot * 2 + 1] = l_all;
+        for (int dt = 0; dt < DT; dt++) *(f32x4_t*)(ws_o + slot * HD + 16 * dt + 4 * g4) = acc_o[dt];
+        if (g4 == 0) {
+            ws_ml[slot * 2] = m_run * c;  // the merge works in the exp2 domain
+            ws_ml[slot * 2 + 1] = l_run;
         }
     }
 }
@@ -311,15 +325,8 @@ __global__ void kv_append_kernel(uint16_t* __restrict__ k_cache, uint16_t* __res
 
 template <int HD>
 hipError_t launch_split_hd(hipStream_t stream, const DecodeSplitParams& p) {
-    dim3 grid(p.n_chunks, p.kv_heads, p.batch), block(256);
-    int g = p.heads / p.kv_heads;
-    switch (g) {
-        case 1: hipLaunchKernelGGL((decode_split_kernel<HD, 1>), grid, block, 0, stream, p); break;
-        case 2: hipLaunchKernelGGL((decode_split_kernel<HD, 2>), grid, block, 0, stream, p); break;
-        case 4: hipLaunchKernelGGL((decode_split_kernel<HD, 4>), grid, block, 0, stream, p); break;
-        case 8: hipLaunchKernelGGL((decode_split_kernel<HD, 8>), grid, block, 0, stream, p); break;
-        default: return hipErrorInvalidValue;
-    }
+    dim3 grid(p.n_chunks, p.kv_heads, p.batch), block(64);
+    hipLaunchKernelGGL(decode_split_kernel<HD>, grid, block, 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(decode_merge_kernel<HD>, dim3(p.heads, p.batch), dim3(HD), 0, stream, p);
@@ -331,7 +338,7 @@ hipError_t launch_split_hd(hipStream_t stream, const DecodeSplitParams& p) {
 bool decode_split_supported(int heads, int kv_heads, int dim) {
     if (kv_heads <= 0 || heads % kv_heads != 0) return false;
     int g = heads / kv_heads;
-    return (dim == 64 || dim == 128) && (g == 1 || g == 2 || g == 4 || g == 8);
+    return (dim == 64 || dim == 128) && g <= 16;
 }
 
 int decode_split_chunk(int max_seq) {
