@@ -52,6 +52,7 @@ int fail_hip(rt_err_detail* e, hipError_t code, const char* where) {
         if (_e != hipSuccess) return fail_hip(err, _e, where); \
     } while (0)
 
+int g_decode_waves = 0;  // one-wave workgroups one launch of the decode kernel keeps resident
 std::mutex g_init_mutex;
 int g_init_status = -1;  // -1: not tried
 char g_init_msg[160];
@@ -88,6 +89,8 @@ int ensure_device(rt_err_detail* err, int device = -1) {
         e = hipSetDevice(dev);
         if (e != hipSuccess) return fail_hip(err, e, "hipSetDevice");
     }
+    // the decode kernel (one wave, ~18 KB LDS, <= 256 VGPRs) fits 8 times on a CU
+    g_decode_waves = prop.multiProcessorCount * 8;
     g_init_status = RT_OK;
     return RT_OK;
 }
@@ -469,9 +472,8 @@ RT_API int rt_gqa_decode_batched_bf16(void* stream, const void* q, const void* k
         p.kv_heads = n_kv;
         p.dim = head_dim;
         p.max_seq = max_seq;
-        p.chunk = rt::decode_split_chunk(max_seq);
-        p.n_chunks = (max_seq + p.chunk - 1) / p.chunk;
-        if (p.n_chunks == 0) p.n_chunks = 1;
+        p.n_part = rt::decode_split_parts(max_seq);
+        p.n_waves = g_decode_waves;
         p.scale_log2e = (1.0f / sqrtf((float)head_dim)) * rt::kLog2eHost;
         HIP_TRY(rt::launch_decode_split((hipStream_t)stream, p), "decode_split launch");
         return RT_OK;

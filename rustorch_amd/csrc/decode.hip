@@ -128,22 +128,69 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(AttnRowsParams p) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Split-K GQA decode, bf16 cache, HD in {64, 128}, up to 16 query heads per kv head.
-// grid (n_chunks, kv_heads, batch), ONE wavefront per workgroup: a wave streams `chunk` key rows of
-// one (sequence, kv head) and serves every query head of the group from that single read.
+// Split-K GQA decode over a ragged batch, bf16 cache, HD in {64, 128}, up to 16 query heads per kv head.
 //
-// Per step of 32 rows the wave loads K and V with fully coalesced 16-byte loads (a load instruction
-// covers 4 whole rows), parks them in its private LDS tile, and runs both products on the matrix
-// cores with the group's query heads as the (zero-padded) 16-wide column block:
+// Work is the flat list of 32-row steps of every (sequence, kv head) segment, in (b, kvh, row) order:
+// S steps in all.  A fixed grid of one-wave workgroups (as many as the GPU holds at once) cuts that
+// list into equal contiguous spans, so every wave streams the same number of bytes whatever the
+// lengths are, no workgroup is launched for rows that do not exist, and a segment is split only where
+// a span boundary falls inside it.  A wave leaves one partial (o, m, l) per segment it touches, at slot
+// (its index - index of the first wave on that segment); the merge kernel folds a head's partials with
+// the online-softmax monoid (crates/rustorch-attention/src/online_softmax.rs:105-131, extended with o).
+//
+// Per step the wave loads K and V with fully coalesced 16-byte loads (a load instruction covers 4
+// whole rows), parks them in its private LDS tile, and runs both products on the matrix cores with
+// the group's query heads as the (zero-padded) 16-wide column block:
 //
 //   S^T[kv, h]  = K[kv, :] . Q[h, :]        v_mfma_f32_16x16x32_bf16, A = K tile, B = Q (registers)
 //   O^T[d, h]  += V^T[d, kv] . P^T[kv, h]    A = V tile read transposed (ds_read_b64_tr_b16), B = P
 //
 // Lane l holds column h = l % 16 and the 8 keys 16*rt + 4*(l/16) + i of the step, which as they
 // stand are the 8 contraction slots of its B operand for the second product; the V operand is
-// fetched with the same slot -> key map.  The memory system sees nothing but long coalesced
-// streams; the VALU work per byte is a small fraction of a lane-per-element formulation.
-constexpr int kDecRows = 32;  // key rows per step
+// fetched with the same slot -> key map.
+constexpr int kDecRows = 32;     // key rows per step
+constexpr int kDecSpanMin = 8;   // a wave takes at least this many steps (bounds the partials per segment)
+
+__device__ __forceinline__ int dec_steps(int len) { return (len + kDecRows - 1) / kDecRows; }
+__device__ __forceinline__ int dec_len(const DecodeSplitParams& p, int b) { return min(max(p.kv_lens[b], 0), p.max_seq); }
+
+__device__ __forceinline__ int wave_sum_i(int x) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off, 64);
+    return x;
+}
+__device__ __forceinline__ int wave_incl_scan_i(int x, int lane) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        int y = __shfl_up(x, off, 64);
+        if (lane >= off) x += y;
+    }
+    return x;
+}
+
+// Steps of all sequences (each counted kv_heads times) and the span every wave takes.
+__device__ __forceinline__ void dec_total(const DecodeSplitParams& p, int lane, int& total, int& span) {
+    int t = 0;
+    for (int r = 0; r < p.batch; r += 64) {
+        int i = r + lane;
+        t += wave_sum_i(i < p.batch ? p.kv_heads * dec_steps(dec_len(p, i)) : 0);
+    }
+    total = t;
+    span = max((t + p.n_waves - 1) / p.n_waves, kDecSpanMin);
+}
+// First step (in the flat list) of sequence b.
+__device__ __forceinline__ int dec_seq_start(const DecodeSplitParams& p, int lane, int b) {
+    int t = 0;
+    for (int r = 0; r < b; r += 64) {
+        int i = r + lane;
+        t += wave_sum_i(i < b ? p.kv_heads * dec_steps(dec_len(p, i)) : 0);
+    }
+    return t;
+}
+
+struct DecCursor {  // position in the flat step list
+    int b, kvh, st, steps_b, len_b;
+};
 
 template <int HD>
 __global__ __launch_bounds__(64) void decode_split_kernel(DecodeSplitParams p) {
@@ -159,55 +206,111 @@ __global__ __launch_bounds__(64) void decode_split_kernel(DecodeSplitParams p) {
 
     const int lane = threadIdx.x;
     const int hcol = lane & 15, g4 = lane >> 4;
-    const int chunk = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    const int w = blockIdx.x;
     const int G = p.heads / p.kv_heads;
-    const int kv_len = min(max(p.kv_lens[b], 0), p.max_seq);
-    const int r_begin = chunk * p.chunk;
-    if (r_begin >= kv_len) return;  // the merge kernel never reads this slot
-    const int r_end = min(kv_len, r_begin + p.chunk);
+    const int Hkv = p.kv_heads;
 
-    const size_t cache_base = ((size_t)b * p.kv_heads + kvh) * (size_t)p.max_seq * HD;
-    const uint16_t* __restrict__ K = p.k_cache + cache_base;
-    const uint16_t* __restrict__ V = p.v_cache + cache_base;
+    int total, span;
+    dec_total(p, lane, total, span);
+    const int first = w * span;
+    const int last = min(total, first + span);
+    if (first >= last) return;
 
-    // Q as B operand: column h = lane % 16 (zero beyond the group), contraction slots 8*(lane/16)..+8
-    bf16x8_t qreg[KS];
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-        u32x4_t z = {0u, 0u, 0u, 0u};
-        if (hcol < G) z = *(const u32x4_t*)(p.q + ((size_t)b * p.heads + (size_t)kvh * G + hcol) * HD + 32 * ks + 8 * g4);
-        qreg[ks] = __builtin_bit_cast(bf16x8_t, z);
+    // ---- locate the sequence that holds step `first`
+    DecCursor cur;
+    int seq_start;  // flat index of the first step of sequence cur.b
+    {
+        int base = 0, b = 0, found_start = 0;
+        for (int r = 0; r < p.batch; r += 64) {
+            int i = r + lane;
+            int st = i < p.batch ? Hkv * dec_steps(dec_len(p, i)) : 0;
+            int incl = wave_incl_scan_i(st, lane) + base;
+            int cnt = __popcll(__ballot(i < p.batch && incl <= first));  // sequences of this round that end before `first`
+            if (cnt < 64) {
+                b = r + cnt;
+                found_start = cnt == 0 ? base : __shfl(incl, cnt - 1, 64);
+                break;
+            }
+            base = __shfl(incl, 63, 64);
+        }
+        cur.b = b;
+        seq_start = found_start;
+        cur.len_b = dec_len(p, b);
+        cur.steps_b = dec_steps(cur.len_b);
+        int local = first - seq_start;
+        cur.kvh = local / cur.steps_b;
+        cur.st = local - cur.kvh * cur.steps_b;
     }
-    f32x4_t acc_o[DT];
-#pragma unroll
-    for (int t = 0; t < DT; t++) acc_o[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    float m_run = neg_inf(), l_run = 0.0f;
+    auto advance = [&](DecCursor& c) {
+        if (++c.st == c.steps_b) {
+            c.st = 0;
+            if (++c.kvh == Hkv) {
+                c.kvh = 0;
+                do {  // skip empty sequences; the caller never advances past the last step of the list
+                    ++c.b;
+                    c.len_b = c.b < p.batch ? dec_len(p, c.b) : kDecRows;
+                    c.steps_b = dec_steps(c.len_b);
+                } while (c.steps_b == 0);
+            }
+        }
+    };
+
     const float c = p.scale_log2e;
     const float lazy_raw = 8.0f / c;
-
     const int ld_row = lane / CH, ld_c = lane % CH;
     const int k_off = hcol * LDK + 8 * g4;
     const int tr_off = (4 * g4 + (hcol >> 2)) * LDV + 4 * (hcol & 3);
 
     u32x4_t kreg[NLD], vreg[NLD];
-    auto issue_loads = [&](int r0) {
+    auto issue_loads = [&](const DecCursor& cc) {
+        const size_t base = ((size_t)cc.b * Hkv + cc.kvh) * (size_t)p.max_seq * HD;
+        const uint16_t* K = p.k_cache + base;
+        const uint16_t* V = p.v_cache + base;
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
-            int r = min(r0 + RPI * i + ld_row, r_end - 1);  // rows past the end re-read the last row; masked below
+            int r = min(cc.st * kDecRows + RPI * i + ld_row, cc.len_b - 1);  // rows past the end re-read the last row; masked below
             kreg[i] = *(const u32x4_t*)(K + (size_t)r * HD + 8 * ld_c);
             vreg[i] = *(const u32x4_t*)(V + (size_t)r * HD + 8 * ld_c);
         }
     };
-    issue_loads(r_begin);
+    // Q as B operand: column h = lane % 16 (zero beyond the group), contraction slots 8*(lane/16)..+8
+    bf16x8_t qreg[KS], qnext[KS];
+    auto load_q = [&](const DecCursor& cc, bf16x8_t (&q)[KS]) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            u32x4_t z = {0u, 0u, 0u, 0u};
+            if (hcol < G) z = *(const u32x4_t*)(p.q + ((size_t)cc.b * p.heads + (size_t)cc.kvh * G + hcol) * HD + 32 * ks + 8 * g4);
+            q[ks] = __builtin_bit_cast(bf16x8_t, z);
+        }
+    };
 
-    for (int r0 = r_begin; r0 < r_end; r0 += kDecRows) {
+    f32x4_t acc_o[DT];
+    float m_run, l_run;
+    auto reset_state = [&]() {
+#pragma unroll
+        for (int t = 0; t < DT; t++) acc_o[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        m_run = neg_inf();
+        l_run = 0.0f;
+    };
+    reset_state();
+
+    DecCursor nxt = cur;  // the prefetch cursor runs one step ahead of `cur`
+    load_q(cur, qreg);
+    issue_loads(nxt);
+    advance(nxt);
+
+    for (int t = first; t < last; t++) {
         // registers -> the wave's LDS tile (the previous step's reads have been consumed by its MFMAs)
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
             *(u32x4_t*)(Kw + (RPI * i + ld_row) * LDK + 8 * ld_c) = kreg[i];
             *(u32x4_t*)(Vw + (RPI * i + ld_row) * LDV + 8 * ld_c) = vreg[i];
         }
-        if (r0 + kDecRows < r_end) issue_loads(r0 + kDecRows);  // next step's rows fly while this one computes
+        const bool more = t + 1 < last;
+        if (more) {  // next step's rows (and, on a segment change, its queries) fly while this one computes
+            issue_loads(nxt);
+            if (nxt.st == 0) load_q(nxt, qnext);
+        }
 
         // ---- S^T = K . Q^T, two 16-key row tiles
         f32x4_t s[2];
@@ -220,12 +323,13 @@ __global__ __launch_bounds__(64) void decode_split_kernel(DecodeSplitParams p) {
                 s[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[ks], s[rt], 0, 0, 0);
             }
         }
-        if (r0 + kDecRows > r_end) {  // ragged last step
+        const int r0 = cur.st * kDecRows;
+        if (r0 + kDecRows > cur.len_b) {  // ragged last step of a segment
 #pragma unroll
             for (int rt = 0; rt < 2; rt++)
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    if (r0 + 16 * rt + 4 * g4 + i >= r_end) s[rt][i] = neg_inf();
+                    if (r0 + 16 * rt + 4 * g4 + i >= cur.len_b) s[rt][i] = neg_inf();
         }
         // ---- column max over the 32 keys: in-lane, then across the four 16-lane groups
         float m_step = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
@@ -243,7 +347,7 @@ __global__ __launch_bounds__(64) void decode_split_kernel(DecodeSplitParams p) {
             m_run = m_new;
             l_run *= alpha;
 #pragma unroll
-            for (int t = 0; t < DT; t++) acc_o[t] *= alpha;
+            for (int tt = 0; tt < DT; tt++) acc_o[tt] *= alpha;
         }
         const float mc = ((m_run == neg_inf()) ? 0.0f : m_run) * c;
         float pe[8];
@@ -266,46 +370,66 @@ __global__ __launch_bounds__(64) void decode_split_kernel(DecodeSplitParams p) {
             u32x4_t av = {lo[0], lo[1], hi[0], hi[1]};
             acc_o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av), pB, acc_o[dt], 0, 0, 0);
         }
-    }
 
-    // ---- row sum across the four lane groups, then the partial (o, m, l) of this chunk
-    {
-        auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
-        l_run = __uint_as_float(r16[0]) + __uint_as_float(r16[1]);
-        auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
-        l_run = __uint_as_float(r32[0]) + __uint_as_float(r32[1]);
-    }
-    if (hcol < G) {
-        float* ws_o = p.ws;
-        float* ws_ml = p.ws + (size_t)p.batch * p.heads * p.n_chunks * HD;
-        const size_t slot = ((size_t)b * p.heads + (size_t)kvh * G + hcol) * p.n_chunks + chunk;
-        // acc_o[dt][i] = O^T[d = 16dt + 4g + i][h]
+        // ---- end of a segment (or of this wave's span): leave the partial and start afresh
+        const bool seg_end = (cur.st == cur.steps_b - 1);
+        if (seg_end || !more) {
+            float l_all = l_run;
+            {
+                auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(l_all), __float_as_uint(l_all), false, false);
+                l_all = __uint_as_float(r16[0]) + __uint_as_float(r16[1]);
+                auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_all), __float_as_uint(l_all), false, false);
+                l_all = __uint_as_float(r32[0]) + __uint_as_float(r32[1]);
+            }
+            const int seg_first = t - cur.st;  // flat index of the segment's first step
+            const int part = w - seg_first / span;
+            if (hcol < G) {
+                float* ws_o = p.ws;
+                float* ws_ml = p.ws + (size_t)p.batch * p.heads * p.n_part * HD;
+                const size_t slot = ((size_t)cur.b * p.heads + (size_t)cur.kvh * G + hcol) * p.n_part + part;
+                // acc_o[dt][i] = O^T[d = 16dt + 4g + i][h]
 #pragma unroll
-        for (int dt = 0; dt < DT; dt++) *(f32x4_t*)(ws_o + slot * HD + 16 * dt + 4 * g4) = acc_o[dt];
-        if (g4 == 0) {
-            ws_ml[slot * 2] = m_run * c;  // the merge works in the exp2 domain
-            ws_ml[slot * 2 + 1] = l_run;
+                for (int dt = 0; dt < DT; dt++) *(f32x4_t*)(ws_o + slot * HD + 16 * dt + 4 * g4) = acc_o[dt];
+                if (g4 == 0) {
+                    ws_ml[slot * 2] = m_run * c;  // the merge works in the exp2 domain
+                    ws_ml[slot * 2 + 1] = l_all;
+                }
+            }
+            reset_state();
+            if (seg_end && more) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) qreg[ks] = qnext[ks];
+            }
         }
+        cur = nxt;
+        if (more) advance(nxt);
     }
 }
 
-// grid (heads, batch), HD threads.
+// grid (heads, batch), 64 * ceil(HD/64) threads: thread d folds element d of the head's partials.
 template <int HD>
-__global__ __launch_bounds__(HD) void decode_merge_kernel(DecodeSplitParams p) {
+__global__ __launch_bounds__(HD < 64 ? 64 : HD) void decode_merge_kernel(DecodeSplitParams p) {
     const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
-    const int kv_len = min(max(p.kv_lens[b], 0), p.max_seq);
-    const int n_valid = (kv_len + p.chunk - 1) / p.chunk;
+    const int lane = threadIdx.x & 63;
+    const int G = p.heads / p.kv_heads;
+    const int kvh = h / G;
+    int total, span;
+    dec_total(p, lane, total, span);
+    const int steps_b = dec_steps(dec_len(p, b));
+    const int seg_first = dec_seq_start(p, lane, b) + kvh * steps_b;
+    const int w_first = seg_first / span;
+    const int n_valid = steps_b > 0 ? (seg_first + steps_b - 1) / span - w_first + 1 : 0;
     const float* ws_o = p.ws;
-    const float* ws_ml = p.ws + (size_t)p.batch * p.heads * p.n_chunks * HD;
-    const size_t slot0 = ((size_t)b * p.heads + h) * p.n_chunks;
+    const float* ws_ml = p.ws + (size_t)p.batch * p.heads * p.n_part * HD;
+    const size_t slot0 = ((size_t)b * p.heads + h) * p.n_part;
     float m_all = neg_inf();
-    for (int c = 0; c < n_valid; c++) m_all = fmaxf(m_all, ws_ml[(slot0 + c) * 2]);
+    for (int k = 0; k < n_valid; k++) m_all = fmaxf(m_all, ws_ml[(slot0 + k) * 2]);
     float m_use = (m_all == neg_inf()) ? 0.0f : m_all;
     float acc = 0.0f, l_all = 0.0f;
-    for (int c = 0; c < n_valid; c++) {
-        float cw = __builtin_amdgcn_exp2f(ws_ml[(slot0 + c) * 2] - m_use);
-        acc += ws_o[(slot0 + c) * HD + d] * cw;
-        l_all += ws_ml[(slot0 + c) * 2 + 1] * cw;
+    for (int k = 0; k < n_valid; k++) {
+        float cw = __builtin_amdgcn_exp2f(ws_ml[(slot0 + k) * 2] - m_use);
+        acc += ws_o[(slot0 + k) * HD + d] * cw;
+        l_all += ws_ml[(slot0 + k) * 2 + 1] * cw;
     }
     // kv_len == 0: no key contributes, the output row is zero (gqa.rs:261; llm_kernels.rs:456)
     float r = n_valid > 0 ? acc / l_all : 0.0f;
@@ -325,8 +449,7 @@ __global__ void kv_append_kernel(uint16_t* __restrict__ k_cache, uint16_t* __res
 
 template <int HD>
 hipError_t launch_split_hd(hipStream_t stream, const DecodeSplitParams& p) {
-    dim3 grid(p.n_chunks, p.kv_heads, p.batch), block(64);
-    hipLaunchKernelGGL(decode_split_kernel<HD>, grid, block, 0, stream, p);
+    hipLaunchKernelGGL(decode_split_kernel<HD>, dim3(p.n_waves), dim3(64), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(decode_merge_kernel<HD>, dim3(p.heads, p.batch), dim3(HD), 0, stream, p);
@@ -341,20 +464,18 @@ bool decode_split_supported(int heads, int kv_heads, int dim) {
     return (dim == 64 || dim == 128) && g <= 16;
 }
 
-int decode_split_chunk(int max_seq) {
-    (void)max_seq;
-    return 512;
+int decode_split_parts(int max_seq) {
+    int steps_max = (max_seq + kDecRows - 1) / kDecRows;
+    return (steps_max + kDecSpanMin - 1) / kDecSpanMin + 1;
 }
 
 size_t decode_split_workspace_bytes(int batch, int heads, int dim, int max_seq) {
-    int chunk = decode_split_chunk(max_seq);
-    size_t n_chunks = ((size_t)max_seq + chunk - 1) / chunk;
-    if (n_chunks == 0) n_chunks = 1;
-    return (size_t)batch * heads * n_chunks * ((size_t)dim + 2) * sizeof(float);
+    return (size_t)batch * heads * decode_split_parts(max_seq) * ((size_t)dim + 2) * sizeof(float);
 }
 
 hipError_t launch_decode_split(hipStream_t stream, const DecodeSplitParams& p) {
     if (p.batch == 0 || p.heads == 0) return hipSuccess;
+    if (p.n_waves <= 0) return hipErrorInvalidValue;
     if (p.dim == 64) return launch_split_hd<64>(stream, p);
     if (p.dim == 128) return launch_split_hd<128>(stream, p);
     return hipErrorInvalidValue;

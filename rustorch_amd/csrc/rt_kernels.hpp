@@ -65,11 +65,12 @@ struct DecodeSplitParams {
     const int32_t* kv_lens;   // device int32[batch]
     float* ws;                // partial (o, m, l) per (b, head, chunk)
     int batch, heads, kv_heads, dim, max_seq;
-    int chunk, n_chunks;
+    int n_part;   // partial slots per (sequence, head): decode_split_parts(max_seq)
+    int n_waves;  // one-wave workgroups launched: what the GPU holds at once
     float scale_log2e;
 };
 bool decode_split_supported(int heads, int kv_heads, int dim);
-int decode_split_chunk(int max_seq);
+int decode_split_parts(int max_seq);
 size_t decode_split_workspace_bytes(int batch, int heads, int dim, int max_seq);
 hipError_t launch_decode_split(hipStream_t stream, const DecodeSplitParams& p);
 
