@@ -52,6 +52,7 @@ int fail_hip(rt_err_detail* e, hipError_t code, const char* where) {
         if (_e != hipSuccess) return fail_hip(err, _e, where); \
     } while (0)
 
+int g_num_cus = 0;
 int g_decode_waves = 0;  // one-wave workgroups one launch of the decode kernel keeps resident
 std::mutex g_init_mutex;
 int g_init_status = -1;  // -1: not tried
@@ -90,6 +91,7 @@ int ensure_device(rt_err_detail* err, int device = -1) {
         if (e != hipSuccess) return fail_hip(err, e, "hipSetDevice");
     }
     // the decode kernel (one wave, ~18 KB LDS, <= 256 VGPRs) fits 8 times on a CU
+    g_num_cus = prop.multiProcessorCount;
     g_decode_waves = prop.multiProcessorCount * 8;
     g_init_status = RT_OK;
     return RT_OK;
@@ -354,6 +356,7 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
     p.ref_bc = (int)(shape->bc == 0 ? 1 : (shape->bc > 0x7fffffffull ? 0x7fffffff : shape->bc));
     p.zero_padded_rows = zero_padded_rows;
     p.scale_log2e = (1.0f / sqrtf((float)shape->dim)) * rt::kLog2eHost;
+    p.n_workers = g_num_cus;
     HIP_TRY(rt::launch_flash_bf16((hipStream_t)stream, p), "flash_fwd_bf16 launch");
     return RT_OK;
 }

@@ -49,10 +49,6 @@ constexpr int NTHREADS = 64 * RT_FA_WAVES;
 constexpr int BR = 32 * RT_FA_WAVES;  // query rows per workgroup
 constexpr int BC = 64;                // key rows per step
 constexpr float kLazyLog2 = 8.0f;
-#ifndef RT_FA_QG
-#define RT_FA_QG 1
-#endif
-constexpr int QG = RT_FA_QG;  // query tiles per scheduling group
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
@@ -110,44 +106,19 @@ __global__ __launch_bounds__(NTHREADS, RT_FA_MIN_BLOCKS) void flash_fwd_bf16_ker
     const int col = lane & 31, hh = lane >> 5;
     RT_PHASE_DECL;
 
-    // ---- block -> (batch*head, query tile).  Workgroups are dealt round-robin to the 8 XCDs (each
-    // with its own L2), so XCD x gets the heads bh = x (mod 8).  Within an XCD the order is: groups of
-    // QG query tiles from the longest (causal) rows down, every head of the XCD per group.  Long jobs
-    // start first and the kernel ends on short ones; a group keeps QG workgroups on one head's K/V.
-    const int n_qtiles = (p.seq + BR - 1) / BR;
-    const int n_bh = p.batch * p.heads;
-    int bh, qt;
-    {
-        int id = blockIdx.x;
-        if ((n_bh & 7) == 0) {
-            const int xcd = id & 7, slot = id >> 3, heads_x = n_bh >> 3;
-            const int per_group = QG * heads_x;       // jobs in one full group of query tiles
-            const int g = slot / per_group;            // group index (0 = longest rows)
-            const int in_g = slot - g * per_group;
-            const int g_tiles = min(QG, n_qtiles - g * QG);  // the last group may be short
-            const int head = in_g / g_tiles;
-            qt = g * QG + (in_g - head * g_tiles);
-            bh = head * 8 + xcd;
-        } else {
-            bh = id / n_qtiles;
-            qt = id % n_qtiles;
-        }
-    }
-    const int qtile = n_qtiles - 1 - qt;  // the longest causal rows first
-    const int b = bh / p.heads, h = bh % p.heads;
-    const int kvh = h / p.group;
+    // ---- jobs.  A job is one (batch*head, 256-row query tile); the grid is persistent (one
+    // workgroup per CU) and every workgroup walks its own list.  Jobs are ranked from the longest
+    // (causal) rows down and dealt to the workers in boustrophedon order (round i: job i*W + w, or
+    // i*W + W-1-w when i is odd), so every worker gets the same number of key tiles to within one job,
+    // starts on a long job and ends on a short one.  Nothing is relaunched between jobs: the next
+    // job's queries and first key tile are requested before the current job's output is stored.
     const int N = p.seq;
-    const int q0 = qtile * BR;
-    const int qw = q0 + wave * 32;  // first query row of this wave
-    const int q_row = qw + col;
-
-    const uint16_t* __restrict__ Qg = p.q + ((size_t)b * p.heads + h) * (size_t)N * HD;
-    const uint16_t* __restrict__ Kg = p.k + ((size_t)b * p.kv_heads + kvh) * (size_t)N * HD;
-    const uint16_t* __restrict__ Vg = p.v + ((size_t)b * p.kv_heads + kvh) * (size_t)N * HD;
-    uint16_t* __restrict__ Og = p.out + ((size_t)b * p.heads + h) * (size_t)N * HD;
-
-    int n_keys = N;  // keys that exist for this sequence
-    if (MODE == kMaskVarlenCausal) n_keys = min(N, max(0, p.seq_lens[b]));
+    const int n_qtiles = (N + BR - 1) / BR;
+    const int n_bh = p.batch * p.heads;
+    const int n_jobs = n_qtiles * n_bh;
+    const int W = gridDim.x, w = blockIdx.x;
+    const float c = p.scale_log2e;
+    const float lazy_raw = kLazyLog2 / c;  // the rescale threshold in raw-score units
 
     bool poison = false;  // a padding mask hiding the reference's whole first key tile: every row NaN
     if (MODE == kMaskPadding) {
@@ -157,47 +128,25 @@ __global__ __launch_bounds__(NTHREADS, RT_FA_MIN_BLOCKS) void flash_fwd_bf16_ker
         poison = !__any(any);
     }
 
-    // ---- Q as B operand, in registers for the whole kernel
-    bf16x8_t qreg[KS];
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-        u32x4_t z = {0u, 0u, 0u, 0u};
-        if (q_row < N) z = *(const u32x4_t*)(Qg + (size_t)q_row * HD + 16 * ks + 8 * hh);
-        qreg[ks] = __builtin_bit_cast(bf16x8_t, z);
-    }
-
+    // state of the current job
+    int q0, qw, q_row, n_keys, n_steps;
+    const uint16_t* __restrict__ Kg;
+    const uint16_t* __restrict__ Vg;
+    uint16_t* __restrict__ Og;
+    bf16x8_t qreg[KS];  // Q as B operand, in registers for the whole job
+    u32x4_t kreg[PASSES], vreg[PASSES];
     f32x16_t acc_o[DT];
-#pragma unroll
-    for (int t = 0; t < DT; t++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) acc_o[t][i] = 0.0f;
-    float m_run = neg_inf(), l_run = 0.0f;
-    const float c = p.scale_log2e;
-    const float lazy_raw = kLazyLog2 / c;  // the rescale threshold in raw-score units
-
-    int kv_end = n_keys;
-    if (kCausal) kv_end = min(n_keys, q0 + BR);
-    if (MODE == kMaskVarlenCausal && q0 >= n_keys) kv_end = 0;  // a tile of padded query rows
-#ifdef RT_EXP_STEPS
-    const int n_steps = min(RT_EXP_STEPS, (kv_end + BC - 1) / BC);
-#else
-    const int n_steps = (kv_end + BC - 1) / BC;
-#endif
+    float m_run, l_run;
 
     // ---- global -> register prefetch of one K/V tile, then register -> LDS.  Rows past the last key
     // are read from the last key instead (no branch); they are masked in the score tile, so their
     // probabilities are zero.
-    u32x4_t kreg[PASSES], vreg[PASSES];
     auto prefetch = [&](int kv0) {
 #pragma unroll
         for (int i = 0; i < PASSES; i++) {
             const int idx = tid + i * NTHREADS;
             if (NCHUNK % NTHREADS == 0 || idx < NCHUNK) {
-#ifdef RT_EXP_SAMETILE
-                int r = min(idx / CH, n_keys - 1);
-#else
                 int r = min(kv0 + idx / CH, n_keys - 1);
-#endif
                 kreg[i] = *(const u32x4_t*)(Kg + (size_t)r * HD + 8 * (idx % CH));
                 vreg[i] = *(const u32x4_t*)(Vg + (size_t)r * HD + 8 * (idx % CH));
             }
@@ -213,16 +162,38 @@ __global__ __launch_bounds__(NTHREADS, RT_FA_MIN_BLOCKS) void flash_fwd_bf16_ker
             }
         }
     };
-    if (n_steps > 0) {
-        prefetch(0);
-        stage(0);
-        if (n_steps > 1) prefetch(BC);
-    }
-    // Drain every outstanding global load once, here: inside the loop the only loads in flight are then
-    // the tile prefetches, and the first MFMA of a step (which reads the Q registers) no longer has to
-    // wait for the prefetch issued just before it.
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    __syncthreads();
+    // job index of round i for this worker, or -1
+    auto job_of_round = [&](int i) {
+        int j = i * W + ((i & 1) ? (W - 1 - w) : w);
+        return j < n_jobs ? j : -1;
+    };
+    // point the state at job j and request its queries and first key tile
+    auto begin_job = [&](int j) {
+        const int rank = j / n_bh, bh = j - rank * n_bh;
+        const int qtile = n_qtiles - 1 - rank;  // rank 0 = the longest causal rows
+        const int b = bh / p.heads, h = bh - b * p.heads;
+        const int kvh = h / p.group;
+        q0 = qtile * BR;
+        qw = q0 + wave * 32;
+        q_row = qw + col;
+        const uint16_t* Qg = p.q + ((size_t)b * p.heads + h) * (size_t)N * HD;
+        Kg = p.k + ((size_t)b * p.kv_heads + kvh) * (size_t)N * HD;
+        Vg = p.v + ((size_t)b * p.kv_heads + kvh) * (size_t)N * HD;
+        Og = p.out + ((size_t)b * p.heads + h) * (size_t)N * HD;
+        n_keys = N;  // keys that exist for this sequence
+        if (MODE == kMaskVarlenCausal) n_keys = min(N, max(0, p.seq_lens[b]));
+        int kv_end = n_keys;
+        if (kCausal) kv_end = min(n_keys, q0 + BR);
+        if (MODE == kMaskVarlenCausal && q0 >= n_keys) kv_end = 0;  // a tile of padded query rows
+        n_steps = (kv_end + BC - 1) / BC;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            u32x4_t z = {0u, 0u, 0u, 0u};
+            if (q_row < N) z = *(const u32x4_t*)(Qg + (size_t)q_row * HD + 16 * ks + 8 * hh);
+            qreg[ks] = __builtin_bit_cast(bf16x8_t, z);
+        }
+        if (n_steps > 0) prefetch(0);
+    };
 
     // per-lane part of the transposing V read: lane -> (row within a group of 4, 4-column chunk)
     const int tr_off = ((lane & 15) >> 2) * LDV + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + 4 * hh * LDV;
@@ -323,54 +294,79 @@ __global__ __launch_bounds__(NTHREADS, RT_FA_MIN_BLOCKS) void flash_fwd_bf16_ker
         RT_PHASE(7);
     };
 
-    for (int step = 0; step < n_steps; step++) {
-        const int kv0 = step * BC;
-        const int buf = step & 1;
-        RT_PHASE(0);
-        // tile step+1 goes into the other buffer (last read in step-1, before the barrier that ended it)
-        if (step + 1 < n_steps) {
-            stage(buf ^ 1);
-            if (step + 2 < n_steps) prefetch(kv0 + 2 * BC);
+    int round = 0;
+    int job = job_of_round(0);
+    if (job >= 0) begin_job(job);
+    while (job >= 0) {
+#pragma unroll
+        for (int t = 0; t < DT; t++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc_o[t][i] = 0.0f;
+        m_run = neg_inf();
+        l_run = 0.0f;
+        if (n_steps > 0) {
+            stage(0);
+            if (n_steps > 1) prefetch(BC);
         }
-        if (!(kCausal && kv0 > qw + 31)) {  // wave-uniform: this wave's rows see something of the tile
-            bool need_mask = (kv0 + BC > n_keys);
-            if (kCausal) need_mask |= (kv0 + BC - 1 > qw);
-            if (MODE == kMaskPadding) need_mask = true;
-#ifdef RT_EXP_NOMASK
-            need_mask = false;
-#endif
-            if (need_mask)
-                tile(Ks[buf], Vs[buf], kv0, std::true_type{});
-            else
-                tile(Ks[buf], Vs[buf], kv0, std::false_type{});
-        }
-        RT_PHASE(8);
-        __syncthreads();  // tile `buf` is free again; tile buf^1 is complete
-        RT_PHASE(9);
-    }
+        // Drain every outstanding global load once per job, here: inside the loop the only loads in
+        // flight are then the tile prefetches, and the first MFMA of a step (which reads the Q registers)
+        // does not wait for the prefetch issued just before it.
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
 
-    RT_PHASE_DUMP;
-    // ---- normalise and store.  acc_o[dt][i] = O^T[d = 32dt + 8(i/4) + 4hh + i%4][q_row]
-    float l = sum_with_other_half(l_run);
-    bool good = (l > 0.0f) && (l < __uint_as_float(0x7f800000u)) && !poison;
-    float inv_l = 1.0f / l;
-    if (q_row < N) {
-        const bool padded_row = (MODE == kMaskVarlenCausal) && (q_row >= n_keys);
-#pragma unroll
-        for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                float o[4];
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    float x = good ? acc_o[dt][4 * j + r] * inv_l : quiet_nan();
-                    if (padded_row) x = p.zero_padded_rows ? 0.0f : quiet_nan();
-                    o[r] = x;
-                }
-                u32x2_t w = {cvt_pk_bf16(o[0], o[1]), cvt_pk_bf16(o[2], o[3])};
-                *(u32x2_t*)(Og + (size_t)q_row * HD + dt * 32 + 8 * j + 4 * hh) = w;
+        for (int step = 0; step < n_steps; step++) {
+            const int kv0 = step * BC;
+            const int buf = step & 1;
+            RT_PHASE(0);
+            // tile step+1 goes into the other buffer (last read in step-1, before the barrier that ended it)
+            if (step + 1 < n_steps) {
+                stage(buf ^ 1);
+                if (step + 2 < n_steps) prefetch(kv0 + 2 * BC);
             }
+            if (!(kCausal && kv0 > qw + 31)) {  // wave-uniform: this wave's rows see something of the tile
+                bool need_mask = (kv0 + BC > n_keys);
+                if (kCausal) need_mask |= (kv0 + BC - 1 > qw);
+                if (MODE == kMaskPadding) need_mask = true;
+                if (need_mask)
+                    tile(Ks[buf], Vs[buf], kv0, std::true_type{});
+                else
+                    tile(Ks[buf], Vs[buf], kv0, std::false_type{});
+            }
+            RT_PHASE(8);
+            __syncthreads();  // tile `buf` is free again; tile buf^1 is complete
+            RT_PHASE(9);
+        }
+
+        // ---- this job's output rows: remember where they go, then turn the loads over to the next job
+        // so that its queries and first key tile travel while the output is normalised and stored
+        uint16_t* __restrict__ out_row = Og + (size_t)q_row * HD;
+        const bool row_ok = q_row < N;
+        const bool padded_row = (MODE == kMaskVarlenCausal) && (q_row >= n_keys);
+        job = job_of_round(++round);
+        if (job >= 0) begin_job(job);
+
+        // acc_o[dt][i] = O^T[d = 32dt + 8(i/4) + 4hh + i%4][q_row]
+        float l = sum_with_other_half(l_run);
+        bool good = (l > 0.0f) && (l < __uint_as_float(0x7f800000u)) && !poison;
+        float inv_l = 1.0f / l;
+        if (row_ok) {
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    float o[4];
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        float x = good ? acc_o[dt][4 * j + r] * inv_l : quiet_nan();
+                        if (padded_row) x = p.zero_padded_rows ? 0.0f : quiet_nan();
+                        o[r] = x;
+                    }
+                    u32x2_t wv = {cvt_pk_bf16(o[0], o[1]), cvt_pk_bf16(o[2], o[3])};
+                    *(u32x2_t*)(out_row + dt * 32 + 8 * j + 4 * hh) = wv;
+                }
+        }
     }
+    RT_PHASE_DUMP;
 }
 
 template <int HD>
@@ -392,7 +388,9 @@ hipError_t launch_hd(hipStream_t stream, const FlashBf16Params& p, dim3 grid, di
 hipError_t launch_flash_bf16(hipStream_t stream, const FlashBf16Params& p) {
     if (p.batch == 0 || p.heads == 0 || p.seq == 0) return hipSuccess;
     int n_qtiles = (p.seq + BR - 1) / BR;
-    dim3 grid((unsigned)((size_t)n_qtiles * p.batch * p.heads)), block(NTHREADS);
+    size_t n_jobs = (size_t)n_qtiles * p.batch * p.heads;
+    size_t workers = p.n_workers > 0 ? (size_t)p.n_workers : 256;
+    dim3 grid((unsigned)(n_jobs < workers ? n_jobs : workers)), block(NTHREADS);
     switch (p.dim) {
         case 64: return launch_hd<64>(stream, p, grid, block);
         case 128: return launch_hd<128>(stream, p, grid, block);

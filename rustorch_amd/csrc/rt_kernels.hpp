@@ -37,6 +37,7 @@ struct FlashBf16Params {
     int ref_bc;
     int zero_padded_rows;
     float scale_log2e;  // (1/sqrt(dim)) * log2(e)
+    int n_workers;      // persistent workgroups to launch: the number of CUs
 };
 // dim in {64, 128}.
 hipError_t launch_flash_bf16(hipStream_t stream, const FlashBf16Params& p);
