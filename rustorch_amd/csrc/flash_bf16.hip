@@ -2,12 +2,14 @@
 // flash_forward_masked (crates/rustorch-attention/src/cpu_forward.rs:193-425) for bf16
 // tensors: bf16 in, f32 accumulation on the matrix cores, bf16 out rounded once.
 //
-// Workgroup = 8 wavefronts (two per SIMD) = 256 query rows of one (batch, head); each wave owns 32
-// rows and the workgroup walks the keys 64 at a time through a double-buffered LDS tile.  A wave
-// treats the tile as two 32-key items and pipelines them so that the matrix cores and the vector
-// ALU work at the same time:
+// Persistent grid, one workgroup of 8 wavefronts (two per SIMD) per CU.  A job is 256 query rows of
+// one (batch, head): each wave owns 32 rows, and the workgroup walks the keys 128 at a time through a
+// double-buffered LDS tile that the waves fill with direct global->LDS loads (no registers, no LDS
+// store instructions).  A wave treats the tile as four 32-key items and pipelines them so that the
+// matrix cores and the vector ALU work at the same time:
 //
-//   S0 = K0.Q^T | softmax(S0) with S1 = K1.Q^T in flight | softmax(S1) with O += V0^T.P0 in flight | O += V1^T.P1
+//   S(i+1) = K(i+1).Q^T  in flight while  P(i) = exp2(S(i) - m)      is computed, then
+//   O     += V(i)^T.P(i) in flight while  m   = max(m, rowmax S(i+1)) is computed.
 //
 //   S^T[kv, q]  = K[kv, :] . Q[q, :]      v_mfma_f32_32x32x16_bf16, A = K tile (LDS), B = Q (registers)
 //   online softmax on S^T: lane l holds 16 scores of query row l % 32, so row max / row sum are
@@ -20,11 +22,13 @@
 // the 16 contraction slots; the V operand is fetched with the same permutation, so P is never
 // written to LDS.
 //
+// LDS tiles are unpadded; bank conflicts are avoided by an XOR swizzle of the 16-byte slots of a row,
+// applied on the global side of the load (lane l of a load instruction always lands at LDS byte 16*l
+// of its 1 KB block, so it fetches the slot that belongs there).
+//
 // The running max is only raised (and O, l rescaled) when some row's item max exceeds it by more
 // than 2^8 in the exp2 domain: P then stays below 2^8, harmless in f32/bf16, and the rescale of the
 // 64 O registers leaves the steady-state loop.
-#include <type_traits>
-
 #include "rt_common.hpp"
 #include "rt_kernels.hpp"
 
@@ -39,15 +43,11 @@ namespace rt {
 
 namespace {
 
-#ifndef RT_FA_WAVES
-#define RT_FA_WAVES 8
-#endif
-#ifndef RT_FA_MIN_BLOCKS
-#define RT_FA_MIN_BLOCKS 1
-#endif
-constexpr int NTHREADS = 64 * RT_FA_WAVES;
-constexpr int BR = 32 * RT_FA_WAVES;  // query rows per workgroup
-constexpr int BC = 64;                // key rows per step
+constexpr int NWAVES = 8;
+constexpr int NTHREADS = 64 * NWAVES;
+constexpr int BR = 32 * NWAVES;  // query rows per job
+constexpr int BC = 128;          // key rows per step (one barrier per step)
+constexpr int NITEMS = BC / 32;  // 32-key items per step
 constexpr float kLazyLog2 = 8.0f;
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
@@ -63,55 +63,78 @@ __device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
 // bytes addressed by lanes 4e + j/4, e = 0..3.  With lane 4e + c pointing at row k0+e, columns
 // n0+4c.., lane j ends up with column n0+j of rows k0..k0+3: a contraction-major MFMA operand
 // fragment out of a row-major tile.
-__device__ __forceinline__ u32x2_t lds_read_tr16(const uint16_t* p) {
+__device__ __forceinline__ u32x2_t lds_read_tr16(const unsigned char* p) {
     s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3)))*)(p));
     return __builtin_bit_cast(u32x2_t, v);
 }
 
+// plain v_max_f32: returns the non-NaN operand, without the canonicalising extra instruction fmaxf gets
+__device__ __forceinline__ float vmax(float a, float b) {
+    float d;
+    asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+}
 // max / sum of a value with the one held by lane l ^ 32, without going through LDS:
 // v_permlane32_swap leaves (lower half, lower half) in one register and (upper, upper) in the other.
 __device__ __forceinline__ float max_with_other_half(float x) {
     auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    return vmax(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 __device__ __forceinline__ float sum_with_other_half(float x) {
     auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
-
 __device__ __forceinline__ float max16(const f32x16_t& s) {
-    float a = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
-    float b = fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7]));
-    float c = fmaxf(fmaxf(s[8], s[9]), fmaxf(s[10], s[11]));
-    float d = fmaxf(fmaxf(s[12], s[13]), fmaxf(s[14], s[15]));
-    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+    float a = vmax(vmax(s[0], s[1]), vmax(s[2], s[3]));
+    float b = vmax(vmax(s[4], s[5]), vmax(s[6], s[7]));
+    float c = vmax(vmax(s[8], s[9]), vmax(s[10], s[11]));
+    float d = vmax(vmax(s[12], s[13]), vmax(s[14], s[15]));
+    return vmax(vmax(a, b), vmax(c, d));
+}
+
+// 16 bytes per lane from global memory straight into LDS: lane l lands at lds_block + 16*l (lds_block
+// is wave-uniform and goes through M0).  Issued as inline assembly so that the compiler's counter
+// bookkeeping does not treat every later LDS read as dependent on it: completion is awaited explicitly
+// (s_waitcnt vmcnt(0) before the barrier that publishes the tile).  Loads the compiler does not know of
+// can only make its own vmcnt waits longer, never shorter, because the counter retires in order.
+__device__ __forceinline__ void load_to_lds(const void* gptr, unsigned char* lds_block) {
+    const uint32_t lds_addr = __builtin_amdgcn_readfirstlane(
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds_block);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(gptr) : "memory");
 }
 
 template <int HD, int MODE>
-__global__ __launch_bounds__(NTHREADS, RT_FA_MIN_BLOCKS) void flash_fwd_bf16_kernel(FlashBf16Params p) {
-    constexpr int LDK = HD + 8;   // K row stride (bf16): +16 B, 16 rows x 16 B tile all 64 banks
-    constexpr int LDV = HD + 32;  // V row stride: = 64 B (mod 256 B), 4 rows x 64 B tile all 64 banks
-    constexpr int KS = HD / 16;   // contraction steps of the score product
-    constexpr int DT = HD / 32;   // 32-row tiles of O^T
-    constexpr int CH = HD / 8;    // 16-byte chunks per row
-    constexpr int NCHUNK = BC * CH;  // 16-byte chunks in one K (or V) tile
-    constexpr int PASSES = (NCHUNK + NTHREADS - 1) / NTHREADS;
+__global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Params p) {
+    constexpr int ROWB = HD * 2;             // bytes per row
+    constexpr int SPR = HD / 8;              // 16-byte slots per row
+    constexpr int RPI = 64 / SPR;            // rows covered by one wave load instruction (1 KB)
+    constexpr int TILE_B = BC * ROWB;        // bytes of one K (or V) tile
+    constexpr int NLD = BC / RPI / NWAVES;   // load instructions per wave, per matrix, per tile
+    constexpr int KS = HD / 16;              // contraction steps of the score product
+    constexpr int DT = HD / 32;              // 32-row tiles of O^T
     constexpr bool kCausal = (MODE == kMaskCausal) || (MODE == kMaskVarlenCausal);
+    static_assert(NLD >= 1 && BC % (RPI * NWAVES) == 0, "tile load split");
 
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[2][BC * LDK];
-    __shared__ __attribute__((aligned(16))) uint16_t Vs[2][BC * LDV];
+    // [stage 0: K, V][stage 1: K, V]
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * TILE_B];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, hh = lane >> 5;
     RT_PHASE_DECL;
 
-    // ---- jobs.  A job is one (batch*head, 256-row query tile); the grid is persistent (one
-    // workgroup per CU) and every workgroup walks its own list.  Jobs are ranked from the longest
-    // (causal) rows down and dealt to the workers in boustrophedon order (round i: job i*W + w, or
-    // i*W + W-1-w when i is odd), so every worker gets the same number of key tiles to within one job,
-    // starts on a long job and ends on a short one.  Nothing is relaunched between jobs: the next
-    // job's queries and first key tile are requested before the current job's output is stored.
+    // slot swizzles (see the header): K rows are read 16 at a time at one slot (b128), V rows 4 at a
+    // time over 4 adjacent slots (transposing b64 reads)
+    auto swz_k = [](int r) { return HD == 128 ? (r & 15) : ((r >> 1) & 7); };
+    auto swz_v = [](int r) { return HD == 128 ? 4 * (r & 3) : 4 * ((r >> 1) & 1); };
+    auto swz_o = [](int r) { return r & (SPR - 1); };
+
+    // ---- jobs.  A job is one (batch*head, 256-row query tile); every workgroup walks its own list.
+    // Jobs are ranked from the longest (causal) rows down and dealt to the workers in boustrophedon
+    // order (round i: job i*W + w, or i*W + W-1-w when i is odd), so every worker gets the same number
+    // of key tiles to within one job, starts on a long job and ends on a short one.  Nothing is
+    // relaunched between jobs: the next job's queries and first key tile are requested before the
+    // current job's output is stored.
     const int N = p.seq;
     const int n_qtiles = (N + BR - 1) / BR;
     const int n_bh = p.batch * p.heads;
@@ -128,38 +151,50 @@ __global__ __launch_bounds__(NTHREADS, RT_FA_MIN_BLOCKS) void flash_fwd_bf16_ker
         poison = !__any(any);
     }
 
+    // ---- per-lane constants of the tile loads: instruction n of this wave fills LDS block
+    // wave + NWAVES*n (rows RPI*block ..), lane l fetching the slot that belongs at byte 16*l
+    int ld_row[NLD];
+    uint32_t ld_k[NLD], ld_v[NLD];  // byte offset inside a global row
+#pragma unroll
+    for (int n = 0; n < NLD; n++) {
+        const int r = (wave + NWAVES * n) * RPI + lane / SPR, s = lane % SPR;
+        ld_row[n] = r;
+        ld_k[n] = (uint32_t)((s ^ swz_k(r)) * 16);
+        ld_v[n] = (uint32_t)((s ^ swz_v(r)) * 16);
+    }
+    // ---- per-lane constants of the operand reads
+    uint32_t koff[KS];  // K A-operand: row col of an item, slot (2ks + hh)
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) koff[ks] = (uint32_t)(col * ROWB + (((2 * ks + hh) ^ swz_k(col)) * 16));
+    uint32_t voff[DT];  // V^T A-operand: lane j of a 16-group addresses row j/4 (+4hh), 4 columns
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+        const int j = lane & 15, grp = (lane >> 4) & 1, row = (j >> 2) + 4 * hh;
+        const int slot = (4 * dt + 2 * grp + ((j & 3) >> 1)) ^ swz_v(row);
+        voff[dt] = (uint32_t)(row * ROWB + slot * 16 + 8 * (j & 1));
+    }
+
     // state of the current job
     int q0, qw, q_row, n_keys, n_steps;
-    const uint16_t* __restrict__ Kg;
-    const uint16_t* __restrict__ Vg;
+    const unsigned char* __restrict__ Kg;
+    const unsigned char* __restrict__ Vg;
     uint16_t* __restrict__ Og;
     bf16x8_t qreg[KS];  // Q as B operand, in registers for the whole job
-    u32x4_t kreg[PASSES], vreg[PASSES];
     f32x16_t acc_o[DT];
     float m_run, l_run;
 
-    // ---- global -> register prefetch of one K/V tile, then register -> LDS.  Rows past the last key
-    // are read from the last key instead (no branch); they are masked in the score tile, so their
-    // probabilities are zero.
-    auto prefetch = [&](int kv0) {
+    // request key tile `kv0` into stage `st`.  Rows past the last key are read from the last key
+    // instead; they are masked in the score tile, so their probabilities are zero.
+    auto load_tile = [&](int kv0, int st) {
+        unsigned char* kdst = lds + st * 2 * TILE_B;
+        unsigned char* vdst = kdst + TILE_B;
 #pragma unroll
-        for (int i = 0; i < PASSES; i++) {
-            const int idx = tid + i * NTHREADS;
-            if (NCHUNK % NTHREADS == 0 || idx < NCHUNK) {
-                int r = min(kv0 + idx / CH, n_keys - 1);
-                kreg[i] = *(const u32x4_t*)(Kg + (size_t)r * HD + 8 * (idx % CH));
-                vreg[i] = *(const u32x4_t*)(Vg + (size_t)r * HD + 8 * (idx % CH));
-            }
-        }
-    };
-    auto stage = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < PASSES; i++) {
-            const int idx = tid + i * NTHREADS;
-            if (NCHUNK % NTHREADS == 0 || idx < NCHUNK) {
-                *(u32x4_t*)(&Ks[buf][(idx / CH) * LDK + 8 * (idx % CH)]) = kreg[i];
-                *(u32x4_t*)(&Vs[buf][(idx / CH) * LDV + 8 * (idx % CH)]) = vreg[i];
-            }
+        for (int n = 0; n < NLD; n++) {
+            const int r = min(kv0 + ld_row[n], n_keys - 1);
+            const size_t row_off = (size_t)r * ROWB;
+            const int blk = (wave + NWAVES * n) * 1024;
+            load_to_lds(Kg + row_off + ld_k[n], kdst + blk);
+            load_to_lds(Vg + row_off + ld_v[n], vdst + blk);
         }
     };
     // job index of round i for this worker, or -1
@@ -167,7 +202,7 @@ __global__ __launch_bounds__(NTHREADS, RT_FA_MIN_BLOCKS) void flash_fwd_bf16_ker
         int j = i * W + ((i & 1) ? (W - 1 - w) : w);
         return j < n_jobs ? j : -1;
     };
-    // point the state at job j and request its queries and first key tile
+    // point the state at job j and request its queries and first key tile (into stage 0)
     auto begin_job = [&](int j) {
         const int rank = j / n_bh, bh = j - rank * n_bh;
         const int qtile = n_qtiles - 1 - rank;  // rank 0 = the longest causal rows
@@ -177,8 +212,8 @@ __global__ __launch_bounds__(NTHREADS, RT_FA_MIN_BLOCKS) void flash_fwd_bf16_ker
         qw = q0 + wave * 32;
         q_row = qw + col;
         const uint16_t* Qg = p.q + ((size_t)b * p.heads + h) * (size_t)N * HD;
-        Kg = p.k + ((size_t)b * p.kv_heads + kvh) * (size_t)N * HD;
-        Vg = p.v + ((size_t)b * p.kv_heads + kvh) * (size_t)N * HD;
+        Kg = (const unsigned char*)(p.k + ((size_t)b * p.kv_heads + kvh) * (size_t)N * HD);
+        Vg = (const unsigned char*)(p.v + ((size_t)b * p.kv_heads + kvh) * (size_t)N * HD);
         Og = p.out + ((size_t)b * p.heads + h) * (size_t)N * HD;
         n_keys = N;  // keys that exist for this sequence
         if (MODE == kMaskVarlenCausal) n_keys = min(N, max(0, p.seq_lens[b]));
@@ -192,19 +227,19 @@ __global__ __launch_bounds__(NTHREADS, RT_FA_MIN_BLOCKS) void flash_fwd_bf16_ker
             if (q_row < N) z = *(const u32x4_t*)(Qg + (size_t)q_row * HD + 16 * ks + 8 * hh);
             qreg[ks] = __builtin_bit_cast(bf16x8_t, z);
         }
-        if (n_steps > 0) prefetch(0);
+        if (n_steps > 0) load_tile(0, 0);
     };
 
-    // per-lane part of the transposing V read: lane -> (row within a group of 4, 4-column chunk)
-    const int tr_off = ((lane & 15) >> 2) * LDV + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + 4 * hh * LDV;
-    const int k_off = col * LDK + 8 * hh;
-
     // ---- pieces of the per-item pipeline -------------------------------------------------------------
-    // scores of one 32-key item: 8 (HD=128) MFMAs accumulating over the head dim
-    auto qk = [&](const uint16_t* Kb, int t, f32x16_t& s) {
+    // scores of one 32-key item: KS MFMAs accumulating over the head dim
+    auto qk = [&](const unsigned char* Kb, int t, f32x16_t& s) {
         bf16x8_t a[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) a[ks] = *(const bf16x8_t*)(Kb + 32 * t * LDK + k_off + 16 * ks);
+#ifdef RT_EXP_NOK
+        for (int ks = 0; ks < KS; ks++) a[ks] = qreg[(ks + t + 1) % KS];
+#else
+        for (int ks = 0; ks < KS; ks++) a[ks] = *(const bf16x8_t*)(Kb + 32 * t * ROWB + koff[ks]);
+#endif
 #pragma unroll
         for (int i = 0; i < 16; i++) s[i] = 0.0f;
 #pragma unroll
@@ -223,8 +258,13 @@ __global__ __launch_bounds__(NTHREADS, RT_FA_MIN_BLOCKS) void flash_fwd_bf16_ker
     // raise the running max when it pays (wave-uniform branch; no MFMA inside)
     auto update_max = [&](const f32x16_t& s) {
         float m_item = max_with_other_half(max16(s));
+#ifdef RT_EXP_NORESCALE
+        if (m_run == neg_inf()) m_run = 0.0f;
+        if (false) {
+#else
         if (__any(m_item > m_run + lazy_raw)) {
-            float m_new = fmaxf(m_run, m_item);
+#endif
+            float m_new = vmax(m_run, m_item);
             float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
             float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);  // m_run = -inf -> 0
             m_run = m_new;
@@ -241,7 +281,11 @@ __global__ __launch_bounds__(NTHREADS, RT_FA_MIN_BLOCKS) void flash_fwd_bf16_ker
         float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int i = 0; i < 16; i++) {
+#ifdef RT_EXP_NOEXP
+            float e = __builtin_fmaf(s[i], c, -mc);
+#else
             float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c, -mc));
+#endif
             s[i] = e;
             part[i & 3] += e;
         }
@@ -255,43 +299,70 @@ __global__ __launch_bounds__(NTHREADS, RT_FA_MIN_BLOCKS) void flash_fwd_bf16_ker
         }
     };
     // O^T += V^T . P^T for one item: 2 contraction steps of 16 keys x DT output tiles
-    auto pv = [&](const uint16_t* Vb, int t, const bf16x8_t (&pB)[2]) {
+    auto pv = [&](const unsigned char* Vb, int t, const bf16x8_t (&pB)[2]) {
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             // contraction slots 0-3 of this lane: keys kv_lo..kv_lo+3; slots 4-7: kv_lo+8..kv_lo+11
-            const uint16_t* vp = Vb + (32 * t + 16 * u) * LDV + tr_off;
+            const unsigned char* vp = Vb + (32 * t + 16 * u) * ROWB;
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
-                u32x2_t lo = lds_read_tr16(vp + dt * 32);
-                u32x2_t hi = lds_read_tr16(vp + dt * 32 + 8 * LDV);
+#ifdef RT_EXP_HALFV
+                u32x2_t lo = lds_read_tr16(vp + voff[dt & ~1]);
+                u32x2_t hi = lo;
+#elif defined(RT_EXP_NOV)
+                u32x2_t lo = {koff[0] + dt, koff[1]}, hi = {koff[2], koff[3] + u};
+#else
+                u32x2_t lo = lds_read_tr16(vp + voff[dt]);
+                u32x2_t hi = lds_read_tr16(vp + voff[dt] + 8 * ROWB);
+#endif
                 u32x4_t av = {lo[0], lo[1], hi[0], hi[1]};
                 acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), pB[u],
                                                                     acc_o[dt], 0, 0, 0);
             }
         }
     };
-    // one 64-key tile; NEED_MASK is a compile-time flag so the steady state carries no mask code
-    auto tile = [&](const uint16_t* Kb, const uint16_t* Vb, int kv0, auto need_mask_tag) {
-        constexpr bool NEED_MASK = decltype(need_mask_tag)::value;
-        f32x16_t s0, s1;
-        bf16x8_t p0[2], p1[2];
+    // One 128-key tile = up to four 32-key items.
+    // Fast path: all four items visible and unmasked.  Straight-line code, so that each product sits in
+    // the same scheduling region as the vector work it is meant to hide (an MFMA only overlaps with the
+    // vector instructions issued right behind it; a branch between them would serialise the two).
+    auto tile_full = [&](const unsigned char* Kb, const unsigned char* Vb) {
+        f32x16_t s_a, s_b;
+        bf16x8_t pB[2];
         RT_PHASE(1);
-        qk(Kb, 0, s0);
-        if (NEED_MASK) mask_item(kv0, s0);
+        qk(Kb, 0, s_a);
+        update_max(s_a);
         RT_PHASE(2);
-        update_max(s0);
+        qk(Kb, 1, s_b);  exp_item(s_a, pB);      // scores of item 1 | probabilities of item 0
+        pv(Vb, 0, pB);   update_max(s_b);        // item 0 into O    | max of item 1 (P(i) is relative to the max
+        qk(Kb, 2, s_a);  exp_item(s_b, pB);      //                  |   BEFORE item i+1 raises it: accumulate first)
+        pv(Vb, 1, pB);   update_max(s_a);
+        qk(Kb, 3, s_b);  exp_item(s_a, pB);
+        pv(Vb, 2, pB);   update_max(s_b);
+        exp_item(s_b, pB);
+        pv(Vb, 3, pB);
         RT_PHASE(3);
-        qk(Kb, 1, s1);       // matrix cores: scores of item 1 ...
-        exp_item(s0, p0);    // ... vector ALU: probabilities of item 0
-        if (NEED_MASK) mask_item(kv0 + 32, s1);
-        RT_PHASE(4);
-        pv(Vb, 0, p0);       // matrix cores: item 0 into O (P0 is relative to the max BEFORE item 1 raises it,
-        update_max(s1);      //   so it must be accumulated before a rescale) ... vector ALU: max of item 1
-        RT_PHASE(5);
-        exp_item(s1, p1);    //   and its probabilities
-        RT_PHASE(6);
-        pv(Vb, 1, p1);
-        RT_PHASE(7);
+    };
+    // General path: n_act items are visible to this wave (a causal mask hides the rest); only the last
+    // visible one can need masking (diagonal or ragged end), unless the mask is a keep vector.
+    auto tile_part = [&](const unsigned char* Kb, const unsigned char* Vb, int kv0, int n_act, bool mask_last) {
+        f32x16_t s_a, s_b;
+        bf16x8_t pB[2];
+        qk(Kb, 0, s_a);
+        if (MODE == kMaskPadding || (mask_last && n_act == 1)) mask_item(kv0, s_a);
+        update_max(s_a);
+#pragma unroll
+        for (int i = 0; i < NITEMS; i++) {
+            f32x16_t& s_cur = (i & 1) ? s_b : s_a;
+            f32x16_t& s_nxt = (i & 1) ? s_a : s_b;
+            const bool more = i + 1 < n_act;  // wave-uniform
+            if (more) qk(Kb, i + 1, s_nxt);
+            exp_item(s_cur, pB);
+            if (more && (MODE == kMaskPadding || (mask_last && i + 2 == n_act)))
+                mask_item(kv0 + 32 * (i + 1), s_nxt);
+            pv(Vb, i, pB);
+            if (!more) break;
+            update_max(s_nxt);
+        }
     };
 
     int round = 0;
@@ -304,67 +375,71 @@ __global__ __launch_bounds__(NTHREADS, RT_FA_MIN_BLOCKS) void flash_fwd_bf16_ker
             for (int i = 0; i < 16; i++) acc_o[t][i] = 0.0f;
         m_run = neg_inf();
         l_run = 0.0f;
-        if (n_steps > 0) {
-            stage(0);
-            if (n_steps > 1) prefetch(BC);
-        }
-        // Drain every outstanding global load once per job, here: inside the loop the only loads in
-        // flight are then the tile prefetches, and the first MFMA of a step (which reads the Q registers)
-        // does not wait for the prefetch issued just before it.
+        // the queries and tile 0 have landed; the barrier also ends the previous job's use of LDS
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
+        RT_PHASE(10);
 
         for (int step = 0; step < n_steps; step++) {
             const int kv0 = step * BC;
-            const int buf = step & 1;
+            const int st = step & 1;
             RT_PHASE(0);
-            // tile step+1 goes into the other buffer (last read in step-1, before the barrier that ended it)
-            if (step + 1 < n_steps) {
-                stage(buf ^ 1);
-                if (step + 2 < n_steps) prefetch(kv0 + 2 * BC);
-            }
-            if (!(kCausal && kv0 > qw + 31)) {  // wave-uniform: this wave's rows see something of the tile
-                bool need_mask = (kv0 + BC > n_keys);
-                if (kCausal) need_mask |= (kv0 + BC - 1 > qw);
-                if (MODE == kMaskPadding) need_mask = true;
-                if (need_mask)
-                    tile(Ks[buf], Vs[buf], kv0, std::true_type{});
+            // tile step+1 goes into the other stage (last read in step-1, before the barrier that ended it)
+            if (step + 1 < n_steps) load_tile(kv0 + BC, st ^ 1);
+            int n_act = NITEMS;
+            if (kCausal) n_act = (kv0 > qw + 31) ? 0 : min(NITEMS, (qw + 31 - kv0) / 32 + 1);  // items starting at or before the wave's last row
+            n_act = min(n_act, (n_keys - kv0 + 31) / 32);                // items that hold an existing key
+            if (n_act > 0) {
+                const int last_kv = kv0 + 32 * n_act - 1;  // last key of the last visible item
+                bool mask_last = last_kv >= n_keys;
+                if (kCausal) mask_last |= last_kv > qw;
+                if (MODE != kMaskPadding && n_act == NITEMS && !mask_last)
+                    tile_full(lds + st * 2 * TILE_B, lds + st * 2 * TILE_B + TILE_B);
                 else
-                    tile(Ks[buf], Vs[buf], kv0, std::false_type{});
+                    tile_part(lds + st * 2 * TILE_B, lds + st * 2 * TILE_B + TILE_B, kv0, n_act, mask_last);
             }
             RT_PHASE(8);
-            __syncthreads();  // tile `buf` is free again; tile buf^1 is complete
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // this wave's share of tile step+1 has landed
+            __syncthreads();                      // stage `st` is free again; stage st^1 is complete
             RT_PHASE(9);
         }
 
-        // ---- this job's output rows: remember where they go, then turn the loads over to the next job
-        // so that its queries and first key tile travel while the output is normalised and stored
-        uint16_t* __restrict__ out_row = Og + (size_t)q_row * HD;
-        const bool row_ok = q_row < N;
+        // ---- this job's output.  Stage 1 of LDS is free (the next job's first tile goes to stage 0): each
+        // wave parks its 32 normalised rows there, swizzled, and streams them out as whole rows.
+        const int qw_out = qw;
+        uint16_t* __restrict__ og_out = Og;
         const bool padded_row = (MODE == kMaskVarlenCausal) && (q_row >= n_keys);
         job = job_of_round(++round);
-        if (job >= 0) begin_job(job);
+        if (job >= 0) begin_job(job);  // its loads travel while the output is normalised and stored
 
-        // acc_o[dt][i] = O^T[d = 32dt + 8(i/4) + 4hh + i%4][q_row]
+        // acc_o[dt][i] = O^T[d = 32dt + 8(i/4) + 4hh + i%4][row col of the wave]
         float l = sum_with_other_half(l_run);
         bool good = (l > 0.0f) && (l < __uint_as_float(0x7f800000u)) && !poison;
         float inv_l = 1.0f / l;
-        if (row_ok) {
+        unsigned char* obuf = lds + 2 * TILE_B + wave * 32 * ROWB;
 #pragma unroll
-            for (int dt = 0; dt < DT; dt++)
+        for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    float o[4];
+            for (int j = 0; j < 4; j++) {
+                float o[4];
 #pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        float x = good ? acc_o[dt][4 * j + r] * inv_l : quiet_nan();
-                        if (padded_row) x = p.zero_padded_rows ? 0.0f : quiet_nan();
-                        o[r] = x;
-                    }
-                    u32x2_t wv = {cvt_pk_bf16(o[0], o[1]), cvt_pk_bf16(o[2], o[3])};
-                    *(u32x2_t*)(out_row + dt * 32 + 8 * j + 4 * hh) = wv;
+                for (int r = 0; r < 4; r++) {
+                    float x = good ? acc_o[dt][4 * j + r] * inv_l : quiet_nan();
+                    if (padded_row) x = p.zero_padded_rows ? 0.0f : quiet_nan();
+                    o[r] = x;
                 }
+                u32x2_t wv = {cvt_pk_bf16(o[0], o[1]), cvt_pk_bf16(o[2], o[3])};
+                *(u32x2_t*)(obuf + col * ROWB + (((4 * dt + j) ^ swz_o(col)) * 16) + 8 * hh) = wv;
+            }
+        // (the same wave wrote and now reads: no barrier needed, the LDS queue is in order)
+#pragma unroll
+        for (int n = 0; n < 32 / RPI; n++) {
+            const int r = n * RPI + lane / SPR, pos = lane % SPR;
+            u32x4_t v = *(const u32x4_t*)(obuf + r * ROWB + pos * 16);
+            if (qw_out + r < N)
+                *(u32x4_t*)((unsigned char*)og_out + (size_t)(qw_out + r) * ROWB + ((pos ^ swz_o(r)) * 16)) = v;
         }
+        RT_PHASE(11);
     }
     RT_PHASE_DUMP;
 }
