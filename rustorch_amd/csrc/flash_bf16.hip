@@ -131,10 +131,9 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
 
     // ---- jobs.  A job is one (batch*head, 256-row query tile); every workgroup walks its own list.
     // Jobs are ranked from the longest (causal) rows down and dealt to the workers in boustrophedon
-    // order (round i: job i*W + w, or i*W + W-1-w when i is odd), so every worker gets the same number
-    // of key tiles to within one job, starts on a long job and ends on a short one.  Nothing is
-    // relaunched between jobs: the next job's queries and first key tile are requested before the
-    // current job's output is stored.
+    // rows (a row runs left to right, the next right to left), so every worker gets the same number of
+    // key tiles to within one job.  Nothing is relaunched between jobs: the next job's queries and first
+    // key tile are requested before the current job's output is stored.
     const int N = p.seq;
     const int n_qtiles = (N + BR - 1) / BR;
     const int n_bh = p.batch * p.heads;
@@ -197,8 +196,20 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             load_to_lds(Vg + row_off + ld_v[n], vdst + blk);
         }
     };
-    // job index of round i for this worker, or -1
+    // Job of round i for this worker, or -1, as rank * n_bh + bh (rank 0 = the longest causal rows).
+    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  When the heads divide evenly,
+    // XCD x owns the heads bh = x (mod 8) and deals ITS job list (head-major, long rows first) to its own
+    // workers in boustrophedon rows: the workers of an XCD then sit on one or two heads at a time and
+    // share their K/V through that L2, and every worker still gets a long job paired with a short one.
+    const bool by_xcd = ((n_bh & 7) == 0) && ((W & 7) == 0);
     auto job_of_round = [&](int i) {
+        if (by_xcd) {
+            const int C = W >> 3, x = w & 7, cw = w >> 3;
+            const int q = i * C + ((i & 1) ? (C - 1 - cw) : cw);
+            if (q >= n_qtiles * (n_bh >> 3)) return -1;
+            const int head = q / n_qtiles, rank = q - head * n_qtiles;
+            return rank * n_bh + head * 8 + x;
+        }
         int j = i * W + ((i & 1) ? (W - 1 - w) : w);
         return j < n_jobs ? j : -1;
     };
