@@ -30,6 +30,11 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+# HBM bytes per launch of the dominant kernels on the bench workloads, from the rocprofv3 --pmc runs
+# summarised under profiles/ (FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB, the factors a 256 MiB copy reads).
+# Counters cannot be read from inside this process; these are the committed measurements, not live values.
+TRAFFIC_PREFILL_BYTES = (289000 * 2.0 + 139800 * 1.0) * 1024
+TRAFFIC_DECODE_BYTES = (624200 * 2.0 + 5313 * 1.0) * 1024
 
 
 class Hip:
@@ -206,7 +211,7 @@ def main():
                              "cache_sets_rotated": n_sets},
                   "roofline": {"bound": "hbm", "achieved": alg_bytes / (ms_kernel * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                                "unit": "GB/s", "frac": alg_bytes / (ms_kernel * 1e-3) / 1e9 / PEAK_HBM_GBS,
-                               "traffic": None, "kernels": "decode_split + decode_merge (one event pair per step)"}}
+                               "traffic": TRAFFIC_DECODE_BYTES, "kernels": "decode_split + decode_merge (one event pair per step)"}}
         if not args.no_cpu:
             threads = min(oracle.max_threads(), 16)
             got = oracle.bf16_to_f32(d_o.download(np.uint16))
@@ -238,7 +243,7 @@ def main():
                                "f32 accumulation", "flop_convention": "4*B*H*D*N*(N+1)/2 (causal-counted)",
                    "tflops_unmasked_convention_4BHN2D": prefill["tflops_unmasked_convention"]},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "flash_fwd_bf16_kernel<128>",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_PREFILL_BYTES, "kernel": "flash_fwd_bf16_kernel<128>",
                      "kernel_ms_mean": prefill["kernel_ms_mean"], "kernel_ms_median": prefill["kernel_ms_median"],
                      "kernel_ms_min": prefill["kernel_ms_min"]},
     }

@@ -154,7 +154,8 @@ int rt_gqa_decode_online_bf16(void *stream, const void *q, const void *k_cache, 
  * Split-K over the context with a second-pass (m, l, o) merge; `workspace` (device, at least
  * rt_gqa_decode_workspace_bytes(...) bytes, 256-byte aligned) holds the partial results.
  * batch = 1 with kv_lens = [kv_len] is the reference call.  A sequence with kv_lens[b] == 0
- * gives NaN rows (0/0, as crates/rustorch-nn/src/gqa.rs:256 would). */
+ * gives rows of +0.0 (the reference kernel ends with o / fmaxf(l, 1e-12f) = 0, llm_kernels.rs:456;
+ * crates/rustorch-nn/src/gqa.rs:260-261 fills the row with 0 before an empty key loop). */
 int rt_gqa_decode_batched_bf16(void *stream, const void *q, const void *k_cache, const void *v_cache, void *out,
                                const int32_t *kv_lens, int32_t batch, int32_t n_heads, int32_t n_kv,
                                int32_t head_dim, int32_t max_seq, void *workspace, size_t workspace_bytes,

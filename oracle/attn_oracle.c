@@ -581,7 +581,8 @@ RO_EXPORT void ro_gqa_decode_online_bf16(const uint16_t *q, const uint16_t *k_ca
 /* ---- Batched, ragged decode: the CPU path (model.rs:638-668 trim + gqa.rs
  * decode_attn_row) applied per sequence b with its own kv_len, in f32 on
  * bf16-rounded inputs.  q [B,Hq,D] bf16, caches [B,Hkv,max_seq,D] bf16,
- * out [B,Hq,D] f32.  kv_len == 0 leaves the row as 0/0 = NaN, as gqa.rs:256 would. */
+ * out [B,Hq,D] f32.  kv_len == 0 gives a row of zeros: gqa.rs:260-261 fills the row with 0
+ * and the key loop is empty (the bf16 kernel's o / fmaxf(l, 1e-12f) gives the same). */
 RO_EXPORT void ro_gqa_decode_batched_bf16(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache,
                                           const int32_t *kv_lens, float *out, int batch, int n_heads, int n_kv,
                                           int head_dim, int max_seq, int threads) {
