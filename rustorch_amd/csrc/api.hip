@@ -335,6 +335,8 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
         return fail(err, RT_ERR_UNSUPPORTED, -1, 128, shape->dim, "bf16 flash kernels cover dim 64 and 128");
     if ((shape->seq + 127) / 128 * shape->batch * shape->heads > 0x7fffffffull)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    if (shape->seq > (1ull << 23))  // the kernel addresses rows of one (batch, head) slab with 32-bit byte offsets
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 1ull << 23, shape->seq, "bf16 flash kernels cover seq <= 2^23");
     if (!q || !k || !v || !out || (mask == rt::kMaskPadding && !keep) || (mask == rt::kMaskVarlenCausal && !seq_lens))
         return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
     rc = ensure_device(err);

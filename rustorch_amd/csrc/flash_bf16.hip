@@ -92,15 +92,18 @@ __device__ __forceinline__ float max16(const f32x16_t& s) {
     return vmax(vmax(a, b), vmax(c, d));
 }
 
-// 16 bytes per lane from global memory straight into LDS: lane l lands at lds_block + 16*l (lds_block
-// is wave-uniform and goes through M0).  Issued as inline assembly so that the compiler's counter
+// 16 bytes per lane from global memory straight into LDS: lane l lands at LDS byte address
+// lds_block + 16*l (lds_block is wave-uniform and goes through M0).  Issued as inline assembly so that the compiler's counter
 // bookkeeping does not treat every later LDS read as dependent on it: completion is awaited explicitly
 // (s_waitcnt vmcnt(0) before the barrier that publishes the tile).  Loads the compiler does not know of
 // can only make its own vmcnt waits longer, never shorter, because the counter retires in order.
-__device__ __forceinline__ void load_to_lds(const void* gptr, unsigned char* lds_block) {
-    const uint32_t lds_addr = __builtin_amdgcn_readfirstlane(
-        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds_block);
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(gptr) : "memory");
+__device__ __forceinline__ void load_to_lds(const void* base, uint32_t byte_off, uint32_t lds_block) {
+    // base is wave-uniform (a scalar register pair); the lane's unsigned 32-bit byte offset is added to it
+    const uint32_t lds_addr = __builtin_amdgcn_readfirstlane(lds_block);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_addr), "v"(byte_off), "s"(base)
+                 : "memory");
 }
 
 template <int HD, int MODE>
@@ -113,7 +116,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     constexpr int KS = HD / 16;              // contraction steps of the score product
     constexpr int DT = HD / 32;              // 32-row tiles of O^T
     constexpr bool kCausal = (MODE == kMaskCausal) || (MODE == kMaskVarlenCausal);
-    static_assert(NLD >= 1 && BC % (RPI * NWAVES) == 0, "tile load split");
+    static_assert(NLD >= 1 && NLD <= NITEMS && BC % (RPI * NWAVES) == 0, "tile load split");
 
     // [stage 0: K, V][stage 1: K, V]
     __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * TILE_B];
@@ -151,16 +154,12 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     }
 
     // ---- per-lane constants of the tile loads: instruction n of this wave fills LDS block
-    // wave + NWAVES*n (rows RPI*block ..), lane l fetching the slot that belongs at byte 16*l
-    int ld_row[NLD];
-    uint32_t ld_k[NLD], ld_v[NLD];  // byte offset inside a global row
-#pragma unroll
-    for (int n = 0; n < NLD; n++) {
-        const int r = (wave + NWAVES * n) * RPI + lane / SPR, s = lane % SPR;
-        ld_row[n] = r;
-        ld_k[n] = (uint32_t)((s ^ swz_k(r)) * 16);
-        ld_v[n] = (uint32_t)((s ^ swz_v(r)) * 16);
-    }
+    // wave + NWAVES*n (rows RPI*block ..), lane l fetching the slot that belongs at byte 16*l.  The
+    // swizzle only looks at the low bits of the row, which do not depend on n.
+    static_assert((NWAVES * RPI) % 16 == 0, "row swizzles must not depend on the load index");
+    const int ld_row0 = wave * RPI + lane / SPR;
+    const uint32_t ld_k0 = (uint32_t)(((lane % SPR) ^ swz_k(ld_row0)) * 16);  // byte offset inside a global row
+    const uint32_t ld_v0 = (uint32_t)(((lane % SPR) ^ swz_v(ld_row0)) * 16);
     // ---- per-lane constants of the operand reads
     uint32_t koff[KS];  // K A-operand: row col of an item, slot (2ks + hh)
 #pragma unroll
@@ -184,17 +183,22 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
 
     // request key tile `kv0` into stage `st`.  Rows past the last key are read from the last key
     // instead; they are masked in the score tile, so their probabilities are zero.
+    // This wave issues NLD K loads and NLD V loads per tile; load_part issues the n-th pair, so that a
+    // tile's requests can be spread over the step before it (eight waves asking for a whole tile at once
+    // queue up behind the CU's one address unit, and a wave cannot issue anything else while it waits).
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    auto load_part = [&](int n, int kv0, int st) {
+        const uint32_t kdst = lds_base + (uint32_t)(st * 2 * TILE_B + (wave + NWAVES * n) * 1024);
+        int r = kv0 + ld_row0 + NWAVES * RPI * n;
+        asm volatile("" : "+v"(r));  // recompute per call: hoisted copies of these offsets only cost registers
+        r = min(r, n_keys - 1);
+        const uint32_t row_off = (uint32_t)r * ROWB;  // a (b, h) slab is below 4 GiB: seq * dim * 2 < 2^32
+        load_to_lds(Kg, row_off + ld_k0, kdst);
+        load_to_lds(Vg, row_off + ld_v0, kdst + TILE_B);
+    };
     auto load_tile = [&](int kv0, int st) {
-        unsigned char* kdst = lds + st * 2 * TILE_B;
-        unsigned char* vdst = kdst + TILE_B;
 #pragma unroll
-        for (int n = 0; n < NLD; n++) {
-            const int r = min(kv0 + ld_row[n], n_keys - 1);
-            const size_t row_off = (size_t)r * ROWB;
-            const int blk = (wave + NWAVES * n) * 1024;
-            load_to_lds(Kg + row_off + ld_k[n], kdst + blk);
-            load_to_lds(Vg + row_off + ld_v[n], vdst + blk);
-        }
+        for (int n = 0; n < NLD; n++) load_part(n, kv0, st);
     };
     // Job of round i for this worker, or -1, as rank * n_bh + bh (rank 0 = the longest causal rows).
     // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  When the heads divide evenly,
@@ -246,11 +250,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     auto qk = [&](const unsigned char* Kb, int t, f32x16_t& s) {
         bf16x8_t a[KS];
 #pragma unroll
-#ifdef RT_EXP_NOK
-        for (int ks = 0; ks < KS; ks++) a[ks] = qreg[(ks + t + 1) % KS];
-#else
         for (int ks = 0; ks < KS; ks++) a[ks] = *(const bf16x8_t*)(Kb + 32 * t * ROWB + koff[ks]);
-#endif
 #pragma unroll
         for (int i = 0; i < 16; i++) s[i] = 0.0f;
 #pragma unroll
@@ -269,12 +269,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     // raise the running max when it pays (wave-uniform branch; no MFMA inside)
     auto update_max = [&](const f32x16_t& s) {
         float m_item = max_with_other_half(max16(s));
-#ifdef RT_EXP_NORESCALE
-        if (m_run == neg_inf()) m_run = 0.0f;
-        if (false) {
-#else
         if (__any(m_item > m_run + lazy_raw)) {
-#endif
             float m_new = vmax(m_run, m_item);
             float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
             float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);  // m_run = -inf -> 0
@@ -292,11 +287,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-#ifdef RT_EXP_NOEXP
-            float e = __builtin_fmaf(s[i], c, -mc);
-#else
             float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c, -mc));
-#endif
             s[i] = e;
             part[i & 3] += e;
         }
@@ -317,15 +308,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             const unsigned char* vp = Vb + (32 * t + 16 * u) * ROWB;
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
-#ifdef RT_EXP_HALFV
-                u32x2_t lo = lds_read_tr16(vp + voff[dt & ~1]);
-                u32x2_t hi = lo;
-#elif defined(RT_EXP_NOV)
-                u32x2_t lo = {koff[0] + dt, koff[1]}, hi = {koff[2], koff[3] + u};
-#else
                 u32x2_t lo = lds_read_tr16(vp + voff[dt]);
                 u32x2_t hi = lds_read_tr16(vp + voff[dt] + 8 * ROWB);
-#endif
                 u32x4_t av = {lo[0], lo[1], hi[0], hi[1]};
                 acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), pB[u],
                                                                     acc_o[dt], 0, 0, 0);
@@ -336,17 +320,21 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     // Fast path: all four items visible and unmasked.  Straight-line code, so that each product sits in
     // the same scheduling region as the vector work it is meant to hide (an MFMA only overlaps with the
     // vector instructions issued right behind it; a branch between them would serialise the two).
-    auto tile_full = [&](const unsigned char* Kb, const unsigned char* Vb) {
+    auto tile_full = [&](const unsigned char* Kb, const unsigned char* Vb, int kv_next, int st_next) {
         f32x16_t s_a, s_b;
         bf16x8_t pB[2];
         RT_PHASE(1);
+        load_part(0, kv_next, st_next);
         qk(Kb, 0, s_a);
         update_max(s_a);
         RT_PHASE(2);
+        if (NLD > 1) load_part(1 % NLD, kv_next, st_next);
         qk(Kb, 1, s_b);  exp_item(s_a, pB);      // scores of item 1 | probabilities of item 0
         pv(Vb, 0, pB);   update_max(s_b);        // item 0 into O    | max of item 1 (P(i) is relative to the max
+        if (NLD > 2) load_part(2 % NLD, kv_next, st_next);
         qk(Kb, 2, s_a);  exp_item(s_b, pB);      //                  |   BEFORE item i+1 raises it: accumulate first)
         pv(Vb, 1, pB);   update_max(s_a);
+        if (NLD > 3) load_part(3 % NLD, kv_next, st_next);
         qk(Kb, 3, s_b);  exp_item(s_a, pB);
         pv(Vb, 2, pB);   update_max(s_b);
         exp_item(s_b, pB);
@@ -396,7 +384,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             const int st = step & 1;
             RT_PHASE(0);
             // tile step+1 goes into the other stage (last read in step-1, before the barrier that ended it)
-            if (step + 1 < n_steps) load_tile(kv0 + BC, st ^ 1);
+            const bool more = step + 1 < n_steps;
             int n_act = NITEMS;
             if (kCausal) n_act = (kv0 > qw + 31) ? 0 : min(NITEMS, (qw + 31 - kv0) / 32 + 1);  // items starting at or before the wave's last row
             n_act = min(n_act, (n_keys - kv0 + 31) / 32);                // items that hold an existing key
@@ -404,10 +392,16 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
                 const int last_kv = kv0 + 32 * n_act - 1;  // last key of the last visible item
                 bool mask_last = last_kv >= n_keys;
                 if (kCausal) mask_last |= last_kv > qw;
-                if (MODE != kMaskPadding && n_act == NITEMS && !mask_last)
-                    tile_full(lds + st * 2 * TILE_B, lds + st * 2 * TILE_B + TILE_B);
-                else
+                if (MODE != kMaskPadding && n_act == NITEMS && !mask_last) {
+                    // the fast path requests the next tile itself, a quarter per item; with no next tile it
+                    // asks for its own tile again (served from cache into the idle stage) to stay branch-free
+                    tile_full(lds + st * 2 * TILE_B, lds + st * 2 * TILE_B + TILE_B, more ? kv0 + BC : kv0, st ^ 1);
+                } else {
+                    if (more) load_tile(kv0 + BC, st ^ 1);
                     tile_part(lds + st * 2 * TILE_B, lds + st * 2 * TILE_B + TILE_B, kv0, n_act, mask_last);
+                }
+            } else if (more) {
+                load_tile(kv0 + BC, st ^ 1);
             }
             RT_PHASE(8);
             __builtin_amdgcn_s_waitcnt(0x0F70);  // this wave's share of tile step+1 has landed
@@ -421,7 +415,9 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         uint16_t* __restrict__ og_out = Og;
         const bool padded_row = (MODE == kMaskVarlenCausal) && (q_row >= n_keys);
         job = job_of_round(++round);
+        RT_PHASE(4);
         if (job >= 0) begin_job(job);  // its loads travel while the output is normalised and stored
+        RT_PHASE(5);
 
         // acc_o[dt][i] = O^T[d = 32dt + 8(i/4) + 4hh + i%4][row col of the wave]
         float l = sum_with_other_half(l_run);
@@ -442,6 +438,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
                 u32x2_t wv = {cvt_pk_bf16(o[0], o[1]), cvt_pk_bf16(o[2], o[3])};
                 *(u32x2_t*)(obuf + col * ROWB + (((4 * dt + j) ^ swz_o(col)) * 16) + 8 * hh) = wv;
             }
+        RT_PHASE(6);
         // (the same wave wrote and now reads: no barrier needed, the LDS queue is in order)
 #pragma unroll
         for (int n = 0; n < 32 / RPI; n++) {
