@@ -5,11 +5,7 @@
 // Persistent grid, one workgroup of 8 wavefronts (two per SIMD) per CU.  A job is 256 query rows of
 // one (batch, head): each wave owns 32 rows, and the workgroup walks the keys 128 at a time through a
 // double-buffered LDS tile that the waves fill with direct global->LDS loads (no registers, no LDS
-// store instructions).  A wave treats the tile as four 32-key items and pipelines them so that the
-// matrix cores and the vector ALU work at the same time:
-//
-//   S(i+1) = K(i+1).Q^T  in flight while  P(i) = exp2(S(i) - m)      is computed, then
-//   O     += V(i)^T.P(i) in flight while  m   = max(m, rowmax S(i+1)) is computed.
+// store instructions).  A wave treats the tile as four 32-key items:
 //
 //   S^T[kv, q]  = K[kv, :] . Q[q, :]      v_mfma_f32_32x32x16_bf16, A = K tile (LDS), B = Q (registers)
 //   online softmax on S^T: lane l holds 16 scores of query row l % 32, so row max / row sum are
@@ -22,6 +18,18 @@
 // the 16 contraction slots; the V operand is fetched with the same permutation, so P is never
 // written to LDS.
 //
+// Schedule.  A wave can start one instruction every four to five cycles whatever its kind, and a
+// matrix instruction keeps the matrix pipe busy for 32 cycles, so a wave that only multiplies leaves
+// most issue slots free while a wave that only does softmax needs all of them.  The two waves of a SIMD
+// therefore alternate, one cluster apart, with one workgroup barrier per cluster:
+//
+//   C(k): S^T(k) = K(k).Q^T and O^T += V(k-1)^T.P(k-1)^T (16 matrix instructions, operands in registers),
+//         with the LDS reads of the NEXT cluster's operands (V(k), K(k+1)) and the global->LDS requests
+//         of the next tile slotted in between;
+//   S(k): row max, rescale check, P(k) = exp2(..), row sums, conversion to bf16: vector work only.
+//
+// Waves 0-3 run C(k) while waves 4-7 run S(k-1), then they swap.
+//
 // LDS tiles are unpadded; bank conflicts are avoided by an XOR swizzle of the 16-byte slots of a row,
 // applied on the global side of the load (lane l of a load instruction always lands at LDS byte 16*l
 // of its 1 KB block, so it fetches the slot that belongs there).
@@ -31,6 +39,8 @@
 // 64 O registers leaves the steady-state loop.
 #include "rt_common.hpp"
 #include "rt_kernels.hpp"
+
+#include <type_traits>
 
 // Phase marker for a timing harness that includes this file with its own definition; nothing here.
 #ifndef RT_PHASE
@@ -84,12 +94,27 @@ __device__ __forceinline__ float sum_with_other_half(float x) {
     auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
+// max of the 16 scores a lane holds: eight three-input maxima in one block of assembly (separate
+// statements would each be fenced by a wait state the hardware does not need between vector instructions)
 __device__ __forceinline__ float max16(const f32x16_t& s) {
-    float a = vmax(vmax(s[0], s[1]), vmax(s[2], s[3]));
-    float b = vmax(vmax(s[4], s[5]), vmax(s[6], s[7]));
-    float c = vmax(vmax(s[8], s[9]), vmax(s[10], s[11]));
-    float d = vmax(vmax(s[12], s[13]), vmax(s[14], s[15]));
-    return vmax(vmax(a, b), vmax(c, d));
+    float t0, t1, t2;
+    asm("v_max3_f32 %0, %3, %4, %5\n\t"
+        "v_max3_f32 %1, %6, %7, %8\n\t"
+        "v_max3_f32 %2, %9, %10, %11\n\t"
+        "v_max3_f32 %0, %0, %12, %13\n\t"
+        "v_max3_f32 %1, %1, %14, %15\n\t"
+        "v_max3_f32 %2, %2, %16, %17\n\t"
+        "v_max3_f32 %0, %0, %1, %2\n\t"
+        "v_max_f32 %0, %0, %18"
+        : "=&v"(t0), "=&v"(t1), "=&v"(t2)
+        : "v"(s[0]), "v"(s[1]), "v"(s[2]), "v"(s[3]), "v"(s[4]), "v"(s[5]), "v"(s[6]), "v"(s[7]), "v"(s[8]),
+          "v"(s[9]), "v"(s[10]), "v"(s[11]), "v"(s[12]), "v"(s[13]), "v"(s[14]), "v"(s[15]));
+    return t0;
+}
+// lo + hi of a packed bf16 pair, added to acc in f32 (v_dot2c_f32_bf16 with a pair of ones)
+__device__ __forceinline__ float add_bf16_pair(uint32_t pair, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pair),
+                                           __builtin_bit_cast(bf16x2_t, 0x3F803F80u), acc, false);
 }
 
 // 16 bytes per lane from global memory straight into LDS: lane l lands at LDS byte address
@@ -106,6 +131,13 @@ __device__ __forceinline__ void load_to_lds(const void* base, uint32_t byte_off,
                  : "memory");
 }
 
+// 16-byte LDS read into the register that `dst` already occupies (a read-write argument keeps the register).
+// The compiler does not see an LDS read here: the caller waits (s_waitcnt lgkmcnt) before using dst.
+template <int OFF>
+__device__ __forceinline__ void lds_read_b128_in_place(bf16x8_t& dst, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "+v"(dst) : "v"(addr), "n"(OFF));
+}
+
 template <int HD, int MODE>
 __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Params p) {
     constexpr int ROWB = HD * 2;             // bytes per row
@@ -118,11 +150,17 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     constexpr bool kCausal = (MODE == kMaskCausal) || (MODE == kMaskVarlenCausal);
     static_assert(NLD >= 1 && NLD <= NITEMS && BC % (RPI * NWAVES) == 0, "tile load split");
 
-    // [stage 0: K, V][stage 1: K, V]
+    // [K stage 0][K stage 1][V stage 0][V stage 1]: with this order every operand read of the steady state
+    // is one per-lane base address plus an immediate offset below 64 KB
     __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * TILE_B];
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: branches on it are scalar
+#ifndef RT_EXP_GRP
+#define RT_EXP_GRP (wave >> 2)
+#endif
+    const int grp = RT_EXP_GRP;                                  // 0: waves 0-3, 1: waves 4-7 (one of each per SIMD)
     const int col = lane & 31, hh = lane >> 5;
     RT_PHASE_DECL;
 
@@ -160,17 +198,23 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     const int ld_row0 = wave * RPI + lane / SPR;
     const uint32_t ld_k0 = (uint32_t)(((lane % SPR) ^ swz_k(ld_row0)) * 16);  // byte offset inside a global row
     const uint32_t ld_v0 = (uint32_t)(((lane % SPR) ^ swz_v(ld_row0)) * 16);
-    // ---- per-lane constants of the operand reads
-    uint32_t koff[KS];  // K A-operand: row col of an item, slot (2ks + hh)
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) koff[ks] = (uint32_t)(col * ROWB + (((2 * ks + hh) ^ swz_k(col)) * 16));
-    uint32_t voff[DT];  // V^T A-operand: lane j of a 16-group addresses row j/4 (+4hh), 4 columns
-#pragma unroll
-    for (int dt = 0; dt < DT; dt++) {
-        const int j = lane & 15, grp = (lane >> 4) & 1, row = (j >> 2) + 4 * hh;
-        const int slot = (4 * dt + 2 * grp + ((j & 3) >> 1)) ^ swz_v(row);
-        voff[dt] = (uint32_t)(row * ROWB + slot * 16 + 8 * (j & 1));
+    // ---- per-lane bases of the operand reads.  The swizzles only permute address bits that the operand
+    // index also occupies, so operand ks (dt) of a lane sits at base ^ 32*ks (base ^ 64*dt): one register
+    // per matrix, one XOR per read.  The stage bit is toggled into the bases once per step; item and
+    // half-item offsets are immediates.
+    static_assert(HD == 128 || HD == 64, "operand address algebra below");
+    // K A-operand: row col of an item, slot (2ks + hh) ^ swz_k(col)
+    uint32_t k_base = (uint32_t)(col * ROWB + ((hh ^ swz_k(col)) * 16));
+    // V^T A-operand: lane j of a 16-group addresses row j/4 (+4hh), 4 columns; slot (4dt + low) ^ swz_v(row)
+    uint32_t v_base;
+    {
+        const int j = lane & 15, g16 = (lane >> 4) & 1, row = (j >> 2) + 4 * hh;
+        const int low = 2 * g16 + ((j & 3) >> 1);
+        v_base = (uint32_t)(2 * TILE_B + row * ROWB + ((low ^ swz_v(row)) * 16) + 8 * (j & 1));
     }
+    // (2ks + hh) ^ x == (hh ^ x) ^ 2ks and (4dt + low) ^ x == (low ^ x) ^ 4dt bit for bit
+    auto k_addr = [&](int ks, int flip) { return lds + (k_base ^ (uint32_t)(32 * ks + flip)); };
+    auto v_addr = [&](int dt) { return lds + (v_base ^ (uint32_t)(64 * dt)); };
 
     // state of the current job
     int q0, qw, q_row, n_keys, n_steps;
@@ -180,21 +224,26 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     bf16x8_t qreg[KS];  // Q as B operand, in registers for the whole job
     f32x16_t acc_o[DT];
     float m_run, l_run;
+    // operands of the next matrix cluster, and the scores / probabilities that travel between clusters
+    bf16x8_t a[KS];      // K(k)
+    u32x4_t vreg[2][DT]; // V(k-1): [16-key half][32-row tile of O^T]
+    bf16x8_t pB[2];      // P(k-1)
+    f32x16_t s;          // S^T(k)
 
-    // request key tile `kv0` into stage `st`.  Rows past the last key are read from the last key
-    // instead; they are masked in the score tile, so their probabilities are zero.
     // This wave issues NLD K loads and NLD V loads per tile; load_part issues the n-th pair, so that a
-    // tile's requests can be spread over the step before it (eight waves asking for a whole tile at once
+    // tile's requests can be spread over several clusters (eight waves asking for a whole tile at once
     // queue up behind the CU's one address unit, and a wave cannot issue anything else while it waits).
+    // Rows past the last key are read from the last key instead; they are masked in the score tile, so
+    // their probabilities are zero.
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
     auto load_part = [&](int n, int kv0, int st) {
-        const uint32_t kdst = lds_base + (uint32_t)(st * 2 * TILE_B + (wave + NWAVES * n) * 1024);
+        const uint32_t kdst = lds_base + (uint32_t)(st * TILE_B + (wave + NWAVES * n) * 1024);
         int r = kv0 + ld_row0 + NWAVES * RPI * n;
         asm volatile("" : "+v"(r));  // recompute per call: hoisted copies of these offsets only cost registers
         r = min(r, n_keys - 1);
         const uint32_t row_off = (uint32_t)r * ROWB;  // a (b, h) slab is below 4 GiB: seq * dim * 2 < 2^32
         load_to_lds(Kg, row_off + ld_k0, kdst);
-        load_to_lds(Vg, row_off + ld_v0, kdst + TILE_B);
+        load_to_lds(Vg, row_off + ld_v0, kdst + 2 * TILE_B);
     };
     auto load_tile = [&](int kv0, int st) {
 #pragma unroll
@@ -245,18 +294,37 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         if (n_steps > 0) load_tile(0, 0);
     };
 
-    // ---- pieces of the per-item pipeline -------------------------------------------------------------
-    // scores of one 32-key item: KS MFMAs accumulating over the head dim
-    auto qk = [&](const unsigned char* Kb, int t, f32x16_t& s) {
-        bf16x8_t a[KS];
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) a[ks] = *(const bf16x8_t*)(Kb + 32 * t * ROWB + koff[ks]);
+    // ---- pieces of the clusters ------------------------------------------------------------------------
+    // operand reads; `off` is an immediate byte offset (item, half item); `flip` = TILE_B reads the other stage
+    // The K operand is refilled IN PLACE: the read is written in assembly with the operand register as a
+    // read-write argument, so it lands in the register the matrix instruction before it has just read (left
+    // to itself the register allocator keeps two sets of K operands and runs out of registers).  The
+    // compiler does not see these as LDS reads, so the wait for them is written out (lds_operands_ready).
+    auto k_read_one = [&](auto off_c, int flip, int ks) {
+        constexpr int OFF = decltype(off_c)::value;
+        const uint32_t addr = lds_base + (k_base ^ (uint32_t)(32 * ks + flip));
+        lds_read_b128_in_place<OFF>(a[ks], addr);
+    };
+    auto lds_operands_ready = [&]() { __builtin_amdgcn_s_waitcnt(0xC07F); };  // lgkmcnt(0)
+    auto v_read_one = [&](int off, int j) {  // operand of the j-th P.V matrix instruction
+        const int u = j / DT, dt = j % DT;
+        // contraction slots 0-3 of a lane: keys kv_lo..kv_lo+3; slots 4-7: kv_lo+8..kv_lo+11
+        const unsigned char* ptr = v_addr(dt) + off + 16 * u * ROWB;
+        u32x2_t lo = lds_read_tr16(ptr);
+        u32x2_t hi = lds_read_tr16(ptr + 8 * ROWB);
+        vreg[u][dt] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+    };
+    auto mfma_qk = [&](int ks) { s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], qreg[ks], s, 0, 0, 0); };
+    auto mfma_pv = [&](int j) {
+        const int u = j / DT, dt = j % DT;
+        acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vreg[u][dt]), pB[u],
+                                                            acc_o[dt], 0, 0, 0);
+    };
+    auto zero_s = [&]() {
 #pragma unroll
         for (int i = 0; i < 16; i++) s[i] = 0.0f;
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], qreg[ks], s, 0, 0, 0);
     };
-    auto mask_item = [&](int kv_base, f32x16_t& s) {
+    auto mask_item = [&](int kv_base) {
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             int kr = kv_base + 8 * (i >> 2) + 4 * hh + (i & 3);
@@ -266,8 +334,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             s[i] = masked ? neg_inf() : s[i];
         }
     };
-    // raise the running max when it pays (wave-uniform branch; no MFMA inside)
-    auto update_max = [&](const f32x16_t& s) {
+    // raise the running max when it pays (wave-uniform branch)
+    auto update_max = [&]() {
         float m_item = max_with_other_half(max16(s));
         if (__any(m_item > m_run + lazy_raw)) {
             float m_new = vmax(m_run, m_item);
@@ -281,9 +349,26 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
                 for (int i = 0; i < 16; i++) acc_o[t][i] *= alpha;
         }
     };
-    // p = exp2(s*c - m*c) in place, row-sum share, and the two B operands of the item
-    auto exp_item = [&](f32x16_t& s, bf16x8_t (&pB)[2]) {
+    // p = exp2(s*c - m*c), row-sum share, and the two B operands of the item
+    auto exp_item = [&]() {
         const float mc = ((m_run == neg_inf()) ? 0.0f : m_run) * c;
+#ifdef RT_EXP_DOT2
+        float part = 0.0f;
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            u32x4_t pb;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * u + 2 * e], c, -mc));
+                const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * u + 2 * e + 1], c, -mc));
+                pb[e] = cvt_pk_bf16(e0, e1);
+                if (u == 0) l_run = add_bf16_pair(pb[e], l_run);
+                else part = add_bf16_pair(pb[e], part);
+            }
+            pB[u] = __builtin_bit_cast(bf16x8_t, pb);
+        }
+        l_run += part;
+#else
         float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int i = 0; i < 16; i++) {
@@ -299,69 +384,90 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             for (int e = 0; e < 4; e++) pb[e] = cvt_pk_bf16(s[8 * u + 2 * e], s[8 * u + 2 * e + 1]);
             pB[u] = __builtin_bit_cast(bf16x8_t, pb);
         }
+#endif
     };
-    // O^T += V^T . P^T for one item: 2 contraction steps of 16 keys x DT output tiles
-    auto pv = [&](const unsigned char* Vb, int t, const bf16x8_t (&pB)[2]) {
+    // one barrier per cluster; nothing may be scheduled across it
+    auto cluster_barrier = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+#ifndef RT_EXP_NOBAR
+        __builtin_amdgcn_s_barrier();
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    static_assert(KS == 2 * DT, "one P.V matrix instruction per score matrix instruction");
+
+    // One step = one 128-key tile = four items, each a C cluster and an S cluster.  Every wave runs every
+    // item of every step of the job (an item hidden from all of a wave's rows by the causal mask is scored,
+    // masked to -inf and contributes exact zeros): all eight waves then meet the same barriers, and a wave
+    // that skipped the work would only wait there.
+    auto run_item = [&](auto i_c, int kv0, int kv_next, int st, int mask_from) {
+        constexpr int i = decltype(i_c)::value;
+        constexpr int item_off = 32 * i * ROWB;
+        // ---- C: the products, and right after each the read that refills its operand for the next C.
+        // Score and P.V instructions alternate: a score instruction accumulates onto the one before it,
+        // and back-to-back dependent matrix instructions would wait for each other.
+        RT_PHASE(0);
+        lds_operands_ready();
+        zero_s();
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
-            // contraction slots 0-3 of this lane: keys kv_lo..kv_lo+3; slots 4-7: kv_lo+8..kv_lo+11
-            const unsigned char* vp = Vb + (32 * t + 16 * u) * ROWB;
+        for (int ks = 0; ks < KS; ks++) {
+#ifndef RT_EXP_NOMFMA
+            mfma_qk(ks);
+#else
+            s[ks] += __builtin_bit_cast(f32x4_t, a[ks])[0]; s[ks + 8] += __builtin_bit_cast(f32x4_t, a[ks])[1];
+#endif
+#ifndef RT_EXP_NOLDS
+            if (i + 1 < NITEMS) k_read_one(std::integral_constant<int, (i + 1 < NITEMS ? item_off + 32 * ROWB : 0)>{}, 0, ks);
+            else k_read_one(std::integral_constant<int, 0>{}, TILE_B, ks);  // item 0 of the next tile, other stage
+#endif
+#ifndef RT_EXP_NOMFMA
+            mfma_pv(ks);
+#else
+            acc_o[ks % DT][ks] += __builtin_bit_cast(f32x4_t, vreg[ks / DT][ks % DT])[0] * __builtin_bit_cast(f32x4_t, pB[ks / DT])[ks % DT];
+#endif
+#ifndef RT_EXP_NOLDS
+            v_read_one(item_off, ks);
+#endif
+        }
+        // the next tile (or, with none left, this tile again: served from cache into the idle stage,
+        // which keeps the cluster free of branches): requested with items 0 and 1, awaited with item 2
+        if (NLD >= 2) {
+            if (i < 2) {
 #pragma unroll
-            for (int dt = 0; dt < DT; dt++) {
-                u32x2_t lo = lds_read_tr16(vp + voff[dt]);
-                u32x2_t hi = lds_read_tr16(vp + voff[dt] + 8 * ROWB);
-                u32x4_t av = {lo[0], lo[1], hi[0], hi[1]};
-                acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), pB[u],
-                                                                    acc_o[dt], 0, 0, 0);
+                for (int n = 0; n < NLD / 2; n++) load_part(i * (NLD / 2) + n, kv_next, st ^ 1);
             }
+        } else if (i == 0) {
+            load_part(0, kv_next, st ^ 1);
         }
-    };
-    // One 128-key tile = up to four 32-key items.
-    // Fast path: all four items visible and unmasked.  Straight-line code, so that each product sits in
-    // the same scheduling region as the vector work it is meant to hide (an MFMA only overlaps with the
-    // vector instructions issued right behind it; a branch between them would serialise the two).
-    auto tile_full = [&](const unsigned char* Kb, const unsigned char* Vb, int kv_next, int st_next) {
-        f32x16_t s_a, s_b;
-        bf16x8_t pB[2];
+        if (i == 2) __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wave's share has landed
+        if (i == NITEMS - 1) __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): stage st may be refilled
         RT_PHASE(1);
-        load_part(0, kv_next, st_next);
-        qk(Kb, 0, s_a);
-        update_max(s_a);
+        cluster_barrier();
         RT_PHASE(2);
-        if (NLD > 1) load_part(1 % NLD, kv_next, st_next);
-        qk(Kb, 1, s_b);  exp_item(s_a, pB);      // scores of item 1 | probabilities of item 0
-        pv(Vb, 0, pB);   update_max(s_b);        // item 0 into O    | max of item 1 (P(i) is relative to the max
-        if (NLD > 2) load_part(2 % NLD, kv_next, st_next);
-        qk(Kb, 2, s_a);  exp_item(s_b, pB);      //                  |   BEFORE item i+1 raises it: accumulate first)
-        pv(Vb, 1, pB);   update_max(s_a);
-        if (NLD > 3) load_part(3 % NLD, kv_next, st_next);
-        qk(Kb, 3, s_b);  exp_item(s_a, pB);
-        pv(Vb, 2, pB);   update_max(s_b);
-        exp_item(s_b, pB);
-        pv(Vb, 3, pB);
+        // ---- S
+        if (MODE == kMaskPadding || kv0 + 32 * i + 31 > mask_from) mask_item(kv0 + 32 * i);
+#ifndef RT_EXP_NOSOFTMAX
+        update_max();
+        exp_item();
+#else
+        // timing experiment: keep the scores alive with two cheap instructions
+        pB[0] = __builtin_bit_cast(bf16x8_t, u32x4_t{__float_as_uint(s[0]) & 0x3f003f00u, __float_as_uint(s[5]) & 0x3f003f00u, __float_as_uint(s[10]) & 0x3f003f00u, __float_as_uint(s[15]) & 0x3f003f00u});
+        pB[1] = pB[0];
+#endif
         RT_PHASE(3);
+        cluster_barrier();
+        RT_PHASE(9);
     };
-    // General path: n_act items are visible to this wave (a causal mask hides the rest); only the last
-    // visible one can need masking (diagonal or ragged end), unless the mask is a keep vector.
-    auto tile_part = [&](const unsigned char* Kb, const unsigned char* Vb, int kv0, int n_act, bool mask_last) {
-        f32x16_t s_a, s_b;
-        bf16x8_t pB[2];
-        qk(Kb, 0, s_a);
-        if (MODE == kMaskPadding || (mask_last && n_act == 1)) mask_item(kv0, s_a);
-        update_max(s_a);
-#pragma unroll
-        for (int i = 0; i < NITEMS; i++) {
-            f32x16_t& s_cur = (i & 1) ? s_b : s_a;
-            f32x16_t& s_nxt = (i & 1) ? s_a : s_b;
-            const bool more = i + 1 < n_act;  // wave-uniform
-            if (more) qk(Kb, i + 1, s_nxt);
-            exp_item(s_cur, pB);
-            if (more && (MODE == kMaskPadding || (mask_last && i + 2 == n_act)))
-                mask_item(kv0 + 32 * (i + 1), s_nxt);
-            pv(Vb, i, pB);
-            if (!more) break;
-            update_max(s_nxt);
-        }
+    // One step = one 128-key tile = four items, each a C cluster and an S cluster.  Every wave runs every
+    // item of every step of the job (an item hidden from all of a wave's rows by the causal mask is scored,
+    // masked to -inf and contributes exact zeros): all eight waves then meet the same barriers, and a wave
+    // that skipped the work would only wait there.
+    auto run_step = [&](int kv0, int kv_next, int st, int mask_from) {
+        static_assert(NITEMS == 4, "items per step");
+        run_item(std::integral_constant<int, 0>{}, kv0, kv_next, st, mask_from);
+        run_item(std::integral_constant<int, 1>{}, kv0, kv_next, st, mask_from);
+        run_item(std::integral_constant<int, 2>{}, kv0, kv_next, st, mask_from);
+        run_item(std::integral_constant<int, 3>{}, kv0, kv_next, st, mask_from);
     };
 
     int round = 0;
@@ -374,40 +480,43 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             for (int i = 0; i < 16; i++) acc_o[t][i] = 0.0f;
         m_run = neg_inf();
         l_run = 0.0f;
+        // the first C of a job has no previous item: it multiplies zeros into O
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            pB[u] = __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u});
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) vreg[u][dt] = u32x4_t{0u, 0u, 0u, 0u};
+        }
         // the queries and tile 0 have landed; the barrier also ends the previous job's use of LDS
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
         RT_PHASE(10);
 
+        // an item needs masking when its last key lies past the last existing key or past the wave's first row
+        const int mask_from = kCausal ? min(n_keys - 1, qw) : n_keys - 1;
+        if (grp == 1) cluster_barrier();  // the second group runs one cluster behind the first
+        if (n_steps > 0) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) k_read_one(std::integral_constant<int, 0>{}, 0, ks);  // K(0)
+        }
+        cluster_barrier();
         for (int step = 0; step < n_steps; step++) {
             const int kv0 = step * BC;
-            const int st = step & 1;
-            RT_PHASE(0);
-            // tile step+1 goes into the other stage (last read in step-1, before the barrier that ended it)
-            const bool more = step + 1 < n_steps;
-            int n_act = NITEMS;
-            if (kCausal) n_act = (kv0 > qw + 31) ? 0 : min(NITEMS, (qw + 31 - kv0) / 32 + 1);  // items starting at or before the wave's last row
-            n_act = min(n_act, (n_keys - kv0 + 31) / 32);                // items that hold an existing key
-            if (n_act > 0) {
-                const int last_kv = kv0 + 32 * n_act - 1;  // last key of the last visible item
-                bool mask_last = last_kv >= n_keys;
-                if (kCausal) mask_last |= last_kv > qw;
-                if (MODE != kMaskPadding && n_act == NITEMS && !mask_last) {
-                    // the fast path requests the next tile itself, a quarter per item; with no next tile it
-                    // asks for its own tile again (served from cache into the idle stage) to stay branch-free
-                    tile_full(lds + st * 2 * TILE_B, lds + st * 2 * TILE_B + TILE_B, more ? kv0 + BC : kv0, st ^ 1);
-                } else {
-                    if (more) load_tile(kv0 + BC, st ^ 1);
-                    tile_part(lds + st * 2 * TILE_B, lds + st * 2 * TILE_B + TILE_B, kv0, n_act, mask_last);
-                }
-            } else if (more) {
-                load_tile(kv0 + BC, st ^ 1);
-            }
-            RT_PHASE(8);
-            __builtin_amdgcn_s_waitcnt(0x0F70);  // this wave's share of tile step+1 has landed
-            __syncthreads();                      // stage `st` is free again; stage st^1 is complete
-            RT_PHASE(9);
+            run_step(kv0, step + 1 < n_steps ? kv0 + BC : kv0, step & 1, mask_from);
+            k_base ^= (uint32_t)TILE_B;  // the other stage
+            v_base ^= (uint32_t)TILE_B;
         }
+        if (n_steps & 1) {  // back to stage 0 for the next job
+            k_base ^= (uint32_t)TILE_B;
+            v_base ^= (uint32_t)TILE_B;
+        }
+        // the last item's P.V
+        if (n_steps > 0) {
+#pragma unroll
+            for (int j = 0; j < KS; j++) mfma_pv(j);
+        }
+        cluster_barrier();
+        if (grp == 0) cluster_barrier();  // the first group waits for the second to finish
 
         // ---- this job's output.  Stage 1 of LDS is free (the next job's first tile goes to stage 0): each
         // wave parks its 32 normalised rows there, swizzled, and streams them out as whole rows.
@@ -423,7 +532,15 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         float l = sum_with_other_half(l_run);
         bool good = (l > 0.0f) && (l < __uint_as_float(0x7f800000u)) && !poison;
         float inv_l = 1.0f / l;
-        unsigned char* obuf = lds + 2 * TILE_B + wave * 32 * ROWB;
+        // waves 0-3 park in the K half of stage 1, waves 4-7 in its V half.  All addresses below are built
+        // from a copy of the lane index the compiler cannot see through: computed once per kernel they would
+        // sit in registers (or scratch) through the whole main loop.
+        int lane_e = lane;
+        asm volatile("" : "+v"(lane_e));
+        const int col_e = lane_e & 31, hh_e = lane_e >> 5;
+        const uint32_t obuf = lds_base + (uint32_t)((grp ? 3 * TILE_B : TILE_B) + (wave & 3) * 32 * ROWB);
+        // row col_e, slot (4dt + j) ^ swz_o(col_e): the slot bits of the base are XORed with a constant
+        const uint32_t park = obuf + (uint32_t)(col_e * ROWB + swz_o(col_e) * 16 + 8 * hh_e);
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
@@ -436,16 +553,22 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
                     o[r] = x;
                 }
                 u32x2_t wv = {cvt_pk_bf16(o[0], o[1]), cvt_pk_bf16(o[2], o[3])};
-                *(u32x2_t*)(obuf + col * ROWB + (((4 * dt + j) ^ swz_o(col)) * 16) + 8 * hh) = wv;
+                *(u32x2_t __attribute__((address_space(3)))*)(uintptr_t)(park ^ (uint32_t)(16 * (4 * dt + j))) = wv;
             }
         RT_PHASE(6);
         // (the same wave wrote and now reads: no barrier needed, the LDS queue is in order)
+        {
+            const int r0 = lane_e / SPR, pos = lane_e % SPR;  // instruction n covers rows n*RPI + r0
+            const uint32_t rd = obuf + (uint32_t)(r0 * ROWB + pos * 16);
+            // global slot pos ^ swz_o(n*RPI + r0): the part of the swizzle that depends on n is XORed in below
+            unsigned char* gp = (unsigned char*)og_out + (size_t)(qw_out + r0) * ROWB + ((pos ^ swz_o(r0)) * 16);
 #pragma unroll
-        for (int n = 0; n < 32 / RPI; n++) {
-            const int r = n * RPI + lane / SPR, pos = lane % SPR;
-            u32x4_t v = *(const u32x4_t*)(obuf + r * ROWB + pos * 16);
-            if (qw_out + r < N)
-                *(u32x4_t*)((unsigned char*)og_out + (size_t)(qw_out + r) * ROWB + ((pos ^ swz_o(r)) * 16)) = v;
+            for (int n = 0; n < 32 / RPI; n++) {
+                u32x4_t v = *(const u32x4_t __attribute__((address_space(3)))*)(uintptr_t)(rd + (uint32_t)(n * RPI * ROWB));
+                const int flip = (swz_o(n * RPI) * 16);  // r0 < RPI and RPI is a power of two: no carry into these bits
+                if (qw_out + n * RPI + r0 < N)
+                    *(u32x4_t*)((unsigned char*)((uintptr_t)(gp + (size_t)n * RPI * ROWB) ^ (uintptr_t)flip)) = v;
+            }
         }
         RT_PHASE(11);
     }
