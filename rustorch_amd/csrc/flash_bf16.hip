@@ -74,8 +74,12 @@ __device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
 // n0+4c.., lane j ends up with column n0+j of rows k0..k0+3: a contraction-major MFMA operand
 // fragment out of a row-major tile.
 __device__ __forceinline__ u32x2_t lds_read_tr16(const unsigned char* p) {
+#ifdef RT_EXP_PLAINV
+    return *(const u32x2_t __attribute__((address_space(3)))*)(p);
+#else
     s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3)))*)(p));
     return __builtin_bit_cast(u32x2_t, v);
+#endif
 }
 
 // plain v_max_f32: returns the non-NaN operand, without the canonicalising extra instruction fmaxf gets
@@ -111,12 +115,6 @@ __device__ __forceinline__ float max16(const f32x16_t& s) {
           "v"(s[9]), "v"(s[10]), "v"(s[11]), "v"(s[12]), "v"(s[13]), "v"(s[14]), "v"(s[15]));
     return t0;
 }
-// lo + hi of a packed bf16 pair, added to acc in f32 (v_dot2c_f32_bf16 with a pair of ones)
-__device__ __forceinline__ float add_bf16_pair(uint32_t pair, float acc) {
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pair),
-                                           __builtin_bit_cast(bf16x2_t, 0x3F803F80u), acc, false);
-}
-
 // 16 bytes per lane from global memory straight into LDS: lane l lands at LDS byte address
 // lds_block + 16*l (lds_block is wave-uniform and goes through M0).  Issued as inline assembly so that the compiler's counter
 // bookkeeping does not treat every later LDS read as dependent on it: completion is awaited explicitly
@@ -352,23 +350,6 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     // p = exp2(s*c - m*c), row-sum share, and the two B operands of the item
     auto exp_item = [&]() {
         const float mc = ((m_run == neg_inf()) ? 0.0f : m_run) * c;
-#ifdef RT_EXP_DOT2
-        float part = 0.0f;
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-            u32x4_t pb;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * u + 2 * e], c, -mc));
-                const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * u + 2 * e + 1], c, -mc));
-                pb[e] = cvt_pk_bf16(e0, e1);
-                if (u == 0) l_run = add_bf16_pair(pb[e], l_run);
-                else part = add_bf16_pair(pb[e], part);
-            }
-            pB[u] = __builtin_bit_cast(bf16x8_t, pb);
-        }
-        l_run += part;
-#else
         float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int i = 0; i < 16; i++) {
@@ -384,7 +365,6 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             for (int e = 0; e < 4; e++) pb[e] = cvt_pk_bf16(s[8 * u + 2 * e], s[8 * u + 2 * e + 1]);
             pB[u] = __builtin_bit_cast(bf16x8_t, pb);
         }
-#endif
     };
     // one barrier per cluster; nothing may be scheduled across it
     auto cluster_barrier = [&]() {
@@ -407,6 +387,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         // Score and P.V instructions alternate: a score instruction accumulates onto the one before it,
         // and back-to-back dependent matrix instructions would wait for each other.
         RT_PHASE(0);
+        __builtin_amdgcn_s_setprio(3);  // the multiplying wave goes first: its next instruction frees the matrix pipe
         lds_operands_ready();
         zero_s();
 #pragma unroll
@@ -416,7 +397,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
 #else
             s[ks] += __builtin_bit_cast(f32x4_t, a[ks])[0]; s[ks + 8] += __builtin_bit_cast(f32x4_t, a[ks])[1];
 #endif
-#ifndef RT_EXP_NOLDS
+#if !defined(RT_EXP_NOLDS) && !defined(RT_EXP_NOKREAD)
             if (i + 1 < NITEMS) k_read_one(std::integral_constant<int, (i + 1 < NITEMS ? item_off + 32 * ROWB : 0)>{}, 0, ks);
             else k_read_one(std::integral_constant<int, 0>{}, TILE_B, ks);  // item 0 of the next tile, other stage
 #endif
@@ -425,9 +406,12 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
 #else
             acc_o[ks % DT][ks] += __builtin_bit_cast(f32x4_t, vreg[ks / DT][ks % DT])[0] * __builtin_bit_cast(f32x4_t, pB[ks / DT])[ks % DT];
 #endif
-#ifndef RT_EXP_NOLDS
+#if !defined(RT_EXP_NOLDS) && !defined(RT_EXP_NOVREAD) && !defined(RT_EXP_VINS)
             v_read_one(item_off, ks);
 #endif
+            // keep this order: two matrix instructions, three reads, and so on (left alone the scheduler
+            // bunches the reads, and the matrix pipe runs dry while a wave issues ten of them in a row)
+            __builtin_amdgcn_sched_barrier(0);
         }
         // the next tile (or, with none left, this tile again: served from cache into the idle stage,
         // which keeps the cluster free of branches): requested with items 0 and 1, awaited with item 2
@@ -442,9 +426,14 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         if (i == 2) __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wave's share has landed
         if (i == NITEMS - 1) __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): stage st may be refilled
         RT_PHASE(1);
+        __builtin_amdgcn_s_setprio(0);
         cluster_barrier();
         RT_PHASE(2);
         // ---- S
+#ifdef RT_EXP_VINS
+#pragma unroll
+        for (int j = 0; j < KS; j++) v_read_one(item_off, j);
+#endif
         if (MODE == kMaskPadding || kv0 + 32 * i + 31 > mask_from) mask_item(kv0 + 32 * i);
 #ifndef RT_EXP_NOSOFTMAX
         update_max();
