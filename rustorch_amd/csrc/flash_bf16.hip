@@ -129,6 +129,16 @@ __device__ __forceinline__ void load_to_lds(const void* base, uint32_t byte_off,
                  : "memory");
 }
 
+// n / d for 0 <= n < 2^22 and d >= 1 with inv = 1.0f / d: the float quotient is off by at most one.  An integer
+// division costs some thirty instructions, and the job bookkeeping does four per job.
+__device__ __forceinline__ int div_small(int n, int d, float inv) {
+    int q = (int)((float)n * inv);
+    const int r = n - q * d;
+    q += (r >= d) ? 1 : 0;
+    q -= (r < 0) ? 1 : 0;
+    return __builtin_amdgcn_readfirstlane(q);  // callers divide wave-uniform values: keep the result scalar
+}
+
 // 16-byte LDS read into the register that `dst` already occupies (a read-write argument keeps the register).
 // The compiler does not see an LDS read here: the caller waits (s_waitcnt lgkmcnt) before using dst.
 template <int OFF>
@@ -253,12 +263,16 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     // workers in boustrophedon rows: the workers of an XCD then sit on one or two heads at a time and
     // share their K/V through that L2, and every worker still gets a long job paired with a short one.
     const bool by_xcd = ((n_bh & 7) == 0) && ((W & 7) == 0);
+    const bool small_ids = n_jobs < (1 << 22);  // quotients below come from div_small
+    const float inv_qtiles = 1.0f / (float)n_qtiles, inv_bh = 1.0f / (float)n_bh;
+    const float inv_heads = 1.0f / (float)p.heads, inv_group = 1.0f / (float)p.group;
+    auto quot = [&](int n, int d, float inv) { return small_ids ? div_small(n, d, inv) : n / d; };
     auto job_of_round = [&](int i) {
         if (by_xcd) {
             const int C = W >> 3, x = w & 7, cw = w >> 3;
             const int q = i * C + ((i & 1) ? (C - 1 - cw) : cw);
             if (q >= n_qtiles * (n_bh >> 3)) return -1;
-            const int head = q / n_qtiles, rank = q - head * n_qtiles;
+            const int head = quot(q, n_qtiles, inv_qtiles), rank = q - head * n_qtiles;
             return rank * n_bh + head * 8 + x;
         }
         int j = i * W + ((i & 1) ? (W - 1 - w) : w);
@@ -266,10 +280,10 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     };
     // point the state at job j and request its queries and first key tile (into stage 0)
     auto begin_job = [&](int j) {
-        const int rank = j / n_bh, bh = j - rank * n_bh;
+        const int rank = quot(j, n_bh, inv_bh), bh = j - rank * n_bh;
         const int qtile = n_qtiles - 1 - rank;  // rank 0 = the longest causal rows
-        const int b = bh / p.heads, h = bh - b * p.heads;
-        const int kvh = h / p.group;
+        const int b = quot(bh, p.heads, inv_heads), h = bh - b * p.heads;
+        const int kvh = quot(h, p.group, inv_group);
         q0 = qtile * BR;
         qw = q0 + wave * 32;
         q_row = qw + col;
@@ -283,13 +297,42 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         if (kCausal) kv_end = min(n_keys, q0 + BR);
         if (MODE == kMaskVarlenCausal && q0 >= n_keys) kv_end = 0;  // a tile of padded query rows
         n_steps = (kv_end + BC - 1) / BC;
+        // The wave's 32 query rows are one contiguous block: fetched in whole rows (load n, lane l: row
+        // RPI*n + l/SPR, slot l%SPR), which costs the address unit a quarter of what row-per-lane loads
+        // would; settle_queries() turns the registers into the operand layout once they have landed.
+        static_assert(32 / RPI == KS, "one raw query register per operand register");
+        {
+            int lane_q = lane;
+            asm volatile("" : "+v"(lane_q));  // (addresses rebuilt per job: see the note at the output stage)
+            const int r0 = lane_q / SPR, slot = lane_q % SPR;
+            const unsigned char* qp = (const unsigned char*)Qg + (size_t)(qw + r0) * ROWB + slot * 16;
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            u32x4_t z = {0u, 0u, 0u, 0u};
-            if (q_row < N) z = *(const u32x4_t*)(Qg + (size_t)q_row * HD + 16 * ks + 8 * hh);
-            qreg[ks] = __builtin_bit_cast(bf16x8_t, z);
+            for (int n = 0; n < KS; n++) {
+                u32x4_t z = {0u, 0u, 0u, 0u};
+                if (qw + RPI * n + r0 < N) z = *(const u32x4_t*)(qp + (size_t)n * RPI * ROWB);
+                qreg[n] = __builtin_bit_cast(bf16x8_t, z);
+            }
         }
         if (n_steps > 0) load_tile(0, 0);
+    };
+    // Raw query registers -> B operands, through the wave's own corner of LDS stage 1 (idle between jobs):
+    // rows are written with the K tile's slot swizzle and read back like a K operand, (row col, slot 2ks+hh).
+    auto settle_queries = [&]() {
+        int lane_q = lane;
+        asm volatile("" : "+v"(lane_q));
+        const uint32_t qbuf = lds_base + (uint32_t)((grp ? 3 * TILE_B : TILE_B) + (wave & 3) * 32 * ROWB);
+        const int r0 = lane_q / SPR, slot = lane_q % SPR;
+#pragma unroll
+        for (int n = 0; n < KS; n++) {
+            const int r = RPI * n + r0;
+            *(bf16x8_t __attribute__((address_space(3)))*)(uintptr_t)(qbuf + (uint32_t)(r * ROWB + ((slot ^ swz_k(r)) * 16))) =
+                qreg[n];
+        }
+        const int col_q = lane_q & 31, hh_q = lane_q >> 5;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++)
+            qreg[ks] = *(const bf16x8_t __attribute__((address_space(3)))*)(uintptr_t)(
+                qbuf + (uint32_t)(col_q * ROWB + (((2 * ks + hh_q) ^ swz_k(col_q)) * 16)));
     };
 
     // ---- pieces of the clusters ------------------------------------------------------------------------
@@ -478,6 +521,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         }
         // the queries and tile 0 have landed; the barrier also ends the previous job's use of LDS
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        settle_queries();
         __syncthreads();
         RT_PHASE(10);
 
