@@ -74,12 +74,8 @@ __device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
 // n0+4c.., lane j ends up with column n0+j of rows k0..k0+3: a contraction-major MFMA operand
 // fragment out of a row-major tile.
 __device__ __forceinline__ u32x2_t lds_read_tr16(const unsigned char* p) {
-#ifdef RT_EXP_PLAINV
-    return *(const u32x2_t __attribute__((address_space(3)))*)(p);
-#else
     s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3)))*)(p));
     return __builtin_bit_cast(u32x2_t, v);
-#endif
 }
 
 // plain v_max_f32: returns the non-NaN operand, without the canonicalising extra instruction fmaxf gets
@@ -165,10 +161,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: branches on it are scalar
-#ifndef RT_EXP_GRP
-#define RT_EXP_GRP (wave >> 2)
-#endif
-    const int grp = RT_EXP_GRP;                                  // 0: waves 0-3, 1: waves 4-7 (one of each per SIMD)
+    const int grp = wave >> 2;                                  // 0: waves 0-3, 1: waves 4-7 (one of each per SIMD)
     const int col = lane & 31, hh = lane >> 5;
     RT_PHASE_DECL;
 
@@ -412,9 +405,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     // one barrier per cluster; nothing may be scheduled across it
     auto cluster_barrier = [&]() {
         __builtin_amdgcn_sched_barrier(0);
-#ifndef RT_EXP_NOBAR
         __builtin_amdgcn_s_barrier();
-#endif
         __builtin_amdgcn_sched_barrier(0);
     };
     static_assert(KS == 2 * DT, "one P.V matrix instruction per score matrix instruction");
@@ -432,26 +423,15 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         RT_PHASE(0);
         __builtin_amdgcn_s_setprio(3);  // the multiplying wave goes first: its next instruction frees the matrix pipe
         lds_operands_ready();
+        __builtin_amdgcn_sched_barrier(0);  // no matrix instruction may be moved ahead of that wait
         zero_s();
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-#ifndef RT_EXP_NOMFMA
             mfma_qk(ks);
-#else
-            s[ks] += __builtin_bit_cast(f32x4_t, a[ks])[0]; s[ks + 8] += __builtin_bit_cast(f32x4_t, a[ks])[1];
-#endif
-#if !defined(RT_EXP_NOLDS) && !defined(RT_EXP_NOKREAD)
             if (i + 1 < NITEMS) k_read_one(std::integral_constant<int, (i + 1 < NITEMS ? item_off + 32 * ROWB : 0)>{}, 0, ks);
             else k_read_one(std::integral_constant<int, 0>{}, TILE_B, ks);  // item 0 of the next tile, other stage
-#endif
-#ifndef RT_EXP_NOMFMA
             mfma_pv(ks);
-#else
-            acc_o[ks % DT][ks] += __builtin_bit_cast(f32x4_t, vreg[ks / DT][ks % DT])[0] * __builtin_bit_cast(f32x4_t, pB[ks / DT])[ks % DT];
-#endif
-#if !defined(RT_EXP_NOLDS) && !defined(RT_EXP_NOVREAD) && !defined(RT_EXP_VINS)
             v_read_one(item_off, ks);
-#endif
             // keep this order: two matrix instructions, three reads, and so on (left alone the scheduler
             // bunches the reads, and the matrix pipe runs dry while a wave issues ten of them in a row)
             __builtin_amdgcn_sched_barrier(0);
@@ -473,19 +453,9 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         cluster_barrier();
         RT_PHASE(2);
         // ---- S
-#ifdef RT_EXP_VINS
-#pragma unroll
-        for (int j = 0; j < KS; j++) v_read_one(item_off, j);
-#endif
         if (MODE == kMaskPadding || kv0 + 32 * i + 31 > mask_from) mask_item(kv0 + 32 * i);
-#ifndef RT_EXP_NOSOFTMAX
         update_max();
         exp_item();
-#else
-        // timing experiment: keep the scores alive with two cheap instructions
-        pB[0] = __builtin_bit_cast(bf16x8_t, u32x4_t{__float_as_uint(s[0]) & 0x3f003f00u, __float_as_uint(s[5]) & 0x3f003f00u, __float_as_uint(s[10]) & 0x3f003f00u, __float_as_uint(s[15]) & 0x3f003f00u});
-        pB[1] = pB[0];
-#endif
         RT_PHASE(3);
         cluster_barrier();
         RT_PHASE(9);
@@ -502,6 +472,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         run_item(std::integral_constant<int, 3>{}, kv0, kv_next, st, mask_from);
     };
 
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) a[ks] = __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u});
     int round = 0;
     int job = job_of_round(0);
     if (job >= 0) begin_job(job);
