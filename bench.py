@@ -33,7 +33,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the dominant kernels on the bench workloads, from the rocprofv3 --pmc runs
 # summarised under profiles/ (FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB, the factors a 256 MiB copy reads).
 # Counters cannot be read from inside this process; these are the committed measurements, not live values.
-TRAFFIC_PREFILL_BYTES = (289000 * 2.0 + 139800 * 1.0) * 1024
+TRAFFIC_PREFILL_BYTES = (284200 * 2.0 + 131100 * 1.0) * 1024
 TRAFFIC_DECODE_BYTES = (624200 * 2.0 + 5313 * 1.0) * 1024
 
 
@@ -96,8 +96,10 @@ def time_steps(hip, stream, launch, steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    # defaults long enough to leave the first ~15 ms after an idle period, in which the clocks first drop and
+    # then recover (launches of the same kernel take 540, 730, then 530 us): 250 launches are 0.15 s
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity sample")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None)
     ap.add_argument("--calibrate-copy", action="store_true",
