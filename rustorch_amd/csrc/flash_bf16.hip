@@ -371,7 +371,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     // raise the running max when it pays (wave-uniform branch)
     auto update_max = [&]() {
         float m_item = max_with_other_half(max16(s));
-        if (__any(m_item > m_run + lazy_raw)) {
+        if (__builtin_expect(__any(m_item > m_run + lazy_raw), 0)) {
             float m_new = vmax(m_run, m_item);
             float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
             float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);  // m_run = -inf -> 0
@@ -386,12 +386,13 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     // p = exp2(s*c - m*c), row-sum share, and the two B operands of the item
     auto exp_item = [&]() {
         const float mc = ((m_run == neg_inf()) ? 0.0f : m_run) * c;
-        float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        float part[4];
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c, -mc));
             s[i] = e;
-            part[i & 3] += e;
+            if (i < 4) part[i] = e;
+            else part[i & 3] += e;
         }
         l_run += (part[0] + part[1]) + (part[2] + part[3]);
 #pragma unroll
@@ -453,9 +454,13 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         cluster_barrier();
         RT_PHASE(2);
         // ---- S
-        if (MODE == kMaskPadding || kv0 + 32 * i + 31 > mask_from) mask_item(kv0 + 32 * i);
+        if (MODE == kMaskPadding || __builtin_expect(kv0 + 32 * i + 31 > mask_from, 0)) mask_item(kv0 + 32 * i);
         update_max();
         exp_item();
+        // P is only used by the next matrix cluster, and the compiler would sink the exponentials and
+        // conversions that make it down to that use, past the barrier and in between the matrix
+        // instructions; pinning the values here keeps the work in this cluster
+        asm volatile("" : "+v"(pB[0]), "+v"(pB[1]), "+v"(l_run));
         RT_PHASE(3);
         cluster_barrier();
         RT_PHASE(9);
