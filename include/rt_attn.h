@@ -111,6 +111,13 @@ int rt_gqa_forward_f32(const float *q, size_t q_len, const float *k, size_t k_le
                        float *out, size_t out_len, size_t batch, size_t n_heads, size_t n_kv_heads, size_t seq_q,
                        size_t seq_kv, size_t head_dim, rt_err_detail *err);
 
+/* rustorch_nn::attention::mha_flash_forward_f32 -- crates/rustorch-nn/src/attention.rs:452-495.  q, k, v
+ * [batch, seq, heads, head_dim] host slices, out [batch, seq, heads*head_dim]; unmasked attention per
+ * (batch, head) with the checks of flash_forward on the shape (batch, heads, seq, head_dim), in its order. */
+int rt_mha_flash_forward_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len,
+                             float *out, size_t out_len, size_t batch, size_t seq, size_t heads, size_t head_dim,
+                             rt_err_detail *err);
+
 /* ---- prefill, device pointers ---------------------------------------------------------------- */
 
 /* flash_forward_masked on device-resident f32 tensors (same semantics; keep is a device
@@ -125,6 +132,18 @@ int rt_flash_forward_f32_dev(void *stream, const rt_attention_shape *shape, uint
 int rt_flash_forward_bf16_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const void *q,
                               const void *k, const void *v, int mask_kind, const uint8_t *keep, void *out,
                               rt_err_detail *err);
+
+/* The same two calls on tensors laid out [batch, seq, heads, dim] (k/v: [batch, seq, n_kv_heads, dim]),
+ * the layout rustorch_nn::MultiHeadAttention holds its projections in: the kernels walk the rows with a
+ * pitch of heads*dim elements, so the four host-side transposes of
+ * crates/rustorch-nn/src/attention.rs:466-486 (transpose_BTHD_to_BHTD_f32 x3, transpose_BHTD_to_BTHD_f32)
+ * have no counterpart here.  out has the layout of q, i.e. [batch, seq, heads*dim]. */
+int rt_flash_forward_bnhd_f32_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const float *q,
+                                  const float *k, const float *v, int mask_kind, const uint8_t *keep, float *out,
+                                  rt_err_detail *err);
+int rt_flash_forward_bnhd_bf16_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const void *q,
+                                   const void *k, const void *v, int mask_kind, const uint8_t *keep, void *out,
+                                   rt_err_detail *err);
 
 /* Padded-batch causal prefill: sequence b has seq_lens[b] <= seq valid positions (device
  * int32[batch]); key j of sequence b is masked iff j > i or j >= seq_lens[b].  Valid rows equal

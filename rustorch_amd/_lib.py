@@ -16,6 +16,7 @@ SYMBOLS = (
     "rt_init", "rt_version", "rt_status_name",
     "rt_flash_forward_f32", "rt_flash_forward_masked_f32", "rt_gqa_forward_f32",
     "rt_flash_forward_f32_dev", "rt_flash_forward_bf16_dev", "rt_flash_forward_varlen_bf16_dev",
+    "rt_mha_flash_forward_f32", "rt_flash_forward_bnhd_f32_dev", "rt_flash_forward_bnhd_bf16_dev",
     "rt_kv_append_bf16", "rt_gqa_decode_online_bf16", "rt_gqa_decode_batched_bf16",
     "rt_gqa_decode_workspace_bytes",
     "rt_buf_alloc", "rt_buf_free", "rt_memcpy_h2d", "rt_memcpy_d2h", "rt_stream_synchronize",
@@ -79,6 +80,9 @@ def lib():
     L.rt_flash_forward_f32_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_flash_forward_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_flash_forward_varlen_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, i32p, C.c_int, vp, errp]
+    L.rt_mha_flash_forward_f32.argtypes = [fp, sz, fp, sz, fp, sz, fp, sz, sz, sz, sz, sz, errp]
+    L.rt_flash_forward_bnhd_f32_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
+    L.rt_flash_forward_bnhd_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_kv_append_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, errp]
     L.rt_gqa_decode_online_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, errp]
     L.rt_gqa_decode_batched_bf16.argtypes = [vp, vp, vp, vp, vp, i32p, i32, i32, i32, i32, i32, vp, sz, errp]

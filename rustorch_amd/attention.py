@@ -130,3 +130,43 @@ def flash_forward_varlen_bf16_dev(shape, q, k, v, seq_lens_dev, out, zero_padded
                                                   dev_ptr(v), dev_ptr(seq_lens_dev), int(bool(zero_padded_rows)),
                                                   dev_ptr(out), C.byref(err))
     raise_for(rc, err)
+
+
+# ---- [batch, seq, heads, dim] tensors: the layout MultiHeadAttention keeps its projections in --------------
+
+
+def mha_flash_forward_f32(q, k, v, batch: int, seq: int, heads: int, head_dim: int, out=None):
+    """rustorch_nn::attention::mha_flash_forward_f32 (crates/rustorch-nn/src/attention.rs:452-495): q, k, v flat
+    f32 [B,T,H,hd]; returns flat f32 [B,T,H*hd].  Unmasked attention per (batch, head); no transposed copies."""
+    q, qp = _f32(q)
+    k, kp = _f32(k)
+    v, vp = _f32(v)
+    if out is None:
+        out = np.zeros(batch * seq * heads * head_dim, dtype=np.float32)
+    assert out.dtype == np.float32 and out.flags.c_contiguous
+    err = L.RtErr()
+    rc = L.lib().rt_mha_flash_forward_f32(qp, q.size, kp, k.size, vp, v.size,
+                                          out.ctypes.data_as(C.POINTER(C.c_float)), out.size, batch, seq, heads,
+                                          head_dim, C.byref(err))
+    raise_for(rc, err)
+    return out
+
+
+def flash_forward_bnhd_f32_dev(shape, q, k, v, out, mask: Mask = None, keep_dev=None, n_kv_heads=0, stream=None):
+    """f32 [B,N,H,D] device tensors (k, v: [B,N,Hkv,D]); `shape` is still (batch, heads, seq, dim)."""
+    mask = mask or Mask.none()
+    err = L.RtErr()
+    s = shape._c()
+    rc = L.lib().rt_flash_forward_bnhd_f32_dev(stream, C.byref(s), n_kv_heads, dev_ptr(q), dev_ptr(k), dev_ptr(v),
+                                               mask.kind, dev_ptr(keep_dev), dev_ptr(out), C.byref(err))
+    raise_for(rc, err)
+
+
+def flash_forward_bnhd_bf16_dev(shape, q, k, v, out, mask: Mask = None, keep_dev=None, n_kv_heads=0, stream=None):
+    """bf16 [B,N,H,D] device tensors (k, v: [B,N,Hkv,D]); `shape` is still (batch, heads, seq, dim)."""
+    mask = mask or Mask.none()
+    err = L.RtErr()
+    s = shape._c()
+    rc = L.lib().rt_flash_forward_bnhd_bf16_dev(stream, C.byref(s), n_kv_heads, dev_ptr(q), dev_ptr(k), dev_ptr(v),
+                                                mask.kind, dev_ptr(keep_dev), dev_ptr(out), C.byref(err))
+    raise_for(rc, err)

@@ -130,9 +130,10 @@ int check_flash_dims(const rt_attention_shape* s, uint64_t n_kv_heads, rt_err_de
     return RT_OK;
 }
 
+// bnhd: tensors are [batch, seq, heads, dim] instead of [batch, heads, seq, dim]
 int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n_kv_heads, const float* q,
                      const float* k, const float* v, int mask_kind, const uint8_t* keep, float* out,
-                     rt_err_detail* err) {
+                     rt_err_detail* err, bool bnhd = false) {
     if (s->dim > 128) return fail(err, RT_ERR_UNSUPPORTED, -1, 128, s->dim, "f32 flash kernel covers dim <= 128");
     rt::FlashF32Params p;
     p.q = q;
@@ -149,6 +150,13 @@ int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n
     p.mask = mask_kind;
     p.ref_bc = (int)(s->bc == 0 ? 1 : (s->bc > 0x7fffffffull ? 0x7fffffff : s->bc));
     p.scale = 1.0f / sqrtf((float)s->dim);
+    if (bnhd) {
+        p.lq = p.lo = rt::layout_bnhd((long long)s->heads, (long long)s->seq, p.dim);
+        p.lkv = rt::layout_bnhd((long long)n_kv_heads, (long long)s->seq, p.dim);
+    } else {
+        p.lq = p.lo = rt::layout_bhnd((long long)s->heads, (long long)s->seq, p.dim);
+        p.lkv = rt::layout_bhnd((long long)n_kv_heads, (long long)s->seq, p.dim);
+    }
     HIP_TRY(rt::launch_flash_f32(stream, p), "flash_fwd_f32 launch");
     return RT_OK;
 }
@@ -323,7 +331,7 @@ RT_API int rt_flash_forward_f32_dev(void* stream, const rt_attention_shape* shap
 
 static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads, const void* q,
                              const void* k, const void* v, int mask, const uint8_t* keep, const int32_t* seq_lens,
-                             int zero_padded_rows, void* out, rt_err_detail* err) {
+                             int zero_padded_rows, void* out, rt_err_detail* err, bool bnhd = false) {
     clear_err(err);
     if (!shape) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "shape is NULL");
     if (shape->dim == 0) return fail(err, RT_ERR_ZERO_DIM, -1, 0, 0, "dim must be > 0");
@@ -335,8 +343,14 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
         return fail(err, RT_ERR_UNSUPPORTED, -1, 128, shape->dim, "bf16 flash kernels cover dim 64 and 128");
     if ((shape->seq + 127) / 128 * shape->batch * shape->heads > 0x7fffffffull)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
-    if (shape->seq > (1ull << 23))  // the kernel addresses rows of one (batch, head) slab with 32-bit byte offsets
-        return fail(err, RT_ERR_UNSUPPORTED, -1, 1ull << 23, shape->seq, "bf16 flash kernels cover seq <= 2^23");
+    {   // the kernel addresses the rows of one (batch, head) slab with 32-bit byte offsets
+        const uint64_t pitch_b = (bnhd ? shape->heads : 1) * shape->dim * 2;
+        if (shape->seq * pitch_b >= (1ull << 32))
+            return fail(err, RT_ERR_UNSUPPORTED, -1, (1ull << 32) / pitch_b, shape->seq,
+                        "bf16 flash kernels need seq * row pitch below 4 GiB");
+    }
+    if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 16, 0, "bf16 flash kernels need 16-byte aligned tensors");
     if (!q || !k || !v || !out || (mask == rt::kMaskPadding && !keep) || (mask == rt::kMaskVarlenCausal && !seq_lens))
         return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
     rc = ensure_device(err);
@@ -359,6 +373,13 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
     p.zero_padded_rows = zero_padded_rows;
     p.scale_log2e = (1.0f / sqrtf((float)shape->dim)) * rt::kLog2eHost;
     p.n_workers = g_num_cus;
+    if (bnhd) {
+        p.lq = p.lo = rt::layout_bnhd((long long)shape->heads, (long long)shape->seq, p.dim);
+        p.lkv = rt::layout_bnhd((long long)n_kv_heads, (long long)shape->seq, p.dim);
+    } else {
+        p.lq = p.lo = rt::layout_bhnd((long long)shape->heads, (long long)shape->seq, p.dim);
+        p.lkv = rt::layout_bhnd((long long)n_kv_heads, (long long)shape->seq, p.dim);
+    }
     HIP_TRY(rt::launch_flash_bf16((hipStream_t)stream, p), "flash_fwd_bf16 launch");
     return RT_OK;
 }
@@ -371,6 +392,65 @@ RT_API int rt_flash_forward_bf16_dev(void* stream, const rt_attention_shape* sha
         return fail(err, RT_ERR_UNSUPPORTED, -1, 0, (uint64_t)mask_kind, "unknown mask kind");
     }
     return flash_bf16_common(stream, shape, n_kv_heads, q, k, v, mask_kind, keep, nullptr, 0, out, err);
+}
+
+RT_API int rt_flash_forward_bnhd_bf16_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,
+                                          const void* q, const void* k, const void* v, int mask_kind,
+                                          const uint8_t* keep, void* out, rt_err_detail* err) {
+    if (mask_kind < RT_MASK_NONE || mask_kind > RT_MASK_PADDING) {
+        clear_err(err);
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, (uint64_t)mask_kind, "unknown mask kind");
+    }
+    return flash_bf16_common(stream, shape, n_kv_heads, q, k, v, mask_kind, keep, nullptr, 0, out, err, true);
+}
+
+RT_API int rt_flash_forward_bnhd_f32_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,
+                                         const float* q, const float* k, const float* v, int mask_kind,
+                                         const uint8_t* keep, float* out, rt_err_detail* err) {
+    clear_err(err);
+    if (!shape) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "shape is NULL");
+    if (shape->dim == 0) return fail(err, RT_ERR_ZERO_DIM, -1, 0, 0, "dim must be > 0");
+    if (mask_kind < RT_MASK_NONE || mask_kind > RT_MASK_PADDING)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, (uint64_t)mask_kind, "unknown mask kind");
+    if (n_kv_heads == 0) n_kv_heads = shape->heads;
+    if (shape->seq == 0 || shape->batch == 0 || shape->heads == 0) return RT_OK;
+    int rc = check_flash_dims(shape, n_kv_heads, err);
+    if (rc) return rc;
+    if (!q || !k || !v || !out || (mask_kind == RT_MASK_PADDING && !keep))
+        return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    rc = ensure_device(err);
+    if (rc) return rc;
+    return flash_f32_device((hipStream_t)stream, shape, n_kv_heads, q, k, v, mask_kind, keep, out, err, true);
+}
+
+RT_API int rt_mha_flash_forward_f32(const float* q, size_t q_len, const float* k, size_t k_len, const float* v,
+                                    size_t v_len, float* out, size_t out_len, size_t batch, size_t seq, size_t heads,
+                                    size_t head_dim, rt_err_detail* err) {
+    clear_err(err);
+    // the reference transposes to [B,H,T,hd] and calls flash_forward (attention.rs:474-483): same checks, same order
+    rt_attention_shape shape = {batch, heads, seq, head_dim, 64, 64};
+    int rc = validate_flash(&shape, q_len, k_len, v_len, out_len, RT_MASK_NONE, 0, err);
+    if (rc) return rc;
+    if (seq == 0 || q_len == 0) return RT_OK;
+    if (!q || !k || !v || !out) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    rc = check_flash_dims(&shape, heads, err);
+    if (rc) return rc;
+    rc = ensure_device(err);
+    if (rc) return rc;
+    DevBuf dq, dk, dv, dout;
+    size_t bytes = q_len * sizeof(float);
+    HIP_TRY(hipMalloc(&dq.p, bytes), "hipMalloc q");
+    HIP_TRY(hipMalloc(&dk.p, bytes), "hipMalloc k");
+    HIP_TRY(hipMalloc(&dv.p, bytes), "hipMalloc v");
+    HIP_TRY(hipMalloc(&dout.p, bytes), "hipMalloc out");
+    HIP_TRY(hipMemcpy(dq.p, q, bytes, hipMemcpyHostToDevice), "copy q");
+    HIP_TRY(hipMemcpy(dk.p, k, bytes, hipMemcpyHostToDevice), "copy k");
+    HIP_TRY(hipMemcpy(dv.p, v, bytes, hipMemcpyHostToDevice), "copy v");
+    rc = flash_f32_device(nullptr, &shape, heads, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p,
+                          RT_MASK_NONE, nullptr, (float*)dout.p, err, true);
+    if (rc) return rc;
+    HIP_TRY(hipMemcpy(out, dout.p, bytes, hipMemcpyDeviceToHost), "copy out");
+    return RT_OK;
 }
 
 RT_API int rt_flash_forward_varlen_bf16_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,

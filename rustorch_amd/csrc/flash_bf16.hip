@@ -182,6 +182,9 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     const int n_jobs = n_qtiles * n_bh;
     const int W = gridDim.x, w = blockIdx.x;
     const float c = p.scale_log2e;
+    // bytes between consecutive rows of a (batch, head) slab: ROWB when the slab is contiguous
+    const uint32_t q_pitch_b = (uint32_t)p.lq.row_pitch * 2u, kv_pitch_b = (uint32_t)p.lkv.row_pitch * 2u;
+    const uint32_t o_pitch_b = (uint32_t)p.lo.row_pitch * 2u;
     const float lazy_raw = kLazyLog2 / c;  // the rescale threshold in raw-score units
 
     bool poison = false;  // a padding mask hiding the reference's whole first key tile: every row NaN
@@ -214,7 +217,6 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         v_base = (uint32_t)(2 * TILE_B + row * ROWB + ((low ^ swz_v(row)) * 16) + 8 * (j & 1));
     }
     // (2ks + hh) ^ x == (hh ^ x) ^ 2ks and (4dt + low) ^ x == (low ^ x) ^ 4dt bit for bit
-    auto k_addr = [&](int ks, int flip) { return lds + (k_base ^ (uint32_t)(32 * ks + flip)); };
     auto v_addr = [&](int dt) { return lds + (v_base ^ (uint32_t)(64 * dt)); };
 
     // state of the current job
@@ -242,7 +244,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         int r = kv0 + ld_row0 + NWAVES * RPI * n;
         asm volatile("" : "+v"(r));  // recompute per call: hoisted copies of these offsets only cost registers
         r = min(r, n_keys - 1);
-        const uint32_t row_off = (uint32_t)r * ROWB;  // a (b, h) slab is below 4 GiB: seq * dim * 2 < 2^32
+        const uint32_t row_off = (uint32_t)r * kv_pitch_b;  // seq * row pitch stays below 4 GiB (checked by the caller)
         load_to_lds(Kg, row_off + ld_k0, kdst);
         load_to_lds(Vg, row_off + ld_v0, kdst + 2 * TILE_B);
     };
@@ -280,10 +282,10 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         q0 = qtile * BR;
         qw = q0 + wave * 32;
         q_row = qw + col;
-        const uint16_t* Qg = p.q + ((size_t)b * p.heads + h) * (size_t)N * HD;
-        Kg = (const unsigned char*)(p.k + ((size_t)b * p.kv_heads + kvh) * (size_t)N * HD);
-        Vg = (const unsigned char*)(p.v + ((size_t)b * p.kv_heads + kvh) * (size_t)N * HD);
-        Og = p.out + ((size_t)b * p.heads + h) * (size_t)N * HD;
+        const uint16_t* Qg = p.q + (size_t)b * p.lq.batch_stride + (size_t)h * p.lq.head_stride;
+        Kg = (const unsigned char*)(p.k + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride);
+        Vg = (const unsigned char*)(p.v + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride);
+        Og = p.out + (size_t)b * p.lo.batch_stride + (size_t)h * p.lo.head_stride;
         n_keys = N;  // keys that exist for this sequence
         if (MODE == kMaskVarlenCausal) n_keys = min(N, max(0, p.seq_lens[b]));
         int kv_end = n_keys;
@@ -298,11 +300,11 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             int lane_q = lane;
             asm volatile("" : "+v"(lane_q));  // (addresses rebuilt per job: see the note at the output stage)
             const int r0 = lane_q / SPR, slot = lane_q % SPR;
-            const unsigned char* qp = (const unsigned char*)Qg + (size_t)(qw + r0) * ROWB + slot * 16;
+            const unsigned char* qp = (const unsigned char*)Qg + (size_t)(qw + r0) * q_pitch_b + slot * 16;
 #pragma unroll
             for (int n = 0; n < KS; n++) {
                 u32x4_t z = {0u, 0u, 0u, 0u};
-                if (qw + RPI * n + r0 < N) z = *(const u32x4_t*)(qp + (size_t)n * RPI * ROWB);
+                if (qw + RPI * n + r0 < N) z = *(const u32x4_t*)(qp + (size_t)n * RPI * q_pitch_b);
                 qreg[n] = __builtin_bit_cast(bf16x8_t, z);
             }
         }
@@ -570,14 +572,15 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         {
             const int r0 = lane_e / SPR, pos = lane_e % SPR;  // instruction n covers rows n*RPI + r0
             const uint32_t rd = obuf + (uint32_t)(r0 * ROWB + pos * 16);
-            // global slot pos ^ swz_o(n*RPI + r0): the part of the swizzle that depends on n is XORed in below
-            unsigned char* gp = (unsigned char*)og_out + (size_t)(qw_out + r0) * ROWB + ((pos ^ swz_o(r0)) * 16);
+            // global slot pos ^ swz_o(n*RPI + r0); r0 < RPI and RPI is a power of two, so the part of the
+            // swizzle that depends on n is a plain XOR into the slot bits of the lane's byte offset
+            const uint32_t slot_off = (uint32_t)((pos ^ swz_o(r0)) * 16);
+            unsigned char* gp = (unsigned char*)og_out + (size_t)(qw_out + r0) * o_pitch_b;
 #pragma unroll
             for (int n = 0; n < 32 / RPI; n++) {
                 u32x4_t v = *(const u32x4_t __attribute__((address_space(3)))*)(uintptr_t)(rd + (uint32_t)(n * RPI * ROWB));
-                const int flip = (swz_o(n * RPI) * 16);  // r0 < RPI and RPI is a power of two: no carry into these bits
                 if (qw_out + n * RPI + r0 < N)
-                    *(u32x4_t*)((unsigned char*)((uintptr_t)(gp + (size_t)n * RPI * ROWB) ^ (uintptr_t)flip)) = v;
+                    *(u32x4_t*)(gp + (size_t)n * RPI * o_pitch_b + (slot_off ^ (uint32_t)(swz_o(n * RPI) * 16))) = v;
             }
         }
         RT_PHASE(11);

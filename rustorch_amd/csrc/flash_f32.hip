@@ -41,10 +41,11 @@ __global__ __launch_bounds__(64) void flash_fwd_f32_kernel(FlashF32Params p) {
     const int q0 = qtile * kRows;
     const int h = blockIdx.y, b = blockIdx.z;
     const int kvh = h / p.group;
-    const float* __restrict__ Qg = p.q + ((size_t)b * p.heads + h) * (size_t)N * D;
-    const float* __restrict__ Kg = p.k + ((size_t)b * p.kv_heads + kvh) * (size_t)N * D;
-    const float* __restrict__ Vg = p.v + ((size_t)b * p.kv_heads + kvh) * (size_t)N * D;
-    float* __restrict__ Og = p.out + ((size_t)b * p.heads + h) * (size_t)N * D;
+    const float* __restrict__ Qg = p.q + (size_t)b * p.lq.batch_stride + (size_t)h * p.lq.head_stride;
+    const float* __restrict__ Kg = p.k + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+    const float* __restrict__ Vg = p.v + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+    float* __restrict__ Og = p.out + (size_t)b * p.lo.batch_stride + (size_t)h * p.lo.head_stride;
+    const size_t q_pitch = p.lq.row_pitch, kv_pitch = p.lkv.row_pitch, o_pitch = p.lo.row_pitch;
 
     // With a padding mask the reference's recurrence turns every row into NaN when its first
     // key tile [0, bc) holds no visible key (cpu_forward.rs:364-384); reproduce that outcome.
@@ -60,7 +61,7 @@ __global__ __launch_bounds__(64) void flash_fwd_f32_kernel(FlashF32Params p) {
     for (int idx = lane; idx < kRows * DPAD; idx += kWave) {
         int r = idx / DPAD, d = idx - r * DPAD;
         int qr = q0 + r;
-        Qs[r * LDQ + d] = (qr < N && d < D) ? Qg[(size_t)qr * D + d] : 0.0f;
+        Qs[r * LDQ + d] = (qr < N && d < D) ? Qg[(size_t)qr * q_pitch + d] : 0.0f;
     }
 
     f32x16_t acc_o[DT];
@@ -81,8 +82,8 @@ __global__ __launch_bounds__(64) void flash_fwd_f32_kernel(FlashF32Params p) {
             int r = idx / DPAD, d = idx - r * DPAD;
             int kr = kv0 + r;
             bool ok = (kr < N && d < D);
-            Ks[r * LDQ + d] = ok ? Kg[(size_t)kr * D + d] : 0.0f;
-            Vs[r * DPAD + d] = ok ? Vg[(size_t)kr * D + d] : 0.0f;
+            Ks[r * LDQ + d] = ok ? Kg[(size_t)kr * kv_pitch + d] : 0.0f;
+            Vs[r * DPAD + d] = ok ? Vg[(size_t)kr * kv_pitch + d] : 0.0f;
         }
         __syncthreads();
 
@@ -154,7 +155,7 @@ __global__ __launch_bounds__(64) void flash_fwd_f32_kernel(FlashF32Params p) {
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 int d = t * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
-                if (d < D) Og[(size_t)q_row * D + d] = good ? acc_o[t][i] * inv_l : quiet_nan();
+                if (d < D) Og[(size_t)q_row * o_pitch + d] = good ? acc_o[t][i] * inv_l : quiet_nan();
             }
     }
 }

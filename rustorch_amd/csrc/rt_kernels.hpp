@@ -9,6 +9,21 @@ namespace rt {
 enum MaskKind : int { kMaskNone = 0, kMaskCausal = 1, kMaskPadding = 2, kMaskVarlenCausal = 3 };
 constexpr float kLog2eHost = 1.4426950408889634f;
 
+// Where element [b, h, row, 0] of a 4-D attention tensor sits (in elements): rows of `dim` contiguous
+// elements, `row_pitch` apart.  [B,H,N,D] row-major: {H*N*D, N*D, D}; [B,N,H,D] row-major (the layout
+// MultiHeadAttention holds its projections in): {N*H*D, D, H*D}.
+struct TensorLayout {
+    long long batch_stride;
+    long long head_stride;
+    int row_pitch;
+};
+inline TensorLayout layout_bhnd(long long heads, long long seq, int dim) {
+    return TensorLayout{heads * seq * dim, seq * dim, dim};
+}
+inline TensorLayout layout_bnhd(long long heads, long long seq, int dim) {
+    return TensorLayout{seq * heads * dim, (long long)dim, (int)(heads * dim)};
+}
+
 struct FlashF32Params {
     const float* q;
     const float* k;
@@ -20,6 +35,7 @@ struct FlashF32Params {
     int mask;
     int ref_bc;  // the reference's key-tile size, for the leading-masked-tile rule
     float scale;
+    TensorLayout lq, lkv, lo;  // layouts of q, of k and v, of out
 };
 // dim <= 128.  Returns hipErrorInvalidValue for an unsupported dim.
 hipError_t launch_flash_f32(hipStream_t stream, const FlashF32Params& p);
@@ -38,6 +54,7 @@ struct FlashBf16Params {
     int zero_padded_rows;
     float scale_log2e;  // (1/sqrt(dim)) * log2(e)
     int n_workers;      // persistent workgroups to launch: the number of CUs
+    TensorLayout lq, lkv, lo;  // layouts of q, of k and v, of out; seq * row_pitch * 2 bytes must stay below 2^32
 };
 // dim in {64, 128}.
 hipError_t launch_flash_bf16(hipStream_t stream, const FlashBf16Params& p);
