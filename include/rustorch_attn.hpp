@@ -1,0 +1,313 @@
+// rustorch_attn.hpp -- C++ host-side mirror of rustorch's attention call surface over the C ABI of
+// librt_attn_hip.so (rt_attn.h).  Header only; link with -lrt_attn_hip.
+//
+// The names, argument meaning and error behaviour follow the Rust items they stand for (paths relative to
+// the reference checkout):
+//
+//   rustorch_attn::AttentionShape, AttentionError, flash_forward, flash_forward_masked
+//                                   crates/rustorch-attention/src/cpu_forward.rs:49-242
+//   rustorch_attn::Mask             crates/rustorch-attention/src/mask.rs:26-78
+//   rustorch_attn::gqa_forward_f32, GQAError
+//                                   crates/rustorch-nn/src/gqa.rs:36-210
+//   rustorch_attn::mha_flash_forward_f32
+//                                   crates/rustorch-nn/src/attention.rs:452-495
+//   rustorch_attn::LlmKernels       crates/rustorch-cuda/src/llm_kernels.rs:874-958 (attention part)
+//   rustorch_attn::HipStorage       the slot of Storage::Cuda, crates/rustorch-core/src/tensor/storage.rs:776-817
+//
+// Where Rust returns Result<(), E>, these functions throw E (a std::exception carrying the enum's fields).
+// There is no CPU fallback: on a machine without a gfx950 device compute calls throw DeviceError.
+#ifndef RUSTORCH_ATTN_HPP
+#define RUSTORCH_ATTN_HPP
+
+#include <array>
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "rt_attn.h"
+
+namespace rustorch_attn {
+
+// ---- errors ------------------------------------------------------------------------------------------
+
+// AttentionError (cpu_forward.rs:93-114) with MaskError folded in as the Mask variant (mask.rs:70-78).
+struct AttentionError : std::runtime_error {
+    enum class Kind { ZeroDim, BufferShapeMismatch, OutputShapeMismatch, MaskPaddingLengthMismatch };
+    Kind kind;
+    std::string which;  // "q" | "k" | "v" for BufferShapeMismatch
+    size_t expected = 0, got = 0;
+    AttentionError(Kind k, std::string w, size_t e, size_t g, const std::string& msg)
+        : std::runtime_error(msg), kind(k), which(std::move(w)), expected(e), got(g) {}
+};
+
+// GQAError (gqa.rs:37-55).
+struct GQAError : std::runtime_error {
+    enum class Kind { HeadCountMismatch, WrongInputLen };
+    Kind kind;
+    std::string which;  // "q" | "k" | "v" | "out" | "flash_forward"
+    size_t expected = 0, got = 0;  // HeadCountMismatch: expected = n_heads, got = n_kv_heads
+    GQAError(Kind k, std::string w, size_t e, size_t g, const std::string& msg)
+        : std::runtime_error(msg), kind(k), which(std::move(w)), expected(e), got(g) {}
+};
+
+// Stands where the reference has CudaError: no device, a failed HIP call, a shape the kernels do not cover.
+struct DeviceError : std::runtime_error {
+    int status;     // rt_status
+    int hip_error;  // hipError_t when status == RT_ERR_HIP
+    DeviceError(int st, int he, const std::string& msg) : std::runtime_error(msg), status(st), hip_error(he) {}
+};
+
+namespace detail {
+inline const char* which_name(int w) {
+    static const char* names[] = {"q", "k", "v", "out", "flash_forward"};
+    return (w >= 0 && w < 5) ? names[w] : "";
+}
+[[noreturn]] inline void throw_device(int rc, const rt_err_detail& e) {
+    throw DeviceError(rc, e.hip_error, std::string(rt_status_name(rc)) + ": " + e.message);
+}
+inline void check_attention(int rc, const rt_err_detail& e) {
+    using K = AttentionError::Kind;
+    switch (rc) {
+        case RT_OK: return;
+        case RT_ERR_ZERO_DIM: throw AttentionError(K::ZeroDim, "", 0, 0, "dim must be > 0");
+        case RT_ERR_BUFFER_SHAPE_MISMATCH: {
+            std::string w = which_name(e.which);
+            throw AttentionError(K::BufferShapeMismatch, w, e.expected, e.got,
+                                 w + " buffer has " + std::to_string(e.got) + " elements, expected " +
+                                     std::to_string(e.expected));
+        }
+        case RT_ERR_OUTPUT_SHAPE_MISMATCH:
+            throw AttentionError(K::OutputShapeMismatch, "", e.expected, e.got,
+                                 "output buffer has " + std::to_string(e.got) + " elements, expected " +
+                                     std::to_string(e.expected));
+        case RT_ERR_PADDING_LENGTH_MISMATCH:
+            throw AttentionError(K::MaskPaddingLengthMismatch, "", e.expected, e.got,
+                                 "mask error: padding mask len " + std::to_string(e.got) + ", expected " +
+                                     std::to_string(e.expected));
+        default: throw_device(rc, e);
+    }
+}
+inline void check_gqa(int rc, const rt_err_detail& e) {
+    using K = GQAError::Kind;
+    switch (rc) {
+        case RT_OK: return;
+        case RT_ERR_HEAD_COUNT_MISMATCH:
+            throw GQAError(K::HeadCountMismatch, "", e.expected, e.got,
+                           "gqa: n_heads " + std::to_string(e.expected) + " not divisible by n_kv_heads " +
+                               std::to_string(e.got));
+        case RT_ERR_WRONG_INPUT_LEN: {
+            std::string w = which_name(e.which);
+            throw GQAError(K::WrongInputLen, w, e.expected, e.got,
+                           "gqa: " + w + " expected " + std::to_string(e.expected) + " f32, got " +
+                               std::to_string(e.got));
+        }
+        default: throw_device(rc, e);
+    }
+}
+inline void check_device(int rc, const rt_err_detail& e) {
+    if (rc != RT_OK) throw_device(rc, e);
+}
+}  // namespace detail
+
+// ---- shapes and masks ------------------------------------------------------------------------------------
+
+// AttentionShape (cpu_forward.rs:49-89): row-major [batch, heads, seq, dim]; br = bc = 64 by default.
+struct AttentionShape {
+    size_t batch = 0, heads = 0, seq = 0, dim = 0, br = 64, bc = 64;
+    static AttentionShape make(size_t batch, size_t heads, size_t seq, size_t dim) {
+        return AttentionShape{batch, heads, seq, dim, 64, 64};
+    }
+    AttentionShape with_tiles(size_t br_, size_t bc_) const {
+        AttentionShape s = *this;
+        s.br = br_;
+        s.bc = bc_;
+        return s;
+    }
+    size_t buffer_len() const { return batch * heads * seq * dim; }
+    std::array<size_t, 4> strides() const { return {heads * seq * dim, seq * dim, dim, 1}; }
+    rt_attention_shape c() const { return rt_attention_shape{batch, heads, seq, dim, br, bc}; }
+};
+
+// Mask (mask.rs:26-65).
+struct Mask {
+    enum class Kind { None = RT_MASK_NONE, Causal = RT_MASK_CAUSAL, Padding = RT_MASK_PADDING };
+    Kind kind = Kind::None;
+    std::vector<uint8_t> keep;  // Padding: one byte per key, non-zero = visible
+    static Mask none() { return Mask{}; }
+    static Mask causal() {
+        Mask m;
+        m.kind = Kind::Causal;
+        return m;
+    }
+    static Mask padding(const std::vector<bool>& keep_mask) {
+        Mask m;
+        m.kind = Kind::Padding;
+        m.keep.assign(keep_mask.begin(), keep_mask.end());
+        return m;
+    }
+    bool is_masked(size_t qi, size_t kj) const {
+        if (kind == Kind::Causal) return kj > qi;
+        if (kind == Kind::Padding) return kj < keep.size() && keep[kj] == 0;
+        return false;
+    }
+};
+
+// ---- prefill on host slices (synchronous, like the Rust functions) ----------------------------------------
+
+inline void flash_forward_masked(const AttentionShape& shape, const float* q, size_t q_len, const float* k,
+                                 size_t k_len, const float* v, size_t v_len, const Mask& mask, float* out,
+                                 size_t out_len) {
+    rt_attention_shape s = shape.c();
+    rt_err_detail e;
+    int rc = rt_flash_forward_masked_f32(&s, q, q_len, k, k_len, v, v_len, (int)mask.kind,
+                                         mask.keep.empty() ? nullptr : mask.keep.data(), mask.keep.size(), out,
+                                         out_len, &e);
+    detail::check_attention(rc, e);
+}
+inline void flash_forward_masked(const AttentionShape& shape, const std::vector<float>& q,
+                                 const std::vector<float>& k, const std::vector<float>& v, const Mask& mask,
+                                 std::vector<float>& out) {
+    flash_forward_masked(shape, q.data(), q.size(), k.data(), k.size(), v.data(), v.size(), mask, out.data(),
+                         out.size());
+}
+inline void flash_forward(const AttentionShape& shape, const std::vector<float>& q, const std::vector<float>& k,
+                          const std::vector<float>& v, std::vector<float>& out) {
+    flash_forward_masked(shape, q, k, v, Mask::none(), out);
+}
+
+// gqa_forward_f32 (gqa.rs:94-210).
+inline void gqa_forward_f32(const std::vector<float>& q, const std::vector<float>& k, const std::vector<float>& v,
+                            std::vector<float>& out, size_t batch, size_t n_heads, size_t n_kv_heads, size_t seq_q,
+                            size_t seq_kv, size_t head_dim) {
+    rt_err_detail e;
+    int rc = rt_gqa_forward_f32(q.data(), q.size(), k.data(), k.size(), v.data(), v.size(), out.data(), out.size(),
+                                batch, n_heads, n_kv_heads, seq_q, seq_kv, head_dim, &e);
+    detail::check_gqa(rc, e);
+}
+
+// mha_flash_forward_f32 (attention.rs:452-495): q, k, v [B,T,H,hd]; returns [B,T,H*hd].
+inline std::vector<float> mha_flash_forward_f32(const std::vector<float>& q, const std::vector<float>& k,
+                                                const std::vector<float>& v, size_t batch, size_t seq, size_t heads,
+                                                size_t head_dim) {
+    std::vector<float> out(batch * seq * heads * head_dim);
+    rt_err_detail e;
+    int rc = rt_mha_flash_forward_f32(q.data(), q.size(), k.data(), k.size(), v.data(), v.size(), out.data(),
+                                      out.size(), batch, seq, heads, head_dim, &e);
+    detail::check_attention(rc, e);
+    return out;
+}
+
+// ---- device memory --------------------------------------------------------------------------------------
+
+class HipStorage {
+public:
+    HipStorage() = default;
+    explicit HipStorage(size_t bytes) : bytes_(bytes) {
+        rt_err_detail e;
+        ptr_ = rt_buf_alloc(bytes, &e);
+        if (!ptr_ && bytes) detail::throw_device(e.hip_error ? RT_ERR_HIP : RT_ERR_NO_DEVICE, e);
+    }
+    template <typename T>
+    static HipStorage from_host(const std::vector<T>& host) {
+        HipStorage s(host.size() * sizeof(T));
+        s.upload(host.data(), host.size() * sizeof(T));
+        return s;
+    }
+    HipStorage(const HipStorage&) = delete;
+    HipStorage& operator=(const HipStorage&) = delete;
+    HipStorage(HipStorage&& o) noexcept : ptr_(o.ptr_), bytes_(o.bytes_) { o.ptr_ = nullptr; o.bytes_ = 0; }
+    HipStorage& operator=(HipStorage&& o) noexcept {
+        if (this != &o) {
+            release();
+            ptr_ = o.ptr_;
+            bytes_ = o.bytes_;
+            o.ptr_ = nullptr;
+            o.bytes_ = 0;
+        }
+        return *this;
+    }
+    ~HipStorage() { release(); }
+    void* ptr() const { return ptr_; }
+    size_t byte_len() const { return bytes_; }
+    void upload(const void* src, size_t bytes, void* stream = nullptr) {
+        rt_err_detail e;
+        detail::check_device(rt_memcpy_h2d(ptr_, src, bytes, stream, &e), e);
+    }
+    void download(void* dst, size_t bytes, void* stream = nullptr) const {
+        rt_err_detail e;
+        detail::check_device(rt_memcpy_d2h(dst, ptr_, bytes, stream, &e), e);
+    }
+    template <typename T>
+    std::vector<T> to_host() const {
+        std::vector<T> h(bytes_ / sizeof(T));
+        download(h.data(), h.size() * sizeof(T));
+        return h;
+    }
+
+private:
+    void release() {
+        if (ptr_) (void)rt_buf_free(ptr_, nullptr);
+        ptr_ = nullptr;
+    }
+    void* ptr_ = nullptr;
+    size_t bytes_ = 0;
+};
+
+inline void synchronize(void* stream = nullptr) {
+    rt_err_detail e;
+    detail::check_device(rt_stream_synchronize(stream, &e), e);
+}
+
+// ---- device-resident prefill (bf16 bit patterns) ------------------------------------------------------------
+
+inline void flash_forward_bf16_dev(const AttentionShape& shape, const void* q, const void* k, const void* v, void* out,
+                                   Mask::Kind mask = Mask::Kind::None, const uint8_t* keep_dev = nullptr,
+                                   size_t n_kv_heads = 0, void* stream = nullptr) {
+    rt_attention_shape s = shape.c();
+    rt_err_detail e;
+    detail::check_attention(rt_flash_forward_bf16_dev(stream, &s, n_kv_heads, q, k, v, (int)mask, keep_dev, out, &e), e);
+}
+inline void flash_forward_varlen_bf16_dev(const AttentionShape& shape, const void* q, const void* k, const void* v,
+                                          const int32_t* seq_lens_dev, void* out, bool zero_padded_rows = true,
+                                          size_t n_kv_heads = 0, void* stream = nullptr) {
+    rt_attention_shape s = shape.c();
+    rt_err_detail e;
+    detail::check_attention(
+        rt_flash_forward_varlen_bf16_dev(stream, &s, n_kv_heads, q, k, v, seq_lens_dev, zero_padded_rows ? 1 : 0, out, &e),
+        e);
+}
+
+// ---- LlmKernels: the attention launchers (llm_kernels.rs:874-958), raw device addresses and i32 dims ----------
+
+struct LlmKernels {
+    static void kv_append_bf16(void* stream, void* k_cache, void* v_cache, const void* k_in, const void* v_in, int32_t pos,
+                               int32_t n_kv, int32_t head_dim, int32_t max_seq) {
+        rt_err_detail e;
+        detail::check_device(rt_kv_append_bf16(stream, k_cache, v_cache, k_in, v_in, pos, n_kv, head_dim, max_seq, &e), e);
+    }
+    static void gqa_decode_online_bf16(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out,
+                                       int32_t n_heads, int32_t n_kv, int32_t kv_len, int32_t head_dim, int32_t max_seq) {
+        rt_err_detail e;
+        detail::check_gqa(
+            rt_gqa_decode_online_bf16(stream, q, k_cache, v_cache, out, n_heads, n_kv, kv_len, head_dim, max_seq, &e), e);
+    }
+    static size_t gqa_decode_workspace_bytes(int32_t batch, int32_t n_heads, int32_t n_kv, int32_t head_dim,
+                                             int32_t max_seq) {
+        return rt_gqa_decode_workspace_bytes(batch, n_heads, n_kv, head_dim, max_seq);
+    }
+    static void gqa_decode_batched_bf16(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out,
+                                        const int32_t* kv_lens, int32_t batch, int32_t n_heads, int32_t n_kv,
+                                        int32_t head_dim, int32_t max_seq, void* workspace, size_t workspace_bytes) {
+        rt_err_detail e;
+        detail::check_gqa(rt_gqa_decode_batched_bf16(stream, q, k_cache, v_cache, out, kv_lens, batch, n_heads, n_kv,
+                                                     head_dim, max_seq, workspace, workspace_bytes, &e),
+                          e);
+    }
+};
+
+}  // namespace rustorch_attn
+
+#endif  // RUSTORCH_ATTN_HPP

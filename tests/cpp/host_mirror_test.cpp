@@ -1,0 +1,223 @@
+// Tests of the C++ host mirror (include/rustorch_attn.hpp), written after the reference's own unit tests
+// (crates/rustorch-attention/src/cpu_forward.rs tests module, crates/rustorch-nn/src/gqa.rs tests).
+//   host_mirror_test errors   error enums and their order: needs no GPU
+//   host_mirror_test gpu      small forwards against a double-precision loop and the reference's closed forms
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <limits>
+#include <vector>
+
+#include "rustorch_attn.hpp"
+
+using namespace rustorch_attn;
+
+static int g_failed = 0;
+#define CHECK(cond)                                                          \
+    do {                                                                     \
+        if (!(cond)) {                                                       \
+            std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);      \
+            ++g_failed;                                                      \
+        }                                                                    \
+    } while (0)
+
+template <typename E, typename F>
+static bool throws(F&& f, E* out = nullptr) {
+    try {
+        f();
+    } catch (const E& e) {
+        if (out) *out = e;
+        return true;
+    } catch (...) {
+        return false;
+    }
+    return false;
+}
+
+static std::vector<float> lcg(size_t n, uint64_t seed) {  // uniform in [-1, 1)
+    std::vector<float> v(n);
+    uint64_t s = seed * 6364136223846793005ull + 1442695040888963407ull;
+    for (size_t i = 0; i < n; i++) {
+        s = s * 6364136223846793005ull + 1442695040888963407ull;
+        v[i] = (float)((double)(s >> 11) / 9007199254740992.0 * 2.0 - 1.0);
+    }
+    return v;
+}
+
+// softmax(q k^T / sqrt(d)) v in double, with the reference's "no visible key -> NaN row" rule
+static std::vector<float> naive(const AttentionShape& s, const std::vector<float>& q, const std::vector<float>& k,
+                                const std::vector<float>& v, const Mask& mask) {
+    std::vector<float> out(s.buffer_len());
+    const double scale = 1.0 / std::sqrt((double)s.dim);
+    std::vector<double> sc(s.seq);
+    for (size_t bh = 0; bh < s.batch * s.heads; bh++) {
+        const float* Q = q.data() + bh * s.seq * s.dim;
+        const float* K = k.data() + bh * s.seq * s.dim;
+        const float* V = v.data() + bh * s.seq * s.dim;
+        for (size_t i = 0; i < s.seq; i++) {
+            double m = -std::numeric_limits<double>::infinity();
+            for (size_t j = 0; j < s.seq; j++) {
+                double d = 0;
+                for (size_t t = 0; t < s.dim; t++) d += (double)Q[i * s.dim + t] * K[j * s.dim + t];
+                sc[j] = mask.is_masked(i, j) ? -std::numeric_limits<double>::infinity() : d * scale;
+                if (sc[j] > m) m = sc[j];
+            }
+            double l = 0;
+            for (size_t j = 0; j < s.seq; j++) l += std::isinf(m) ? 0.0 : std::exp(sc[j] - m);
+            for (size_t t = 0; t < s.dim; t++) {
+                double o = 0;
+                for (size_t j = 0; j < s.seq; j++) o += (std::isinf(m) ? 0.0 : std::exp(sc[j] - m)) * V[j * s.dim + t];
+                out[(bh * s.seq + i) * s.dim + t] = l > 0 ? (float)(o / l) : std::numeric_limits<float>::quiet_NaN();
+            }
+        }
+    }
+    return out;
+}
+
+static void test_errors() {
+    {   // ZeroDim comes first (cpu_forward.rs:142-169)
+        std::vector<float> e, out;
+        AttentionError err(AttentionError::Kind::ZeroDim, "", 0, 0, "");
+        CHECK(throws<AttentionError>([&] { flash_forward(AttentionShape::make(1, 1, 4, 0), e, e, e, out); }, &err));
+        CHECK(err.kind == AttentionError::Kind::ZeroDim);
+    }
+    {   // then q, k, v lengths, then the output, then the padding mask
+        AttentionShape s = AttentionShape::make(1, 1, 4, 8);
+        std::vector<float> good(32), bad(16), out(32);
+        const char* which[3] = {"q", "k", "v"};
+        for (int i = 0; i < 3; i++) {
+            AttentionError err(AttentionError::Kind::ZeroDim, "", 0, 0, "");
+            const std::vector<float>& a = i == 0 ? bad : good;
+            const std::vector<float>& b = i <= 1 ? bad : good;
+            CHECK(throws<AttentionError>([&] { flash_forward(s, a, b, bad, out); }, &err));
+            CHECK(err.kind == AttentionError::Kind::BufferShapeMismatch && err.which == which[i]);
+            CHECK(err.expected == 32 && err.got == 16);
+            CHECK(std::string(err.what()) == std::string(which[i]) + " buffer has 16 elements, expected 32");
+        }
+        std::vector<float> short_out(31);
+        AttentionError err(AttentionError::Kind::ZeroDim, "", 0, 0, "");
+        CHECK(throws<AttentionError>([&] { flash_forward(s, good, good, good, short_out); }, &err));
+        CHECK(err.kind == AttentionError::Kind::OutputShapeMismatch && err.expected == 32 && err.got == 31);
+        AttentionShape s4 = AttentionShape::make(1, 1, 4, 4);
+        std::vector<float> out16(16);
+        CHECK(throws<AttentionError>(
+            [&] { flash_forward_masked(s4, bad, bad, bad, Mask::padding({true, true, true}), out16); }, &err));
+        CHECK(err.kind == AttentionError::Kind::MaskPaddingLengthMismatch && err.expected == 4 && err.got == 3);
+    }
+    {   // seq == 0 is Ok and touches nothing (cpu_forward.rs:203-206)
+        std::vector<float> e, out;
+        flash_forward(AttentionShape::make(2, 4, 0, 16), e, e, e, out);
+    }
+    {   // GQA: head counts first, then q, k, v, out (gqa.rs:106-141)
+        std::vector<float> q(20), kv(8), out(20);
+        GQAError err(GQAError::Kind::WrongInputLen, "", 0, 0, "");
+        CHECK(throws<GQAError>([&] { gqa_forward_f32(q, kv, kv, out, 1, 5, 2, 1, 1, 4); }, &err));
+        CHECK(err.kind == GQAError::Kind::HeadCountMismatch && err.expected == 5 && err.got == 2);
+        std::vector<float> q16(16), q7(7), kv9(9), out15(15);
+        CHECK(throws<GQAError>([&] { gqa_forward_f32(q7, kv, kv, q16, 1, 4, 2, 1, 1, 4); }, &err));
+        CHECK(err.which == "q" && err.expected == 16 && err.got == 7);
+        CHECK(throws<GQAError>([&] { gqa_forward_f32(q16, kv9, kv, q16, 1, 4, 2, 1, 1, 4); }, &err));
+        CHECK(err.which == "k" && err.expected == 8 && err.got == 9);
+        CHECK(throws<GQAError>([&] { gqa_forward_f32(q16, kv, kv9, q16, 1, 4, 2, 1, 1, 4); }, &err));
+        CHECK(err.which == "v");
+        CHECK(throws<GQAError>([&] { gqa_forward_f32(q16, kv, kv, out15, 1, 4, 2, 1, 1, 4); }, &err));
+        CHECK(err.which == "out" && err.expected == 16 && err.got == 15);
+    }
+    {   // shape helpers
+        AttentionShape s = AttentionShape::make(2, 3, 5, 7);
+        CHECK(s.buffer_len() == 210 && s.br == 64 && s.bc == 64);
+        auto st = s.strides();
+        CHECK(st[0] == 105 && st[1] == 35 && st[2] == 7 && st[3] == 1);
+        CHECK(Mask::causal().is_masked(1, 2) && !Mask::causal().is_masked(2, 2));
+        CHECK(Mask::padding({true, false}).is_masked(0, 1) && !Mask::padding({true, false}).is_masked(0, 0));
+    }
+}
+
+static float max_abs_diff(const std::vector<float>& a, const std::vector<float>& b, bool* nan_same) {
+    float m = 0;
+    *nan_same = true;
+    for (size_t i = 0; i < a.size(); i++) {
+        if (std::isnan(a[i]) != std::isnan(b[i])) *nan_same = false;
+        if (!std::isnan(a[i]) && !std::isnan(b[i])) m = std::fmax(m, std::fabs(a[i] - b[i]));
+    }
+    return m;
+}
+
+static void test_gpu() {
+    const size_t shapes[][4] = {{1, 1, 1, 4}, {1, 2, 7, 8}, {2, 3, 33, 16}, {1, 2, 130, 64}, {1, 1, 65, 128}};
+    for (auto& sh : shapes) {
+        AttentionShape s = AttentionShape::make(sh[0], sh[1], sh[2], sh[3]);
+        auto q = lcg(s.buffer_len(), 1), k = lcg(s.buffer_len(), 2), v = lcg(s.buffer_len(), 3);
+        std::vector<bool> keep(s.seq);
+        for (size_t j = 0; j < s.seq; j++) keep[j] = (j % 3 != 1);
+        const Mask masks[3] = {Mask::none(), Mask::causal(), Mask::padding(keep)};
+        for (const Mask& m : masks) {
+            std::vector<float> out(s.buffer_len(), -7.0f);
+            flash_forward_masked(s, q, k, v, m, out);
+            bool nan_same;
+            float d = max_abs_diff(out, naive(s, q, k, v, m), &nan_same);
+            CHECK(nan_same);
+            CHECK(d <= 1e-5f);
+        }
+    }
+    {   // N == 1: out == v (reference test single_token_returns_v)
+        AttentionShape s = AttentionShape::make(1, 1, 1, 4);
+        std::vector<float> q = {1, 2, 3, 4}, k = {4, 3, 2, 1}, v = {0.5f, -1.5f, 2.5f, 7.0f}, out(4);
+        flash_forward(s, q, k, v, out);
+        for (int i = 0; i < 4; i++) CHECK(out[i] == v[i]);
+    }
+    {   // keep = [T, F, F, T] with equal scores: the mean of V rows 0 and 3
+        AttentionShape s = AttentionShape::make(1, 1, 4, 1);
+        std::vector<float> q(4, 0.0f), k(4, 0.0f), v = {10, 99, 99, 30}, out(4);
+        flash_forward_masked(s, q, k, v, Mask::padding({true, false, false, true}), out);
+        for (int i = 0; i < 4; i++) CHECK(std::fabs(out[i] - 20.0f) <= 1e-5f);
+    }
+    {   // mha_flash_forward_f32 == flash_forward on transposed copies
+        size_t b = 2, t = 9, h = 3, d = 8;
+        auto q = lcg(b * t * h * d, 5), k = lcg(b * t * h * d, 6), v = lcg(b * t * h * d, 7);
+        auto tr = [&](const std::vector<float>& x) {  // [B,T,H,D] -> [B,H,T,D]
+            std::vector<float> y(x.size());
+            for (size_t bi = 0; bi < b; bi++)
+                for (size_t ti = 0; ti < t; ti++)
+                    for (size_t hi = 0; hi < h; hi++)
+                        for (size_t di = 0; di < d; di++)
+                            y[((bi * h + hi) * t + ti) * d + di] = x[((bi * t + ti) * h + hi) * d + di];
+            return y;
+        };
+        AttentionShape s = AttentionShape::make(b, h, t, d);
+        auto want = naive(s, tr(q), tr(k), tr(v), Mask::none());
+        auto got = mha_flash_forward_f32(q, k, v, b, t, h, d);
+        float m = 0;
+        for (size_t bi = 0; bi < b; bi++)
+            for (size_t ti = 0; ti < t; ti++)
+                for (size_t hi = 0; hi < h; hi++)
+                    for (size_t di = 0; di < d; di++)
+                        m = std::fmax(m, std::fabs(got[((bi * t + ti) * h + hi) * d + di] -
+                                                    want[((bi * h + hi) * t + ti) * d + di]));
+        CHECK(m <= 1e-5f);
+    }
+    {   // device buffers round-trip
+        std::vector<float> h = lcg(1000, 9);
+        HipStorage s = HipStorage::from_host(h);
+        auto back = s.to_host<float>();
+        CHECK(back == h);
+    }
+}
+
+int main(int argc, char** argv) {
+    const char* mode = argc > 1 ? argv[1] : "errors";
+    try {
+        if (!std::strcmp(mode, "errors")) test_errors();
+        else if (!std::strcmp(mode, "gpu")) test_gpu();
+        else {
+            std::printf("usage: %s errors|gpu\n", argv[0]);
+            return 2;
+        }
+    } catch (const std::exception& e) {
+        std::printf("FAIL: unexpected exception: %s\n", e.what());
+        return 1;
+    }
+    std::printf(g_failed ? "%d check(s) failed\n" : "ok\n", g_failed);
+    return g_failed ? 1 : 0;
+}
