@@ -370,18 +370,13 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             s[i] = masked ? neg_inf() : s[i];
         }
     };
-    // The softmax of an item is split over the two clusters.  The part that needs nothing but the finished
-    // scores runs in the second half of the matrix cluster, in the issue slots between the P.V
-    // instructions: the row max of the item, and t = s*c - m*c against the running max AS IT STANDS.  The
-    // softmax cluster then only raises the max when it pays (rarely: then t is shifted by the difference,
-    // and O and l are rescaled), takes exp2(t), the row sums and the bf16 conversion.
+    // The softmax of an item is split over the two clusters.  Its row max needs nothing but the finished
+    // scores and is taken in the second half of the matrix cluster, in the issue slots between the P.V
+    // instructions.  The softmax cluster then raises the running max when it pays (rarely: O and l are
+    // rescaled), and takes exp2(s*c - m*c), the row sums and the bf16 conversion.
     auto item_max = [&]() { return max_with_other_half(max16(s)); };
-    auto prescale = [&](int lo, int hi, float neg_mc) {
-#pragma unroll
-        for (int i = lo; i < hi; i++) s[i] = __builtin_fmaf(s[i], c, neg_mc);
-    };
-    // raise the running max when it pays (wave-uniform branch); mc_used is what prescale() subtracted
-    auto update_max = [&](float m_item, float mc_used) {
+    // raise the running max when it pays (wave-uniform branch)
+    auto update_max = [&](float m_item) {
         if (__builtin_expect(__any(m_item > m_run + lazy_raw), 0)) {
             float m_new = vmax(m_run, m_item);
             float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
@@ -392,17 +387,15 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             for (int t = 0; t < DT; t++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) acc_o[t][i] *= alpha;
-            const float shift = mc_used - m_use * c;  // t was taken against the old max
-#pragma unroll
-            for (int i = 0; i < 16; i++) s[i] += shift;
         }
     };
-    // p = exp2(t), row-sum share, and the two B operands of the item
+    // p = exp2(s*c - m*c), row-sum share, and the two B operands of the item
     auto exp_item = [&]() {
+        const float mc = ((m_run == neg_inf()) ? 0.0f : m_run) * c;
         float part[4];
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            float e = __builtin_amdgcn_exp2f(s[i]);
+            float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c, -mc));
             s[i] = e;
             if (i < 4) part[i] = e;
             else part[i & 3] += e;
@@ -447,8 +440,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             else k_read_one(std::integral_constant<int, 0>{}, TILE_B, ks);  // item 0 of the next tile, other stage
             __builtin_amdgcn_sched_barrier(0);  // keep this order (left alone the scheduler bunches the reads)
         }
-        // two P.V instructions cover the time the last score instruction needs to finish; then the first
-        // half of this item's softmax goes between the others
+        // two P.V instructions cover the time the last score instruction needs to finish; then this item's
+        // row max goes between the others
         static_assert(KS >= 4, "needs P.V instructions to hide the vector work behind");
 #pragma unroll
         for (int j = 0; j < 2; j++) {
@@ -458,35 +451,31 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         }
         if (MODE == kMaskPadding || __builtin_expect(kv0 + 32 * i + 31 > mask_from, 0)) mask_item(kv0 + 32 * i);
         float m_item = item_max();
-        const float mc_used = ((m_run == neg_inf()) ? 0.0f : m_run) * c;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 2; j < KS; j++) {
             mfma_pv(j);
             v_read_one(item_off, j);
-            prescale(16 * (j - 2) / (KS - 2), 16 * (j - 1) / (KS - 2), -mc_used);
             __builtin_amdgcn_sched_barrier(0);
         }
         // (pinned: the compiler would otherwise sink this work to its use in the softmax cluster)
-        asm volatile("" : "+v"(s), "+v"(m_item));
-        // the next tile (or, with none left, this tile again: served from cache into the idle stage,
-        // which keeps the cluster free of branches): requested with items 0 and 1, awaited with item 2
-        if (NLD >= 2) {
-            if (i < 2) {
-#pragma unroll
-                for (int n = 0; n < NLD / 2; n++) load_part(i * (NLD / 2) + n, kv_next, st ^ 1);
-            }
-        } else if (i == 0) {
-            load_part(0, kv_next, st ^ 1);
-        }
-        if (i == 2) __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wave's share has landed
+        asm volatile("" : "+v"(m_item));
+        if (i == 2) __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wave's share of the next tile has landed
         if (i == NITEMS - 1) __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): stage st may be refilled
         RT_PHASE(1);
         __builtin_amdgcn_s_setprio(0);
         cluster_barrier();
         RT_PHASE(2);
         // ---- S
-        update_max(m_item, mc_used);
+        // The next tile (or, with none left, this tile again: served from cache into the idle stage, which
+        // keeps the cluster free of branches) is requested here, where issue slots are free, with item 0, and
+        // awaited at the end of the matrix cluster of item 2.  Stage st^1 is idle by now: its last readers
+        // were the matrix clusters of the previous step's item 3, the later of which ended one barrier ago.
+        if (i == 0) {
+#pragma unroll
+            for (int n = 0; n < NLD; n++) load_part(n, kv_next, st ^ 1);
+        }
+        update_max(m_item);
         exp_item();
         // P is only used by the next matrix cluster, and the compiler would sink the exponentials and
         // conversions that make it down to that use, past the barrier and in between the matrix
