@@ -249,8 +249,21 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         load_to_lds(Vg, row_off + ld_v0, kdst + 2 * TILE_B);
     };
     auto load_tile = [&](int kv0, int st) {
+        if (kv0 + BC <= n_keys) {
+            // every row of the tile exists: one multiply for the tile, additions from there on
+            const uint32_t kdst = lds_base + (uint32_t)(st * TILE_B + wave * 1024);
+            uint32_t off = (uint32_t)(kv0 + ld_row0) * kv_pitch_b;
+            const uint32_t stride = (uint32_t)(NWAVES * RPI) * kv_pitch_b;
 #pragma unroll
-        for (int n = 0; n < NLD; n++) load_part(n, kv0, st);
+            for (int n = 0; n < NLD; n++) {
+                load_to_lds(Kg, off + ld_k0, kdst + (uint32_t)(NWAVES * n * 1024));
+                load_to_lds(Vg, off + ld_v0, kdst + (uint32_t)(NWAVES * n * 1024 + 2 * TILE_B));
+                off += stride;
+            }
+        } else {
+#pragma unroll
+            for (int n = 0; n < NLD; n++) load_part(n, kv0, st);
+        }
     };
     // Job of round i for this worker, or -1, as rank * n_bh + bh (rank 0 = the longest causal rows).
     // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  When the heads divide evenly,
@@ -467,14 +480,11 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         cluster_barrier();
         RT_PHASE(2);
         // ---- S
-        // The next tile (or, with none left, this tile again: served from cache into the idle stage, which
-        // keeps the cluster free of branches) is requested here, where issue slots are free, with item 0, and
+        // The next tile (or, with none left, this tile again: served from cache into the idle stage) is
+        // requested here, where issue slots are free, with item 0, and
         // awaited at the end of the matrix cluster of item 2.  Stage st^1 is idle by now: its last readers
         // were the matrix clusters of the previous step's item 3, the later of which ended one barrier ago.
-        if (i == 0) {
-#pragma unroll
-            for (int n = 0; n < NLD; n++) load_part(n, kv_next, st ^ 1);
-        }
+        if (i == 0) load_tile(kv_next, st ^ 1);
         update_max(m_item);
         exp_item();
         // P is only used by the next matrix cluster, and the compiler would sink the exponentials and
