@@ -249,21 +249,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         load_to_lds(Vg, row_off + ld_v0, kdst + 2 * TILE_B);
     };
     auto load_tile = [&](int kv0, int st) {
-        if (kv0 + BC <= n_keys) {
-            // every row of the tile exists: one multiply for the tile, additions from there on
-            const uint32_t kdst = lds_base + (uint32_t)(st * TILE_B + wave * 1024);
-            uint32_t off = (uint32_t)(kv0 + ld_row0) * kv_pitch_b;
-            const uint32_t stride = (uint32_t)(NWAVES * RPI) * kv_pitch_b;
 #pragma unroll
-            for (int n = 0; n < NLD; n++) {
-                load_to_lds(Kg, off + ld_k0, kdst + (uint32_t)(NWAVES * n * 1024));
-                load_to_lds(Vg, off + ld_v0, kdst + (uint32_t)(NWAVES * n * 1024 + 2 * TILE_B));
-                off += stride;
-            }
-        } else {
-#pragma unroll
-            for (int n = 0; n < NLD; n++) load_part(n, kv0, st);
-        }
+        for (int n = 0; n < NLD; n++) load_part(n, kv0, st);
     };
     // Job of round i for this worker, or -1, as rank * n_bh + bh (rank 0 = the longest causal rows).
     // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  When the heads divide evenly,
@@ -383,13 +370,9 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             s[i] = masked ? neg_inf() : s[i];
         }
     };
-    // The softmax of an item is split over the two clusters.  Its row max needs nothing but the finished
-    // scores and is taken in the second half of the matrix cluster, in the issue slots between the P.V
-    // instructions.  The softmax cluster then raises the running max when it pays (rarely: O and l are
-    // rescaled), and takes exp2(s*c - m*c), the row sums and the bf16 conversion.
-    auto item_max = [&]() { return max_with_other_half(max16(s)); };
     // raise the running max when it pays (wave-uniform branch)
-    auto update_max = [&](float m_item) {
+    auto update_max = [&]() {
+        float m_item = max_with_other_half(max16(s));
         if (__builtin_expect(__any(m_item > m_run + lazy_raw), 0)) {
             float m_new = vmax(m_run, m_item);
             float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
@@ -445,47 +428,36 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         lds_operands_ready();
         __builtin_amdgcn_sched_barrier(0);  // no matrix instruction may be moved ahead of that wait
         zero_s();
-        // the score instructions first, each followed by the read that refills its K operand
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
             mfma_qk(ks);
             if (i + 1 < NITEMS) k_read_one(std::integral_constant<int, (i + 1 < NITEMS ? item_off + 32 * ROWB : 0)>{}, 0, ks);
             else k_read_one(std::integral_constant<int, 0>{}, TILE_B, ks);  // item 0 of the next tile, other stage
-            __builtin_amdgcn_sched_barrier(0);  // keep this order (left alone the scheduler bunches the reads)
-        }
-        // two P.V instructions cover the time the last score instruction needs to finish; then this item's
-        // row max goes between the others
-        static_assert(KS >= 4, "needs P.V instructions to hide the vector work behind");
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            mfma_pv(j);
-            v_read_one(item_off, j);
+            mfma_pv(ks);
+            v_read_one(item_off, ks);
+            // keep this order: two matrix instructions, three reads, and so on (left alone the scheduler
+            // bunches the reads, and the matrix pipe runs dry while a wave issues ten of them in a row)
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (MODE == kMaskPadding || __builtin_expect(kv0 + 32 * i + 31 > mask_from, 0)) mask_item(kv0 + 32 * i);
-        float m_item = item_max();
-        __builtin_amdgcn_sched_barrier(0);
+        // the next tile (or, with none left, this tile again: served from cache into the idle stage,
+        // which keeps the cluster free of branches): requested with items 0 and 1, awaited with item 2
+        if (NLD >= 2) {
+            if (i < 2) {
 #pragma unroll
-        for (int j = 2; j < KS; j++) {
-            mfma_pv(j);
-            v_read_one(item_off, j);
-            __builtin_amdgcn_sched_barrier(0);
+                for (int n = 0; n < NLD / 2; n++) load_part(i * (NLD / 2) + n, kv_next, st ^ 1);
+            }
+        } else if (i == 0) {
+            load_part(0, kv_next, st ^ 1);
         }
-        // (pinned: the compiler would otherwise sink this work to its use in the softmax cluster)
-        asm volatile("" : "+v"(m_item));
-        if (i == 2) __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wave's share of the next tile has landed
+        if (i == 2) __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wave's share has landed
         if (i == NITEMS - 1) __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): stage st may be refilled
         RT_PHASE(1);
         __builtin_amdgcn_s_setprio(0);
         cluster_barrier();
         RT_PHASE(2);
         // ---- S
-        // The next tile (or, with none left, this tile again: served from cache into the idle stage) is
-        // requested here, where issue slots are free, with item 0, and
-        // awaited at the end of the matrix cluster of item 2.  Stage st^1 is idle by now: its last readers
-        // were the matrix clusters of the previous step's item 3, the later of which ended one barrier ago.
-        if (i == 0) load_tile(kv_next, st ^ 1);
-        update_max(m_item);
+        if (MODE == kMaskPadding || __builtin_expect(kv0 + 32 * i + 31 > mask_from, 0)) mask_item(kv0 + 32 * i);
+        update_max();
         exp_item();
         // P is only used by the next matrix cluster, and the compiler would sink the exponentials and
         // conversions that make it down to that use, past the barrier and in between the matrix
