@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-A step is one pass of the bf16 causal prefill kernel over BASELINE's workload
+A step is one pass of the bf16 causal prefill kernel over the headline workload
 B=4, H=32, N=4096, D=128 (inputs resident in HBM before the timed region); the same run also
 times the batched GQA decode workload (batch 64, 32 query / 8 kv heads, D=128, context lengths
 uniform in [512, 8192], Lmax 8192) and reports it under "decode".
@@ -20,6 +20,7 @@ import argparse
 import ctypes as C
 import json
 import os
+import subprocess
 import sys
 import time
 
@@ -33,7 +34,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the dominant kernels on the bench workloads, from the rocprofv3 --pmc runs
 # summarised under profiles/ (FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB, the factors a 256 MiB copy reads).
 # Counters cannot be read from inside this process; these are the committed measurements, not live values.
-TRAFFIC_PREFILL_BYTES = (284200 * 2.0 + 131100 * 1.0) * 1024
+TRAFFIC_PREFILL_BYTES = (260500 * 2.0 + 131100 * 1.0) * 1024
 TRAFFIC_DECODE_BYTES = (624200 * 2.0 + 5313 * 1.0) * 1024
 
 
@@ -93,6 +94,25 @@ def time_steps(hip, stream, launch, steps, warmup):
     return wall_ms, per
 
 
+def sustained_mfma():
+    """Rate and shader clock of a pure bf16 MFMA loop on changing N(0,1)-like operands, launched back to back for
+    about a second (a child process: rustorch_amd/lib/mfma_sustained, built with the library).  None when the
+    program is missing or fails; the bench line is complete without it."""
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "rustorch_amd", "lib", "mfma_sustained")
+    if not os.path.exists(exe):
+        return None
+    try:
+        r = subprocess.run([exe, "2", "12"], capture_output=True, text=True, timeout=60)
+        last = r.stdout.strip().splitlines()[-1].split()
+        if r.returncode != 0 or last[0] != "sustained":
+            return None
+        return {"tflops": float(last[1]), "shader_mhz": float(last[2]),
+                "how": "v_mfma_f32_32x32x16_bf16 only, 8 waves/CU, operands changing per instruction, median of "
+                       "launches 600-1199"}
+    except (OSError, subprocess.SubprocessError, IndexError, ValueError):
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -102,6 +122,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity sample")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None)
+    ap.add_argument("--no-ceiling", action="store_true",
+                    help="skip the run of rustorch_amd/lib/mfma_sustained (what a loop of nothing but bf16 MFMA "
+                         "sustains on this GPU, reported beside the data-sheet peak)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also issue one 256 MiB device-to-device copy (a dispatch of known traffic, to scale the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -236,6 +259,7 @@ def main():
                               dtype="bf16", data="synthetic", vs_baseline=None)))
         return
     achieved = prefill["tflops_kernel"]
+    sustained = None if args.no_ceiling else sustained_mfma()
     out = {
         "metric": "prefill attn TFLOP/s (% bf16 MFMA peak); decode attn HBM GB/s (% peak)",
         "value": prefill["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -249,6 +273,9 @@ def main():
                      "kernel_ms_mean": prefill["kernel_ms_mean"], "kernel_ms_median": prefill["kernel_ms_median"],
                      "kernel_ms_min": prefill["kernel_ms_min"]},
     }
+    if sustained is not None:
+        # context for `frac`: under load the power limit, not the 2.4 GHz of the data sheet, sets the clock
+        out["roofline"]["sustained_mfma"] = dict(sustained, frac_of_sustained=achieved / sustained["tflops"])
     if "cpu" in prefill:
         out["cpu_baseline"] = prefill["cpu"]
         out["parity_max_abs"] = prefill["parity_max_abs"]

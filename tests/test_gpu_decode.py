@@ -116,7 +116,7 @@ def test_decode_workspace_too_small_is_an_error():
 
 
 def test_config_decode_b64_h32_kv8_d128_lmax8192(oracle):
-    """BASELINE configs[3] at full size: lengths uniform in [512, 8192] from a seed, N(0,1) bf16
+    """The decode workload of the benchmark set at full size: lengths uniform in [512, 8192] from a seed, N(0,1) bf16
     caches in the contiguous (B, Hkv, Lmax, D) layout."""
     b, hq, hkv, d, max_seq = 64, 32, 8, 128, 8192
     lens = np.random.default_rng(4).integers(512, 8193, size=b).astype(np.int32)

@@ -111,7 +111,7 @@ def test_varlen_small(oracle):
 
 
 def test_config_padded_batch_b16_h16_n1024_d64(oracle):
-    """BASELINE configs[2]: lengths uniform in [128, 1024] from a seed, key padding + causal,
+    """The variable-length workload of the benchmark set: lengths uniform in [128, 1024] from a seed, key padding + causal,
     padded query rows exactly 0."""
     b, h, n, d = 16, 16, 1024, 64
     lens = np.random.default_rng(2026).integers(128, 1025, size=b).astype(np.int32)
@@ -125,7 +125,7 @@ def test_config_padded_batch_b16_h16_n1024_d64(oracle):
 
 
 def test_config_prefill_b4_h32_n4096_d128(oracle):
-    """BASELINE configs[1] at full size.  The oracle (which computes every tile, as the reference
+    """The headline prefill workload at full size.  The oracle (which computes every tile, as the reference
     does) checks a sample of (b,h) slabs in full; size-independent properties cover all slabs:
     causal row 0 == V[0] exactly, and a second run with V := const gives const."""
     b, h, n, d = 4, 32, 4096, 128
@@ -147,7 +147,7 @@ def test_config_prefill_b4_h32_n4096_d128(oracle):
 
 
 def test_config_long_context_b1_h32_n16384_d128(oracle):
-    """BASELINE configs[4]: Q scaled by 2.0 before rounding.  Checked against the oracle on the
+    """The large-logit workload of the benchmark set: Q scaled by 2.0 before rounding.  Checked against the oracle on the
     first 2048 rows of two heads (causal rows depend only on their prefix, so the truncated problem
     is the same computation) and on sampled late rows through the reference's single-row decode
     function (row i of causal attention == unmasked attention of q_i over keys [0, i])."""

@@ -179,7 +179,7 @@ def test_flash_matches_oracle_random_shapes(oracle):
 
 
 def test_config_f32_causal_b1_h8_n2048_d64(oracle):
-    """BASELINE configs[0]: the reference's own CPU-runnable case, N(0,1) inputs, causal."""
+    """Workload 0 of the benchmark set: the reference's own CPU-runnable case, N(0,1) inputs, causal."""
     bhnd = (1, 8, 2048, 64)
     q, k, v = (seeded_normal(bhnd, s) for s in (101, 102, 103))
     shape = ra.AttentionShape.new(*bhnd)
