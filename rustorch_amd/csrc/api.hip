@@ -90,9 +90,10 @@ int ensure_device(rt_err_detail* err, int device = -1) {
         e = hipSetDevice(dev);
         if (e != hipSuccess) return fail_hip(err, e, "hipSetDevice");
     }
-    // the decode kernel (one wave, ~18 KB LDS, <= 256 VGPRs) fits 8 times on a CU
+    // the decode kernel (one wave, ~18 KB LDS, <= 256 VGPRs) fits 8 times on a CU; one wave per SIMD already
+    // streams at the rate the memory system gives, and fewer waves leave fewer partials to merge
     g_num_cus = prop.multiProcessorCount;
-    g_decode_waves = prop.multiProcessorCount * 8;
+    g_decode_waves = prop.multiProcessorCount * 4;
     g_init_status = RT_OK;
     return RT_OK;
 }

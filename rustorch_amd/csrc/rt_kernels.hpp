@@ -84,7 +84,7 @@ struct DecodeSplitParams {
     float* ws;                // partial (o, m, l) per (b, head, chunk)
     int batch, heads, kv_heads, dim, max_seq;
     int n_part;   // partial slots per (sequence, head): decode_split_parts(max_seq)
-    int n_waves;  // one-wave workgroups launched: what the GPU holds at once
+    int n_waves;  // one-wave workgroups launched (all resident at once)
     float scale_log2e;
 };
 bool decode_split_supported(int heads, int kv_heads, int dim);
