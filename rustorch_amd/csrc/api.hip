@@ -151,6 +151,7 @@ int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n
     p.mask = mask_kind;
     p.ref_bc = (int)(s->bc == 0 ? 1 : (s->bc > 0x7fffffffull ? 0x7fffffff : s->bc));
     p.scale = 1.0f / sqrtf((float)s->dim);
+    p.n_cus = g_num_cus;
     if (bnhd) {
         p.lq = p.lo = rt::layout_bnhd((long long)s->heads, (long long)s->seq, p.dim);
         p.lkv = rt::layout_bnhd((long long)n_kv_heads, (long long)s->seq, p.dim);

@@ -160,12 +160,268 @@ __global__ __launch_bounds__(64) void flash_fwd_f32_kernel(FlashF32Params p) {
     }
 }
 
+
+// ---- head dims that are a multiple of 32, 16-byte aligned rows: the fast kernel ---------------------------
+//
+// One workgroup of four waves owns 32 query rows; wave w walks the key tiles t = w, w+4, ... (32 keys each) on its
+// own, with a private LDS tile and no workgroup barrier in the loop, and the four partial (O, m, l) states are
+// merged through LDS at the end with the online-softmax monoid (online_softmax.rs:105-131 extended with O).
+// Splitting the keys rather than the query rows over the waves shortens the longest chain of dependent steps
+// four times, which is what a small problem (8 heads x 2048 rows) is bound by.  The next tile travels from
+// global memory into registers (16-byte loads) while the current one is multiplied.
+//
+// The contraction index of the score product is walked in the order d = 8j + 4*half + i (i = 0..3) for both
+// operands, so that a lane fetches its four K values of a chunk with one 16-byte LDS read and Q stays in
+// registers for the whole job.
+template <int DT>
+__global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_kernel(FlashF32Params p) {
+    constexpr int DPAD = 32 * DT;       // == dim
+    constexpr int LDK = DPAD + 4;       // row stride of the K tile: 16-byte reads of 16 rows tile all banks
+    constexpr int CH = DPAD / 4;        // 16-byte chunks per row
+    constexpr int NLD = 32 * CH / 64;   // 16-byte loads per lane, per matrix, per tile
+    constexpr int KTILE = kRows * LDK, VTILE = kRows * DPAD;
+    constexpr int NW = 4;
+    __shared__ __attribute__((aligned(16))) float lds[NW * (KTILE + VTILE)];
+    __shared__ float red_m[NW][kRows], red_l[NW][kRows];
+    __shared__ float fin_inv[kRows];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, hh = lane >> 5;
+    const int N = p.seq;
+    const int h = blockIdx.y, b = blockIdx.z;
+    // longest causal rows first; when the whole grid is resident at once (p.zigzag), every other head runs the
+    // other way round, so that the workgroups that end up sharing a CU are a long one and a short one
+    int qtile = (int)gridDim.x - 1 - (int)blockIdx.x;
+    if (p.zigzag && ((h + b * (int)gridDim.y) * 2 >= (int)(gridDim.y * gridDim.z))) qtile = (int)blockIdx.x;
+    const int q0 = qtile * kRows;
+    const int kvh = h / p.group;
+    const float* __restrict__ Qg = p.q + (size_t)b * p.lq.batch_stride + (size_t)h * p.lq.head_stride;
+    const float* __restrict__ Kg = p.k + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+    const float* __restrict__ Vg = p.v + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+    float* __restrict__ Og = p.out + (size_t)b * p.lo.batch_stride + (size_t)h * p.lo.head_stride;
+    const size_t q_pitch = p.lq.row_pitch, kv_pitch = p.lkv.row_pitch, o_pitch = p.lo.row_pitch;
+    float* Kw = lds + wave * (KTILE + VTILE);
+    float* Vw = Kw + KTILE;
+
+    // leading-masked-tile rule of the reference's recurrence (cpu_forward.rs:364-384), as in the kernel above
+    bool poison = false;
+    if (p.mask == kMaskPadding) {
+        int lim = p.ref_bc < N ? p.ref_bc : N;
+        bool any = false;
+        for (int j = lane; j < lim; j += kWave) any |= (p.keep[j] != 0);
+        poison = !__any(any);
+    }
+
+    // Q as B operand, in registers: qreg[4j + i] = Q[q0 + col][8j + 4hh + i]
+    const int q_row = q0 + col;
+    float qreg[DPAD / 2];
+#pragma unroll
+    for (int j = 0; j < DPAD / 8; j++) {
+        f32x4_t z = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (q_row < N) z = *(const f32x4_t*)(Qg + (size_t)q_row * q_pitch + 8 * j + 4 * hh);
+#pragma unroll
+        for (int i = 0; i < 4; i++) qreg[4 * j + i] = z[i];
+    }
+
+    f32x16_t acc_o[DT];
+#pragma unroll
+    for (int t = 0; t < DT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc_o[t][i] = 0.0f;
+    float m_run = neg_inf();
+    float l_run = 0.0f;  // this lane's share of the row sum
+
+    int kv_end = N;
+    if (p.mask == kMaskCausal) kv_end = min(N, q0 + kRows);
+    const int n_tiles = (kv_end + kRows - 1) / kRows;
+
+    // lane's chunks of a tile: load n covers row (64n + lane) / CH, chunk (64n + lane) % CH.  When CH divides 64
+    // that is row n * (64/CH) + lane / CH, chunk lane % CH: one per-lane offset, everything else is uniform.
+    constexpr bool kEvenRows = (64 % CH == 0);
+    constexpr int RPL = kEvenRows ? 64 / CH : 0;  // rows per load instruction
+    const int ld_r = lane / CH, ld_c = lane % CH;
+    const uint32_t ld_off = (uint32_t)ld_r * (uint32_t)kv_pitch * 4u + (uint32_t)ld_c * 16u;  // bytes; a few rows: fits
+    f32x4_t kreg[NLD], vreg[NLD];
+    auto issue_loads = [&](int tile) {
+#pragma unroll
+        for (int n = 0; n < NLD; n++) {
+            f32x4_t zk = {0.0f, 0.0f, 0.0f, 0.0f}, zv = zk;
+            if constexpr (kEvenRows) {
+                const int row0 = tile * kRows + RPL * n;  // uniform
+                const size_t base = (size_t)row0 * kv_pitch * sizeof(float);
+                if (row0 + ld_r < N) {  // rows past the end are zeros (and masked below)
+                    zk = *(const f32x4_t*)((const char*)Kg + base + ld_off);
+                    zv = *(const f32x4_t*)((const char*)Vg + base + ld_off);
+                }
+            } else {
+                const int idx = 64 * n + lane, r = idx / CH, c = idx % CH;
+                const int kr = tile * kRows + r;
+                if (kr < N) {
+                    zk = *(const f32x4_t*)(Kg + (size_t)kr * kv_pitch + 4 * c);
+                    zv = *(const f32x4_t*)(Vg + (size_t)kr * kv_pitch + 4 * c);
+                }
+            }
+            kreg[n] = zk;
+            vreg[n] = zv;
+        }
+    };
+    if (wave < n_tiles) issue_loads(wave);
+
+    for (int tile = wave; tile < n_tiles; tile += NW) {
+        const int kv0 = tile * kRows;
+        // registers -> this wave's LDS tile (its reads of the previous tile are behind it: same wave, in order)
+#pragma unroll
+        for (int n = 0; n < NLD; n++) {
+            const int idx = 64 * n + lane, r = idx / CH, c = idx % CH;
+            *(f32x4_t*)(Kw + r * LDK + 4 * c) = kreg[n];
+            *(f32x4_t*)(Vw + r * DPAD + 4 * c) = vreg[n];
+        }
+        if (tile + NW < n_tiles) issue_loads(tile + NW);
+
+        // S^T = K . Q^T
+        f32x16_t s;
+#pragma unroll
+        for (int i = 0; i < 16; i++) s[i] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < DPAD / 8; j++) {
+            const f32x4_t a = *(const f32x4_t*)(Kw + col * LDK + 8 * j + 4 * hh);
+#pragma unroll
+            for (int i = 0; i < 4; i++) s = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], qreg[4 * j + i], s, 0, 0, 0);
+        }
+        // register i of the accumulator holds key row 8*(i/4) + 4*hh + (i%4), query row `col`
+        float m_tile = neg_inf();
+        const bool edge = (kv0 + kRows > N) || (p.mask == kMaskCausal && kv0 + kRows - 1 > q0) || (p.mask == kMaskPadding);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            float x = s[i] * p.scale;
+            if (edge) {
+                int kr = kv0 + 8 * (i >> 2) + 4 * hh + (i & 3);
+                bool masked = kr >= N;
+                if (p.mask == kMaskCausal) masked |= kr > q_row;
+                if (p.mask == kMaskPadding) masked |= (kr < N) && (p.keep[kr] == 0);
+                x = masked ? neg_inf() : x;
+            }
+            s[i] = x;
+            m_tile = (x > m_tile) ? x : m_tile;  // NaN never wins, as in the reference's `if x > m`
+        }
+        {
+            float o = other_half(m_tile);
+            m_tile = (o > m_tile) ? o : m_tile;
+        }
+        float m_new = (m_tile > m_run) ? m_tile : m_run;
+        float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+        float alpha = (m_run == neg_inf()) ? 0.0f : expf(m_run - m_use);
+        m_run = m_new;
+        // exp(x) as exp2(x * log2 e) on the hardware exp2: the difference is taken first (exact for the terms
+        // that matter), so the argument carries one rounding, about 1e-7 relative on each weight
+        float part[4];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            float e = __builtin_amdgcn_exp2f((s[i] - m_use) * kLog2e);
+            s[i] = e;
+            if (i < 4) part[i] = e;
+            else part[i & 3] += e;
+        }
+        l_run = l_run * alpha + ((part[0] + part[1]) + (part[2] + part[3]));
+        if (__any(alpha != 1.0f)) {  // wave-uniform: the reference also rescales only when alpha != 1 (cpu_forward.rs:372)
+#pragma unroll
+            for (int t = 0; t < DT; t++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc_o[t][i] *= alpha;
+        }
+        // O^T += V^T . P^T, two keys per instruction: the lower half of the wave feeds key 8j+r, the upper 8j+4+r
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int kr = 8 * (i >> 2) + 4 * hh + (i & 3);
+#pragma unroll
+            for (int t = 0; t < DT; t++) {
+                float a = Vw[kr * DPAD + t * 32 + col];
+                acc_o[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s[i], acc_o[t], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- merge the four partial states
+    {
+        float l = l_run + other_half(l_run);
+        if (hh == 0) {
+            red_m[wave][col] = m_run;
+            red_l[wave][col] = l;
+        }
+    }
+    __syncthreads();  // also: every wave is done with its tiles
+    float m_all = neg_inf();
+#pragma unroll
+    for (int w2 = 0; w2 < NW; w2++) {
+        float mw = red_m[w2][col];
+        m_all = (mw > m_all) ? mw : m_all;
+    }
+    float l_all = 0.0f, my_f = 0.0f;
+#pragma unroll
+    for (int w2 = 0; w2 < NW; w2++) {
+        float mw = red_m[w2][col];
+        float f = (mw == neg_inf()) ? 0.0f : expf(mw - m_all);  // an empty partial weighs nothing
+        l_all += red_l[w2][col] * f;
+        if (w2 == wave) my_f = f;
+    }
+    if (wave == 0 && hh == 0) {
+        bool good = (l_all > 0.0f) && (fabsf(l_all) != __uint_as_float(0x7f800000u)) && (l_all == l_all) && !poison;
+        fin_inv[col] = good ? 1.0f / l_all : quiet_nan();
+    }
+    // this wave's weighted O, as rows [col][d], into its own K tile
+#pragma unroll
+    for (int t = 0; t < DT; t++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            f32x4_t o = {acc_o[t][4 * g] * my_f, acc_o[t][4 * g + 1] * my_f, acc_o[t][4 * g + 2] * my_f, acc_o[t][4 * g + 3] * my_f};
+            *(f32x4_t*)(Kw + col * LDK + t * 32 + 8 * g + 4 * hh) = o;
+        }
+    __syncthreads();
+    // all 256 threads: sum the four partial tiles, normalise, store whole rows
+#pragma unroll
+    for (int n = 0; n < (kRows * CH + 255) / 256; n++) {
+        const int idx = 256 * n + tid;
+        if (idx < kRows * CH) {
+            const int r = idx / CH, c = idx % CH;
+            f32x4_t sum = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int w2 = 0; w2 < NW; w2++) sum += *(const f32x4_t*)(lds + w2 * (KTILE + VTILE) + r * LDK + 4 * c);
+            const float inv = fin_inv[r];
+            // a NaN in fin_inv marks a row without a valid sum: the whole row is NaN, whatever O holds
+            f32x4_t o;
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[i] = (inv == inv) ? sum[i] * inv : quiet_nan();
+            if (q0 + r < N) *(f32x4_t*)(Og + (size_t)(q0 + r) * o_pitch + 4 * c) = o;
+        }
+    }
+}
+
 }  // namespace
 
 hipError_t launch_flash_f32(hipStream_t stream, const FlashF32Params& p) {
     if (p.batch == 0 || p.heads == 0 || p.seq == 0) return hipSuccess;
     dim3 grid((p.seq + kRows - 1) / kRows, p.heads, p.batch), block(64);
     int dt = (p.dim + 31) / 32;
+    // the fast kernel reads whole 16-byte chunks: head dim a multiple of 32, rows and bases 16-byte aligned
+    auto aligned = [](const void* ptr, const TensorLayout& l) {
+        return ((uintptr_t)ptr % 16 == 0) && (l.batch_stride % 4 == 0) && (l.head_stride % 4 == 0) && (l.row_pitch % 4 == 0);
+    };
+    if (p.dim % 32 == 0 && aligned(p.q, p.lq) && aligned(p.k, p.lkv) && aligned(p.v, p.lkv) && aligned(p.out, p.lo)) {
+        dim3 block4(256);
+        FlashF32Params pz = p;
+        // 8 (dim <= 64) or 4 waves fit on a CU: is every workgroup resident from the start?
+        const long long resident = (long long)p.n_cus * (dt <= 2 ? 2 : 1);
+        pz.zigzag = (p.mask == kMaskCausal) && ((long long)grid.x * grid.y * grid.z <= resident) ? 1 : 0;
+        switch (dt) {
+            case 1: hipLaunchKernelGGL(flash_fwd_f32_splitk_kernel<1>, grid, block4, 0, stream, pz); break;
+            case 2: hipLaunchKernelGGL(flash_fwd_f32_splitk_kernel<2>, grid, block4, 0, stream, pz); break;
+            case 3: hipLaunchKernelGGL(flash_fwd_f32_splitk_kernel<3>, grid, block4, 0, stream, pz); break;
+            case 4: hipLaunchKernelGGL(flash_fwd_f32_splitk_kernel<4>, grid, block4, 0, stream, pz); break;
+            default: return hipErrorInvalidValue;
+        }
+        return hipGetLastError();
+    }
     switch (dt) {
         case 1: hipLaunchKernelGGL(flash_fwd_f32_kernel<1>, grid, block, 0, stream, p); break;
         case 2: hipLaunchKernelGGL(flash_fwd_f32_kernel<2>, grid, block, 0, stream, p); break;

@@ -36,6 +36,8 @@ struct FlashF32Params {
     int ref_bc;  // the reference's key-tile size, for the leading-masked-tile rule
     float scale;
     TensorLayout lq, lkv, lo;  // layouts of q, of k and v, of out
+    int n_cus;   // CUs of the device (0: unknown)
+    int zigzag;  // set by the launcher
 };
 // dim <= 128.  Returns hipErrorInvalidValue for an unsupported dim.
 hipError_t launch_flash_f32(hipStream_t stream, const FlashF32Params& p);
