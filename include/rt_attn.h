@@ -51,6 +51,8 @@ enum rt_status {
     RT_ERR_WRONG_INPUT_LEN = 6,         /* GQAError::WrongInputLen{which,expected,got} */
     RT_ERR_KV_OVERFLOW = 7,             /* KVCacheError::Overflow{requested=got,max=expected} */
     RT_ERR_KV_WRONG_INPUT_LEN = 8,      /* KVCacheError::WrongInputLen{expected,got_k=got,got_v=got2} */
+    RT_ERR_ROPE_WRONG_INPUT_LEN = 9,    /* RoPEError::WrongInputLen{expected,got} */
+    RT_ERR_ROPE_POSITION_OVERFLOW = 10, /* RoPEError::PositionOverflow{max_seq=expected,requested=got} */
     RT_ERR_NULL_POINTER = 20,
     RT_ERR_UNSUPPORTED = 21,            /* shape outside what the kernels cover; message says which */
     RT_ERR_WORKSPACE_TOO_SMALL = 22,    /* expected = bytes needed, got = bytes given */
@@ -160,6 +162,25 @@ int rt_flash_forward_varlen_bf16_dev(void *stream, const rt_attention_shape *sha
  * cache[kv_h*max_seq*head_dim + pos*head_dim + i] = in[kv_h*head_dim + i] for K and V. */
 int rt_kv_append_bf16(void *stream, void *k_cache, void *v_cache, const void *k_in, const void *v_in, int32_t pos,
                       int32_t n_kv, int32_t head_dim, int32_t max_seq, rt_err_detail *err);
+
+/* Steps 2a, 2b and 3 of LlamaModel::decode_step -- crates/rustorch-llm/src/model.rs:575-636 -- in one launch,
+ * for a batch of sequences on bf16 storage: per-head RMSNorm of q and k (rms_norm_per_head, model.rs:862-897;
+ * gamma f32[head_dim] shared by the heads, NULL = no norm), half-split RoPE (RoPE::apply_inplace_half_split,
+ * crates/rustorch-nn/src/rope.rs:162-205; cos/sin f32[table_rows, head_dim/2] as RoPE::new builds them,
+ * rope.rs:63-90) and the cache append (kv_append_bf16, llm_kernels.rs:353-372).  Replaces the
+ * rope_half_split_bf16 x2 + kv_append_bf16 launches of crates/rustorch-llm/src/cuda_backend.rs:486-540.
+ * q [batch,n_heads,head_dim] is rewritten in place; k_in/v_in [batch,n_kv,head_dim]; caches
+ * [batch,n_kv,max_seq,head_dim]; sequence b uses position positions[b] (device int32[batch]) or, with
+ * positions == NULL, `pos`.  f32 arithmetic in the reference's order, one rounding to bf16 at the end.
+ * Errors: `pos` >= table_rows -> RT_ERR_ROPE_POSITION_OVERFLOW (RoPEError::PositionOverflow{max_seq=expected,
+ * requested=got}); `pos` >= max_seq -> RT_ERR_KV_OVERFLOW; odd head_dim or head_dim > 512 -> RT_ERR_UNSUPPORTED
+ * (RoPE::new panics on an odd head_dim).  Positions on the device cannot be checked by the host: a sequence
+ * whose position is out of range is left untouched. */
+int rt_qk_norm_rope_kv_append_bf16(void *stream, void *q, const void *k_in, const void *v_in, void *k_cache,
+                                   void *v_cache, const int32_t *positions, int32_t pos, const float *q_gamma,
+                                   const float *k_gamma, float eps, const float *cos_table, const float *sin_table,
+                                   int32_t table_rows, int32_t batch, int32_t n_heads, int32_t n_kv, int32_t head_dim,
+                                   int32_t max_seq, rt_err_detail *err);
 
 /* LlmKernels::gqa_decode_online_bf16 -- llm_kernels.rs:396-457, :915-958.  q/out
  * [n_heads,head_dim] bf16, caches [n_kv,max_seq,head_dim] bf16 of which [..kv_len] is read;

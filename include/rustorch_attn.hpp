@@ -12,6 +12,7 @@
 //   rustorch_attn::mha_flash_forward_f32
 //                                   crates/rustorch-nn/src/attention.rs:452-495
 //   rustorch_attn::LlmKernels       crates/rustorch-cuda/src/llm_kernels.rs:874-958 (attention part)
+//   rustorch_attn::RoPE, RoPEError  crates/rustorch-nn/src/rope.rs:33-241 (tables and errors; the rotation runs on the device)
 //   rustorch_attn::HipStorage       the slot of Storage::Cuda, crates/rustorch-core/src/tensor/storage.rs:776-817
 //
 // Where Rust returns Result<(), E>, these functions throw E (a std::exception carrying the enum's fields).
@@ -20,6 +21,7 @@
 #define RUSTORCH_ATTN_HPP
 
 #include <array>
+#include <cmath>
 #include <cstddef>
 #include <cstdint>
 #include <stdexcept>
@@ -51,6 +53,21 @@ struct GQAError : std::runtime_error {
     size_t expected = 0, got = 0;  // HeadCountMismatch: expected = n_heads, got = n_kv_heads
     GQAError(Kind k, std::string w, size_t e, size_t g, const std::string& msg)
         : std::runtime_error(msg), kind(k), which(std::move(w)), expected(e), got(g) {}
+};
+
+// RoPEError (crates/rustorch-nn/src/rope.rs:208-241) and KVCacheError::Overflow (kv_cache.rs:229-256), the two
+// errors the decode preparation step can return.
+struct RoPEError : std::runtime_error {
+    enum class Kind { WrongInputLen, PositionOverflow };
+    Kind kind;
+    size_t expected = 0, got = 0;  // PositionOverflow: expected = max_seq, got = requested
+    RoPEError(Kind k, size_t e, size_t g, const std::string& msg) : std::runtime_error(msg), kind(k), expected(e), got(g) {}
+};
+struct KVCacheOverflow : std::runtime_error {
+    size_t requested = 0, max = 0;
+    KVCacheOverflow(size_t r, size_t m)
+        : std::runtime_error("kv_cache overflow: requested " + std::to_string(r) + " positions, max " + std::to_string(m)),
+          requested(r), max(m) {}
 };
 
 // Stands where the reference has CudaError: no device, a failed HIP call, a shape the kernels do not cover.
@@ -109,6 +126,19 @@ inline void check_gqa(int rc, const rt_err_detail& e) {
 }
 inline void check_device(int rc, const rt_err_detail& e) {
     if (rc != RT_OK) throw_device(rc, e);
+}
+inline void check_prepare(int rc, const rt_err_detail& e) {
+    switch (rc) {
+        case RT_OK: return;
+        case RT_ERR_ROPE_WRONG_INPUT_LEN:
+            throw RoPEError(RoPEError::Kind::WrongInputLen, e.expected, e.got,
+                            "rope: expected buffer of " + std::to_string(e.expected) + " f32, got " + std::to_string(e.got));
+        case RT_ERR_ROPE_POSITION_OVERFLOW:
+            throw RoPEError(RoPEError::Kind::PositionOverflow, e.expected, e.got,
+                            "rope: position " + std::to_string(e.got) + " exceeds max_seq " + std::to_string(e.expected));
+        case RT_ERR_KV_OVERFLOW: throw KVCacheOverflow(e.got, e.expected);
+        default: throw_device(rc, e);
+    }
 }
 }  // namespace detail
 
@@ -280,6 +310,43 @@ inline void flash_forward_varlen_bf16_dev(const AttentionShape& shape, const voi
         e);
 }
 
+// ---- RoPE tables (crates/rustorch-nn/src/rope.rs:33-90) ----------------------------------------------------
+//
+// RoPE::new: theta_k = 1 / base^(2k / head_dim), angle = p * theta_k, cos and sin per (position, k), all in f32.
+// The tables are uploaded on first use and read by LlmKernels::qk_norm_rope_kv_append_bf16.
+class RoPE {
+public:
+    RoPE(size_t head_dim, size_t max_seq, float base = 10000.0f) : head_dim_(head_dim), max_seq_(max_seq) {
+        if (head_dim % 2 != 0) throw std::invalid_argument("RoPE: head_dim must be even, got " + std::to_string(head_dim));
+        const size_t half = head_dim / 2;
+        cos_.resize(max_seq * half);
+        sin_.resize(max_seq * half);
+        for (size_t p = 0; p < max_seq; p++)
+            for (size_t k = 0; k < half; k++) {
+                const float inv_theta = 1.0f / std::pow(base, (float)(2 * k) / (float)head_dim);
+                const float angle = (float)p * inv_theta;
+                cos_[p * half + k] = std::cos(angle);
+                sin_[p * half + k] = std::sin(angle);
+            }
+    }
+    size_t head_dim() const { return head_dim_; }
+    size_t max_seq() const { return max_seq_; }
+    const std::vector<float>& cos_table() const { return cos_; }
+    const std::vector<float>& sin_table() const { return sin_; }
+    const void* device_cos() { upload(); return dcos_.ptr(); }
+    const void* device_sin() { upload(); return dsin_.ptr(); }
+
+private:
+    void upload() {
+        if (dcos_.ptr() || cos_.empty()) return;
+        dcos_ = HipStorage::from_host(cos_);
+        dsin_ = HipStorage::from_host(sin_);
+    }
+    size_t head_dim_, max_seq_;
+    std::vector<float> cos_, sin_;
+    HipStorage dcos_, dsin_;
+};
+
 // ---- LlmKernels: the attention launchers (llm_kernels.rs:874-958), raw device addresses and i32 dims ----------
 
 struct LlmKernels {
@@ -287,6 +354,27 @@ struct LlmKernels {
                                int32_t n_kv, int32_t head_dim, int32_t max_seq) {
         rt_err_detail e;
         detail::check_device(rt_kv_append_bf16(stream, k_cache, v_cache, k_in, v_in, pos, n_kv, head_dim, max_seq, &e), e);
+    }
+    // Steps 2a, 2b, 3 of LlamaModel::decode_step (crates/rustorch-llm/src/model.rs:575-636) in one launch: per-head
+    // q/k RMSNorm (device f32 gammas or nullptr), half-split RoPE, cache append.  `positions` is a device
+    // int32[batch] array, or nullptr to use `pos` for every sequence (then checked here, like the reference).
+    static void qk_norm_rope_kv_append_bf16(void* stream, void* q, const void* k_in, const void* v_in, void* k_cache,
+                                            void* v_cache, const int32_t* positions, int32_t pos, const float* q_gamma,
+                                            const float* k_gamma, float eps, RoPE& rope, int32_t batch, int32_t n_heads,
+                                            int32_t n_kv, int32_t head_dim, int32_t max_seq) {
+        if (!positions) {  // the reference's checks, before anything touches the device (rope.rs:179-184, kv_cache.rs:88-95)
+            if (pos < 0 || (size_t)pos >= rope.max_seq())
+                throw RoPEError(RoPEError::Kind::PositionOverflow, rope.max_seq(), (size_t)((int64_t)pos + 1),
+                                "rope: position " + std::to_string((int64_t)pos + 1) + " exceeds max_seq " +
+                                    std::to_string(rope.max_seq()));
+            if (pos >= max_seq) throw KVCacheOverflow((size_t)((int64_t)pos + 1), (size_t)max_seq);
+        }
+        rt_err_detail e;
+        detail::check_prepare(
+            rt_qk_norm_rope_kv_append_bf16(stream, q, k_in, v_in, k_cache, v_cache, positions, pos, q_gamma, k_gamma, eps,
+                                           (const float*)rope.device_cos(), (const float*)rope.device_sin(),
+                                           (int32_t)rope.max_seq(), batch, n_heads, n_kv, head_dim, max_seq, &e),
+            e);
     }
     static void gqa_decode_online_bf16(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out,
                                        int32_t n_heads, int32_t n_kv, int32_t kv_len, int32_t head_dim, int32_t max_seq) {

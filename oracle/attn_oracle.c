@@ -19,6 +19,12 @@
  *   ro_kv_trim                crates/rustorch-llm/src/model.rs:638-650
  *   ro_gqa_decode_online_bf16 crates/rustorch-cuda/src/llm_kernels.rs:396-457
  *   ro_kv_append_bf16         crates/rustorch-cuda/src/llm_kernels.rs:353-372
+ *   ro_rope_tables            crates/rustorch-nn/src/rope.rs:63-90 (RoPE::new)
+ *   ro_rope_half_split        crates/rustorch-nn/src/rope.rs:162-205 (apply_inplace_half_split)
+ *   ro_rope_interleaved       crates/rustorch-nn/src/rope.rs:96-142 (apply_inplace)
+ *   ro_rms_norm_per_head      crates/rustorch-llm/src/model.rs:862-897
+ *   ro_decode_prepare_bf16    crates/rustorch-llm/src/model.rs:575-636 (steps 2a, 2b, 3 of decode_step:
+ *                             per-head q/k RMSNorm, half-split RoPE, cache append) on bf16 storage
  *   ro_f32_to_bf16            half 2.7.1 bf16::from_f32 (round to nearest even),
  *                             the rule crates/rustorch-amp/src/bf16_kernels.rs:266-267 uses
  *
@@ -55,6 +61,8 @@ enum {
     RO_ERR_WRONG_INPUT_LEN = 6,
     RO_ERR_KV_OVERFLOW = 7,
     RO_ERR_KV_WRONG_INPUT_LEN = 8,
+    RO_ERR_ROPE_WRONG_INPUT_LEN = 9,
+    RO_ERR_ROPE_POSITION_OVERFLOW = 10,
 };
 
 enum { RO_MASK_NONE = 0, RO_MASK_CAUSAL = 1, RO_MASK_PADDING = 2 };
@@ -619,4 +627,143 @@ RO_EXPORT int ro_max_threads(void) {
 #else
     return 1;
 #endif
+}
+
+
+/* ---- RoPE and per-head RMSNorm: the steps between the QKV projection and decode attention ------------- */
+
+/* RoPE::new (rope.rs:63-90): theta_k = 1 / base^(2k / head_dim), angle = p * theta_k, all in f32. */
+RO_EXPORT void ro_rope_tables(int head_dim, int max_seq, float base, float *cos_t, float *sin_t) {
+    const int half = head_dim / 2;
+    for (int p = 0; p < max_seq; p++)
+        for (int k = 0; k < half; k++) {
+            float inv_theta = 1.0f / powf(base, (float)(2 * k) / (float)head_dim);
+            float angle = (float)p * inv_theta;
+            cos_t[(size_t)p * half + k] = cosf(angle);
+            sin_t[(size_t)p * half + k] = sinf(angle);
+        }
+}
+
+static int rope_check(size_t x_len, size_t batch, size_t n_heads, size_t seq, size_t d, size_t position_offset,
+                      size_t table_rows, ro_err *err) {
+    size_t expected = batch * n_heads * seq * d;
+    if (x_len != expected) { /* rope.rs:173-178 */
+        set_err(err, -1, expected, x_len);
+        return RO_ERR_ROPE_WRONG_INPUT_LEN;
+    }
+    if (position_offset + seq > table_rows) { /* rope.rs:179-184: expected = max_seq, got = requested */
+        set_err(err, -1, table_rows, position_offset + seq);
+        return RO_ERR_ROPE_POSITION_OVERFLOW;
+    }
+    return RO_OK;
+}
+
+/* apply_inplace_half_split (rope.rs:162-205): dim k pairs with dim k + D/2. */
+RO_EXPORT int ro_rope_half_split(float *x, size_t x_len, size_t batch, size_t n_heads, size_t seq, size_t head_dim,
+                                 size_t position_offset, const float *cos_t, const float *sin_t, size_t table_rows,
+                                 ro_err *err) {
+    int rc = rope_check(x_len, batch, n_heads, seq, head_dim, position_offset, table_rows, err);
+    if (rc != RO_OK) return rc;
+    const size_t d = head_dim, half = d / 2;
+    for (size_t b = 0; b < batch; b++)
+        for (size_t h = 0; h < n_heads; h++)
+            for (size_t s = 0; s < seq; s++) {
+                size_t p = position_offset + s;
+                size_t row_off = b * n_heads * seq * d + h * seq * d + s * d;
+                size_t table_off = p * half;
+                for (size_t k = 0; k < half; k++) {
+                    float c = cos_t[table_off + k], si = sin_t[table_off + k];
+                    float x0 = x[row_off + k], x1 = x[row_off + k + half];
+                    x[row_off + k] = x0 * c - x1 * si;
+                    x[row_off + k + half] = x1 * c + x0 * si;
+                }
+            }
+    return RO_OK;
+}
+
+/* apply_inplace (rope.rs:96-142): pairs (2k, 2k+1). */
+RO_EXPORT int ro_rope_interleaved(float *x, size_t x_len, size_t batch, size_t n_heads, size_t seq, size_t head_dim,
+                                  size_t position_offset, const float *cos_t, const float *sin_t, size_t table_rows,
+                                  ro_err *err) {
+    int rc = rope_check(x_len, batch, n_heads, seq, head_dim, position_offset, table_rows, err);
+    if (rc != RO_OK) return rc;
+    const size_t d = head_dim, half = d / 2;
+    for (size_t b = 0; b < batch; b++)
+        for (size_t h = 0; h < n_heads; h++)
+            for (size_t s = 0; s < seq; s++) {
+                size_t p = position_offset + s;
+                size_t row_off = b * n_heads * seq * d + h * seq * d + s * d;
+                size_t table_off = p * half;
+                for (size_t k = 0; k < half; k++) {
+                    float c = cos_t[table_off + k], si = sin_t[table_off + k];
+                    float x0 = x[row_off + 2 * k], x1 = x[row_off + 2 * k + 1];
+                    x[row_off + 2 * k] = x0 * c - x1 * si;
+                    x[row_off + 2 * k + 1] = x0 * si + x1 * c;
+                }
+            }
+    return RO_OK;
+}
+
+/* rms_norm_inplace (model.rs:862-885, default convention) on one head. */
+static void rms_norm_head(float *x, const float *gamma, size_t d, float eps) {
+    float inv_d = 1.0f / (float)d;
+    float sq = 0.0f;
+    for (size_t i = 0; i < d; i++) sq += x[i] * x[i];
+    float inv_rms = 1.0f / sqrtf(sq * inv_d + eps);
+    for (size_t i = 0; i < d; i++) x[i] = x[i] * inv_rms * gamma[i];
+}
+
+/* rms_norm_per_head (model.rs:890-897): gamma [head_dim] shared by the heads. */
+RO_EXPORT void ro_rms_norm_per_head(float *x, const float *gamma, size_t n_heads, size_t head_dim, float eps) {
+    for (size_t h = 0; h < n_heads; h++) rms_norm_head(x + h * head_dim, gamma, head_dim, eps);
+}
+
+/* Steps 2a, 2b and 3 of decode_step (model.rs:575-636) for a batch of sequences on bf16 storage: every value is
+ * widened to f32, normalised per head (when a gamma is given), rotated (half-split) at the sequence's position and
+ * rounded to bf16 once; q is rewritten in place, k and v go to row positions[b] of the caches
+ * [batch, n_kv, max_seq, head_dim] (the index rule of kv_append_bf16, llm_kernels.rs:353-372, per sequence).
+ * Positions must satisfy 0 <= p < min(max_seq, table_rows); returns the overflow error otherwise, having written
+ * nothing. */
+RO_EXPORT int ro_decode_prepare_bf16(uint16_t *q, const uint16_t *k_in, const uint16_t *v_in, uint16_t *k_cache,
+                                     uint16_t *v_cache, const int32_t *positions, const float *q_gamma,
+                                     const float *k_gamma, float eps, const float *cos_t, const float *sin_t, int batch,
+                                     int n_heads, int n_kv, int head_dim, int max_seq, int table_rows, ro_err *err) {
+    const size_t d = (size_t)head_dim;
+    for (int b = 0; b < batch; b++) {
+        int p = positions[b];
+        if (p < 0 || p >= table_rows) {
+            set_err(err, -1, (uint64_t)table_rows, (uint64_t)((int64_t)p + 1));
+            return RO_ERR_ROPE_POSITION_OVERFLOW;
+        }
+        if (p >= max_seq) { /* kv_cache.rs:88-95 */
+            set_err(err, -1, (uint64_t)max_seq, (uint64_t)((int64_t)p + 1));
+            return RO_ERR_KV_OVERFLOW;
+        }
+    }
+    float *row = (float *)malloc(d * sizeof(float));
+    if (!row) return -1;
+    ro_err e2;
+    for (int b = 0; b < batch; b++) {
+        const size_t p = (size_t)positions[b];
+        for (int h = 0; h < n_heads + n_kv; h++) {
+            const int is_q = h < n_heads;
+            uint16_t *src = is_q ? q + ((size_t)b * n_heads + h) * d : (uint16_t *)k_in + ((size_t)b * n_kv + (h - n_heads)) * d;
+            const float *gamma = is_q ? q_gamma : k_gamma;
+            for (size_t i = 0; i < d; i++) row[i] = ro_bf16_to_f32(src[i]);
+            if (gamma) rms_norm_head(row, gamma, d, eps);
+            ro_rope_half_split(row, d, 1, 1, 1, d, p, cos_t, sin_t, (size_t)table_rows, &e2);
+            if (is_q) {
+                for (size_t i = 0; i < d; i++) src[i] = ro_f32_to_bf16(row[i]);
+            } else {
+                const size_t off = (((size_t)b * n_kv + (h - n_heads)) * (size_t)max_seq + p) * d;
+                const uint16_t *vs = v_in + ((size_t)b * n_kv + (h - n_heads)) * d;
+                for (size_t i = 0; i < d; i++) {
+                    k_cache[off + i] = ro_f32_to_bf16(row[i]);
+                    v_cache[off + i] = vs[i];
+                }
+            }
+        }
+    }
+    free(row);
+    return RO_OK;
 }

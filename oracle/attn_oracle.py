@@ -32,6 +32,8 @@ ERR_HEAD_COUNT_MISMATCH = 5
 ERR_WRONG_INPUT_LEN = 6
 ERR_KV_OVERFLOW = 7
 ERR_KV_WRONG_INPUT_LEN = 8
+ERR_ROPE_WRONG_INPUT_LEN = 9
+ERR_ROPE_POSITION_OVERFLOW = 10
 
 WHICH = {0: "q", 1: "k", 2: "v", 3: "out", 4: "flash_forward", -1: ""}
 
@@ -111,6 +113,15 @@ def lib():
         L.ro_osm_full.argtypes = [fp, sz, C.POINTER(_Osm)]
         L.ro_osm_full.restype = None
         L.ro_max_threads.restype = C.c_int
+        L.ro_rope_tables.argtypes = [C.c_int, C.c_int, C.c_float, fp, fp]
+        L.ro_rope_tables.restype = None
+        rope_args = [fp, sz, sz, sz, sz, sz, sz, fp, fp, sz, C.POINTER(_Err)]
+        L.ro_rope_half_split.argtypes = rope_args
+        L.ro_rope_interleaved.argtypes = rope_args
+        L.ro_rms_norm_per_head.argtypes = [fp, fp, sz, sz, C.c_float]
+        L.ro_rms_norm_per_head.restype = None
+        L.ro_decode_prepare_bf16.argtypes = [u16p, u16p, u16p, u16p, u16p, i32p, fp, fp, C.c_float, fp, fp] + \
+            [C.c_int] * 6 + [C.POINTER(_Err)]
         _lib = L
     return _lib
 
@@ -349,6 +360,73 @@ def online_softmax_full(xs) -> OnlineSoftmaxState:
     r = OnlineSoftmaxState()
     lib().ro_osm_full(xp, xs.size, C.byref(r._s))
     return r
+
+
+class RoPE:
+    """RoPE::new and its two apply functions (crates/rustorch-nn/src/rope.rs:63-205) on float32 arrays."""
+
+    def __init__(self, head_dim: int, max_seq: int, base: float = 10000.0):
+        if head_dim % 2 != 0:
+            raise ValueError(f"RoPE: head_dim must be even, got {head_dim}")  # rope.rs:64-68 panics
+        self.head_dim, self.max_seq = head_dim, max_seq
+        half = head_dim // 2
+        self.cos = np.zeros(max_seq * half, dtype=np.float32)
+        self.sin = np.zeros(max_seq * half, dtype=np.float32)
+        lib().ro_rope_tables(head_dim, max_seq, base, self.cos.ctypes.data_as(C.POINTER(C.c_float)),
+                             self.sin.ctypes.data_as(C.POINTER(C.c_float)))
+
+    def _apply(self, fn, x, batch, n_heads, seq, position_offset):
+        x = np.ascontiguousarray(np.ravel(x), dtype=np.float32).copy()
+        err = _Err()
+        fp = C.POINTER(C.c_float)
+        rc = fn(x.ctypes.data_as(fp), x.size, batch, n_heads, seq, self.head_dim, position_offset,
+                self.cos.ctypes.data_as(fp), self.sin.ctypes.data_as(fp), self.max_seq, C.byref(err))
+        _raise(rc, err)
+        return x
+
+    def apply_half_split(self, x, batch, n_heads, seq, position_offset):
+        return self._apply(lib().ro_rope_half_split, x, batch, n_heads, seq, position_offset)
+
+    def apply_interleaved(self, x, batch, n_heads, seq, position_offset):
+        return self._apply(lib().ro_rope_interleaved, x, batch, n_heads, seq, position_offset)
+
+
+def rms_norm_per_head(x, gamma, n_heads, head_dim, eps):
+    """model.rs:862-897; returns a new float32 array."""
+    x, _ = _f32(x)
+    x = x.copy()
+    g, gp = _f32(gamma)
+    assert x.size == n_heads * head_dim and g.size == head_dim
+    lib().ro_rms_norm_per_head(x.ctypes.data_as(C.POINTER(C.c_float)), gp, n_heads, head_dim, eps)
+    return x
+
+
+def decode_prepare_bf16(q, k_in, v_in, k_cache, v_cache, positions, q_gamma, k_gamma, eps, rope, batch, n_heads, n_kv,
+                        head_dim, max_seq):
+    """Steps 2a, 2b, 3 of decode_step (model.rs:575-636) on bf16 bit patterns: returns the new q; the caches
+    (uint16 arrays) are updated in place."""
+    assert k_cache.dtype == np.uint16 and v_cache.dtype == np.uint16
+    q, qp = _u16(q)
+    q = q.copy()
+    qp = q.ctypes.data_as(C.POINTER(C.c_uint16))
+    ki, kip = _u16(k_in)
+    vi, vip = _u16(v_in)
+    pos = np.ascontiguousarray(positions, dtype=np.int32)
+    fp = C.POINTER(C.c_float)
+    qg = gp_q = None
+    if q_gamma is not None:
+        qg, gp_q = _f32(q_gamma)
+    kg = gp_k = None
+    if k_gamma is not None:
+        kg, gp_k = _f32(k_gamma)
+    err = _Err()
+    rc = lib().ro_decode_prepare_bf16(qp, kip, vip, k_cache.ctypes.data_as(C.POINTER(C.c_uint16)),
+                                      v_cache.ctypes.data_as(C.POINTER(C.c_uint16)),
+                                      pos.ctypes.data_as(C.POINTER(C.c_int32)), gp_q, gp_k, eps,
+                                      rope.cos.ctypes.data_as(fp), rope.sin.ctypes.data_as(fp), batch, n_heads, n_kv,
+                                      head_dim, max_seq, rope.max_seq, C.byref(err))
+    _raise(rc, err)
+    return q
 
 
 def max_threads() -> int:

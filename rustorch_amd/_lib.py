@@ -17,7 +17,7 @@ SYMBOLS = (
     "rt_flash_forward_f32", "rt_flash_forward_masked_f32", "rt_gqa_forward_f32",
     "rt_flash_forward_f32_dev", "rt_flash_forward_bf16_dev", "rt_flash_forward_varlen_bf16_dev",
     "rt_mha_flash_forward_f32", "rt_flash_forward_bnhd_f32_dev", "rt_flash_forward_bnhd_bf16_dev",
-    "rt_kv_append_bf16", "rt_gqa_decode_online_bf16", "rt_gqa_decode_batched_bf16",
+    "rt_kv_append_bf16", "rt_qk_norm_rope_kv_append_bf16", "rt_gqa_decode_online_bf16", "rt_gqa_decode_batched_bf16",
     "rt_gqa_decode_workspace_bytes",
     "rt_buf_alloc", "rt_buf_free", "rt_memcpy_h2d", "rt_memcpy_d2h", "rt_stream_synchronize",
 )
@@ -31,6 +31,8 @@ RT_ERR_HEAD_COUNT_MISMATCH = 5
 RT_ERR_WRONG_INPUT_LEN = 6
 RT_ERR_KV_OVERFLOW = 7
 RT_ERR_KV_WRONG_INPUT_LEN = 8
+RT_ERR_ROPE_WRONG_INPUT_LEN = 9
+RT_ERR_ROPE_POSITION_OVERFLOW = 10
 RT_ERR_NULL_POINTER = 20
 RT_ERR_UNSUPPORTED = 21
 RT_ERR_WORKSPACE_TOO_SMALL = 22
@@ -84,6 +86,8 @@ def lib():
     L.rt_flash_forward_bnhd_f32_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_flash_forward_bnhd_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_kv_append_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, errp]
+    L.rt_qk_norm_rope_kv_append_bf16.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, vp, vp, C.c_float, vp, vp, i32, i32,
+                                                 i32, i32, i32, i32, errp]
     L.rt_gqa_decode_online_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, errp]
     L.rt_gqa_decode_batched_bf16.argtypes = [vp, vp, vp, vp, vp, i32p, i32, i32, i32, i32, i32, vp, sz, errp]
     L.rt_gqa_decode_workspace_bytes.argtypes = [i32, i32, i32, i32, i32]

@@ -185,6 +185,8 @@ RT_API const char* rt_status_name(int status) {
         case RT_ERR_WRONG_INPUT_LEN: return "WrongInputLen";
         case RT_ERR_KV_OVERFLOW: return "Overflow";
         case RT_ERR_KV_WRONG_INPUT_LEN: return "KvWrongInputLen";
+        case RT_ERR_ROPE_WRONG_INPUT_LEN: return "RopeWrongInputLen";
+        case RT_ERR_ROPE_POSITION_OVERFLOW: return "PositionOverflow";
         case RT_ERR_NULL_POINTER: return "NullPointer";
         case RT_ERR_UNSUPPORTED: return "Unsupported";
         case RT_ERR_WORKSPACE_TOO_SMALL: return "WorkspaceTooSmall";
@@ -477,6 +479,53 @@ RT_API int rt_kv_append_bf16(void* stream, void* k_cache, void* v_cache, const v
     HIP_TRY(rt::launch_kv_append_bf16((hipStream_t)stream, (uint16_t*)k_cache, (uint16_t*)v_cache,
                                       (const uint16_t*)k_in, (const uint16_t*)v_in, pos, n_kv, head_dim, max_seq),
             "kv_append_bf16 launch");
+    return RT_OK;
+}
+
+RT_API int rt_qk_norm_rope_kv_append_bf16(void* stream, void* q, const void* k_in, const void* v_in, void* k_cache,
+                                          void* v_cache, const int32_t* positions, int32_t pos, const float* q_gamma,
+                                          const float* k_gamma, float eps, const float* cos_table,
+                                          const float* sin_table, int32_t table_rows, int32_t batch, int32_t n_heads,
+                                          int32_t n_kv, int32_t head_dim, int32_t max_seq, rt_err_detail* err) {
+    clear_err(err);
+    if (batch < 0 || n_heads < 0 || n_kv < 0 || head_dim < 0 || max_seq < 0 || table_rows < 0)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "negative dimension");
+    if ((head_dim & 1) || head_dim > 512)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 512, (uint64_t)head_dim, "head_dim must be even and <= 512");
+    if (batch > 65535 || n_heads + n_kv > 65535) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    if (!positions) {
+        // the checks of RoPE::apply_inplace_half_split (rope.rs:179-184), then of KVLayerCache::append (kv_cache.rs:88-95)
+        if (pos < 0 || pos >= table_rows)
+            return fail(err, RT_ERR_ROPE_POSITION_OVERFLOW, -1, (uint64_t)table_rows, (uint64_t)((int64_t)pos + 1),
+                        "position outside the RoPE tables");
+        if (pos >= max_seq)
+            return fail(err, RT_ERR_KV_OVERFLOW, -1, (uint64_t)max_seq, (uint64_t)((int64_t)pos + 1), "position outside the cache");
+    }
+    if (batch == 0 || n_heads + n_kv == 0 || head_dim == 0) return RT_OK;
+    if ((n_heads > 0 && !q) || (n_kv > 0 && (!k_in || !v_in || !k_cache || !v_cache)) || !cos_table || !sin_table)
+        return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    int rc = ensure_device(err);
+    if (rc) return rc;
+    rt::DecodePrepareParams p;
+    p.q = (uint16_t*)q;
+    p.k_in = (const uint16_t*)k_in;
+    p.v_in = (const uint16_t*)v_in;
+    p.k_cache = (uint16_t*)k_cache;
+    p.v_cache = (uint16_t*)v_cache;
+    p.positions = positions;
+    p.q_gamma = q_gamma;
+    p.k_gamma = k_gamma;
+    p.cos_table = cos_table;
+    p.sin_table = sin_table;
+    p.eps = eps;
+    p.pos = pos;
+    p.batch = batch;
+    p.n_heads = n_heads;
+    p.n_kv = n_kv;
+    p.head_dim = head_dim;
+    p.max_seq = max_seq;
+    p.table_rows = table_rows;
+    HIP_TRY(rt::launch_decode_prepare((hipStream_t)stream, p), "decode_prepare launch");
     return RT_OK;
 }
 

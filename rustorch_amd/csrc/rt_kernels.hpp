@@ -94,6 +94,25 @@ int decode_split_parts(int max_seq);
 size_t decode_split_workspace_bytes(int batch, int heads, int dim, int max_seq);
 hipError_t launch_decode_split(hipStream_t stream, const DecodeSplitParams& p);
 
+// Per-head q/k RMSNorm, half-split RoPE and the cache append of one decode step (prepare.hip).
+struct DecodePrepareParams {
+    uint16_t* q;              // [batch, n_heads, head_dim], rewritten in place
+    const uint16_t* k_in;     // [batch, n_kv, head_dim]
+    const uint16_t* v_in;
+    uint16_t* k_cache;        // [batch, n_kv, max_seq, head_dim]
+    uint16_t* v_cache;
+    const int32_t* positions; // device int32[batch], or null: `pos` for every sequence
+    const float* q_gamma;     // f32[head_dim] or null (no norm)
+    const float* k_gamma;
+    const float* cos_table;   // f32[table_rows, head_dim / 2]
+    const float* sin_table;
+    float eps;
+    int pos;
+    int batch, n_heads, n_kv, head_dim, max_seq, table_rows;
+};
+// head_dim even and <= 512
+hipError_t launch_decode_prepare(hipStream_t stream, const DecodePrepareParams& p);
+
 hipError_t launch_kv_append_bf16(hipStream_t stream, uint16_t* k_cache, uint16_t* v_cache, const uint16_t* k_in,
                                  const uint16_t* v_in, int pos, int n_kv, int head_dim, int max_seq);
 

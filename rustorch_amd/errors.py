@@ -2,6 +2,7 @@
 
 AttentionError / MaskError: crates/rustorch-attention/src/cpu_forward.rs:93-114, mask.rs:70-78.
 GQAError: crates/rustorch-nn/src/gqa.rs:37-55.  KVCacheError: crates/rustorch-nn/src/kv_cache.rs:229-256.
+RoPEError: crates/rustorch-nn/src/rope.rs:208-241.
 DeviceError stands where the reference has CudaError (NoDeviceFound / Driver / Unsupported).
 """
 from __future__ import annotations
@@ -94,6 +95,26 @@ class LayerOutOfRange(KVCacheError):
         return f"kv_cache layer {self.layer} out of range (have {self.num_layers})"
 
 
+class RoPEError(Exception):
+    pass
+
+
+class RopeWrongInputLen(RoPEError):
+    def __init__(self, expected, got):
+        self.expected, self.got = expected, got
+
+    def __str__(self):
+        return f"rope: expected buffer of {self.expected} f32, got {self.got}"
+
+
+class PositionOverflow(RoPEError):
+    def __init__(self, max_seq, requested):
+        self.max_seq, self.requested = max_seq, requested
+
+    def __str__(self):
+        return f"rope: position {self.requested} exceeds max_seq {self.max_seq}"
+
+
 class DeviceError(Exception):
     """NoDeviceFound / Driver / Unsupported / workspace and pointer errors of the HIP library."""
 
@@ -125,4 +146,8 @@ def raise_for(status: int, err: "L.RtErr"):
         raise Overflow(err.got, err.expected)
     if status == L.RT_ERR_KV_WRONG_INPUT_LEN:
         raise KVWrongInputLen(err.expected, err.got, err.got2)
+    if status == L.RT_ERR_ROPE_WRONG_INPUT_LEN:
+        raise RopeWrongInputLen(err.expected, err.got)
+    if status == L.RT_ERR_ROPE_POSITION_OVERFLOW:
+        raise PositionOverflow(err.expected, err.got)
     raise DeviceError(status, err.message.decode(errors="replace"), err.hip_error, err.expected, err.got)

@@ -132,6 +132,27 @@ static void test_errors() {
         CHECK(Mask::causal().is_masked(1, 2) && !Mask::causal().is_masked(2, 2));
         CHECK(Mask::padding({true, false}).is_masked(0, 1) && !Mask::padding({true, false}).is_masked(0, 0));
     }
+    {   // RoPE::new: position 0 is cos 1 / sin 0, theta_0 = 1, odd head_dim refused (rope.rs:63-90)
+        RoPE rope(4, 8);
+        CHECK(rope.cos_table().size() == 16 && rope.cos_table()[0] == 1.0f && rope.sin_table()[1] == 0.0f);
+        CHECK(std::fabs(rope.cos_table()[2 * 3] - std::cos(3.0f)) < 1e-6f);
+        bool threw = false;
+        try { RoPE bad(5, 4); } catch (const std::invalid_argument&) { threw = true; }
+        CHECK(threw);
+    }
+    {   // a host position is checked like the reference: the RoPE tables first, then the cache (no device needed)
+        RoPE rope(8, 16);
+        uint16_t dummy[8] = {0};
+        bool ok = false;
+        try {
+            LlmKernels::qk_norm_rope_kv_append_bf16(nullptr, dummy, dummy, dummy, dummy, dummy, nullptr, 16, nullptr, nullptr,
+                                                    1e-6f, rope, 1, 1, 1, 8, 32);
+        } catch (const RoPEError& e) {
+            ok = e.kind == RoPEError::Kind::PositionOverflow && e.expected == 16 && e.got == 17;
+        } catch (const DeviceError&) {
+        }
+        CHECK(ok);
+    }
 }
 
 static float max_abs_diff(const std::vector<float>& a, const std::vector<float>& b, bool* nan_same) {
@@ -196,6 +217,31 @@ static void test_gpu() {
                         m = std::fmax(m, std::fabs(got[((bi * t + ti) * h + hi) * d + di] -
                                                     want[((bi * h + hi) * t + ti) * d + di]));
         CHECK(m <= 1e-5f);
+    }
+    {   // decode preparation: at position 0 without norms the rotation is the identity (rope.rs:247-256), so q is
+        // unchanged and row 0 of the caches holds k_in / v_in; at position 1, theta_0 = 1 rotates the pair (0, D/2)
+        // of a unit vector to (cos 1, sin 1)
+        const int hq = 2, hkv = 1, d = 8, lmax = 4;
+        auto bf = [](float x) { uint32_t u; std::memcpy(&u, &x, 4); return (uint16_t)(u >> 16); };
+        auto fb = [](uint16_t h) { uint32_t u = (uint32_t)h << 16; float f; std::memcpy(&f, &u, 4); return f; };
+        std::vector<uint16_t> q(hq * d), k(hkv * d), v(hkv * d), cache(hkv * lmax * d, bf(9.0f));
+        for (int i = 0; i < hq * d; i++) q[i] = bf(0.25f * (float)(i % 7) - 0.5f);
+        for (int i = 0; i < hkv * d; i++) { k[i] = bf(i == 0 ? 1.0f : 0.0f); v[i] = bf(0.5f * (float)i); }
+        RoPE rope(d, 16);
+        HipStorage dq = HipStorage::from_host(q), dk = HipStorage::from_host(k), dv = HipStorage::from_host(v);
+        HipStorage dkc = HipStorage::from_host(cache), dvc = HipStorage::from_host(cache);
+        LlmKernels::qk_norm_rope_kv_append_bf16(nullptr, dq.ptr(), dk.ptr(), dv.ptr(), dkc.ptr(), dvc.ptr(), nullptr, 0, nullptr,
+                                                nullptr, 1e-6f, rope, 1, hq, hkv, d, lmax);
+        synchronize();
+        CHECK(dq.to_host<uint16_t>() == q);
+        auto kc = dkc.to_host<uint16_t>(), vc = dvc.to_host<uint16_t>();
+        for (int i = 0; i < d; i++) CHECK(kc[i] == k[i] && vc[i] == v[i] && kc[d + i] == bf(9.0f));
+        LlmKernels::qk_norm_rope_kv_append_bf16(nullptr, dq.ptr(), dk.ptr(), dv.ptr(), dkc.ptr(), dvc.ptr(), nullptr, 1, nullptr,
+                                                nullptr, 1e-6f, rope, 1, hq, hkv, d, lmax);
+        synchronize();
+        kc = dkc.to_host<uint16_t>();
+        CHECK(std::fabs(fb(kc[d + 0]) - std::cos(1.0f)) < 4e-3f && std::fabs(fb(kc[d + d / 2]) - std::sin(1.0f)) < 4e-3f);
+        for (int i = 1; i < d / 2; i++) CHECK(kc[d + i] == 0 && kc[d + d / 2 + i] == 0);
     }
     {   // device buffers round-trip
         std::vector<float> h = lcg(1000, 9);
