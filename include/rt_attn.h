@@ -163,6 +163,16 @@ int rt_flash_forward_varlen_bf16_dev(void *stream, const rt_attention_shape *sha
 int rt_kv_append_bf16(void *stream, void *k_cache, void *v_cache, const void *k_in, const void *v_in, int32_t pos,
                       int32_t n_kv, int32_t head_dim, int32_t max_seq, rt_err_detail *err);
 
+/* KVLayerCache::append -- crates/rustorch-nn/src/kv_cache.rs:77-112 -- on device buffers: new_k / new_v
+ * [batch, n_heads, seq_added, head_dim] are written at row current_len of the caches [batch, n_heads, max_seq,
+ * head_dim]; elem_bytes is 2 (bf16) or 4 (f32).  Checks in the reference's order: current_len + seq_added > max_seq
+ * -> RT_ERR_KV_OVERFLOW {requested = got, max = expected}; new_k_len or new_v_len (elements) != batch * n_heads *
+ * seq_added * head_dim -> RT_ERR_KV_WRONG_INPUT_LEN {expected, got_k = got, got_v = got2}.  Asynchronous on `stream`. */
+int rt_kv_cache_append_dev(void *stream, void *k_cache, void *v_cache, const void *new_k, size_t new_k_len,
+                           const void *new_v, size_t new_v_len, size_t batch, size_t n_heads, size_t max_seq,
+                           size_t head_dim, size_t current_len, size_t seq_added, size_t elem_bytes,
+                           rt_err_detail *err);
+
 /* Steps 2a, 2b and 3 of LlamaModel::decode_step -- crates/rustorch-llm/src/model.rs:575-636 -- in one launch,
  * for a batch of sequences on bf16 storage: per-head RMSNorm of q and k (rms_norm_per_head, model.rs:862-897;
  * gamma f32[head_dim] shared by the heads, NULL = no norm), half-split RoPE (RoPE::apply_inplace_half_split,
@@ -206,6 +216,10 @@ size_t rt_gqa_decode_workspace_bytes(int32_t batch, int32_t n_heads, int32_t n_k
 /* ---- device buffers (the slot of Storage::Cuda, crates/rustorch-core/src/tensor/storage.rs:776-817) */
 void *rt_buf_alloc(size_t bytes, rt_err_detail *err);
 int rt_buf_free(void *ptr, rt_err_detail *err);
+/* Zero-fills `bytes` bytes at `ptr` (a multiple of 4, `ptr` 4-byte aligned), asynchronously on `stream`, with a
+ * fill kernel (safe to record into a HIP graph).  The reference's caches start as vec![0.0; n]
+ * (crates/rustorch-nn/src/kv_cache.rs:63-66). */
+int rt_buf_zero(void *ptr, size_t bytes, void *stream, rt_err_detail *err);
 int rt_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream, rt_err_detail *err);
 int rt_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream, rt_err_detail *err);
 int rt_stream_synchronize(void *stream, rt_err_detail *err);

@@ -12,6 +12,7 @@
 //   rustorch_attn::mha_flash_forward_f32
 //                                   crates/rustorch-nn/src/attention.rs:452-495
 //   rustorch_attn::LlmKernels       crates/rustorch-cuda/src/llm_kernels.rs:874-958 (attention part)
+//   rustorch_attn::KVCache          crates/rustorch-nn/src/kv_cache.rs:49-256, buffers in HBM
 //   rustorch_attn::RoPE, RoPEError  crates/rustorch-nn/src/rope.rs:33-241 (tables and errors; the rotation runs on the device)
 //   rustorch_attn::HipStorage       the slot of Storage::Cuda, crates/rustorch-core/src/tensor/storage.rs:776-817
 //
@@ -68,6 +69,20 @@ struct KVCacheOverflow : std::runtime_error {
     KVCacheOverflow(size_t r, size_t m)
         : std::runtime_error("kv_cache overflow: requested " + std::to_string(r) + " positions, max " + std::to_string(m)),
           requested(r), max(m) {}
+};
+// The other two variants of KVCacheError.
+struct KVCacheWrongInputLen : std::runtime_error {
+    size_t expected = 0, got_k = 0, got_v = 0;
+    KVCacheWrongInputLen(size_t e, size_t k, size_t v)
+        : std::runtime_error("kv_cache append: expected " + std::to_string(e) + ", got K=" + std::to_string(k) +
+                             " V=" + std::to_string(v)),
+          expected(e), got_k(k), got_v(v) {}
+};
+struct KVCacheLayerOutOfRange : std::runtime_error {
+    size_t layer = 0, num_layers = 0;
+    KVCacheLayerOutOfRange(size_t l, size_t n)
+        : std::runtime_error("kv_cache layer " + std::to_string(l) + " out of range (have " + std::to_string(n) + ")"),
+          layer(l), num_layers(n) {}
 };
 
 // Stands where the reference has CudaError: no device, a failed HIP call, a shape the kernels do not cover.
@@ -137,6 +152,7 @@ inline void check_prepare(int rc, const rt_err_detail& e) {
             throw RoPEError(RoPEError::Kind::PositionOverflow, e.expected, e.got,
                             "rope: position " + std::to_string(e.got) + " exceeds max_seq " + std::to_string(e.expected));
         case RT_ERR_KV_OVERFLOW: throw KVCacheOverflow(e.got, e.expected);
+        case RT_ERR_KV_WRONG_INPUT_LEN: throw KVCacheWrongInputLen(e.expected, e.got, e.got2);
         default: throw_device(rc, e);
     }
 }
@@ -309,6 +325,51 @@ inline void flash_forward_varlen_bf16_dev(const AttentionShape& shape, const voi
         rt_flash_forward_varlen_bf16_dev(stream, &s, n_kv_heads, q, k, v, seq_lens_dev, zero_padded_rows ? 1 : 0, out, &e),
         e);
 }
+
+// ---- KVCache (crates/rustorch-nn/src/kv_cache.rs:49-256) with its buffers in HBM ---------------------------
+//
+// Same protocol as the reference: append(layer, seq_added, new_k, new_v) for every layer, then advance(seq_added).
+// Buffers are [batch, n_heads, max_seq, head_dim] of 2-byte (bf16, the decode kernels' storage) or 4-byte (f32)
+// elements, zero-filled at construction; new_k / new_v are device buffers and their element counts are checked
+// as the reference checks slice lengths.  k_buffer / v_buffer are what the decode entry points take as caches.
+class KVCache {
+public:
+    KVCache(size_t num_layers, size_t batch, size_t n_heads, size_t head_dim, size_t max_seq, size_t elem_bytes = 2)
+        : batch_(batch), n_heads_(n_heads), head_dim_(head_dim), max_seq_(max_seq), elem_bytes_(elem_bytes) {
+        const size_t bytes = batch * n_heads * max_seq * head_dim * elem_bytes;
+        for (size_t i = 0; i < num_layers; i++) {
+            k_.emplace_back(bytes);
+            v_.emplace_back(bytes);
+            rt_err_detail e;
+            detail::check_device(rt_buf_zero(k_.back().ptr(), bytes, nullptr, &e), e);
+            detail::check_device(rt_buf_zero(v_.back().ptr(), bytes, nullptr, &e), e);
+        }
+    }
+    size_t num_layers() const { return k_.size(); }
+    size_t max_seq() const { return max_seq_; }
+    size_t current_len() const { return current_len_; }
+    void clear() { current_len_ = 0; }
+    void append(size_t layer_idx, size_t seq_added, const HipStorage& new_k, const HipStorage& new_v, void* stream = nullptr) {
+        if (layer_idx >= k_.size()) throw KVCacheLayerOutOfRange(layer_idx, k_.size());
+        rt_err_detail e;
+        detail::check_prepare(
+            rt_kv_cache_append_dev(stream, k_[layer_idx].ptr(), v_[layer_idx].ptr(), new_k.ptr(), new_k.byte_len() / elem_bytes_,
+                                   new_v.ptr(), new_v.byte_len() / elem_bytes_, batch_, n_heads_, max_seq_, head_dim_,
+                                   current_len_, seq_added, elem_bytes_, &e),
+            e);
+    }
+    void advance(size_t seq_added) {
+        if (current_len_ + seq_added > max_seq_) throw KVCacheOverflow(current_len_ + seq_added, max_seq_);
+        current_len_ += seq_added;
+    }
+    const HipStorage* k_buffer(size_t layer_idx) const { return layer_idx < k_.size() ? &k_[layer_idx] : nullptr; }
+    const HipStorage* v_buffer(size_t layer_idx) const { return layer_idx < v_.size() ? &v_[layer_idx] : nullptr; }
+    std::array<size_t, 4> dims() const { return {batch_, n_heads_, max_seq_, head_dim_}; }
+
+private:
+    size_t batch_, n_heads_, head_dim_, max_seq_, elem_bytes_, current_len_ = 0;
+    std::vector<HipStorage> k_, v_;
+};
 
 // ---- RoPE tables (crates/rustorch-nn/src/rope.rs:33-90) ----------------------------------------------------
 //

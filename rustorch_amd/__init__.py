@@ -10,9 +10,11 @@ from .attention import (AttentionShape, Mask, flash_forward, flash_forward_bf16_
                         flash_forward_varlen_bf16_dev, mha_flash_forward_f32)
 from .device import HipStorage, init, synchronize
 from .errors import (AttentionError, BufferShapeMismatch, DeviceError, GQAError, HeadCountMismatch, KVCacheError,
+                     KVWrongInputLen, LayerOutOfRange,
                      MaskError, OutputShapeMismatch, Overflow, PaddingLengthMismatch, PositionOverflow, RoPEError,
                      RopeWrongInputLen, WrongInputLen, ZeroDim)
 from .gqa import gqa_forward_f32
+from .kv_cache import KVCache
 from .llm_kernels import LlmKernels
 from .rope import RoPE
 

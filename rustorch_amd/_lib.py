@@ -17,9 +17,9 @@ SYMBOLS = (
     "rt_flash_forward_f32", "rt_flash_forward_masked_f32", "rt_gqa_forward_f32",
     "rt_flash_forward_f32_dev", "rt_flash_forward_bf16_dev", "rt_flash_forward_varlen_bf16_dev",
     "rt_mha_flash_forward_f32", "rt_flash_forward_bnhd_f32_dev", "rt_flash_forward_bnhd_bf16_dev",
-    "rt_kv_append_bf16", "rt_qk_norm_rope_kv_append_bf16", "rt_gqa_decode_online_bf16", "rt_gqa_decode_batched_bf16",
+    "rt_kv_append_bf16", "rt_kv_cache_append_dev", "rt_qk_norm_rope_kv_append_bf16", "rt_gqa_decode_online_bf16", "rt_gqa_decode_batched_bf16",
     "rt_gqa_decode_workspace_bytes",
-    "rt_buf_alloc", "rt_buf_free", "rt_memcpy_h2d", "rt_memcpy_d2h", "rt_stream_synchronize",
+    "rt_buf_alloc", "rt_buf_free", "rt_buf_zero", "rt_memcpy_h2d", "rt_memcpy_d2h", "rt_stream_synchronize",
 )
 
 RT_OK = 0
@@ -86,6 +86,7 @@ def lib():
     L.rt_flash_forward_bnhd_f32_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_flash_forward_bnhd_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_kv_append_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, errp]
+    L.rt_kv_cache_append_dev.argtypes = [vp, vp, vp, vp, sz, vp, sz, sz, sz, sz, sz, sz, sz, sz, errp]
     L.rt_qk_norm_rope_kv_append_bf16.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, vp, vp, C.c_float, vp, vp, i32, i32,
                                                  i32, i32, i32, i32, errp]
     L.rt_gqa_decode_online_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, errp]
@@ -95,6 +96,7 @@ def lib():
     L.rt_buf_alloc.argtypes = [sz, errp]
     L.rt_buf_alloc.restype = vp
     L.rt_buf_free.argtypes = [vp, errp]
+    L.rt_buf_zero.argtypes = [vp, sz, vp, errp]
     L.rt_memcpy_h2d.argtypes = [vp, vp, sz, vp, errp]
     L.rt_memcpy_d2h.argtypes = [vp, vp, sz, vp, errp]
     L.rt_stream_synchronize.argtypes = [vp, errp]

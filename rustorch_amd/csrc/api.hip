@@ -6,6 +6,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <algorithm>
 #include <mutex>
 
 #include "../../include/rt_attn.h"
@@ -482,6 +483,31 @@ RT_API int rt_kv_append_bf16(void* stream, void* k_cache, void* v_cache, const v
     return RT_OK;
 }
 
+RT_API int rt_kv_cache_append_dev(void* stream, void* k_cache, void* v_cache, const void* new_k, size_t new_k_len,
+                                  const void* new_v, size_t new_v_len, size_t batch, size_t n_heads, size_t max_seq,
+                                  size_t head_dim, size_t current_len, size_t seq_added, size_t elem_bytes,
+                                  rt_err_detail* err) {
+    clear_err(err);
+    if (current_len + seq_added > max_seq)  // kv_cache.rs:84-89
+        return fail(err, RT_ERR_KV_OVERFLOW, -1, (uint64_t)max_seq, (uint64_t)(current_len + seq_added), "append beyond max_seq");
+    const size_t bhsd = batch * n_heads * seq_added * head_dim;
+    if (new_k_len != bhsd || new_v_len != bhsd) {  // kv_cache.rs:90-97
+        int rc = fail(err, RT_ERR_KV_WRONG_INPUT_LEN, -1, (uint64_t)bhsd, (uint64_t)new_k_len, "new_k / new_v length");
+        if (err) err->got2 = (uint64_t)new_v_len;
+        return rc;
+    }
+    if (elem_bytes != 2 && elem_bytes != 4) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, (uint64_t)elem_bytes, "elem_bytes must be 2 or 4");
+    if (batch * n_heads > 65535) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    if (bhsd == 0) return RT_OK;
+    if (!k_cache || !v_cache || !new_k || !new_v) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    int rc = ensure_device(err);
+    if (rc) return rc;
+    HIP_TRY(rt::launch_kv_block_append((hipStream_t)stream, k_cache, v_cache, new_k, new_v, batch * n_heads, max_seq, head_dim,
+                                       current_len, seq_added, elem_bytes),
+            "kv_cache_append launch");
+    return RT_OK;
+}
+
 RT_API int rt_qk_norm_rope_kv_append_bf16(void* stream, void* q, const void* k_in, const void* v_in, void* k_cache,
                                           void* v_cache, const int32_t* positions, int32_t pos, const float* q_gamma,
                                           const float* k_gamma, float eps, const float* cos_table,
@@ -653,6 +679,34 @@ RT_API int rt_buf_free(void* ptr, rt_err_detail* err) {
     clear_err(err);
     if (!ptr) return RT_OK;
     HIP_TRY(hipFree(ptr), "hipFree");
+    return RT_OK;
+}
+
+namespace {
+__global__ __launch_bounds__(256) void zero_fill_kernel(uint32_t* p, size_t n_words) {
+    const size_t n4 = n_words / 4;
+    uint4* p4 = (uint4*)p;
+    const size_t stride = (size_t)gridDim.x * blockDim.x, t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (((uintptr_t)p & 15) == 0) {
+        for (size_t i = t; i < n4; i += stride) p4[i] = make_uint4(0u, 0u, 0u, 0u);
+        for (size_t i = 4 * n4 + t; i < n_words; i += stride) p[i] = 0u;
+    } else {
+        for (size_t i = t; i < n_words; i += stride) p[i] = 0u;
+    }
+}
+}  // namespace
+
+RT_API int rt_buf_zero(void* ptr, size_t bytes, void* stream, rt_err_detail* err) {
+    clear_err(err);
+    if (bytes == 0) return RT_OK;
+    if (!ptr) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    if ((bytes & 3) || ((uintptr_t)ptr & 3)) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, (uint64_t)bytes, "zero fill works on 4-byte words");
+    int rc = ensure_device(err);
+    if (rc) return rc;
+    const size_t n_words = bytes / 4;
+    const unsigned blocks = (unsigned)std::min<size_t>((n_words / 4 + 255) / 256 + 1, 4096);
+    hipLaunchKernelGGL(zero_fill_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint32_t*)ptr, n_words);
+    HIP_TRY(hipGetLastError(), "zero_fill launch");
     return RT_OK;
 }
 

@@ -10,6 +10,9 @@
 //                         online-softmax monoid (crates/rustorch-attention/src/online_softmax.rs:105-131,
 //                         extended with o).
 //   kv_append_kernel      llm_kernels.rs:353-372.
+//   kv_block_append_kernel  KVLayerCache::append, crates/rustorch-nn/src/kv_cache.rs:77-112 (seq_added rows per head).
+#include <algorithm>
+
 #include "rt_common.hpp"
 #include "rt_kernels.hpp"
 
@@ -449,6 +452,25 @@ __global__ void kv_append_kernel(uint16_t* __restrict__ k_cache, uint16_t* __res
     v_cache[off] = v_in[idx];
 }
 
+// KVLayerCache::append (kv_cache.rs:97-110): per (b, h) one contiguous run of seq_added * head_dim elements goes
+// from new[b, h, 0.., :] to cache[b, h, current_len.., :].  T is the copy unit (16 bytes when everything is
+// aligned, else the element); run_units / dst_stride_units / dst_first_unit are in units of T.
+template <typename T>
+__global__ __launch_bounds__(256) void kv_block_append_kernel(T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                                              const T* __restrict__ new_k, const T* __restrict__ new_v,
+                                                              size_t run_units, size_t dst_stride_units,
+                                                              size_t dst_first_unit) {
+    const size_t bh = blockIdx.y;
+    const T* sk = new_k + bh * run_units;
+    const T* sv = new_v + bh * run_units;
+    T* dk = k_cache + bh * dst_stride_units + dst_first_unit;
+    T* dv = v_cache + bh * dst_stride_units + dst_first_unit;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < run_units; i += (size_t)gridDim.x * blockDim.x) {
+        dk[i] = sk[i];
+        dv[i] = sv[i];
+    }
+}
+
 template <int HD>
 hipError_t launch_split_hd(hipStream_t stream, const DecodeSplitParams& p) {
     hipLaunchKernelGGL(decode_split_kernel<HD>, dim3(p.n_waves), dim3(64), 0, stream, p);
@@ -503,6 +525,35 @@ hipError_t launch_kv_append_bf16(hipStream_t stream, uint16_t* k_cache, uint16_t
     if (n <= 0) return hipSuccess;
     hipLaunchKernelGGL(kv_append_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, k_cache, v_cache, k_in, v_in,
                        pos, n_kv, head_dim, max_seq);
+    return hipGetLastError();
+}
+
+hipError_t launch_kv_block_append(hipStream_t stream, void* k_cache, void* v_cache, const void* new_k, const void* new_v,
+                                  size_t batch_heads, size_t max_seq, size_t head_dim, size_t current_len,
+                                  size_t seq_added, size_t elem_bytes) {
+    const size_t run_bytes = seq_added * head_dim * elem_bytes;
+    if (batch_heads == 0 || run_bytes == 0) return hipSuccess;
+    if (batch_heads > 65535) return hipErrorInvalidValue;
+    const size_t stride_bytes = max_seq * head_dim * elem_bytes, first_bytes = current_len * head_dim * elem_bytes;
+    auto al16 = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+    const bool wide = al16(k_cache) && al16(v_cache) && al16(new_k) && al16(new_v) && run_bytes % 16 == 0 &&
+                      stride_bytes % 16 == 0 && first_bytes % 16 == 0;
+    const size_t unit = wide ? 16 : elem_bytes;
+    const size_t run_units = run_bytes / unit;
+    const unsigned gx = (unsigned)std::min<size_t>((run_units + 255) / 256, 1024);
+    dim3 grid(gx, (unsigned)batch_heads), block(256);
+    if (wide) {
+        hipLaunchKernelGGL(kv_block_append_kernel<u32x4_t>, grid, block, 0, stream, (u32x4_t*)k_cache, (u32x4_t*)v_cache,
+                           (const u32x4_t*)new_k, (const u32x4_t*)new_v, run_units, stride_bytes / 16, first_bytes / 16);
+    } else if (elem_bytes == 2) {
+        hipLaunchKernelGGL(kv_block_append_kernel<uint16_t>, grid, block, 0, stream, (uint16_t*)k_cache, (uint16_t*)v_cache,
+                           (const uint16_t*)new_k, (const uint16_t*)new_v, run_units, stride_bytes / 2, first_bytes / 2);
+    } else if (elem_bytes == 4) {
+        hipLaunchKernelGGL(kv_block_append_kernel<uint32_t>, grid, block, 0, stream, (uint32_t*)k_cache, (uint32_t*)v_cache,
+                           (const uint32_t*)new_k, (const uint32_t*)new_v, run_units, stride_bytes / 4, first_bytes / 4);
+    } else {
+        return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

@@ -94,6 +94,12 @@ int decode_split_parts(int max_seq);
 size_t decode_split_workspace_bytes(int batch, int heads, int dim, int max_seq);
 hipError_t launch_decode_split(hipStream_t stream, const DecodeSplitParams& p);
 
+// KVLayerCache::append on device buffers of 2- or 4-byte elements: [batch_heads, seq_added, head_dim] into
+// [batch_heads, max_seq, head_dim] at row current_len.
+hipError_t launch_kv_block_append(hipStream_t stream, void* k_cache, void* v_cache, const void* new_k, const void* new_v,
+                                  size_t batch_heads, size_t max_seq, size_t head_dim, size_t current_len,
+                                  size_t seq_added, size_t elem_bytes);
+
 // Per-head q/k RMSNorm, half-split RoPE and the cache append of one decode step (prepare.hip).
 struct DecodePrepareParams {
     uint16_t* q;              // [batch, n_heads, head_dim], rewritten in place

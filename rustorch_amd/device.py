@@ -28,6 +28,14 @@ class HipStorage:
         s.upload(a, stream)
         return s
 
+    @classmethod
+    def zeros(cls, byte_len: int, stream=None) -> "HipStorage":
+        """A zero-filled buffer (byte_len a multiple of 4); the fill is enqueued on `stream`."""
+        s = cls(byte_len)
+        err = L.RtErr()
+        raise_for(L.lib().rt_buf_zero(s.ptr, s.byte_len, stream, C.byref(err)), err)
+        return s
+
     def upload(self, a: np.ndarray, stream=None):
         a = np.ascontiguousarray(a)
         assert a.nbytes <= self.byte_len

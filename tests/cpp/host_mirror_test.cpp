@@ -243,6 +243,27 @@ static void test_gpu() {
         CHECK(std::fabs(fb(kc[d + 0]) - std::cos(1.0f)) < 4e-3f && std::fabs(fb(kc[d + d / 2]) - std::sin(1.0f)) < 4e-3f);
         for (int i = 1; i < d / 2; i++) CHECK(kc[d + i] == 0 && kc[d + d / 2 + i] == 0);
     }
+    {   // KVCache: the reference's index table (kv_cache.rs:306-322) and errors (:326-348) on device buffers
+        KVCache c(1, 1, 1, 2, 4, 4);
+        std::vector<float> k1 = {1, 2}, v1 = {10, 20}, k2 = {3, 4}, v2 = {30, 40};
+        c.append(0, 1, HipStorage::from_host(k1), HipStorage::from_host(v1));
+        c.advance(1);
+        c.append(0, 1, HipStorage::from_host(k2), HipStorage::from_host(v2));
+        c.advance(1);
+        synchronize();
+        auto kb = c.k_buffer(0)->to_host<float>(), vb = c.v_buffer(0)->to_host<float>();
+        CHECK(kb[0] == 1 && kb[1] == 2 && kb[2] == 3 && kb[3] == 4 && kb[4] == 0);
+        CHECK(vb[0] == 10 && vb[1] == 20 && vb[2] == 30 && vb[3] == 40 && c.current_len() == 2);
+        bool overflow = false, wrong = false, layer = false;
+        std::vector<float> six(6, 0.0f), three(3, 0.0f);
+        try { c.append(0, 3, HipStorage::from_host(six), HipStorage::from_host(six)); }
+        catch (const KVCacheOverflow& e) { overflow = e.requested == 5 && e.max == 4; }
+        try { c.append(0, 1, HipStorage::from_host(three), HipStorage::from_host(k1)); }
+        catch (const KVCacheWrongInputLen& e) { wrong = e.expected == 2 && e.got_k == 3 && e.got_v == 2; }
+        try { c.append(7, 1, HipStorage::from_host(k1), HipStorage::from_host(v1)); }
+        catch (const KVCacheLayerOutOfRange& e) { layer = e.layer == 7 && e.num_layers == 1; }
+        CHECK(overflow && wrong && layer && c.k_buffer(3) == nullptr);
+    }
     {   // device buffers round-trip
         std::vector<float> h = lcg(1000, 9);
         HipStorage s = HipStorage::from_host(h);
