@@ -177,20 +177,24 @@ int rt_kv_cache_append_dev(void *stream, void *k_cache, void *v_cache, const voi
  * for a batch of sequences on bf16 storage: per-head RMSNorm of q and k (rms_norm_per_head, model.rs:862-897;
  * gamma f32[head_dim] shared by the heads, NULL = no norm), half-split RoPE (RoPE::apply_inplace_half_split,
  * crates/rustorch-nn/src/rope.rs:162-205; cos/sin f32[table_rows, head_dim/2] as RoPE::new builds them,
- * rope.rs:63-90) and the cache append (kv_append_bf16, llm_kernels.rs:353-372).  Replaces the
- * rope_half_split_bf16 x2 + kv_append_bf16 launches of crates/rustorch-llm/src/cuda_backend.rs:486-540.
- * q [batch,n_heads,head_dim] is rewritten in place; k_in/v_in [batch,n_kv,head_dim]; caches
- * [batch,n_kv,max_seq,head_dim]; sequence b uses position positions[b] (device int32[batch]) or, with
- * positions == NULL, `pos`.  f32 arithmetic in the reference's order, one rounding to bf16 at the end.
- * Errors: `pos` >= table_rows -> RT_ERR_ROPE_POSITION_OVERFLOW (RoPEError::PositionOverflow{max_seq=expected,
- * requested=got}); `pos` >= max_seq -> RT_ERR_KV_OVERFLOW; odd head_dim or head_dim > 512 -> RT_ERR_UNSUPPORTED
- * (RoPE::new panics on an odd head_dim).  Positions on the device cannot be checked by the host: a sequence
- * whose position is out of range is left untouched. */
+ * rope.rs:63-90) and the cache append (KVLayerCache::append, crates/rustorch-nn/src/kv_cache.rs:77-112; for
+ * seq == 1 the index rule of kv_append_bf16, llm_kernels.rs:353-372).  Replaces the rope_half_split_bf16 x2 +
+ * kv_append_bf16 launches of crates/rustorch-llm/src/cuda_backend.rs:486-540.
+ * `seq` new tokens per sequence (1 when decoding, the prompt length when prefilling): q [batch,n_heads,seq,
+ * head_dim] is rewritten in place; k_in/v_in [batch,n_kv,seq,head_dim]; caches [batch,n_kv,max_seq,head_dim].
+ * Token s of sequence b sits at position p_b + s, with p_b = positions[b] (device int32[batch]) or, with
+ * positions == NULL, `pos`; k and v go to cache rows p_b .. p_b + seq - 1.  f32 arithmetic in the reference's
+ * order, one rounding to bf16 at the end.
+ * Errors (host `pos` only): pos + seq > table_rows -> RT_ERR_ROPE_POSITION_OVERFLOW (RoPEError::PositionOverflow
+ * {max_seq = expected, requested = got}, rope.rs:179-184); pos + seq > max_seq -> RT_ERR_KV_OVERFLOW
+ * (kv_cache.rs:84-89); odd head_dim or head_dim > 512 -> RT_ERR_UNSUPPORTED (RoPE::new panics on an odd head_dim).
+ * Positions on the device cannot be checked by the host: a sequence whose rows would leave the tables or the
+ * cache is left untouched. */
 int rt_qk_norm_rope_kv_append_bf16(void *stream, void *q, const void *k_in, const void *v_in, void *k_cache,
                                    void *v_cache, const int32_t *positions, int32_t pos, const float *q_gamma,
                                    const float *k_gamma, float eps, const float *cos_table, const float *sin_table,
-                                   int32_t table_rows, int32_t batch, int32_t n_heads, int32_t n_kv, int32_t head_dim,
-                                   int32_t max_seq, rt_err_detail *err);
+                                   int32_t table_rows, int32_t batch, int32_t seq, int32_t n_heads, int32_t n_kv,
+                                   int32_t head_dim, int32_t max_seq, rt_err_detail *err);
 
 /* LlmKernels::gqa_decode_online_bf16 -- llm_kernels.rs:396-457, :915-958.  q/out
  * [n_heads,head_dim] bf16, caches [n_kv,max_seq,head_dim] bf16 of which [..kv_len] is read;

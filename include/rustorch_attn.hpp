@@ -417,24 +417,26 @@ struct LlmKernels {
         detail::check_device(rt_kv_append_bf16(stream, k_cache, v_cache, k_in, v_in, pos, n_kv, head_dim, max_seq, &e), e);
     }
     // Steps 2a, 2b, 3 of LlamaModel::decode_step (crates/rustorch-llm/src/model.rs:575-636) in one launch: per-head
-    // q/k RMSNorm (device f32 gammas or nullptr), half-split RoPE, cache append.  `positions` is a device
-    // int32[batch] array, or nullptr to use `pos` for every sequence (then checked here, like the reference).
+    // q/k RMSNorm (device f32 gammas or nullptr), half-split RoPE, cache append, for `seq` new tokens per sequence
+    // ([batch, heads, seq, head_dim] buffers; 1 when decoding).  `positions` is a device int32[batch] array (position
+    // of each sequence's first new token), or nullptr to use `pos` for every sequence (then checked here, like the
+    // reference).
     static void qk_norm_rope_kv_append_bf16(void* stream, void* q, const void* k_in, const void* v_in, void* k_cache,
                                             void* v_cache, const int32_t* positions, int32_t pos, const float* q_gamma,
                                             const float* k_gamma, float eps, RoPE& rope, int32_t batch, int32_t n_heads,
-                                            int32_t n_kv, int32_t head_dim, int32_t max_seq) {
-        if (!positions) {  // the reference's checks, before anything touches the device (rope.rs:179-184, kv_cache.rs:88-95)
-            if (pos < 0 || (size_t)pos >= rope.max_seq())
-                throw RoPEError(RoPEError::Kind::PositionOverflow, rope.max_seq(), (size_t)((int64_t)pos + 1),
-                                "rope: position " + std::to_string((int64_t)pos + 1) + " exceeds max_seq " +
-                                    std::to_string(rope.max_seq()));
-            if (pos >= max_seq) throw KVCacheOverflow((size_t)((int64_t)pos + 1), (size_t)max_seq);
+                                            int32_t n_kv, int32_t head_dim, int32_t max_seq, int32_t seq = 1) {
+        if (!positions) {  // the reference's checks, before anything touches the device (rope.rs:179-184, kv_cache.rs:84-89)
+            const int64_t end = (int64_t)pos + seq;
+            if (pos < 0 || end > (int64_t)rope.max_seq())
+                throw RoPEError(RoPEError::Kind::PositionOverflow, rope.max_seq(), (size_t)end,
+                                "rope: position " + std::to_string(end) + " exceeds max_seq " + std::to_string(rope.max_seq()));
+            if (end > max_seq) throw KVCacheOverflow((size_t)end, (size_t)max_seq);
         }
         rt_err_detail e;
         detail::check_prepare(
             rt_qk_norm_rope_kv_append_bf16(stream, q, k_in, v_in, k_cache, v_cache, positions, pos, q_gamma, k_gamma, eps,
                                            (const float*)rope.device_cos(), (const float*)rope.device_sin(),
-                                           (int32_t)rope.max_seq(), batch, n_heads, n_kv, head_dim, max_seq, &e),
+                                           (int32_t)rope.max_seq(), batch, seq, n_heads, n_kv, head_dim, max_seq, &e),
             e);
     }
     static void gqa_decode_online_bf16(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out,

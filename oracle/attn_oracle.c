@@ -718,52 +718,56 @@ RO_EXPORT void ro_rms_norm_per_head(float *x, const float *gamma, size_t n_heads
     for (size_t h = 0; h < n_heads; h++) rms_norm_head(x + h * head_dim, gamma, head_dim, eps);
 }
 
-/* Steps 2a, 2b and 3 of decode_step (model.rs:575-636) for a batch of sequences on bf16 storage: every value is
- * widened to f32, normalised per head (when a gamma is given), rotated (half-split) at the sequence's position and
- * rounded to bf16 once; q is rewritten in place, k and v go to row positions[b] of the caches
- * [batch, n_kv, max_seq, head_dim] (the index rule of kv_append_bf16, llm_kernels.rs:353-372, per sequence).
- * Positions must satisfy 0 <= p < min(max_seq, table_rows); returns the overflow error otherwise, having written
- * nothing. */
+/* Steps 2a, 2b and 3 of decode_step (model.rs:575-636) for a batch of sequences with `seq` new tokens each, on bf16
+ * storage: every value is widened to f32, normalised per head (when a gamma is given), rotated (half-split) at
+ * position positions[b] + s (rope.rs:192-193) and rounded to bf16 once; q [batch, n_heads, seq, head_dim] is
+ * rewritten in place, k and v [batch, n_kv, seq, head_dim] go to rows positions[b] .. + seq - 1 of the caches
+ * [batch, n_kv, max_seq, head_dim] (KVLayerCache::append, kv_cache.rs:97-110; for seq == 1 the index rule of
+ * kv_append_bf16, llm_kernels.rs:353-372).  Every sequence must satisfy 0 <= p and p + seq <= min(max_seq,
+ * table_rows); returns the overflow error otherwise, having written nothing. */
 RO_EXPORT int ro_decode_prepare_bf16(uint16_t *q, const uint16_t *k_in, const uint16_t *v_in, uint16_t *k_cache,
                                      uint16_t *v_cache, const int32_t *positions, const float *q_gamma,
                                      const float *k_gamma, float eps, const float *cos_t, const float *sin_t, int batch,
-                                     int n_heads, int n_kv, int head_dim, int max_seq, int table_rows, ro_err *err) {
+                                     int seq, int n_heads, int n_kv, int head_dim, int max_seq, int table_rows,
+                                     ro_err *err) {
     const size_t d = (size_t)head_dim;
     for (int b = 0; b < batch; b++) {
-        int p = positions[b];
-        if (p < 0 || p >= table_rows) {
-            set_err(err, -1, (uint64_t)table_rows, (uint64_t)((int64_t)p + 1));
+        int64_t p = positions[b];
+        if (p < 0 || p + seq > table_rows) { /* rope.rs:179-184 */
+            set_err(err, -1, (uint64_t)table_rows, (uint64_t)(p + seq));
             return RO_ERR_ROPE_POSITION_OVERFLOW;
         }
-        if (p >= max_seq) { /* kv_cache.rs:88-95 */
-            set_err(err, -1, (uint64_t)max_seq, (uint64_t)((int64_t)p + 1));
+        if (p + seq > max_seq) { /* kv_cache.rs:84-89 */
+            set_err(err, -1, (uint64_t)max_seq, (uint64_t)(p + seq));
             return RO_ERR_KV_OVERFLOW;
         }
     }
     float *row = (float *)malloc(d * sizeof(float));
     if (!row) return -1;
     ro_err e2;
-    for (int b = 0; b < batch; b++) {
-        const size_t p = (size_t)positions[b];
-        for (int h = 0; h < n_heads + n_kv; h++) {
-            const int is_q = h < n_heads;
-            uint16_t *src = is_q ? q + ((size_t)b * n_heads + h) * d : (uint16_t *)k_in + ((size_t)b * n_kv + (h - n_heads)) * d;
-            const float *gamma = is_q ? q_gamma : k_gamma;
-            for (size_t i = 0; i < d; i++) row[i] = ro_bf16_to_f32(src[i]);
-            if (gamma) rms_norm_head(row, gamma, d, eps);
-            ro_rope_half_split(row, d, 1, 1, 1, d, p, cos_t, sin_t, (size_t)table_rows, &e2);
-            if (is_q) {
-                for (size_t i = 0; i < d; i++) src[i] = ro_f32_to_bf16(row[i]);
-            } else {
-                const size_t off = (((size_t)b * n_kv + (h - n_heads)) * (size_t)max_seq + p) * d;
-                const uint16_t *vs = v_in + ((size_t)b * n_kv + (h - n_heads)) * d;
-                for (size_t i = 0; i < d; i++) {
-                    k_cache[off + i] = ro_f32_to_bf16(row[i]);
-                    v_cache[off + i] = vs[i];
+    for (int b = 0; b < batch; b++)
+        for (int h = 0; h < n_heads + n_kv; h++)
+            for (int s = 0; s < seq; s++) {
+                const size_t p = (size_t)positions[b] + (size_t)s;
+                const int is_q = h < n_heads;
+                const int kvh = h - n_heads;
+                uint16_t *src = is_q ? q + (((size_t)b * n_heads + h) * seq + s) * d
+                                     : (uint16_t *)k_in + (((size_t)b * n_kv + kvh) * seq + s) * d;
+                const float *gamma = is_q ? q_gamma : k_gamma;
+                for (size_t i = 0; i < d; i++) row[i] = ro_bf16_to_f32(src[i]);
+                if (gamma) rms_norm_head(row, gamma, d, eps);
+                ro_rope_half_split(row, d, 1, 1, 1, d, p, cos_t, sin_t, (size_t)table_rows, &e2);
+                if (is_q) {
+                    for (size_t i = 0; i < d; i++) src[i] = ro_f32_to_bf16(row[i]);
+                } else {
+                    const size_t off = (((size_t)b * n_kv + kvh) * (size_t)max_seq + p) * d;
+                    const uint16_t *vs = v_in + (((size_t)b * n_kv + kvh) * seq + s) * d;
+                    for (size_t i = 0; i < d; i++) {
+                        k_cache[off + i] = ro_f32_to_bf16(row[i]);
+                        v_cache[off + i] = vs[i];
+                    }
                 }
             }
-        }
-    }
     free(row);
     return RO_OK;
 }

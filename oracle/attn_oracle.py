@@ -121,7 +121,7 @@ def lib():
         L.ro_rms_norm_per_head.argtypes = [fp, fp, sz, sz, C.c_float]
         L.ro_rms_norm_per_head.restype = None
         L.ro_decode_prepare_bf16.argtypes = [u16p, u16p, u16p, u16p, u16p, i32p, fp, fp, C.c_float, fp, fp] + \
-            [C.c_int] * 6 + [C.POINTER(_Err)]
+            [C.c_int] * 7 + [C.POINTER(_Err)]
         _lib = L
     return _lib
 
@@ -402,9 +402,9 @@ def rms_norm_per_head(x, gamma, n_heads, head_dim, eps):
 
 
 def decode_prepare_bf16(q, k_in, v_in, k_cache, v_cache, positions, q_gamma, k_gamma, eps, rope, batch, n_heads, n_kv,
-                        head_dim, max_seq):
-    """Steps 2a, 2b, 3 of decode_step (model.rs:575-636) on bf16 bit patterns: returns the new q; the caches
-    (uint16 arrays) are updated in place."""
+                        head_dim, max_seq, seq=1):
+    """Steps 2a, 2b, 3 of decode_step (model.rs:575-636) on bf16 bit patterns, `seq` new tokens per sequence
+    ([batch, heads, seq, head_dim] inputs): returns the new q; the caches (uint16 arrays) are updated in place."""
     assert k_cache.dtype == np.uint16 and v_cache.dtype == np.uint16
     q, qp = _u16(q)
     q = q.copy()
@@ -423,8 +423,8 @@ def decode_prepare_bf16(q, k_in, v_in, k_cache, v_cache, positions, q_gamma, k_g
     rc = lib().ro_decode_prepare_bf16(qp, kip, vip, k_cache.ctypes.data_as(C.POINTER(C.c_uint16)),
                                       v_cache.ctypes.data_as(C.POINTER(C.c_uint16)),
                                       pos.ctypes.data_as(C.POINTER(C.c_int32)), gp_q, gp_k, eps,
-                                      rope.cos.ctypes.data_as(fp), rope.sin.ctypes.data_as(fp), batch, n_heads, n_kv,
-                                      head_dim, max_seq, rope.max_seq, C.byref(err))
+                                      rope.cos.ctypes.data_as(fp), rope.sin.ctypes.data_as(fp), batch, seq, n_heads,
+                                      n_kv, head_dim, max_seq, rope.max_seq, C.byref(err))
     _raise(rc, err)
     return q
 

@@ -88,7 +88,7 @@ def lib():
     L.rt_kv_append_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, errp]
     L.rt_kv_cache_append_dev.argtypes = [vp, vp, vp, vp, sz, vp, sz, sz, sz, sz, sz, sz, sz, sz, errp]
     L.rt_qk_norm_rope_kv_append_bf16.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, vp, vp, C.c_float, vp, vp, i32, i32,
-                                                 i32, i32, i32, i32, errp]
+                                                 i32, i32, i32, i32, i32, errp]
     L.rt_gqa_decode_online_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, errp]
     L.rt_gqa_decode_batched_bf16.argtypes = [vp, vp, vp, vp, vp, i32p, i32, i32, i32, i32, i32, vp, sz, errp]
     L.rt_gqa_decode_workspace_bytes.argtypes = [i32, i32, i32, i32, i32]

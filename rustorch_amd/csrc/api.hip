@@ -511,23 +511,25 @@ RT_API int rt_kv_cache_append_dev(void* stream, void* k_cache, void* v_cache, co
 RT_API int rt_qk_norm_rope_kv_append_bf16(void* stream, void* q, const void* k_in, const void* v_in, void* k_cache,
                                           void* v_cache, const int32_t* positions, int32_t pos, const float* q_gamma,
                                           const float* k_gamma, float eps, const float* cos_table,
-                                          const float* sin_table, int32_t table_rows, int32_t batch, int32_t n_heads,
-                                          int32_t n_kv, int32_t head_dim, int32_t max_seq, rt_err_detail* err) {
+                                          const float* sin_table, int32_t table_rows, int32_t batch, int32_t seq,
+                                          int32_t n_heads, int32_t n_kv, int32_t head_dim, int32_t max_seq,
+                                          rt_err_detail* err) {
     clear_err(err);
-    if (batch < 0 || n_heads < 0 || n_kv < 0 || head_dim < 0 || max_seq < 0 || table_rows < 0)
+    if (batch < 0 || seq < 0 || n_heads < 0 || n_kv < 0 || head_dim < 0 || max_seq < 0 || table_rows < 0)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "negative dimension");
     if ((head_dim & 1) || head_dim > 512)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 512, (uint64_t)head_dim, "head_dim must be even and <= 512");
-    if (batch > 65535 || n_heads + n_kv > 65535) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    if (batch > 65535 || seq > 65535 || n_heads + n_kv > 65535)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
     if (!positions) {
-        // the checks of RoPE::apply_inplace_half_split (rope.rs:179-184), then of KVLayerCache::append (kv_cache.rs:88-95)
-        if (pos < 0 || pos >= table_rows)
-            return fail(err, RT_ERR_ROPE_POSITION_OVERFLOW, -1, (uint64_t)table_rows, (uint64_t)((int64_t)pos + 1),
-                        "position outside the RoPE tables");
-        if (pos >= max_seq)
-            return fail(err, RT_ERR_KV_OVERFLOW, -1, (uint64_t)max_seq, (uint64_t)((int64_t)pos + 1), "position outside the cache");
+        // the checks of RoPE::apply_inplace_half_split (rope.rs:179-184), then of KVLayerCache::append (kv_cache.rs:84-89)
+        if (pos < 0 || (int64_t)pos + seq > table_rows)
+            return fail(err, RT_ERR_ROPE_POSITION_OVERFLOW, -1, (uint64_t)table_rows, (uint64_t)((int64_t)pos + seq),
+                        "positions outside the RoPE tables");
+        if ((int64_t)pos + seq > max_seq)
+            return fail(err, RT_ERR_KV_OVERFLOW, -1, (uint64_t)max_seq, (uint64_t)((int64_t)pos + seq), "rows outside the cache");
     }
-    if (batch == 0 || n_heads + n_kv == 0 || head_dim == 0) return RT_OK;
+    if (batch == 0 || seq == 0 || n_heads + n_kv == 0 || head_dim == 0) return RT_OK;
     if ((n_heads > 0 && !q) || (n_kv > 0 && (!k_in || !v_in || !k_cache || !v_cache)) || !cos_table || !sin_table)
         return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
     int rc = ensure_device(err);
@@ -546,6 +548,7 @@ RT_API int rt_qk_norm_rope_kv_append_bf16(void* stream, void* q, const void* k_i
     p.eps = eps;
     p.pos = pos;
     p.batch = batch;
+    p.seq = seq;
     p.n_heads = n_heads;
     p.n_kv = n_kv;
     p.head_dim = head_dim;

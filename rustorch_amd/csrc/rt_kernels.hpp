@@ -102,21 +102,21 @@ hipError_t launch_kv_block_append(hipStream_t stream, void* k_cache, void* v_cac
 
 // Per-head q/k RMSNorm, half-split RoPE and the cache append of one decode step (prepare.hip).
 struct DecodePrepareParams {
-    uint16_t* q;              // [batch, n_heads, head_dim], rewritten in place
-    const uint16_t* k_in;     // [batch, n_kv, head_dim]
+    uint16_t* q;              // [batch, n_heads, seq, head_dim], rewritten in place
+    const uint16_t* k_in;     // [batch, n_kv, seq, head_dim]
     const uint16_t* v_in;
     uint16_t* k_cache;        // [batch, n_kv, max_seq, head_dim]
     uint16_t* v_cache;
-    const int32_t* positions; // device int32[batch], or null: `pos` for every sequence
+    const int32_t* positions; // device int32[batch] (position of a sequence's first new token), or null: `pos` for all
     const float* q_gamma;     // f32[head_dim] or null (no norm)
     const float* k_gamma;
     const float* cos_table;   // f32[table_rows, head_dim / 2]
     const float* sin_table;
     float eps;
     int pos;
-    int batch, n_heads, n_kv, head_dim, max_seq, table_rows;
+    int batch, seq, n_heads, n_kv, head_dim, max_seq, table_rows;
 };
-// head_dim even and <= 512
+// head_dim even and <= 512; seq, batch <= 65535
 hipError_t launch_decode_prepare(hipStream_t stream, const DecodePrepareParams& p);
 
 hipError_t launch_kv_append_bf16(hipStream_t stream, uint16_t* k_cache, uint16_t* v_cache, const uint16_t* k_in,

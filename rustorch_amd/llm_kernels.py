@@ -24,25 +24,27 @@ class LlmKernels:
 
     @staticmethod
     def qk_norm_rope_kv_append_bf16(stream, q, k_in, v_in, k_cache, v_cache, positions, rope, batch, n_heads, n_kv,
-                                    head_dim, max_seq, q_gamma=None, k_gamma=None, eps=1e-6):
+                                    head_dim, max_seq, q_gamma=None, k_gamma=None, eps=1e-6, seq=1):
         """Steps 2a, 2b, 3 of decode_step (crates/rustorch-llm/src/model.rs:575-636) in one launch: per-head
         RMSNorm of q and k (device f32 gammas, or None), half-split RoPE with `rope`'s tables, cache append.
-        `positions` is a device int32[batch] buffer, or an int used for every sequence (checked on the host)."""
+        `seq` new tokens per sequence ([batch, heads, seq, head_dim] buffers; 1 when decoding).  `positions` is a
+        device int32[batch] buffer (position of each sequence's first new token), or an int used for every
+        sequence (checked on the host)."""
         err = L.RtErr()
         if isinstance(positions, (int, np.integer)):
             pos_ptr, pos = None, int(positions)
             # the reference's checks, before anything touches the device (rope.rs:179-184, kv_cache.rs:88-95)
-            if pos < 0 or pos >= rope.max_seq:
-                raise PositionOverflow(rope.max_seq, pos + 1)
-            if pos >= max_seq:
-                raise Overflow(pos + 1, max_seq)
+            if pos < 0 or pos + seq > rope.max_seq:
+                raise PositionOverflow(rope.max_seq, pos + seq)
+            if pos + seq > max_seq:
+                raise Overflow(pos + seq, max_seq)
         else:
             pos_ptr, pos = dev_ptr(positions), 0
         cos, sin = rope.device_tables()
         raise_for(L.lib().rt_qk_norm_rope_kv_append_bf16(
             stream, dev_ptr(q), dev_ptr(k_in), dev_ptr(v_in), dev_ptr(k_cache), dev_ptr(v_cache), pos_ptr, pos,
             dev_ptr(q_gamma) if q_gamma is not None else None, dev_ptr(k_gamma) if k_gamma is not None else None,
-            eps, dev_ptr(cos), dev_ptr(sin), rope.max_seq, batch, n_heads, n_kv, head_dim, max_seq, C.byref(err)), err)
+            eps, dev_ptr(cos), dev_ptr(sin), rope.max_seq, batch, seq, n_heads, n_kv, head_dim, max_seq, C.byref(err)), err)
 
     @staticmethod
     def gqa_decode_online_bf16(stream, q, k_cache, v_cache, out, n_heads, n_kv, kv_len, head_dim, max_seq):

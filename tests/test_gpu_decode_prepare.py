@@ -9,13 +9,13 @@ import rustorch_amd as ra
 pytestmark = pytest.mark.gpu
 
 
-def _case(oracle, rng, b_, hq, hkv, d, lmax, positions, norms, eps=1e-6, base=10000.0, table_rows=None):
+def _case(oracle, rng, b_, hq, hkv, d, lmax, positions, norms, eps=1e-6, base=10000.0, table_rows=None, seq=1):
     rope = ra.RoPE(d, table_rows or lmax, base)
     oro = oracle.RoPE(d, table_rows or lmax, base)
     oro.cos, oro.sin = rope.cos.copy(), rope.sin.copy()  # the caller's tables are an input of the kernel
-    q = oracle.f32_to_bf16(rng.standard_normal(b_ * hq * d).astype(np.float32))
-    k = oracle.f32_to_bf16(rng.standard_normal(b_ * hkv * d).astype(np.float32))
-    v = oracle.f32_to_bf16(rng.standard_normal(b_ * hkv * d).astype(np.float32))
+    q = oracle.f32_to_bf16(rng.standard_normal(b_ * hq * seq * d).astype(np.float32))
+    k = oracle.f32_to_bf16(rng.standard_normal(b_ * hkv * seq * d).astype(np.float32))
+    v = oracle.f32_to_bf16(rng.standard_normal(b_ * hkv * seq * d).astype(np.float32))
     kc = oracle.f32_to_bf16(rng.standard_normal(b_ * hkv * lmax * d).astype(np.float32))
     vc = oracle.f32_to_bf16(rng.standard_normal(b_ * hkv * lmax * d).astype(np.float32))
     qg = (1.0 + 0.1 * rng.standard_normal(d)).astype(np.float32) if norms[0] else None
@@ -23,17 +23,18 @@ def _case(oracle, rng, b_, hq, hkv, d, lmax, positions, norms, eps=1e-6, base=10
     return rope, oro, q, k, v, kc, vc, qg, kg
 
 
-def _run(oracle, rope, oro, q, k, v, kc, vc, qg, kg, positions, b_, hq, hkv, d, lmax, eps, scalar_pos=False):
+def _run(oracle, rope, oro, q, k, v, kc, vc, qg, kg, positions, b_, hq, hkv, d, lmax, eps, scalar_pos=False, seq=1):
     K = ra.LlmKernels()
     dq, dk, dv, dkc, dvc = (ra.HipStorage.from_numpy(x) for x in (q, k, v, kc, vc))
     dqg = ra.HipStorage.from_numpy(qg) if qg is not None else None
     dkg = ra.HipStorage.from_numpy(kg) if kg is not None else None
     pos_arg = int(positions[0]) if scalar_pos else ra.HipStorage.from_numpy(np.asarray(positions, dtype=np.int32))
     K.qk_norm_rope_kv_append_bf16(None, dq, dk, dv, dkc, dvc, pos_arg, rope, b_, hq, hkv, d, lmax, q_gamma=dqg,
-                                  k_gamma=dkg, eps=eps)
+                                  k_gamma=dkg, eps=eps, seq=seq)
     ra.synchronize()
     want_kc, want_vc = kc.copy(), vc.copy()
-    want_q = oracle.decode_prepare_bf16(q, k, v, want_kc, want_vc, positions, qg, kg, eps, oro, b_, hq, hkv, d, lmax)
+    want_q = oracle.decode_prepare_bf16(q, k, v, want_kc, want_vc, positions, qg, kg, eps, oro, b_, hq, hkv, d, lmax,
+                                        seq=seq)
     got_q, got_kc, got_vc = dq.download(np.uint16), dkc.download(np.uint16), dvc.download(np.uint16)
     assert np.array_equal(got_q, want_q)
     assert np.array_equal(got_kc, want_kc)
@@ -49,6 +50,28 @@ def test_matches_oracle_bit_for_bit(oracle, norms, b_, hq, hkv, d, lmax):
     positions[-1] = lmax - 1
     rope, oro, q, k, v, kc, vc, qg, kg = _case(oracle, rng, b_, hq, hkv, d, lmax, positions, norms)
     _run(oracle, rope, oro, q, k, v, kc, vc, qg, kg, positions, b_, hq, hkv, d, lmax, 1e-6)
+
+
+@pytest.mark.parametrize("b_,hq,hkv,d,lmax,seq", [(2, 3, 1, 16, 24, 5), (2, 8, 2, 128, 700, 300), (1, 4, 4, 64, 64, 64)])
+def test_several_new_tokens_match_oracle_bit_for_bit(oracle, b_, hq, hkv, d, lmax, seq):
+    """A prompt: [batch, heads, seq, head_dim] inputs, token s at position p + s and cache row p + s."""
+    rng = np.random.default_rng(300 + seq)
+    positions = rng.integers(0, lmax - seq + 1, size=b_).astype(np.int32)
+    positions[-1] = lmax - seq
+    rope, oro, q, k, v, kc, vc, qg, kg = _case(oracle, rng, b_, hq, hkv, d, lmax, positions, (True, True), seq=seq)
+    _run(oracle, rope, oro, q, k, v, kc, vc, qg, kg, positions, b_, hq, hkv, d, lmax, 1e-6, seq=seq)
+
+
+def test_prompt_overflow_is_reported_for_the_last_token():
+    rope = ra.RoPE(8, 16)
+    K = ra.LlmKernels()
+    buf = ra.HipStorage(4096)
+    with pytest.raises(ra.Overflow) as e:
+        K.qk_norm_rope_kv_append_bf16(None, buf, buf, buf, buf, buf, 3, rope, 1, 1, 1, 8, 7, seq=5)
+    assert (e.value.requested, e.value.max) == (8, 7)
+    with pytest.raises(ra.PositionOverflow) as e:
+        K.qk_norm_rope_kv_append_bf16(None, buf, buf, buf, buf, buf, 12, rope, 1, 1, 1, 8, 32, seq=5)
+    assert (e.value.max_seq, e.value.requested) == (16, 17)
 
 
 def test_scalar_position_is_the_reference_call(oracle):

@@ -218,3 +218,36 @@ def test_decode_prepare_position_errors(oracle):
         oracle.decode_prepare_bf16(z, z, z, kc, vc, [16], None, None, 0.0, rope, 1, 1, 1, d, lmax)
     assert e.value.code == oracle.ERR_ROPE_POSITION_OVERFLOW
     assert not kc.any() and not vc.any()
+
+
+def test_decode_prepare_with_several_new_tokens(oracle):
+    """seq > 1 (a prompt): token s of a sequence is rotated at position p + s (rope.rs:192-193) and lands in cache
+    row p + s (kv_cache.rs:97-110); assembled here from the batched RoPE call and the f32 cache append."""
+    rng = np.random.default_rng(31)
+    b_, hq, hkv, d, lmax, seq = 2, 3, 2, 8, 16, 5
+    rope = oracle.RoPE(d, lmax, 10000.0)
+    q = oracle.f32_to_bf16(rng.standard_normal(b_ * hq * seq * d).astype(np.float32))
+    k = oracle.f32_to_bf16(rng.standard_normal(b_ * hkv * seq * d).astype(np.float32))
+    v = oracle.f32_to_bf16(rng.standard_normal(b_ * hkv * seq * d).astype(np.float32))
+    kc = oracle.f32_to_bf16(rng.standard_normal(b_ * hkv * lmax * d).astype(np.float32))
+    vc = oracle.f32_to_bf16(rng.standard_normal(b_ * hkv * lmax * d).astype(np.float32))
+    kg = (1.0 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    pos = np.array([3, 11], dtype=np.int32)
+    kc2, vc2 = kc.copy(), vc.copy()
+    got_q = oracle.decode_prepare_bf16(q, k, v, kc2, vc2, pos, None, kg, 1e-6, rope, b_, hq, hkv, d, lmax, seq=seq)
+    want_kc = oracle.bf16_to_f32(kc).reshape(b_, hkv * lmax * d).copy()
+    want_vc = oracle.bf16_to_f32(vc).reshape(b_, hkv * lmax * d).copy()
+    for b in range(b_):
+        qb = oracle.bf16_to_f32(q).reshape(b_, hq * seq * d)[b]
+        want_q = oracle.f32_to_bf16(rope.apply_half_split(qb, 1, hq, seq, int(pos[b])))
+        assert np.array_equal(got_q.reshape(b_, -1)[b], want_q)
+        kb = oracle.bf16_to_f32(k).reshape(b_, hkv * seq, d)[b]
+        kb = oracle.rms_norm_per_head(kb, kg, hkv * seq, d, 1e-6)
+        kb = oracle.bf16_to_f32(oracle.f32_to_bf16(rope.apply_half_split(kb, 1, hkv, seq, int(pos[b]))))
+        vb = oracle.bf16_to_f32(v).reshape(b_, hkv * seq * d)[b]
+        oracle.kv_cache_append(want_kc[b], want_vc[b], 1, hkv, lmax, d, int(pos[b]), seq, kb, vb)
+    assert np.array_equal(oracle.bf16_to_f32(kc2), want_kc.ravel())
+    assert np.array_equal(oracle.bf16_to_f32(vc2), want_vc.ravel())
+    with pytest.raises(oracle.OracleError) as e:  # the last token would sit at row 16 of a 16-row cache
+        oracle.decode_prepare_bf16(q, k, v, kc2, vc2, [3, 12], None, kg, 1e-6, rope, b_, hq, hkv, d, lmax, seq=seq)
+    assert e.value.code == oracle.ERR_ROPE_POSITION_OVERFLOW and (e.value.expected, e.value.got) == (16, 17)
