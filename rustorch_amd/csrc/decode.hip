@@ -427,14 +427,34 @@ __global__ __launch_bounds__(HD < 64 ? 64 : HD) void decode_merge_kernel(DecodeS
     const float* ws_o = p.ws;
     const float* ws_ml = p.ws + (size_t)p.batch * p.heads * p.n_part * HD;
     const size_t slot0 = ((size_t)b * p.heads + h) * p.n_part;
-    float m_all = neg_inf();
-    for (int k = 0; k < n_valid; k++) m_all = fmaxf(m_all, ws_ml[(slot0 + k) * 2]);
-    float m_use = (m_all == neg_inf()) ? 0.0f : m_all;
-    float acc = 0.0f, l_all = 0.0f;
-    for (int k = 0; k < n_valid; k++) {
-        float cw = __builtin_amdgcn_exp2f(ws_ml[(slot0 + k) * 2] - m_use);
-        acc += ws_o[(slot0 + k) * HD + d] * cw;
-        l_all += ws_ml[(slot0 + k) * 2 + 1] * cw;
+    // One pass over the partials, eight at a time: the loads of a group are independent of each other (a head of a
+    // long sequence has a hundred partials, and one dependent load after the other would cost more than the
+    // split kernel), and the running (m, acc, l) is rescaled once per group.
+    constexpr int kGroup = 8;
+    float m_all = neg_inf(), acc = 0.0f, l_all = 0.0f;
+    for (int k0 = 0; k0 < n_valid; k0 += kGroup) {
+        float mv[kGroup], lv[kGroup], ov[kGroup];
+#pragma unroll
+        for (int j = 0; j < kGroup; j++) {
+            const int k = min(k0 + j, n_valid - 1);  // repeats of the last partial are given weight 0 below
+            mv[j] = ws_ml[(slot0 + k) * 2];
+            lv[j] = ws_ml[(slot0 + k) * 2 + 1];
+            ov[j] = ws_o[(slot0 + k) * HD + d];
+        }
+        float m_new = m_all;
+#pragma unroll
+        for (int j = 0; j < kGroup; j++) m_new = fmaxf(m_new, mv[j]);
+        const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+        const float rescale = (m_all == neg_inf()) ? 0.0f : __builtin_amdgcn_exp2f(m_all - m_use);
+        acc *= rescale;
+        l_all *= rescale;
+#pragma unroll
+        for (int j = 0; j < kGroup; j++) {
+            const float cw = (k0 + j < n_valid) ? __builtin_amdgcn_exp2f(mv[j] - m_use) : 0.0f;
+            acc += ov[j] * cw;
+            l_all += lv[j] * cw;
+        }
+        m_all = m_new;
     }
     // kv_len == 0: no key contributes, the output row is zero (gqa.rs:261; llm_kernels.rs:456)
     float r = n_valid > 0 ? acc / l_all : 0.0f;
