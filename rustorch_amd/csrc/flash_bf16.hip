@@ -188,11 +188,29 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     const float lazy_raw = kLazyLog2 / c;  // the rescale threshold in raw-score units
 
     bool poison = false;  // a padding mask hiding the reference's whole first key tile: every row NaN
+    // The keep vector as one bit per key, a word per 32-key item, built once per workgroup (masks of up to
+    // kKeepWords * 32 keys; longer ones are read byte by byte where they are applied).  A word of ones is the
+    // common case -- padding sits at the tail -- and costs the softmax cluster nothing.
+    constexpr int kKeepWords = 2048;
+    __shared__ uint32_t keep_bits[MODE == kMaskPadding ? kKeepWords : 1];
+    const bool keep_in_lds = (MODE == kMaskPadding) && (N <= 32 * kKeepWords);
     if (MODE == kMaskPadding) {
         int lim = p.ref_bc < N ? p.ref_bc : N;
         bool any = false;
         for (int j = lane; j < lim; j += kWave) any |= (p.keep[j] != 0);
         poison = !__any(any);
+        if (keep_in_lds) {
+            for (int chunk = wave; chunk * 64 < N; chunk += NWAVES) {
+                const int j = chunk * 64 + lane;
+                // keys past the end count as kept here: they are masked by the length test
+                const unsigned long long bits = __ballot(j >= N || p.keep[j] != 0);
+                if (lane == 0) {
+                    keep_bits[2 * chunk] = (uint32_t)bits;
+                    keep_bits[2 * chunk + 1] = (uint32_t)(bits >> 32);
+                }
+            }
+            __syncthreads();
+        }
     }
 
     // ---- per-lane constants of the tile loads: instruction n of this wave fills LDS block
@@ -370,6 +388,18 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             s[i] = masked ? neg_inf() : s[i];
         }
     };
+    // the same for a padding mask held as bits: `word` covers keys kv_base .. kv_base + 31
+    auto mask_item_bits = [&](int kv_base, uint32_t word) {
+        const uint32_t mine = word >> (4 * hh);  // bit 8(i/4) + i%4 of `mine` is key 8(i/4) + 4hh + i%4
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int kr = kv_base + 8 * (i >> 2) + 4 * hh + (i & 3);
+            const uint32_t kept = 0u - ((mine >> (8 * (i >> 2) + (i & 3))) & 1u);  // all ones or zero
+            uint32_t x = (__float_as_uint(s[i]) & kept) | (0xff800000u & ~kept);
+            if (kv_base + 31 >= n_keys) x = (kr >= n_keys) ? 0xff800000u : x;
+            s[i] = __uint_as_float(x);
+        }
+    };
     // raise the running max when it pays (wave-uniform branch)
     auto update_max = [&]() {
         float m_item = max_with_other_half(max16(s));
@@ -456,7 +486,16 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         cluster_barrier();
         RT_PHASE(2);
         // ---- S
-        if (MODE == kMaskPadding || __builtin_expect(kv0 + 32 * i + 31 > mask_from, 0)) mask_item(kv0 + 32 * i);
+        if (MODE == kMaskPadding) {
+            if (keep_in_lds) {
+                const uint32_t word = __builtin_amdgcn_readfirstlane(keep_bits[(kv0 + 32 * i) >> 5]);
+                if (word != 0xffffffffu || kv0 + 32 * i + 31 >= n_keys) mask_item_bits(kv0 + 32 * i, word);
+            } else {
+                mask_item(kv0 + 32 * i);
+            }
+        } else if (__builtin_expect(kv0 + 32 * i + 31 > mask_from, 0)) {
+            mask_item(kv0 + 32 * i);
+        }
         update_max();
         exp_item();
         // P is only used by the next matrix cluster, and the compiler would sink the exponentials and
