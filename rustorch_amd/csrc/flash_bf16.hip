@@ -551,20 +551,32 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             for (int ks = 0; ks < KS; ks++) k_read_one(std::integral_constant<int, 0>{}, 0, ks);  // K(0)
         }
         cluster_barrier();
-        for (int step = 0; step < n_steps; step++) {
+        // With a causal mask the job's last key tile starts past the last row of the waves that own the upper
+        // half of the query tile: for them every score of that step would be masked.  Such a wave finishes its
+        // last live item and then only keeps the barriers company for a step (no matrix, LDS or vector work: on a
+        // part whose clock is set by power the idle wave is worth more than its cycles).
+        const bool dead_last = kCausal && n_steps > 0 && (n_steps - 1) * BC > qw + 31;
+        const int n_run = n_steps - (dead_last ? 1 : 0);
+        for (int step = 0; step < n_run; step++) {
             const int kv0 = step * BC;
             run_step(kv0, step + 1 < n_steps ? kv0 + BC : kv0, step & 1, mask_from);
             k_base ^= (uint32_t)TILE_B;  // the other stage
             v_base ^= (uint32_t)TILE_B;
         }
-        if (n_steps & 1) {  // back to stage 0 for the next job
+        // the last item's P.V
+        if (n_run > 0) {
+#pragma unroll
+            for (int j = 0; j < KS; j++) mfma_pv(j);
+        }
+        if (dead_last) {
+#pragma unroll 1
+            for (int cl = 0; cl < 2 * NITEMS; cl++) cluster_barrier();
             k_base ^= (uint32_t)TILE_B;
             v_base ^= (uint32_t)TILE_B;
         }
-        // the last item's P.V
-        if (n_steps > 0) {
-#pragma unroll
-            for (int j = 0; j < KS; j++) mfma_pv(j);
+        if (n_steps & 1) {  // back to stage 0 for the next job
+            k_base ^= (uint32_t)TILE_B;
+            v_base ^= (uint32_t)TILE_B;
         }
         cluster_barrier();
         if (grp == 0) cluster_barrier();  // the first group waits for the second to finish
