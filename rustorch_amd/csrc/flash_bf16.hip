@@ -443,10 +443,10 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     };
     static_assert(KS == 2 * DT, "one P.V matrix instruction per score matrix instruction");
 
-    // One step = one 128-key tile = four items, each a C cluster and an S cluster.  Every wave runs every
-    // item of every step of the job (an item hidden from all of a wave's rows by the causal mask is scored,
-    // masked to -inf and contributes exact zeros): all eight waves then meet the same barriers, and a wave
-    // that skipped the work would only wait there.
+    // One step = one 128-key tile = four items, each a C cluster and an S cluster.  A wave runs every item of
+    // a step it takes part in (an item hidden from all of its rows by the causal mask is scored, masked to
+    // -inf and contributes exact zeros): all eight waves then meet the same barriers.  The one exception is
+    // taken a whole step at a time, in the job loop: a last key tile that lies wholly past a wave's rows.
     auto run_item = [&](auto i_c, int kv0, int kv_next, int st, int mask_from) {
         constexpr int i = decltype(i_c)::value;
         constexpr int item_off = 32 * i * ROWB;
@@ -506,10 +506,6 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         cluster_barrier();
         RT_PHASE(9);
     };
-    // One step = one 128-key tile = four items, each a C cluster and an S cluster.  Every wave runs every
-    // item of every step of the job (an item hidden from all of a wave's rows by the causal mask is scored,
-    // masked to -inf and contributes exact zeros): all eight waves then meet the same barriers, and a wave
-    // that skipped the work would only wait there.
     auto run_step = [&](int kv0, int kv_next, int st, int mask_from) {
         static_assert(NITEMS == 4, "items per step");
         run_item(std::integral_constant<int, 0>{}, kv0, kv_next, st, mask_from);
