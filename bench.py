@@ -34,7 +34,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the dominant kernels on the bench workloads, from the rocprofv3 --pmc runs
 # summarised under profiles/ (FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB, the factors a 256 MiB copy reads).
 # Counters cannot be read from inside this process; these are the committed measurements, not live values.
-TRAFFIC_PREFILL_BYTES = (260500 * 2.0 + 131100 * 1.0) * 1024
+TRAFFIC_PREFILL_BYTES = (270900 * 2.0 + 131100 * 1.0) * 1024
 TRAFFIC_DECODE_BYTES = (623700 * 2.0 + 3224 * 1.0) * 1024
 
 
