@@ -89,3 +89,60 @@ def test_no_device_is_reported_not_hidden():
     with pytest.raises(ra.DeviceError) as ei:
         ra.flash_forward(shape, z, z, z)
     assert ei.value.status == L.RT_ERR_NO_DEVICE
+
+
+def test_bf16_prefill_argument_errors_before_any_device_use():
+    """Unsupported head dim, misaligned tensors and rows beyond 32-bit offsets are refused by the host checks."""
+    import ctypes as C
+    lib = L.lib()
+
+    def call(fn, b, h, n, d, q=0x1000, k=0x2000, v=0x3000, o=0x4000):
+        err = L.RtErr()
+        s = ra.AttentionShape.new(b, h, n, d)._c()
+        return fn(None, C.byref(s), 0, q, k, v, 1, None, o, C.byref(err)), err
+
+    rc, err = call(lib.rt_flash_forward_bf16_dev, 1, 1, 8, 96)
+    assert rc == L.RT_ERR_UNSUPPORTED and b"64 and 128" in err.message
+    rc, err = call(lib.rt_flash_forward_bf16_dev, 1, 1, 8, 128, q=0x1008)
+    assert rc == L.RT_ERR_UNSUPPORTED and b"aligned" in err.message
+    rc, err = call(lib.rt_flash_forward_bf16_dev, 1, 1, 1 << 24, 128)  # 2^24 rows x 256 B = 4 GiB
+    assert rc == L.RT_ERR_UNSUPPORTED and b"4 GiB" in err.message
+    rc, err = call(lib.rt_flash_forward_bnhd_bf16_dev, 1, 64, 1 << 18, 128)  # row pitch 16 KiB in [B,N,H,D]
+    assert rc == L.RT_ERR_UNSUPPORTED and b"4 GiB" in err.message
+    rc, err = call(lib.rt_flash_forward_bf16_dev, 1, 1, 8, 0)
+    assert rc == L.RT_ERR_ZERO_DIM
+    rc, err = call(lib.rt_flash_forward_bf16_dev, 1, 1, 0, 128, q=None)  # seq == 0: Ok, nothing touched
+    assert rc == L.RT_OK
+
+
+def test_prepare_and_cache_argument_errors_before_any_device_use():
+    import ctypes as C
+    lib = L.lib()
+    err = L.RtErr()
+    p = 0x1000  # never dereferenced: every call below fails (or returns) in the host checks
+
+    def prepare(pos, table_rows, batch, seq, hq, hkv, d, max_seq, positions=None):
+        return lib.rt_qk_norm_rope_kv_append_bf16(None, p, p, p, p, p, positions, pos, None, None, 1e-6, p, p,
+                                                  table_rows, batch, seq, hq, hkv, d, max_seq, C.byref(err))
+
+    assert prepare(16, 16, 1, 1, 1, 1, 8, 32) == L.RT_ERR_ROPE_POSITION_OVERFLOW and (err.expected, err.got) == (16, 17)
+    assert prepare(12, 16, 1, 5, 1, 1, 8, 32) == L.RT_ERR_ROPE_POSITION_OVERFLOW and (err.expected, err.got) == (16, 17)
+    assert prepare(4, 16, 1, 1, 1, 1, 8, 4) == L.RT_ERR_KV_OVERFLOW and (err.expected, err.got) == (4, 5)
+    assert prepare(-1, 16, 1, 1, 1, 1, 8, 4) == L.RT_ERR_ROPE_POSITION_OVERFLOW
+    assert prepare(0, 16, 1, 1, 1, 1, 7, 4) == L.RT_ERR_UNSUPPORTED
+    assert prepare(0, 16, 1, 1, 1, 1, 514, 4) == L.RT_ERR_UNSUPPORTED
+    assert prepare(0, 16, 0, 1, 1, 1, 8, 4) == L.RT_OK  # empty batch
+    assert prepare(0, 16, 1, 0, 1, 1, 8, 4) == L.RT_OK  # no new token
+
+    def append(cur, add, nk, nv, elem=2, batch=1, heads=2, max_seq=8, d=4):
+        return lib.rt_kv_cache_append_dev(None, p, p, p, nk, p, nv, batch, heads, max_seq, d, cur, add, elem, C.byref(err))
+
+    assert append(7, 2, 16, 16) == L.RT_ERR_KV_OVERFLOW and (err.expected, err.got) == (8, 9)
+    assert append(0, 2, 15, 16) == L.RT_ERR_KV_WRONG_INPUT_LEN and (err.expected, err.got, err.got2) == (16, 15, 16)
+    assert append(7, 2, 15, 16) == L.RT_ERR_KV_OVERFLOW  # the overflow is checked first (kv_cache.rs:84-97)
+    assert append(0, 2, 16, 16, elem=3) == L.RT_ERR_UNSUPPORTED
+    assert append(0, 0, 0, 0) == L.RT_OK
+    assert lib.rt_buf_zero(None, 0, None, C.byref(err)) == L.RT_OK
+    assert lib.rt_buf_zero(None, 16, None, C.byref(err)) == L.RT_ERR_NULL_POINTER
+    assert lib.rt_buf_zero(p, 6, None, C.byref(err)) == L.RT_ERR_UNSUPPORTED
+    assert L.status_name(L.RT_ERR_ROPE_POSITION_OVERFLOW) == "PositionOverflow"
