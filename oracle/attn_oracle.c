@@ -36,6 +36,11 @@
  * reference's own flash-vs-naive tolerance (1e-4), the closed forms and the
  * edge/NaN rules (see tests/test_oracle_*.py).
  *
+ * Also "parity unpinned": the last bit of powf / cosf / sinf in
+ * ro_rope_tables (this file uses the C library's; the reference Rust's
+ * std).  One ulp of theta is 5e-4 rad at position 8192.  The tables are an
+ * input of everything downstream, which is pinned given the tables.
+ *
  * Built with -ffp-contract=off so that mul and add stay separate roundings,
  * as in the reference's scalar Rust loops.
  */
