@@ -1,0 +1,109 @@
+"""Randomised parity sweep through the C ABI: shapes, masks, layouts and head groupings drawn from a seed, every
+case compared with the oracle (f32 max-abs <= 1e-5, bf16 <= 2e-2, NaN patterns exact).  Sizes are kept small so
+that the oracle answers in milliseconds; the full-size cases live in the other GPU test files."""
+import numpy as np
+import pytest
+
+import rustorch_amd as ra
+
+pytestmark = pytest.mark.gpu
+
+
+def _bf(oracle, x):
+    return oracle.f32_to_bf16(np.asarray(x, dtype=np.float32))
+
+
+def _compare(name, got, want, tol):
+    assert np.array_equal(np.isnan(got), np.isnan(want)), f"{name}: NaN pattern differs"
+    if np.isfinite(want).any():
+        err = float(np.nanmax(np.abs(got - want)))
+        assert err <= tol, f"{name}: max-abs {err} > {tol}"
+
+
+def _mask(rng, n):
+    kind = int(rng.integers(0, 3))
+    if kind == 0:
+        return ra.Mask.none(), None, None
+    if kind == 1:
+        return ra.Mask.causal(), "causal", None
+    keep = rng.random(n) > 0.3
+    keep[int(rng.integers(0, n))] = True
+    return ra.Mask.padding(keep), ("padding", keep), keep
+
+
+def _bf16_prefill(oracle, rng):
+    b, hkv, g = int(rng.integers(1, 4)), int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 4]))
+    h, n, d = hkv * g, int(rng.choice([1, 31, 64, 127, 128, 129, 255, 256, 257, 300, 511, 640, 777])), int(rng.choice([64, 128]))
+    bnhd = bool(rng.integers(0, 2))
+    qb = _bf(oracle, rng.standard_normal(b * h * n * d) * rng.choice([1.0, 2.0]))
+    kb, vb = _bf(oracle, rng.standard_normal(b * hkv * n * d)), _bf(oracle, rng.standard_normal(b * hkv * n * d))
+    m, om, keep = _mask(rng, n)
+    kf = np.repeat(oracle.bf16_to_f32(kb).reshape(b, hkv, n, d), g, axis=1).ravel()
+    vf = np.repeat(oracle.bf16_to_f32(vb).reshape(b, hkv, n, d), g, axis=1).ravel()
+    want = oracle.flash_forward_masked(oracle.AttentionShape(b, h, n, d), oracle.bf16_to_f32(qb), kf, vf, om)
+    if bnhd:
+        def tr(x, hh):
+            return np.ascontiguousarray(x.reshape(b, hh, n, d).transpose(0, 2, 1, 3)).ravel()
+        qb, kb, vb = tr(qb, h), tr(kb, hkv), tr(vb, hkv)
+    dq, dk, dv = (ra.HipStorage.from_numpy(x) for x in (qb, kb, vb))
+    do = ra.HipStorage(b * h * n * d * 2)
+    kd = ra.HipStorage.from_numpy(keep.astype(np.uint8)) if keep is not None else None
+    fn = ra.flash_forward_bnhd_bf16_dev if bnhd else ra.flash_forward_bf16_dev
+    fn(ra.AttentionShape.new(b, h, n, d), dq, dk, dv, do, m, keep_dev=kd, n_kv_heads=hkv)
+    ra.synchronize()
+    got = oracle.bf16_to_f32(do.download(np.uint16))
+    if bnhd:
+        got = got.reshape(b, n, h, d).transpose(0, 2, 1, 3).ravel()
+    _compare(f"bf16 prefill B{b} H{h}/{hkv} N{n} D{d} {m.kind} bnhd={bnhd}", got, want, 2e-2)
+
+
+def _f32_prefill(oracle, rng):
+    b, h = int(rng.integers(1, 3)), int(rng.integers(1, 4))
+    n, d = int(rng.choice([1, 5, 33, 64, 65, 100, 129, 200])), int(rng.choice([4, 8, 24, 32, 40, 64, 96, 128]))
+    q, k, v = (rng.standard_normal(b * h * n * d).astype(np.float32) for _ in range(3))
+    m, om, _ = _mask(rng, n)
+    got = ra.flash_forward_masked(ra.AttentionShape.new(b, h, n, d), q, k, v, m)
+    want = oracle.flash_forward_masked(oracle.AttentionShape(b, h, n, d), q, k, v, om)
+    _compare(f"f32 prefill B{b} H{h} N{n} D{d} {m.kind}", got, want, 1e-5)
+
+
+def _decode(oracle, rng):
+    b, hkv, g = int(rng.integers(1, 9)), int(rng.choice([1, 2, 8])), int(rng.choice([1, 2, 4, 8]))
+    hq, d, lmax = hkv * g, int(rng.choice([64, 128])), int(rng.choice([16, 100, 257, 1024]))
+    lens = rng.integers(0, lmax + 1, size=b).astype(np.int32)
+    kc, vc = _bf(oracle, rng.standard_normal(b * hkv * lmax * d)), _bf(oracle, rng.standard_normal(b * hkv * lmax * d))
+    q = _bf(oracle, rng.standard_normal(b * hq * d))
+    K = ra.LlmKernels()
+    dq, dk, dv, dl = (ra.HipStorage.from_numpy(x) for x in (q, kc, vc, lens))
+    do = ra.HipStorage(b * hq * d * 2)
+    ws = ra.HipStorage(max(K.gqa_decode_workspace_bytes(b, hq, hkv, d, lmax), 256))
+    K.gqa_decode_batched_bf16(None, dq, dk, dv, do, dl, b, hq, hkv, d, lmax, ws, ws.byte_len)
+    ra.synchronize()
+    want = oracle.gqa_decode_batched_bf16(q, kc, vc, lens, b, hq, hkv, d, lmax)
+    _compare(f"decode B{b} Hq{hq}/{hkv} D{d} Lmax{lmax} lens={lens.tolist()}", oracle.bf16_to_f32(do.download(np.uint16)),
+             want, 2e-2)
+
+
+def _varlen(oracle, rng):
+    b, h, n, d = int(rng.integers(1, 5)), int(rng.choice([1, 2, 4])), int(rng.choice([64, 130, 256, 300, 513])), int(rng.choice([64, 128]))
+    lens = rng.integers(1, n + 1, size=b).astype(np.int32)
+    q, k, v = (_bf(oracle, rng.standard_normal(b * h * n * d)) for _ in range(3))
+    dq, dk, dv, dl = (ra.HipStorage.from_numpy(x) for x in (q, k, v, lens))
+    do = ra.HipStorage(b * h * n * d * 2)
+    ra.flash_forward_varlen_bf16_dev(ra.AttentionShape.new(b, h, n, d), dq, dk, dv, dl, do, zero_padded_rows=True)
+    ra.synchronize()
+    want = oracle.varlen_causal_forward(oracle.bf16_to_f32(q), oracle.bf16_to_f32(k), oracle.bf16_to_f32(v), lens, b, h, n, d,
+                                        zero_padded_rows=True)
+    got = oracle.bf16_to_f32(do.download(np.uint16))
+    _compare(f"varlen B{b} H{h} N{n} D{d} lens={lens.tolist()}", got, np.asarray(want, dtype=np.float32), 2e-2)
+    # padded rows are exact zeros, not merely small
+    pad = np.concatenate([np.arange(n)[None, :] >= lens[:, None]] * 1).reshape(b, 1, n, 1)
+    assert not got.reshape(b, h, n, d)[np.broadcast_to(pad, (b, h, n, d))].any()
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13, 14])
+def test_random_cases_match_oracle(oracle, seed):
+    rng = np.random.default_rng(seed)
+    cases = (_bf16_prefill, _f32_prefill, _decode, _varlen)
+    for _ in range(60):
+        cases[int(rng.integers(0, len(cases)))](oracle, rng)
