@@ -68,7 +68,7 @@ enum rt_mask_kind {
 };
 
 /* `which` of BufferShapeMismatch / WrongInputLen. */
-enum rt_which { RT_WHICH_Q = 0, RT_WHICH_K = 1, RT_WHICH_V = 2, RT_WHICH_OUT = 3, RT_WHICH_FLASH = 4 };
+enum rt_which { RT_WHICH_Q = 0, RT_WHICH_K = 1, RT_WHICH_V = 2, RT_WHICH_OUT = 3, RT_WHICH_FLASH = 4, RT_WHICH_MASK = 5 };
 
 /* Payload of the error enums above.  May be NULL. */
 typedef struct rt_err_detail {
@@ -155,6 +155,21 @@ int rt_flash_forward_bnhd_bf16_dev(void *stream, const rt_attention_shape *shape
 int rt_flash_forward_varlen_bf16_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads,
                                      const void *q, const void *k, const void *v, const int32_t *seq_lens,
                                      int zero_padded_rows, void *out, rt_err_detail *err);
+
+/* The masked / cross-attention core of MultiHeadAttention::forward, steps 2-8 of the composed path --
+ * crates/rustorch-nn/src/attention.rs:371-399: scores = (Q.K^T) * (1/sqrt(head_dim)), + additive mask, softmax over
+ * the keys (crates/rustorch-cpu/src/kernels/softmax.rs:146-180), . V -- on the projected tensors as the module holds
+ * them: q, out [batch, t_q, heads*head_dim], k, v [batch, t_kv, heads*head_dim] (t_q != t_kv is cross-attention).
+ * `mask` is the additive bias the module adds (crates/rustorch-nn/src/masks.rs:22-80 builds them: 0 keeps, -1e4
+ * masks): NULL / mask_len 0 for none, t_q*t_kv elements for [T,T] or [1,T,T], batch*heads*t_q*t_kv for [B*H,T,T].
+ * No transposed copies are made and the score matrix is never materialised.  Checks, in order: head_dim == 0 ->
+ * RT_ERR_ZERO_DIM; q, k, v lengths -> RT_ERR_BUFFER_SHAPE_MISMATCH{which}; out length ->
+ * RT_ERR_OUTPUT_SHAPE_MISMATCH; mask length -> RT_ERR_WRONG_INPUT_LEN{which = 5 ("mask"), expected = t_q*t_kv}.
+ * t_kv == 0 gives rows of zeros (an empty softmax times an empty V, as the composed path computes it).
+ * Synchronous, host slices. */
+int rt_mha_forward_masked_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len,
+                              const float *mask, size_t mask_len, float *out, size_t out_len, size_t batch,
+                              size_t t_q, size_t t_kv, size_t heads, size_t head_dim, rt_err_detail *err);
 
 /* ---- decode, device pointers ------------------------------------------------------------------ */
 

@@ -9,8 +9,10 @@
 //   rustorch_attn::Mask             crates/rustorch-attention/src/mask.rs:26-78
 //   rustorch_attn::gqa_forward_f32, GQAError
 //                                   crates/rustorch-nn/src/gqa.rs:36-210
-//   rustorch_attn::mha_flash_forward_f32
-//                                   crates/rustorch-nn/src/attention.rs:452-495
+//   rustorch_attn::mha_flash_forward_f32, mha_forward_masked_f32
+//                                   crates/rustorch-nn/src/attention.rs:371-399, :452-495
+//   rustorch_attn::causal_mask, sliding_window_mask, bool_to_additive
+//                                   crates/rustorch-nn/src/masks.rs:22-82
 //   rustorch_attn::LlmKernels       crates/rustorch-cuda/src/llm_kernels.rs:874-958 (attention part)
 //   rustorch_attn::KVCache          crates/rustorch-nn/src/kv_cache.rs:49-256, buffers in HBM
 //   rustorch_attn::RoPE, RoPEError  crates/rustorch-nn/src/rope.rs:33-241 (tables and errors; the rotation runs on the device)
@@ -94,8 +96,8 @@ struct DeviceError : std::runtime_error {
 
 namespace detail {
 inline const char* which_name(int w) {
-    static const char* names[] = {"q", "k", "v", "out", "flash_forward"};
-    return (w >= 0 && w < 5) ? names[w] : "";
+    static const char* names[] = {"q", "k", "v", "out", "flash_forward", "mask"};
+    return (w >= 0 && w < 6) ? names[w] : "";
 }
 [[noreturn]] inline void throw_device(int rc, const rt_err_detail& e) {
     throw DeviceError(rc, e.hip_error, std::string(rt_status_name(rc)) + ": " + e.message);
@@ -242,6 +244,44 @@ inline std::vector<float> mha_flash_forward_f32(const std::vector<float>& q, con
     rt_err_detail e;
     int rc = rt_mha_flash_forward_f32(q.data(), q.size(), k.data(), k.size(), v.data(), v.size(), out.data(),
                                       out.size(), batch, seq, heads, head_dim, &e);
+    detail::check_attention(rc, e);
+    return out;
+}
+
+// Additive attention masks (crates/rustorch-nn/src/masks.rs:22-82): 0 keeps, kMaskNeg masks.
+constexpr float kMaskNeg = -1.0e4f;
+inline std::vector<float> causal_mask(size_t seq_len) {
+    std::vector<float> m(seq_len * seq_len, 0.0f);
+    for (size_t i = 0; i < seq_len; i++)
+        for (size_t j = i + 1; j < seq_len; j++) m[i * seq_len + j] = kMaskNeg;
+    return m;
+}
+inline std::vector<float> sliding_window_mask(size_t seq_len, size_t window) {
+    if (window < 1) throw std::invalid_argument("sliding_window_mask: window must be >= 1");
+    std::vector<float> m(seq_len * seq_len, kMaskNeg);
+    for (size_t i = 0; i < seq_len; i++)
+        for (size_t j = 0; j <= i; j++)
+            if (i - j < window) m[i * seq_len + j] = 0.0f;
+    return m;
+}
+inline std::vector<float> bool_to_additive(const std::vector<float>& keep) {
+    std::vector<float> m(keep.size());
+    for (size_t i = 0; i < keep.size(); i++) m[i] = keep[i] >= 0.5f ? 0.0f : kMaskNeg;
+    return m;
+}
+
+// Steps 2-8 of MultiHeadAttention::forward's composed path (attention.rs:371-399): softmax(Q.K^T/sqrt(hd) + mask).V on
+// the projected tensors q [B,t_q,H*hd], k, v [B,t_kv,H*hd]; `attn_mask` empty, t_q*t_kv or B*H*t_q*t_kv elements.
+inline std::vector<float> mha_forward_masked_f32(const std::vector<float>& q, const std::vector<float>& k,
+                                                 const std::vector<float>& v, size_t batch, size_t t_q, size_t t_kv,
+                                                 size_t heads, size_t head_dim,
+                                                 const std::vector<float>& attn_mask = std::vector<float>()) {
+    std::vector<float> out(batch * t_q * heads * head_dim);
+    rt_err_detail e;
+    int rc = rt_mha_forward_masked_f32(q.data(), q.size(), k.data(), k.size(), v.data(), v.size(),
+                                       attn_mask.empty() ? nullptr : attn_mask.data(), attn_mask.size(), out.data(),
+                                       out.size(), batch, t_q, t_kv, heads, head_dim, &e);
+    if (rc == RT_ERR_WRONG_INPUT_LEN) detail::check_gqa(rc, e);  // which = "mask"
     detail::check_attention(rc, e);
     return out;
 }

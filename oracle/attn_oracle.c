@@ -25,6 +25,11 @@
  *   ro_rms_norm_per_head      crates/rustorch-llm/src/model.rs:862-897
  *   ro_decode_prepare_bf16    crates/rustorch-llm/src/model.rs:575-636 (steps 2a, 2b, 3 of decode_step:
  *                             per-head q/k RMSNorm, half-split RoPE, cache append) on bf16 storage
+ *   ro_causal_mask, ro_sliding_window_mask, ro_bool_to_additive
+ *                             crates/rustorch-nn/src/masks.rs:22-82
+ *   ro_softmax_row            crates/rustorch-cpu/src/kernels/softmax.rs:146-180 (softmax_row_online_f32)
+ *   ro_mha_forward_masked     crates/rustorch-nn/src/attention.rs:371-399 (steps 2-8 of the composed
+ *                             MultiHeadAttention path: bmm, scale, additive mask, softmax, bmm)
  *   ro_f32_to_bf16            half 2.7.1 bf16::from_f32 (round to nearest even),
  *                             the rule crates/rustorch-amp/src/bf16_kernels.rs:266-267 uses
  *
@@ -775,4 +780,84 @@ RO_EXPORT int ro_decode_prepare_bf16(uint16_t *q, const uint16_t *k_in, const ui
             }
     free(row);
     return RO_OK;
+}
+
+
+/* ---- MultiHeadAttention's composed path: additive masks, row softmax, the two batched products ---------------- */
+
+#define RO_MASK_NEG (-1.0e4f) /* masks.rs:22 */
+
+/* causal_mask (masks.rs:30-40) */
+RO_EXPORT void ro_causal_mask(size_t seq_len, float *out) {
+    for (size_t i = 0; i < seq_len; i++)
+        for (size_t j = 0; j < seq_len; j++) out[i * seq_len + j] = (j > i) ? RO_MASK_NEG : 0.0f;
+}
+
+/* sliding_window_mask (masks.rs:52-65); window >= 1 is the caller's to guarantee (an assert there) */
+RO_EXPORT void ro_sliding_window_mask(size_t seq_len, size_t window, float *out) {
+    for (size_t i = 0; i < seq_len; i++)
+        for (size_t j = 0; j < seq_len; j++) {
+            int inside_causal = j <= i;
+            size_t back = i >= j ? i - j : 0; /* saturating_sub */
+            int inside_window = back < window;
+            out[i * seq_len + j] = (inside_causal && inside_window) ? 0.0f : RO_MASK_NEG;
+        }
+}
+
+/* bool_to_additive (masks.rs:73-82) */
+RO_EXPORT void ro_bool_to_additive(const float *mask, float *out, size_t n) {
+    for (size_t i = 0; i < n; i++) out[i] = (mask[i] >= 0.5f) ? 0.0f : RO_MASK_NEG;
+}
+
+/* softmax_row_online_f32 (softmax.rs:146-180), the non-log form */
+RO_EXPORT void ro_softmax_row(const float *row_in, float *row_out, size_t n) {
+    if (n == 0) return;
+    float mx = -INFINITY, sum = 0.0f;
+    for (size_t i = 0; i < n; i++) {
+        float x = row_in[i];
+        if (x > mx) {
+            sum *= expf(mx - x);
+            mx = x;
+        }
+        sum += expf(x - mx);
+    }
+    float inv_sum = 1.0f / sum;
+    for (size_t i = 0; i < n; i++) row_out[i] = expf(row_in[i] - mx) * inv_sum;
+}
+
+/* Steps 2-8 of MultiHeadAttention::forward's composed path (attention.rs:371-399) on the projected tensors
+ * q [batch, t_q, heads*hd], k, v [batch, t_kv, heads*hd]: per (b, h) raw = Q.K^T (the two bmm calls go to the `gemm`
+ * crate, restated as ascending-order f32 sums), scores = raw * (1/sqrt(hd)), + mask (broadcast over the leading
+ * batch*heads axis when mask_bh_stride == 0), softmax over the last axis, context = attn.V, heads merged back.
+ * mask may be NULL. */
+RO_EXPORT void ro_mha_forward_masked(const float *q, const float *k, const float *v, const float *mask,
+                                     size_t mask_bh_stride, float *out, size_t batch, size_t t_q, size_t t_kv,
+                                     size_t heads, size_t hd) {
+    const size_t e = heads * hd;
+    const float inv_scale = 1.0f / sqrtf((float)hd);
+    float *scores = (float *)malloc((t_kv ? t_kv : 1) * sizeof(float));
+    float *attn = (float *)malloc((t_kv ? t_kv : 1) * sizeof(float));
+    for (size_t b = 0; b < batch; b++)
+        for (size_t h = 0; h < heads; h++)
+            for (size_t i = 0; i < t_q; i++) {
+                const float *qr = q + (b * t_q + i) * e + h * hd;
+                const float *mrow = mask ? mask + (b * heads + h) * mask_bh_stride + i * t_kv : NULL;
+                for (size_t j = 0; j < t_kv; j++) {
+                    const float *kr = k + (b * t_kv + j) * e + h * hd;
+                    float dot = 0.0f;
+                    for (size_t d = 0; d < hd; d++) dot += qr[d] * kr[d];
+                    float s = dot * inv_scale;
+                    if (mrow) s = s + mrow[j];
+                    scores[j] = s;
+                }
+                ro_softmax_row(scores, attn, t_kv);
+                float *o = out + (b * t_q + i) * e + h * hd;
+                for (size_t d = 0; d < hd; d++) {
+                    float acc = 0.0f;
+                    for (size_t j = 0; j < t_kv; j++) acc += attn[j] * v[(b * t_kv + j) * e + h * hd + d];
+                    o[d] = acc;
+                }
+            }
+    free(scores);
+    free(attn);
 }

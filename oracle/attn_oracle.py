@@ -113,6 +113,16 @@ def lib():
         L.ro_osm_full.argtypes = [fp, sz, C.POINTER(_Osm)]
         L.ro_osm_full.restype = None
         L.ro_max_threads.restype = C.c_int
+        L.ro_causal_mask.argtypes = [sz, fp]
+        L.ro_causal_mask.restype = None
+        L.ro_sliding_window_mask.argtypes = [sz, sz, fp]
+        L.ro_sliding_window_mask.restype = None
+        L.ro_bool_to_additive.argtypes = [fp, fp, sz]
+        L.ro_bool_to_additive.restype = None
+        L.ro_softmax_row.argtypes = [fp, fp, sz]
+        L.ro_softmax_row.restype = None
+        L.ro_mha_forward_masked.argtypes = [fp, fp, fp, fp, sz, fp, sz, sz, sz, sz, sz]
+        L.ro_mha_forward_masked.restype = None
         L.ro_rope_tables.argtypes = [C.c_int, C.c_int, C.c_float, fp, fp]
         L.ro_rope_tables.restype = None
         rope_args = [fp, sz, sz, sz, sz, sz, sz, fp, fp, sz, C.POINTER(_Err)]
@@ -427,6 +437,58 @@ def decode_prepare_bf16(q, k_in, v_in, k_cache, v_cache, positions, q_gamma, k_g
                                       n_kv, head_dim, max_seq, rope.max_seq, C.byref(err))
     _raise(rc, err)
     return q
+
+
+MASK_NEG = np.float32(-1.0e4)
+
+
+def causal_mask(seq_len):
+    """masks.rs:30-40."""
+    out = np.zeros(seq_len * seq_len, dtype=np.float32)
+    lib().ro_causal_mask(seq_len, out.ctypes.data_as(C.POINTER(C.c_float)))
+    return out.reshape(seq_len, seq_len)
+
+
+def sliding_window_mask(seq_len, window):
+    """masks.rs:52-65."""
+    assert window >= 1
+    out = np.zeros(seq_len * seq_len, dtype=np.float32)
+    lib().ro_sliding_window_mask(seq_len, window, out.ctypes.data_as(C.POINTER(C.c_float)))
+    return out.reshape(seq_len, seq_len)
+
+
+def bool_to_additive(mask):
+    """masks.rs:73-82."""
+    m, mp = _f32(np.asarray(mask, dtype=np.float32))
+    out = np.zeros(m.size, dtype=np.float32)
+    lib().ro_bool_to_additive(mp, out.ctypes.data_as(C.POINTER(C.c_float)), m.size)
+    return out.reshape(m.shape)
+
+
+def softmax_row(x):
+    """softmax_row_online_f32 (crates/rustorch-cpu/src/kernels/softmax.rs:146-180)."""
+    x, xp = _f32(np.ravel(x))
+    out = np.zeros(x.size, dtype=np.float32)
+    lib().ro_softmax_row(xp, out.ctypes.data_as(C.POINTER(C.c_float)), x.size)
+    return out
+
+
+def mha_forward_masked(q, k, v, batch, t_q, t_kv, heads, head_dim, attn_mask=None):
+    """Steps 2-8 of the composed MultiHeadAttention path (attention.rs:371-399); q [B,t_q,H*hd], k, v [B,t_kv,H*hd];
+    attn_mask None, t_q*t_kv elements, or B*H*t_q*t_kv elements.  Returns flat float32 [B,t_q,H*hd]."""
+    q, qp = _f32(np.ravel(q))
+    k, kp = _f32(np.ravel(k))
+    v, vp = _f32(np.ravel(v))
+    assert q.size == batch * t_q * heads * head_dim and k.size == v.size == batch * t_kv * heads * head_dim
+    mp, stride = None, 0
+    if attn_mask is not None:
+        m, mp = _f32(np.ravel(attn_mask))
+        assert m.size in (t_q * t_kv, batch * heads * t_q * t_kv)
+        stride = t_q * t_kv if (m.size == batch * heads * t_q * t_kv and batch * heads > 1) else 0
+    out = np.zeros(q.size, dtype=np.float32)
+    lib().ro_mha_forward_masked(qp, kp, vp, mp, stride, out.ctypes.data_as(C.POINTER(C.c_float)), batch, t_q, t_kv,
+                                heads, head_dim)
+    return out
 
 
 def max_threads() -> int:

@@ -7,7 +7,7 @@ no CPU fallback.
 from . import _lib
 from .attention import (AttentionShape, Mask, flash_forward, flash_forward_bf16_dev, flash_forward_bnhd_bf16_dev,
                         flash_forward_bnhd_f32_dev, flash_forward_f32_dev, flash_forward_masked,
-                        flash_forward_varlen_bf16_dev, mha_flash_forward_f32)
+                        flash_forward_varlen_bf16_dev, mha_flash_forward_f32, mha_forward_masked_f32)
 from .device import HipStorage, init, synchronize
 from .errors import (AttentionError, BufferShapeMismatch, DeviceError, GQAError, HeadCountMismatch, KVCacheError,
                      KVWrongInputLen, LayerOutOfRange,
@@ -16,6 +16,7 @@ from .errors import (AttentionError, BufferShapeMismatch, DeviceError, GQAError,
 from .gqa import gqa_forward_f32
 from .kv_cache import KVCache
 from .llm_kernels import LlmKernels
+from .masks import MASK_NEG, bool_to_additive, causal_mask, sliding_window_mask
 from .rope import RoPE
 
 __all__ = [n for n in dir() if not n.startswith("_")]

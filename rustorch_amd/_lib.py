@@ -16,7 +16,7 @@ SYMBOLS = (
     "rt_init", "rt_version", "rt_status_name",
     "rt_flash_forward_f32", "rt_flash_forward_masked_f32", "rt_gqa_forward_f32",
     "rt_flash_forward_f32_dev", "rt_flash_forward_bf16_dev", "rt_flash_forward_varlen_bf16_dev",
-    "rt_mha_flash_forward_f32", "rt_flash_forward_bnhd_f32_dev", "rt_flash_forward_bnhd_bf16_dev",
+    "rt_mha_flash_forward_f32", "rt_mha_forward_masked_f32", "rt_flash_forward_bnhd_f32_dev", "rt_flash_forward_bnhd_bf16_dev",
     "rt_kv_append_bf16", "rt_kv_cache_append_dev", "rt_qk_norm_rope_kv_append_bf16", "rt_gqa_decode_online_bf16", "rt_gqa_decode_batched_bf16",
     "rt_gqa_decode_workspace_bytes",
     "rt_buf_alloc", "rt_buf_free", "rt_buf_zero", "rt_memcpy_h2d", "rt_memcpy_d2h", "rt_stream_synchronize",
@@ -40,7 +40,7 @@ RT_ERR_NO_DEVICE = 30
 RT_ERR_HIP = 31
 
 RT_MASK_NONE, RT_MASK_CAUSAL, RT_MASK_PADDING = 0, 1, 2
-WHICH = {0: "q", 1: "k", 2: "v", 3: "out", 4: "flash_forward", -1: ""}
+WHICH = {0: "q", 1: "k", 2: "v", 3: "out", 4: "flash_forward", 5: "mask", -1: ""}
 
 
 class RtShape(C.Structure):
@@ -83,6 +83,7 @@ def lib():
     L.rt_flash_forward_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_flash_forward_varlen_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, i32p, C.c_int, vp, errp]
     L.rt_mha_flash_forward_f32.argtypes = [fp, sz, fp, sz, fp, sz, fp, sz, sz, sz, sz, sz, errp]
+    L.rt_mha_forward_masked_f32.argtypes = [fp, sz, fp, sz, fp, sz, fp, sz, fp, sz, sz, sz, sz, sz, sz, errp]
     L.rt_flash_forward_bnhd_f32_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_flash_forward_bnhd_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_kv_append_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, errp]

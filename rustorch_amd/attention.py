@@ -152,6 +152,28 @@ def mha_flash_forward_f32(q, k, v, batch: int, seq: int, heads: int, head_dim: i
     return out
 
 
+def mha_forward_masked_f32(q, k, v, batch: int, t_q: int, t_kv: int, heads: int, head_dim: int, attn_mask=None,
+                           out=None):
+    """Steps 2-8 of `MultiHeadAttention::forward`'s composed path (crates/rustorch-nn/src/attention.rs:371-399):
+    softmax((Q.K^T)/sqrt(hd) + attn_mask).V per (batch, head) on the projected tensors q [B,t_q,H*hd], k, v
+    [B,t_kv,H*hd] (flat f32; t_q != t_kv is cross-attention).  `attn_mask` is an additive f32 bias with t_q*t_kv
+    ([T,T] / [1,T,T]) or B*H*t_q*t_kv ([B*H,T,T]) elements, e.g. from `masks.causal_mask`, or None.  Returns flat
+    f32 [B,t_q,H*hd]."""
+    q, qp = _f32(q)
+    k, kp = _f32(k)
+    v, vp = _f32(v)
+    m, mp = (None, None) if attn_mask is None else _f32(np.ravel(attn_mask))
+    if out is None:
+        out = np.zeros(batch * t_q * heads * head_dim, dtype=np.float32)
+    assert out.dtype == np.float32 and out.flags.c_contiguous
+    err = L.RtErr()
+    rc = L.lib().rt_mha_forward_masked_f32(qp, q.size, kp, k.size, vp, v.size, mp, 0 if m is None else m.size,
+                                           out.ctypes.data_as(C.POINTER(C.c_float)), out.size, batch, t_q, t_kv, heads,
+                                           head_dim, C.byref(err))
+    raise_for(rc, err)
+    return out
+
+
 def flash_forward_bnhd_f32_dev(shape, q, k, v, out, mask: Mask = None, keep_dev=None, n_kv_heads=0, stream=None):
     """f32 [B,N,H,D] device tensors (k, v: [B,N,Hkv,D]); `shape` is still (batch, heads, seq, dim)."""
     mask = mask or Mask.none()

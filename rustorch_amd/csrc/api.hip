@@ -292,7 +292,7 @@ RT_API int rt_gqa_forward_f32(const float* q, size_t q_len, const float* k, size
     } else {
         if (head_dim > 512) return fail(err, RT_ERR_UNSUPPORTED, -1, 512, head_dim, "decode rows kernel covers dim <= 512");
         if (seq_q > 65535 * 32ull) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, seq_q, "seq_q too large");
-        rt::AttnRowsParams p;
+        rt::AttnRowsParams p{};
         p.q = dq.p;
         p.k = dk.p;
         p.v = dv.p;
@@ -458,6 +458,68 @@ RT_API int rt_mha_flash_forward_f32(const float* q, size_t q_len, const float* k
     return RT_OK;
 }
 
+RT_API int rt_mha_forward_masked_f32(const float* q, size_t q_len, const float* k, size_t k_len, const float* v,
+                                     size_t v_len, const float* mask, size_t mask_len, float* out, size_t out_len,
+                                     size_t batch, size_t t_q, size_t t_kv, size_t heads, size_t head_dim,
+                                     rt_err_detail* err) {
+    clear_err(err);
+    if (head_dim == 0) return fail(err, RT_ERR_ZERO_DIM, -1, 0, 0, "dim must be > 0");
+    const size_t embed = heads * head_dim;
+    const size_t q_expected = batch * t_q * embed, kv_expected = batch * t_kv * embed;
+    if (q_len != q_expected) return fail(err, RT_ERR_BUFFER_SHAPE_MISMATCH, RT_WHICH_Q, q_expected, q_len, "q length");
+    if (k_len != kv_expected) return fail(err, RT_ERR_BUFFER_SHAPE_MISMATCH, RT_WHICH_K, kv_expected, k_len, "k length");
+    if (v_len != kv_expected) return fail(err, RT_ERR_BUFFER_SHAPE_MISMATCH, RT_WHICH_V, kv_expected, v_len, "v length");
+    if (out_len != q_expected) return fail(err, RT_ERR_OUTPUT_SHAPE_MISMATCH, -1, q_expected, out_len, "out length");
+    const size_t one_mask = t_q * t_kv, all_masks = batch * heads * one_mask;
+    if (!mask) mask_len = 0;
+    if (mask_len != 0 && mask_len != one_mask && mask_len != all_masks)
+        return fail(err, RT_ERR_WRONG_INPUT_LEN, RT_WHICH_MASK, one_mask, mask_len, "mask length");
+    if (q_expected == 0) return RT_OK;
+    if (!q || !out || (kv_expected && (!k || !v))) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    if (head_dim > 512) return fail(err, RT_ERR_UNSUPPORTED, -1, 512, head_dim, "rows kernel covers dim <= 512");
+    if (heads > 65535 || batch > 65535 || t_q > 0x7fffffffull || t_kv > 0x7fffffffull || embed > 0x7fffffffull)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    int rc = ensure_device(err);
+    if (rc) return rc;
+    DevBuf dq, dk, dv, dm, dout;
+    HIP_TRY(hipMalloc(&dq.p, q_expected * 4), "hipMalloc q");
+    HIP_TRY(hipMalloc(&dout.p, q_expected * 4), "hipMalloc out");
+    HIP_TRY(hipMemcpy(dq.p, q, q_expected * 4, hipMemcpyHostToDevice), "copy q");
+    if (kv_expected) {
+        HIP_TRY(hipMalloc(&dk.p, kv_expected * 4), "hipMalloc k");
+        HIP_TRY(hipMalloc(&dv.p, kv_expected * 4), "hipMalloc v");
+        HIP_TRY(hipMemcpy(dk.p, k, kv_expected * 4, hipMemcpyHostToDevice), "copy k");
+        HIP_TRY(hipMemcpy(dv.p, v, kv_expected * 4, hipMemcpyHostToDevice), "copy v");
+    }
+    if (mask_len) {
+        HIP_TRY(hipMalloc(&dm.p, mask_len * 4), "hipMalloc mask");
+        HIP_TRY(hipMemcpy(dm.p, mask, mask_len * 4, hipMemcpyHostToDevice), "copy mask");
+    }
+    rt::AttnRowsParams p{};
+    p.q = dq.p;
+    p.k = dk.p;
+    p.v = dv.p;
+    p.out = dout.p;
+    p.kv_lens = nullptr;
+    p.batch = (int)batch;
+    p.heads = (int)heads;
+    p.kv_heads = (int)heads;
+    p.seq_q = (int)t_q;
+    p.kv_len = (int)t_kv;
+    p.kv_stride = (int)t_kv;
+    p.dim = (int)head_dim;
+    p.head_map = 0;
+    p.scale = 1.0f / sqrtf((float)head_dim);
+    p.bias = mask_len ? (const float*)dm.p : nullptr;
+    p.bias_bh_stride = (mask_len == all_masks && all_masks != one_mask) ? (long long)one_mask : 0;
+    p.use_layout = 1;
+    p.lq = p.lo = rt::layout_bnhd((long long)heads, (long long)t_q, (int)head_dim);
+    p.lkv = rt::layout_bnhd((long long)heads, (long long)t_kv, (int)head_dim);
+    HIP_TRY(rt::launch_attn_rows_f32(nullptr, p), "attn_rows_f32 launch");
+    HIP_TRY(hipMemcpy(out, dout.p, q_expected * 4, hipMemcpyDeviceToHost), "copy out");
+    return RT_OK;
+}
+
 RT_API int rt_flash_forward_varlen_bf16_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,
                                             const void* q, const void* k, const void* v, const int32_t* seq_lens,
                                             int zero_padded_rows, void* out, rt_err_detail* err) {
@@ -583,7 +645,7 @@ RT_API int rt_gqa_decode_online_bf16(void* stream, const void* q, const void* k_
     if (!q || !out || (kv_len > 0 && (!k_cache || !v_cache))) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
     rc = ensure_device(err);
     if (rc) return rc;
-    rt::AttnRowsParams p;
+    rt::AttnRowsParams p{};
     p.q = q;
     p.k = k_cache;
     p.v = v_cache;
@@ -645,7 +707,7 @@ RT_API int rt_gqa_decode_batched_bf16(void* stream, const void* q, const void* k
     }
     // shapes outside the split-K kernel: one workgroup per (sequence, head), no workspace
     if (head_dim > 512) return fail(err, RT_ERR_UNSUPPORTED, -1, 512, (uint64_t)head_dim, "decode rows kernel covers dim <= 512");
-    rt::AttnRowsParams p;
+    rt::AttnRowsParams p{};
     p.q = q;
     p.k = k_cache;
     p.v = v_cache;

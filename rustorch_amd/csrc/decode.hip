@@ -66,6 +66,17 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(AttnRowsParams p) {
     const T* __restrict__ K = (const T*)p.k + ((size_t)b * p.kv_heads + kvh) * (size_t)p.kv_stride * D;
     const T* __restrict__ V = (const T*)p.v + ((size_t)b * p.kv_heads + kvh) * (size_t)p.kv_stride * D;
     T* __restrict__ O = (T*)p.out + (((size_t)b * p.heads + h) * p.seq_q + qi) * D;
+    size_t kv_pitch = (size_t)D;  // elements between consecutive key rows
+    if (p.use_layout) {
+        Q = (const T*)p.q + (size_t)b * p.lq.batch_stride + (size_t)h * p.lq.head_stride + (size_t)qi * p.lq.row_pitch;
+        K = (const T*)p.k + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+        V = (const T*)p.v + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+        O = (T*)p.out + (size_t)b * p.lo.batch_stride + (size_t)h * p.lo.head_stride + (size_t)qi * p.lo.row_pitch;
+        kv_pitch = (size_t)p.lkv.row_pitch;
+    }
+    // scores = (q . k) * scale, then the additive bias (crates/rustorch-nn/src/attention.rs:378-392)
+    const float* __restrict__ bias_row =
+        p.bias ? p.bias + ((size_t)b * p.heads + h) * (size_t)p.bias_bh_stride + (size_t)qi * (size_t)kv_len : nullptr;
 
     float qv[kMaxDJ], o[kMaxDJ];
 #pragma unroll
@@ -80,9 +91,10 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(AttnRowsParams p) {
 #pragma unroll
         for (int j = 0; j < kMaxDJ; j++) {
             int d = lane + 64 * j;
-            if (d < D) part += qv[j] * load_elem<T>(K, (size_t)t * D + d);
+            if (d < D) part += qv[j] * load_elem<T>(K, (size_t)t * kv_pitch + d);
         }
         float s = wave_sum(part) * p.scale;
+        if (bias_row) s += bias_row[t];
         float m_new = s > m ? s : m;
         float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
         float alpha = (m == neg_inf()) ? 0.0f : expf(m - m_use);
@@ -92,7 +104,7 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(AttnRowsParams p) {
 #pragma unroll
         for (int j = 0; j < kMaxDJ; j++) {
             int d = lane + 64 * j;
-            if (d < D) o[j] = o[j] * alpha + e * load_elem<T>(V, (size_t)t * D + d);
+            if (d < D) o[j] = o[j] * alpha + e * load_elem<T>(V, (size_t)t * kv_pitch + d);
         }
     }
     __shared__ float sm[4], sl[4];

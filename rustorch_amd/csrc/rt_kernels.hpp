@@ -73,6 +73,11 @@ struct AttnRowsParams {
     int seq_q, kv_len, kv_stride, dim;
     int head_map;  // 0: kv_h = h / (heads/kv_heads) (gqa.rs:233); 1: kv_h = h*kv_heads/heads (llm_kernels.rs:410)
     float scale;
+    // optional (zero-initialise the struct to leave them off):
+    const float* bias;         // additive score bias [seq_q, kv_len] rows, added after scaling; f32 tensors only
+    long long bias_bh_stride;  // elements between the biases of consecutive (batch, head) pairs; 0 = one bias for all
+    int use_layout;            // != 0: q/out and k/v are addressed through the layouts below instead of [B,H,S,D]
+    TensorLayout lq, lkv, lo;
 };
 hipError_t launch_attn_rows_f32(hipStream_t stream, const AttnRowsParams& p);
 hipError_t launch_attn_rows_bf16(hipStream_t stream, const AttnRowsParams& p);

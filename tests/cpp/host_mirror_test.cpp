@@ -132,6 +132,16 @@ static void test_errors() {
         CHECK(Mask::causal().is_masked(1, 2) && !Mask::causal().is_masked(2, 2));
         CHECK(Mask::padding({true, false}).is_masked(0, 1) && !Mask::padding({true, false}).is_masked(0, 0));
     }
+    {   // additive masks (masks.rs:88-208)
+        auto c = causal_mask(3);
+        CHECK(c[0] == 0 && c[1] == kMaskNeg && c[3] == 0 && c[4] == 0 && c[5] == kMaskNeg && c[8] == 0);
+        CHECK(sliding_window_mask(5, 100) == causal_mask(5));
+        auto w = sliding_window_mask(4, 1);
+        for (int i = 0; i < 4; i++)
+            for (int j = 0; j < 4; j++) CHECK((w[i * 4 + j] == 0.0f) == (i == j));
+        auto a = bool_to_additive({1.0f, 0.0f, 1.0f, 1.0f});
+        CHECK(a[0] == 0 && a[1] == kMaskNeg && a[2] == 0 && a[3] == 0);
+    }
     {   // RoPE::new: position 0 is cos 1 / sin 0, theta_0 = 1, odd head_dim refused (rope.rs:63-90)
         RoPE rope(4, 8);
         CHECK(rope.cos_table().size() == 16 && rope.cos_table()[0] == 1.0f && rope.sin_table()[1] == 0.0f);
@@ -242,6 +252,23 @@ static void test_gpu() {
         kc = dkc.to_host<uint16_t>();
         CHECK(std::fabs(fb(kc[d + 0]) - std::cos(1.0f)) < 4e-3f && std::fabs(fb(kc[d + d / 2]) - std::sin(1.0f)) < 4e-3f);
         for (int i = 1; i < d / 2; i++) CHECK(kc[d + i] == 0 && kc[d + d / 2 + i] == 0);
+    }
+    {   // masked core of MultiHeadAttention: zero q/k + causal mask gives prefix means of V; sliding window 1 gives V itself
+        size_t b = 1, t = 5, h = 2, d = 4;
+        std::vector<float> z(b * t * h * d, 0.0f), v = lcg(b * t * h * d, 13);
+        auto got = mha_forward_masked_f32(z, z, v, b, t, t, h, d, causal_mask(t));
+        for (size_t i = 0; i < t; i++)
+            for (size_t c = 0; c < h * d; c++) {
+                double mean = 0;
+                for (size_t j = 0; j <= i; j++) mean += v[j * h * d + c];
+                CHECK(std::fabs(got[i * h * d + c] - (float)(mean / (double)(i + 1))) <= 1e-5f);
+            }
+        auto diag = mha_forward_masked_f32(z, z, v, b, t, t, h, d, sliding_window_mask(t, 1));
+        for (size_t i = 0; i < v.size(); i++) CHECK(std::fabs(diag[i] - v[i]) <= 1e-6f);
+        bool threw = false;
+        try { mha_forward_masked_f32(z, z, v, b, t, t, h, d, std::vector<float>(7)); }
+        catch (const GQAError& e) { threw = e.which == "mask" && e.expected == t * t && e.got == 7; }
+        CHECK(threw);
     }
     {   // KVCache: the reference's index table (kv_cache.rs:306-322) and errors (:326-348) on device buffers
         KVCache c(1, 1, 1, 2, 4, 4);
