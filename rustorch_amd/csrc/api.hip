@@ -135,9 +135,11 @@ int check_flash_dims(const rt_attention_shape* s, uint64_t n_kv_heads, rt_err_de
 // bnhd: tensors are [batch, seq, heads, dim] instead of [batch, heads, seq, dim]
 int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n_kv_heads, const float* q,
                      const float* k, const float* v, int mask_kind, const uint8_t* keep, float* out,
-                     rt_err_detail* err, bool bnhd = false) {
+                     rt_err_detail* err, bool bnhd = false, const float* bias = nullptr, long long bias_bh_stride = 0) {
     if (s->dim > 128) return fail(err, RT_ERR_UNSUPPORTED, -1, 128, s->dim, "f32 flash kernel covers dim <= 128");
-    rt::FlashF32Params p;
+    rt::FlashF32Params p{};
+    p.bias = bias;
+    p.bias_bh_stride = bias_bh_stride;
     p.q = q;
     p.k = k;
     p.v = v;
@@ -495,6 +497,18 @@ RT_API int rt_mha_forward_masked_f32(const float* q, size_t q_len, const float* 
         HIP_TRY(hipMalloc(&dm.p, mask_len * 4), "hipMalloc mask");
         HIP_TRY(hipMemcpy(dm.p, mask, mask_len * 4, hipMemcpyHostToDevice), "copy mask");
     }
+    const long long bias_bh_stride = (mask_len == all_masks && all_masks != one_mask) ? (long long)one_mask : 0;
+    if (t_q == t_kv && head_dim % 32 == 0 && head_dim <= 128) {
+        // self-attention with a head dim the tiled f32 kernel covers: the same kernel as the unmasked path, with
+        // the mask's row added to the scaled scores
+        rt_attention_shape shape = {batch, heads, t_q, head_dim, 64, 64};
+        rc = flash_f32_device(nullptr, &shape, heads, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p,
+                              RT_MASK_NONE, nullptr, (float*)dout.p, err, true, mask_len ? (const float*)dm.p : nullptr,
+                              bias_bh_stride);
+        if (rc) return rc;
+        HIP_TRY(hipMemcpy(out, dout.p, q_expected * 4, hipMemcpyDeviceToHost), "copy out");
+        return RT_OK;
+    }
     rt::AttnRowsParams p{};
     p.q = dq.p;
     p.k = dk.p;
@@ -511,7 +525,7 @@ RT_API int rt_mha_forward_masked_f32(const float* q, size_t q_len, const float* 
     p.head_map = 0;
     p.scale = 1.0f / sqrtf((float)head_dim);
     p.bias = mask_len ? (const float*)dm.p : nullptr;
-    p.bias_bh_stride = (mask_len == all_masks && all_masks != one_mask) ? (long long)one_mask : 0;
+    p.bias_bh_stride = bias_bh_stride;
     p.use_layout = 1;
     p.lq = p.lo = rt::layout_bnhd((long long)heads, (long long)t_q, (int)head_dim);
     p.lkv = rt::layout_bnhd((long long)heads, (long long)t_kv, (int)head_dim);

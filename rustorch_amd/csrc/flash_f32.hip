@@ -235,6 +235,11 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
     int kv_end = N;
     if (p.mask == kMaskCausal) kv_end = min(N, q0 + kRows);
     const int n_tiles = (kv_end + kRows - 1) / kRows;
+    // additive bias row of this lane's query (MultiHeadAttention's attn_mask, added to the scaled scores)
+    const float* __restrict__ bias_row = nullptr;
+    if (p.bias && q_row < N)
+        bias_row = p.bias + ((size_t)b * p.heads + h) * (size_t)p.bias_bh_stride + (size_t)q_row * (size_t)N;
+    const bool bias_vec = ((N & 3) == 0) && ((((uintptr_t)p.bias) & 15) == 0) && ((p.bias_bh_stride & 3) == 0);
 
     // lane's chunks of a tile: load n covers row (64n + lane) / CH, chunk (64n + lane) % CH.  When CH divides 64
     // that is row n * (64/CH) + lane / CH, chunk lane % CH: one per-lane offset, everything else is uniform.
@@ -292,9 +297,27 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
         // register i of the accumulator holds key row 8*(i/4) + 4*hh + (i%4), query row `col`
         float m_tile = neg_inf();
         const bool edge = (kv0 + kRows > N) || (p.mask == kMaskCausal && kv0 + kRows - 1 > q0) || (p.mask == kMaskPadding);
+        f32x16_t bias;
+#pragma unroll
+        for (int i = 0; i < 16; i++) bias[i] = 0.0f;
+        if (bias_row) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int kr0 = kv0 + 8 * g + 4 * hh;
+                if (bias_vec && kr0 + 3 < N) {
+                    const f32x4_t bv = *(const f32x4_t*)(bias_row + kr0);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) bias[4 * g + r] = bv[r];
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (kr0 + r < N) bias[4 * g + r] = bias_row[kr0 + r];
+                }
+            }
+        }
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            float x = s[i] * p.scale;
+            float x = s[i] * p.scale + bias[i];
             if (edge) {
                 int kr = kv0 + 8 * (i >> 2) + 4 * hh + (i & 3);
                 bool masked = kr >= N;
@@ -422,6 +445,7 @@ hipError_t launch_flash_f32(hipStream_t stream, const FlashF32Params& p) {
         }
         return hipGetLastError();
     }
+    if (p.bias) return hipErrorInvalidValue;  // only the tiled kernel above adds a bias
     switch (dt) {
         case 1: hipLaunchKernelGGL(flash_fwd_f32_kernel<1>, grid, block, 0, stream, p); break;
         case 2: hipLaunchKernelGGL(flash_fwd_f32_kernel<2>, grid, block, 0, stream, p); break;

@@ -38,6 +38,9 @@ struct FlashF32Params {
     TensorLayout lq, lkv, lo;  // layouts of q, of k and v, of out
     int n_cus;   // CUs of the device (0: unknown)
     int zigzag;  // set by the launcher
+    // optional additive score bias, rows of `seq` f32 per query row, added after scaling (zero-initialise to leave off)
+    const float* bias;
+    long long bias_bh_stride;  // elements between the biases of consecutive (batch, head) pairs; 0 = one for all
 };
 // dim <= 128.  Returns hipErrorInvalidValue for an unsupported dim.
 hipError_t launch_flash_f32(hipStream_t stream, const FlashF32Params& p);
