@@ -4,9 +4,10 @@
 A step is one pass of the bf16 causal prefill kernel over the headline workload
 B=4, H=32, N=4096, D=128 (inputs resident in HBM before the timed region); the same run also
 times the batched GQA decode workload (batch 64, 32 query / 8 kv heads, D=128, context lengths
-uniform in [512, 8192], Lmax 8192) and reports it under "decode".
+uniform in [512, 8192], Lmax 8192) and reports it under "decode", and the f32 causal prefill of
+B=1, H=8, N=2048, D=64 (the reference's own CPU-runnable case) under "f32_prefill".
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only prefill|decode|f32]
 
 Prints ONE JSON line.  `value` is prefill TFLOP/s with causal-counted FLOPs
 (4*B*H*D*N*(N+1)/2: skipped tiles are not credited); `roofline` prices it against the dense bf16
@@ -31,6 +32,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+PEAK_F32_TFLOPS = 157.3     # MI355X dense f32 MFMA
 # HBM bytes per launch of the dominant kernels on the bench workloads, from the rocprofv3 --pmc runs
 # summarised under profiles/ (FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB, the factors a 256 MiB copy reads).
 # Counters cannot be read from inside this process; these are the committed measurements, not live values.
@@ -146,7 +148,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity sample")
-    ap.add_argument("--only", choices=["prefill", "decode"], default=None)
+    ap.add_argument("--only", choices=["prefill", "decode", "f32"], default=None)
     ap.add_argument("--no-ceiling", action="store_true",
                     help="skip the run of rustorch_amd/lib/mfma_sustained (what a loop of nothing but bf16 MFMA "
                          "sustains on this GPU, reported beside the data-sheet peak)")
@@ -280,6 +282,52 @@ def main():
                 print(f"PARITY FAILURE: decode max-abs {err}", file=sys.stderr)
                 sys.exit(1)
 
+    # ------------------------------------------------------------------ f32 prefill, the reference's own CPU-runnable case
+    f32 = None
+    if args.only in (None, "f32"):
+        Bf, Hf, Nf, Df = 1, 8, 2048, 64
+        rng_f = np.random.default_rng(77)
+        qf, kf, vf = (rng_f.standard_normal(Bf * Hf * Nf * Df, dtype=np.float32) for _ in range(3))
+        dqf, dkf, dvf = (ra.HipStorage.from_numpy(x) for x in (qf, kf, vf))
+        dof = ra.HipStorage(Bf * Hf * Nf * Df * 4)
+        shape_f = ra.AttentionShape.new(Bf, Hf, Nf, Df)
+        causal_f = ra.Mask.causal()
+        tm = time_steps(hip, stream, lambda i: ra.flash_forward_f32_dev(shape_f, dqf, dkf, dvf, dof, causal_f, stream=stream),
+                        args.steps, args.warmup)
+        flops_f = 4.0 * Bf * Hf * Df * (Nf * (Nf + 1) / 2.0)
+        f32 = {"metric": "f32 prefill attn TFLOP/s", "value": flops_f / (tm.wall_ms / args.steps * 1e-3) / 1e12,
+               "unit": "TFLOP/s", "ms_per_step": tm.wall_ms / args.steps, "kernel_ms_mean": tm.mean_ms, **spread(tm.per),
+               "config": {"workload": "f32 causal flash-attention forward, B=1 H=8 N=2048 D=64, N(0,1) inputs (seed 77), "
+                                      "tensors resident in HBM", "flop_convention": "4*B*H*D*N*(N+1)/2 (causal-counted)"},
+               "roofline": {"bound": "mfma", "achieved": flops_f / (tm.mean_ms * 1e-3) / 1e12, "peak": PEAK_F32_TFLOPS,
+                            "unit": "TFLOP/s", "frac": flops_f / (tm.mean_ms * 1e-3) / 1e12 / PEAK_F32_TFLOPS,
+                            "traffic": None, "kernel": "flash_fwd_f32_splitk_kernel<2>"}}
+        if not args.no_cpu:
+            threads = min(oracle.max_threads(), 16)
+            got = dof.download(np.float32)
+            oracle.flash_forward_masked(oracle.AttentionShape(Bf, Hf, Nf, Df), qf, kf, vf, "causal", threads=threads)  # warm
+            reps = 5
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                want = oracle.flash_forward_masked(oracle.AttentionShape(Bf, Hf, Nf, Df), qf, kf, vf, "causal",
+                                                   threads=threads)
+            cpu_s = (time.perf_counter() - t0) / reps
+            err = float(np.abs(got - want).max())
+            f32["parity_max_abs"] = err
+            f32["cpu_baseline"] = {"value": flops_f / cpu_s / 1e12, "unit": "TFLOP/s", "cores": min(threads, Bf * Hf),
+                                   "kind": "port",
+                                   "sample": f"the whole workload, mean of {reps} runs ({cpu_s * 1e3:.0f} ms each): one task "
+                                             f"per (b,h) slab as rayon does, so at most B*H = 8 threads work; every tile "
+                                             f"computed, causal-counted FLOPs, as in the reference"}
+            if not err <= 1e-5:
+                print(f"PARITY FAILURE: f32 prefill max-abs {err}", file=sys.stderr)
+                sys.exit(1)
+        del dqf, dkf, dvf, dof
+
+    if prefill is None and decode is None:  # --only f32
+        print(json.dumps(dict(f32, n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True,
+                              dtype="f32", data="synthetic", vs_baseline=None)))
+        return
     if prefill is None:  # --only decode: report the decode line as the main one
         print(json.dumps(dict(decode, n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True,
                               dtype="bf16", data="synthetic", vs_baseline=None)))
@@ -307,6 +355,8 @@ def main():
         out["parity_max_abs"] = prefill["parity_max_abs"]
     if decode is not None:
         out["decode"] = decode
+    if f32 is not None:
+        out["f32_prefill"] = f32
     print(json.dumps(out))
 
 
