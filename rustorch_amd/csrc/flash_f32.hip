@@ -189,11 +189,25 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
     const int lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, hh = lane >> 5;
     const int N = p.seq;
-    const int h = blockIdx.y, b = blockIdx.z;
-    // longest causal rows first; when the whole grid is resident at once (p.zigzag), every other head runs the
-    // other way round, so that the workgroups that end up sharing a CU are a long one and a short one
-    int qtile = (int)gridDim.x - 1 - (int)blockIdx.x;
-    if (p.zigzag && ((h + b * (int)gridDim.y) * 2 >= (int)(gridDim.y * gridDim.z))) qtile = (int)blockIdx.x;
+    // Which (batch, head, query tile) this workgroup takes.  Workgroups are dealt round-robin to the 8 XCDs, each
+    // with its own L2: when the heads divide evenly, XCD x takes the heads bh = x (mod 8) and walks them one after
+    // the other, longest causal rows first, so that a head's K and V are fetched into one L2 only.  When the whole
+    // grid is resident at once (p.zigzag) the second half of an XCD's list runs shortest-first, so that the two
+    // workgroups that end up sharing a CU (list positions r and r + half) are a long one and a short one.
+    const int nq = (int)gridDim.x, n_bh = (int)(gridDim.y * gridDim.z);
+    int h = blockIdx.y, b = blockIdx.z;
+    int qtile = nq - 1 - (int)blockIdx.x;
+    if ((n_bh & 7) == 0) {
+        const int lin = (int)blockIdx.x + nq * ((int)blockIdx.y + (int)gridDim.y * (int)blockIdx.z);
+        const int xcd = lin & 7, r = lin >> 3, half = (nq * (n_bh >> 3)) >> 1;
+        int bh = (r / nq) * 8 + xcd;
+        qtile = nq - 1 - r % nq;
+        if (p.zigzag && r >= half && (half % nq == 0 || nq == 2 * half)) qtile = (r - half) % nq;
+        h = bh % (int)gridDim.y;
+        b = bh / (int)gridDim.y;
+    } else if (p.zigzag && ((h + b * (int)gridDim.y) * 2 >= n_bh)) {
+        qtile = (int)blockIdx.x;
+    }
     const int q0 = qtile * kRows;
     const int kvh = h / p.group;
     const float* __restrict__ Qg = p.q + (size_t)b * p.lq.batch_stride + (size_t)h * p.lq.head_stride;
