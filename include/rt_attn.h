@@ -68,7 +68,15 @@ enum rt_mask_kind {
 };
 
 /* `which` of BufferShapeMismatch / WrongInputLen. */
-enum rt_which { RT_WHICH_Q = 0, RT_WHICH_K = 1, RT_WHICH_V = 2, RT_WHICH_OUT = 3, RT_WHICH_FLASH = 4, RT_WHICH_MASK = 5 };
+enum rt_which {
+    RT_WHICH_Q = 0,
+    RT_WHICH_K = 1,
+    RT_WHICH_V = 2,
+    RT_WHICH_OUT = 3,
+    RT_WHICH_FLASH = 4,
+    RT_WHICH_MASK = 5,
+    RT_WHICH_DO = 6 /* the upstream gradient of rt_flash_backward_f32 */
+};
 
 /* Payload of the error enums above.  May be NULL. */
 typedef struct rt_err_detail {
@@ -120,7 +128,24 @@ int rt_mha_flash_forward_f32(const float *q, size_t q_len, const float *k, size_
                              float *out, size_t out_len, size_t batch, size_t seq, size_t heads, size_t head_dim,
                              rt_err_detail *err);
 
+/* rustorch_attention::flash_backward -- crates/rustorch-attention/src/cpu_backward.rs:46-185.  (dQ, dK, dV) of
+ * unmasked attention from q, k, v and the upstream gradient d_out, all [batch,heads,seq,dim] host slices.
+ * Check order: q, k, v, d_out lengths (RT_ERR_BUFFER_SHAPE_MISMATCH, which = q/k/v/do), then the three outputs
+ * (RT_ERR_OUTPUT_SHAPE_MISMATCH, got = the longest of them); seq == 0 returns RT_OK without touching the outputs.
+ * The outputs are overwritten, not accumulated into.  dim <= 128. */
+int rt_flash_backward_f32(const rt_attention_shape *shape, const float *q, size_t q_len, const float *k,
+                          size_t k_len, const float *v, size_t v_len, const float *d_out, size_t d_out_len, float *dq,
+                          size_t dq_len, float *dk, size_t dk_len, float *dv, size_t dv_len, rt_err_detail *err);
+
 /* ---- prefill, device pointers ---------------------------------------------------------------- */
+
+/* flash_backward (cpu_backward.rs:46-185) on device-resident f32 tensors.  `workspace` is device memory of at least
+ * rt_flash_backward_workspace_bytes(shape) bytes, 16-byte aligned (the recomputed forward output and two per-row
+ * statistics); RT_ERR_WORKSPACE_TOO_SMALL otherwise.  Everything runs on `stream`. */
+size_t rt_flash_backward_workspace_bytes(const rt_attention_shape *shape);
+int rt_flash_backward_f32_dev(void *stream, const rt_attention_shape *shape, const float *q, const float *k,
+                              const float *v, const float *d_out, float *dq, float *dk, float *dv, void *workspace,
+                              size_t workspace_bytes, rt_err_detail *err);
 
 /* flash_forward_masked on device-resident f32 tensors (same semantics; keep is a device
  * pointer to `seq` bytes).  n_kv_heads = 0 means n_kv_heads = heads. */

@@ -30,6 +30,7 @@
  *   ro_softmax_row            crates/rustorch-cpu/src/kernels/softmax.rs:146-180 (softmax_row_online_f32)
  *   ro_mha_forward_masked     crates/rustorch-nn/src/attention.rs:371-399 (steps 2-8 of the composed
  *                             MultiHeadAttention path: bmm, scale, additive mask, softmax, bmm)
+ *   ro_flash_backward         crates/rustorch-attention/src/cpu_backward.rs:46-185
  *   ro_f32_to_bf16            half 2.7.1 bf16::from_f32 (round to nearest even),
  *                             the rule crates/rustorch-amp/src/bf16_kernels.rs:266-267 uses
  *
@@ -76,7 +77,7 @@ enum {
 };
 
 enum { RO_MASK_NONE = 0, RO_MASK_CAUSAL = 1, RO_MASK_PADDING = 2 };
-enum { RO_WHICH_Q = 0, RO_WHICH_K = 1, RO_WHICH_V = 2, RO_WHICH_OUT = 3, RO_WHICH_FLASH = 4 };
+enum { RO_WHICH_Q = 0, RO_WHICH_K = 1, RO_WHICH_V = 2, RO_WHICH_OUT = 3, RO_WHICH_FLASH = 4, RO_WHICH_DO = 6 };
 
 typedef struct {
     uint64_t batch, heads, seq, dim, br, bc;
@@ -860,4 +861,102 @@ RO_EXPORT void ro_mha_forward_masked(const float *q, const float *k, const float
             }
     free(scores);
     free(attn);
+}
+
+/* ---- cpu_backward.rs:46-185 ----------------------------------------------
+ * (dQ, dK, dV) of unmasked attention from Q, K, V and the upstream gradient
+ * dO.  P is recomputed per (b,h) as a full seq x seq matrix, exactly as the
+ * reference does; every sum runs in the reference's loop order.  The length
+ * checks come first and in the reference's order (q, k, v, "do", then the
+ * three outputs with got = the longest); seq == 0 returns before anything is
+ * written. */
+RO_EXPORT int ro_flash_backward(const ro_shape *s, const float *q, size_t qn, const float *k, size_t kn,
+                                const float *v, size_t vn, const float *d_out, size_t don, float *dq, size_t dqn,
+                                float *dk, size_t dkn, float *dv, size_t dvn, ro_err *err) {
+    const size_t n = s->seq, d = s->dim;
+    const uint64_t expected = s->batch * s->heads * s->seq * s->dim;
+    const size_t lens[4] = {qn, kn, vn, don};
+    const int which[4] = {RO_WHICH_Q, RO_WHICH_K, RO_WHICH_V, RO_WHICH_DO};
+    for (int i = 0; i < 4; i++)
+        if (lens[i] != expected) {
+            set_err(err, which[i], expected, lens[i]);
+            return RO_ERR_BUFFER_SHAPE_MISMATCH;
+        }
+    if (dqn != expected || dkn != expected || dvn != expected) {
+        size_t got = dqn > dkn ? dqn : dkn;
+        if (dvn > got) got = dvn;
+        set_err(err, RO_WHICH_OUT, expected, got);
+        return RO_ERR_OUTPUT_SHAPE_MISMATCH;
+    }
+    if (n == 0) return RO_OK;
+    const float scale = 1.0f / sqrtf((float)d);
+    for (size_t i = 0; i < expected; i++) dq[i] = dk[i] = dv[i] = 0.0f;
+    float *p = (float *)malloc(sizeof(float) * n * n);
+    float *dp = (float *)malloc(sizeof(float) * n * n);
+    float *ds = (float *)malloc(sizeof(float) * n * n);
+    for (size_t bh = 0; bh < s->batch * s->heads; bh++) {
+        const size_t base = bh * n * d;
+        for (size_t i = 0; i < n; i++) {
+            float row_max = -INFINITY;
+            const float *qi = q + base + i * d;
+            for (size_t j = 0; j < n; j++) {
+                const float *kj = k + base + j * d;
+                float acc = 0.0f;
+                for (size_t t = 0; t < d; t++) acc += qi[t] * kj[t];
+                float scaled = acc * scale;
+                p[i * n + j] = scaled;
+                if (scaled > row_max) row_max = scaled;
+            }
+            float row_sum = 0.0f;
+            for (size_t j = 0; j < n; j++) {
+                float e = expf(p[i * n + j] - row_max);
+                p[i * n + j] = e;
+                row_sum += e;
+            }
+            if (row_sum > 0.0f && isfinite(row_sum))
+                for (size_t j = 0; j < n; j++) p[i * n + j] /= row_sum;
+        }
+        for (size_t j = 0; j < n; j++) {
+            float *dvj = dv + base + j * d;
+            for (size_t i = 0; i < n; i++) {
+                const float pij = p[i * n + j];
+                const float *doi = d_out + base + i * d;
+                for (size_t t = 0; t < d; t++) dvj[t] += pij * doi[t];
+            }
+        }
+        for (size_t i = 0; i < n; i++) {
+            const float *doi = d_out + base + i * d;
+            for (size_t j = 0; j < n; j++) {
+                const float *vj = v + base + j * d;
+                float acc = 0.0f;
+                for (size_t t = 0; t < d; t++) acc += doi[t] * vj[t];
+                dp[i * n + j] = acc;
+            }
+        }
+        for (size_t i = 0; i < n; i++) {
+            float row_dot = 0.0f;
+            for (size_t j = 0; j < n; j++) row_dot += p[i * n + j] * dp[i * n + j];
+            for (size_t j = 0; j < n; j++) ds[i * n + j] = p[i * n + j] * (dp[i * n + j] - row_dot);
+        }
+        for (size_t i = 0; i < n; i++) {
+            float *dqi = dq + base + i * d;
+            for (size_t j = 0; j < n; j++) {
+                const float *kj = k + base + j * d;
+                const float dsij = ds[i * n + j];
+                for (size_t t = 0; t < d; t++) dqi[t] += scale * dsij * kj[t];
+            }
+        }
+        for (size_t j = 0; j < n; j++) {
+            float *dkj = dk + base + j * d;
+            for (size_t i = 0; i < n; i++) {
+                const float *qi = q + base + i * d;
+                const float dsij = ds[i * n + j];
+                for (size_t t = 0; t < d; t++) dkj[t] += scale * dsij * qi[t];
+            }
+        }
+    }
+    free(p);
+    free(dp);
+    free(ds);
+    return RO_OK;
 }

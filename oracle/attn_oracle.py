@@ -35,7 +35,7 @@ ERR_KV_WRONG_INPUT_LEN = 8
 ERR_ROPE_WRONG_INPUT_LEN = 9
 ERR_ROPE_POSITION_OVERFLOW = 10
 
-WHICH = {0: "q", 1: "k", 2: "v", 3: "out", 4: "flash_forward", -1: ""}
+WHICH = {0: "q", 1: "k", 2: "v", 3: "out", 4: "flash_forward", 6: "do", -1: ""}
 
 
 class _Shape(C.Structure):
@@ -132,6 +132,7 @@ def lib():
         L.ro_rms_norm_per_head.restype = None
         L.ro_decode_prepare_bf16.argtypes = [u16p, u16p, u16p, u16p, u16p, i32p, fp, fp, C.c_float, fp, fp] + \
             [C.c_int] * 7 + [C.POINTER(_Err)]
+        L.ro_flash_backward.argtypes = [C.POINTER(_Shape)] + [fp, sz] * 7 + [C.POINTER(_Err)]
         _lib = L
     return _lib
 
@@ -213,6 +214,23 @@ def naive_forward_masked(shape, q, k, v, mask=None):
 
 def naive_forward(shape, q, k, v):
     return naive_forward_masked(shape, q, k, v, None)
+
+
+def flash_backward(shape, q, k, v, d_out, out_lens=None):
+    """cpu_backward.rs:46-185.  Returns flat ``(dq, dk, dv)``; ``out_lens`` overrides the three output lengths
+    (to exercise the length checks)."""
+    ins = [_f32(np.ravel(a)) for a in (q, k, v, d_out)]
+    lens = [shape.buffer_len()] * 3 if out_lens is None else list(out_lens)
+    outs = [np.zeros(n, dtype=np.float32) for n in lens]
+    err = _Err()
+    s = shape._c()
+    args = []
+    for a, ptr in ins:
+        args += [ptr, a.size]
+    for o in outs:
+        args += [o.ctypes.data_as(C.POINTER(C.c_float)), o.size]
+    _raise(lib().ro_flash_backward(C.byref(s), *args, C.byref(err)), err)
+    return tuple(outs)
 
 
 def mask_is_masked(mask, qi, kj) -> bool:

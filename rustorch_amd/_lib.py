@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "librt_attn_hip.so")
 SYMBOLS = (
     "rt_init", "rt_version", "rt_status_name",
     "rt_flash_forward_f32", "rt_flash_forward_masked_f32", "rt_gqa_forward_f32",
+    "rt_flash_backward_f32", "rt_flash_backward_f32_dev", "rt_flash_backward_workspace_bytes",
     "rt_flash_forward_f32_dev", "rt_flash_forward_bf16_dev", "rt_flash_forward_varlen_bf16_dev",
     "rt_mha_flash_forward_f32", "rt_mha_forward_masked_f32", "rt_flash_forward_bnhd_f32_dev", "rt_flash_forward_bnhd_bf16_dev",
     "rt_kv_append_bf16", "rt_kv_cache_append_dev", "rt_qk_norm_rope_kv_append_bf16", "rt_gqa_decode_online_bf16", "rt_gqa_decode_batched_bf16",
@@ -40,7 +41,7 @@ RT_ERR_NO_DEVICE = 30
 RT_ERR_HIP = 31
 
 RT_MASK_NONE, RT_MASK_CAUSAL, RT_MASK_PADDING = 0, 1, 2
-WHICH = {0: "q", 1: "k", 2: "v", 3: "out", 4: "flash_forward", 5: "mask", -1: ""}
+WHICH = {0: "q", 1: "k", 2: "v", 3: "out", 4: "flash_forward", 5: "mask", 6: "do", -1: ""}
 
 
 class RtShape(C.Structure):
@@ -79,6 +80,10 @@ def lib():
     L.rt_flash_forward_f32.argtypes = [shp, fp, sz, fp, sz, fp, sz, fp, sz, errp]
     L.rt_flash_forward_masked_f32.argtypes = [shp, fp, sz, fp, sz, fp, sz, C.c_int, u8p, sz, fp, sz, errp]
     L.rt_gqa_forward_f32.argtypes = [fp, sz, fp, sz, fp, sz, fp, sz, sz, sz, sz, sz, sz, sz, errp]
+    L.rt_flash_backward_f32.argtypes = [shp] + [fp, sz] * 7 + [errp]
+    L.rt_flash_backward_f32_dev.argtypes = [vp, shp] + [vp] * 8 + [sz, errp]
+    L.rt_flash_backward_workspace_bytes.argtypes = [shp]
+    L.rt_flash_backward_workspace_bytes.restype = sz
     L.rt_flash_forward_f32_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_flash_forward_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_flash_forward_varlen_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, i32p, C.c_int, vp, errp]

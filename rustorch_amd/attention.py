@@ -99,6 +99,38 @@ def flash_forward(shape: AttentionShape, q, k, v, out=None):
     return flash_forward_masked(shape, q, k, v, Mask.none(), out)
 
 
+def flash_backward(shape: AttentionShape, q, k, v, d_out, dq=None, dk=None, dv=None):
+    """rustorch_attention::flash_backward (crates/rustorch-attention/src/cpu_backward.rs:46-185): gradients of
+    unmasked attention.  q, k, v, d_out: flat f32 [B,H,N,D]; fills (overwrites) and returns flat f32 (dq, dk, dv)."""
+    ins = [_f32(a) for a in (q, k, v, d_out)]
+    outs = [np.zeros(shape.buffer_len(), dtype=np.float32) if o is None else o for o in (dq, dk, dv)]
+    args = []
+    for a, ptr in ins:
+        args += [ptr, a.size]
+    for o in outs:
+        assert o.dtype == np.float32 and o.flags.c_contiguous
+        args += [o.ctypes.data_as(C.POINTER(C.c_float)), o.size]
+    err = L.RtErr()
+    s = shape._c()
+    raise_for(L.lib().rt_flash_backward_f32(C.byref(s), *args, C.byref(err)), err)
+    return tuple(outs)
+
+
+def flash_backward_workspace_bytes(shape: AttentionShape) -> int:
+    s = shape._c()
+    return int(L.lib().rt_flash_backward_workspace_bytes(C.byref(s)))
+
+
+def flash_backward_f32_dev(shape, q, k, v, d_out, dq, dk, dv, workspace, workspace_bytes, stream=None):
+    """flash_backward on device-resident f32 [B,H,N,D] tensors; enqueues on `stream` and returns."""
+    err = L.RtErr()
+    s = shape._c()
+    rc = L.lib().rt_flash_backward_f32_dev(stream, C.byref(s), dev_ptr(q), dev_ptr(k), dev_ptr(v), dev_ptr(d_out),
+                                           dev_ptr(dq), dev_ptr(dk), dev_ptr(dv), dev_ptr(workspace),
+                                           workspace_bytes, C.byref(err))
+    raise_for(rc, err)
+
+
 # ---- device-resident tensors (torch GPU tensors, HipStorage, or raw addresses) ---------------------------
 
 

@@ -315,6 +315,104 @@ RT_API int rt_gqa_forward_f32(const float* q, size_t q_len, const float* k, size
     return RT_OK;
 }
 
+// ---- backward (cpu_backward.rs:46-185) ----------------------------------------------------------------
+
+namespace {
+
+int flash_bwd_device(hipStream_t stream, const rt_attention_shape* s, const float* q, const float* k, const float* v,
+                     const float* d_out, float* dq, float* dk, float* dv, float* workspace, rt_err_detail* err) {
+    if (s->dim > 128) return fail(err, RT_ERR_UNSUPPORTED, -1, 128, s->dim, "f32 backward kernels cover dim <= 128");
+    rt::FlashBwdF32Params p{};
+    p.q = q;
+    p.k = k;
+    p.v = v;
+    p.d_out = d_out;
+    p.dq = dq;
+    p.dk = dk;
+    p.dv = dv;
+    p.batch = (int)s->batch;
+    p.heads = (int)s->heads;
+    p.seq = (int)s->seq;
+    p.dim = (int)s->dim;
+    p.scale = 1.0f / sqrtf((float)s->dim);
+    HIP_TRY(rt::launch_flash_bwd_f32(stream, p, workspace, g_num_cus), "flash_bwd_f32 launch");
+    return RT_OK;
+}
+
+}  // namespace
+
+RT_API size_t rt_flash_backward_workspace_bytes(const rt_attention_shape* shape) {
+    if (!shape) return 0;
+    if (!fits_int(shape->batch) || !fits_int(shape->heads) || !fits_int(shape->seq) || !fits_int(shape->dim)) return 0;
+    return rt::flash_bwd_f32_workspace_floats((int)shape->batch, (int)shape->heads, (int)shape->seq, (int)shape->dim) *
+           sizeof(float);
+}
+
+RT_API int rt_flash_backward_f32(const rt_attention_shape* shape, const float* q, size_t q_len, const float* k,
+                                 size_t k_len, const float* v, size_t v_len, const float* d_out, size_t d_out_len,
+                                 float* dq, size_t dq_len, float* dk, size_t dk_len, float* dv, size_t dv_len,
+                                 rt_err_detail* err) {
+    clear_err(err);
+    if (!shape) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "shape is NULL");
+    // cpu_backward.rs:59-74: no ZeroDim check here, unlike the forward
+    const uint64_t expected = shape->batch * shape->heads * shape->seq * shape->dim;
+    const size_t lens[4] = {q_len, k_len, v_len, d_out_len};
+    static const char* names[4] = {"q", "k", "v", "do"};
+    static const int which[4] = {RT_WHICH_Q, RT_WHICH_K, RT_WHICH_V, RT_WHICH_DO};
+    for (int i = 0; i < 4; i++)
+        if (lens[i] != expected) {
+            char msg[96];
+            snprintf(msg, sizeof(msg), "%s buffer has %zu elements, expected %llu", names[i], lens[i],
+                     (unsigned long long)expected);
+            return fail(err, RT_ERR_BUFFER_SHAPE_MISMATCH, which[i], expected, lens[i], msg);
+        }
+    if (dq_len != expected || dk_len != expected || dv_len != expected) {
+        size_t got = dq_len > dk_len ? dq_len : dk_len;
+        if (dv_len > got) got = dv_len;
+        return fail(err, RT_ERR_OUTPUT_SHAPE_MISMATCH, RT_WHICH_OUT, expected, got, "gradient buffer length");
+    }
+    if (shape->seq == 0 || expected == 0) return RT_OK;
+    if (!q || !k || !v || !d_out || !dq || !dk || !dv) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    int rc = check_flash_dims(shape, shape->heads, err);
+    if (rc) return rc;
+    rc = ensure_device(err);
+    if (rc) return rc;
+
+    const size_t bytes = (size_t)expected * sizeof(float);
+    DevBuf in[4], out[3], ws;
+    const float* host_in[4] = {q, k, v, d_out};
+    for (int i = 0; i < 4; i++) {
+        HIP_TRY(hipMalloc(&in[i].p, bytes), "hipMalloc input");
+        HIP_TRY(hipMemcpy(in[i].p, host_in[i], bytes, hipMemcpyHostToDevice), "copy input");
+    }
+    for (int i = 0; i < 3; i++) HIP_TRY(hipMalloc(&out[i].p, bytes), "hipMalloc gradient");
+    HIP_TRY(hipMalloc(&ws.p, rt_flash_backward_workspace_bytes(shape)), "hipMalloc workspace");
+    rc = flash_bwd_device(nullptr, shape, (const float*)in[0].p, (const float*)in[1].p, (const float*)in[2].p,
+                          (const float*)in[3].p, (float*)out[0].p, (float*)out[1].p, (float*)out[2].p, (float*)ws.p, err);
+    if (rc) return rc;
+    float* host_out[3] = {dq, dk, dv};
+    for (int i = 0; i < 3; i++) HIP_TRY(hipMemcpy(host_out[i], out[i].p, bytes, hipMemcpyDeviceToHost), "copy gradient");
+    return RT_OK;
+}
+
+RT_API int rt_flash_backward_f32_dev(void* stream, const rt_attention_shape* shape, const float* q, const float* k,
+                                     const float* v, const float* d_out, float* dq, float* dk, float* dv,
+                                     void* workspace, size_t workspace_bytes, rt_err_detail* err) {
+    clear_err(err);
+    if (!shape) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "shape is NULL");
+    if (shape->seq == 0 || shape->batch == 0 || shape->heads == 0 || shape->dim == 0) return RT_OK;
+    int rc = check_flash_dims(shape, shape->heads, err);
+    if (rc) return rc;
+    if (!q || !k || !v || !d_out || !dq || !dk || !dv || !workspace)
+        return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    const size_t need = rt_flash_backward_workspace_bytes(shape);
+    if (workspace_bytes < need || ((uintptr_t)workspace & 15))
+        return fail(err, RT_ERR_WORKSPACE_TOO_SMALL, -1, need, workspace_bytes, "backward workspace");
+    rc = ensure_device(err);
+    if (rc) return rc;
+    return flash_bwd_device((hipStream_t)stream, shape, q, k, v, d_out, dq, dk, dv, (float*)workspace, err);
+}
+
 // ---- prefill, device pointers -----------------------------------------------------------------------
 
 RT_API int rt_flash_forward_f32_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,

@@ -1,0 +1,363 @@
+// f32 attention backward for gfx950: the device counterpart of flash_backward
+// (crates/rustorch-attention/src/cpu_backward.rs:46-185).
+//
+// The reference rebuilds the full seq x seq matrices P, dP and dS per (batch, head).  Here nothing of that
+// size exists: the forward kernel is run once more to leave O and the row statistic L_i = m_i + ln(l_i), and
+//
+//   delta_i = sum_j P_ij dP_ij = dO_i . O_i                                   (flash_bwd_delta_kernel)
+//   P_ij    = exp(scale * Q_i.K_j - L_i),   dP_ij = dO_i . V_j,   dS_ij = P_ij (dP_ij - delta_i)
+//   dV_j = sum_i P_ij dO_i,   dK_j = scale * sum_i dS_ij Q_i                  (flash_bwd_f32_dkdv_kernel)
+//   dQ_i = scale * sum_j dS_ij K_j                                            (flash_bwd_f32_dq_kernel)
+//
+// are recomputed 32 x 32 tile by tile on the f32 matrix cores (v_mfma_f32_32x32x2_f32).  Each output row is owned
+// by exactly one workgroup, so there are no atomics and the result does not depend on scheduling.
+//
+// Both kernels give a workgroup of four waves one tile of 32 "owner" rows (keys for dK/dV, queries for dQ); wave w
+// walks the tiles w, w+4, ... of the other side with a private pair of LDS tiles and no workgroup barrier in the
+// loop, and the four partial sums are added through LDS at the end.  The owner rows sit in registers as the
+// B operand of the two score-shaped products; the accumulator of those products is already in the B-operand
+// layout the two gradient products need, so P and dS never leave the register file:
+//
+//   dK/dV kernel:  S[q, kv] = Q.K^T and dP[q, kv] = dO.V^T   (A = Q / dO tile from LDS, B = K / V registers)
+//                  dV^T[d, kv] += dO^T.P,  dK^T[d, kv] += Q^T.dS   (A = the same LDS tiles read along d)
+//   dQ kernel:     S^T[kv, q] = K.Q^T and dP^T[kv, q] = V.dO^T     (A = K / V tile from LDS, B = Q / dO registers)
+//                  dQ^T[d, q] += K^T.dS^T                          (A = the K tile read along d)
+#include "rt_common.hpp"
+#include "rt_kernels.hpp"
+
+namespace rt {
+
+namespace {
+
+constexpr int kRows = 32;
+constexpr int kNW = 4;  // waves per workgroup
+
+// Copies rows [row0, row0 + 32) x [0, dim) of a [seq, dim] matrix into a 32 x LD LDS tile, zero beyond seq and dim.
+template <int DPAD, int LD>
+__device__ __forceinline__ void stage_tile(float* dst, const float* __restrict__ src, int row0, int N, int D, int lane,
+                                           bool vec) {
+    constexpr int CH = DPAD / 4;
+    if (vec) {
+#pragma unroll
+        for (int n = 0; n < kRows * CH / kWave; n++) {
+            const int idx = kWave * n + lane, r = idx / CH, c = idx % CH;
+            f32x4_t z = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (row0 + r < N && 4 * c < D) z = *(const f32x4_t*)(src + (size_t)(row0 + r) * D + 4 * c);
+            *(f32x4_t*)(dst + r * LD + 4 * c) = z;
+        }
+    } else {
+        for (int idx = lane; idx < kRows * DPAD; idx += kWave) {
+            const int r = idx / DPAD, d = idx - r * DPAD;
+            dst[r * LD + d] = (row0 + r < N && d < D) ? src[(size_t)(row0 + r) * D + d] : 0.0f;
+        }
+    }
+}
+
+// Adds the four waves' 32 x DPAD partial tiles (each at `tile_off` inside its wave's LDS block) and stores rows
+// [row0, row0 + 32) of a [seq, dim] matrix.
+template <int DPAD, int LD, int WAVE_STRIDE>
+__device__ __forceinline__ void reduce_store(const float* lds, int tile_off, float* __restrict__ dst, int row0, int N,
+                                             int D, int tid, bool vec) {
+    constexpr int CH = DPAD / 4;
+#pragma unroll
+    for (int n = 0; n < (kRows * CH + 255) / 256; n++) {
+        const int idx = 256 * n + tid;
+        if (idx < kRows * CH) {
+            const int r = idx / CH, c = idx % CH;
+            f32x4_t sum = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int w = 0; w < kNW; w++) sum += *(const f32x4_t*)(lds + w * WAVE_STRIDE + tile_off + r * LD + 4 * c);
+            if (row0 + r < N) {
+                float* o = dst + (size_t)(row0 + r) * D + 4 * c;
+                if (vec) {
+                    if (4 * c < D) *(f32x4_t*)o = sum;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        if (4 * c + i < D) o[i] = sum[i];
+                }
+            }
+        }
+    }
+}
+
+// accumulator tiles (rows d = 32t + 8g + 4hh + i of column `col`) -> rows [col][d] of an LDS tile
+template <int DT, int LD>
+__device__ __forceinline__ void spill_transposed(float* tile, const f32x16_t* acc, int col, int hh) {
+#pragma unroll
+    for (int t = 0; t < DT; t++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            f32x4_t o = {acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
+            *(f32x4_t*)(tile + col * LD + t * 32 + 8 * g + 4 * hh) = o;
+        }
+}
+
+// one wave per row: delta[row] = sum_d dO[row][d] * O[row][d]
+__global__ __launch_bounds__(256) void flash_bwd_delta_kernel(const float* __restrict__ o, const float* __restrict__ d_out,
+                                                              float* __restrict__ delta, long long rows, int D) {
+    const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= rows) return;
+    float acc = 0.0f;
+    for (int d = lane; d < D; d += kWave) acc += d_out[row * D + d] * o[row * D + d];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (lane == 0) delta[row] = acc;
+}
+
+template <int DT>  // DT = ceil(dim / 32); the head dim is zero-padded to DPAD = 32 * DT in LDS
+__global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dkdv_kernel(FlashBwdF32Params p) {
+    constexpr int DPAD = 32 * DT;
+    constexpr int LD = DPAD + 4;  // 16-byte reads of 16 rows tile all banks
+    constexpr int TILE = kRows * LD;
+    __shared__ __attribute__((aligned(16))) float lds[kNW * 2 * TILE];
+    __shared__ float stat[kNW][2][kRows];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, hh = lane >> 5;
+    const int N = p.seq, D = p.dim;
+    const bool vec = p.vec != 0;
+    const int kv0 = (int)blockIdx.x * kRows;
+    const size_t bh = (size_t)blockIdx.z * gridDim.y + blockIdx.y;
+    const size_t base = bh * (size_t)N * D;
+    const float* __restrict__ Qg = p.q + base;
+    const float* __restrict__ Kg = p.k + base;
+    const float* __restrict__ Vg = p.v + base;
+    const float* __restrict__ dOg = p.d_out + base;
+    const float* __restrict__ lse = p.lse + bh * (size_t)N;
+    const float* __restrict__ delta = p.delta + bh * (size_t)N;
+    float* Qt = lds + wave * 2 * TILE;  // this wave's Q tile
+    float* Ot = Qt + TILE;              // this wave's dO tile
+
+    // the owner rows K[kv0 + col], V[kv0 + col] as B operands; contraction order d = 8j + 4hh + i
+    stage_tile<DPAD, LD>(Qt, Kg, kv0, N, D, lane, vec);
+    stage_tile<DPAD, LD>(Ot, Vg, kv0, N, D, lane, vec);
+    float kreg[DPAD / 2], vreg[DPAD / 2];
+#pragma unroll
+    for (int j = 0; j < DPAD / 8; j++) {
+        const f32x4_t a = *(const f32x4_t*)(Qt + col * LD + 8 * j + 4 * hh);
+        const f32x4_t c = *(const f32x4_t*)(Ot + col * LD + 8 * j + 4 * hh);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            kreg[4 * j + i] = a[i];
+            vreg[4 * j + i] = c[i];
+        }
+    }
+
+    f32x16_t acc_dv[DT], acc_dk[DT];
+#pragma unroll
+    for (int t = 0; t < DT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc_dv[t][i] = acc_dk[t][i] = 0.0f;
+
+    const bool key_ok = kv0 + col < N;
+    const float sl2 = p.scale * kLog2e;
+    const int n_qt = (N + kRows - 1) / kRows;
+    for (int qt = wave; qt < n_qt; qt += kNW) {
+        const int q0 = qt * kRows;
+        stage_tile<DPAD, LD>(Qt, Qg, q0, N, D, lane, vec);
+        stage_tile<DPAD, LD>(Ot, dOg, q0, N, D, lane, vec);
+        if (hh == 0) {
+            const bool ok = q0 + col < N;
+            stat[wave][0][col] = ok ? lse[q0 + col] * kLog2e : 0.0f;
+            stat[wave][1][col] = ok ? delta[q0 + col] : 0.0f;
+        }
+        f32x16_t s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; i++) s[i] = dp[i] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < DPAD / 8; j++) {
+            const f32x4_t a = *(const f32x4_t*)(Qt + col * LD + 8 * j + 4 * hh);
+            const f32x4_t c = *(const f32x4_t*)(Ot + col * LD + 8 * j + 4 * hh);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], kreg[4 * j + i], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x2f32(c[i], vreg[4 * j + i], dp, 0, 0, 0);
+            }
+        }
+        // register i holds query row 8*(i/4) + 4*hh + (i%4) of the tile, key kv0 + col
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int qr = 8 * (i >> 2) + 4 * hh + (i & 3);
+            const bool ok = key_ok && (q0 + qr < N);
+            const float pv = ok ? __builtin_amdgcn_exp2f(s[i] * sl2 - stat[wave][0][qr]) : 0.0f;
+            s[i] = pv;
+            dp[i] = pv * (dp[i] - stat[wave][1][qr]) * p.scale;
+        }
+        // dV^T += dO^T . P and dK^T += Q^T . dS, two query rows per instruction
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int qr = 8 * (i >> 2) + 4 * hh + (i & 3);
+#pragma unroll
+            for (int t = 0; t < DT; t++) {
+                acc_dv[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(Ot[qr * LD + t * 32 + col], s[i], acc_dv[t], 0, 0, 0);
+                acc_dk[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(Qt[qr * LD + t * 32 + col], dp[i], acc_dk[t], 0, 0, 0);
+            }
+        }
+    }
+
+    spill_transposed<DT, LD>(Ot, acc_dv, col, hh);
+    spill_transposed<DT, LD>(Qt, acc_dk, col, hh);
+    __syncthreads();
+    reduce_store<DPAD, LD, 2 * TILE>(lds, TILE, p.dv + base, kv0, N, D, tid, vec);
+    reduce_store<DPAD, LD, 2 * TILE>(lds, 0, p.dk + base, kv0, N, D, tid, vec);
+}
+
+template <int DT>
+__global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dq_kernel(FlashBwdF32Params p) {
+    constexpr int DPAD = 32 * DT;
+    constexpr int LD = DPAD + 4;
+    constexpr int TILE = kRows * LD;
+    __shared__ __attribute__((aligned(16))) float lds[kNW * 2 * TILE];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, hh = lane >> 5;
+    const int N = p.seq, D = p.dim;
+    const bool vec = p.vec != 0;
+    const int q0 = (int)blockIdx.x * kRows;
+    const size_t bh = (size_t)blockIdx.z * gridDim.y + blockIdx.y;
+    const size_t base = bh * (size_t)N * D;
+    const float* __restrict__ Qg = p.q + base;
+    const float* __restrict__ Kg = p.k + base;
+    const float* __restrict__ Vg = p.v + base;
+    const float* __restrict__ dOg = p.d_out + base;
+    float* Kt = lds + wave * 2 * TILE;
+    float* Vt = Kt + TILE;
+
+    // the owner rows Q[q0 + col], dO[q0 + col] as B operands
+    stage_tile<DPAD, LD>(Kt, Qg, q0, N, D, lane, vec);
+    stage_tile<DPAD, LD>(Vt, dOg, q0, N, D, lane, vec);
+    float qreg[DPAD / 2], oreg[DPAD / 2];
+#pragma unroll
+    for (int j = 0; j < DPAD / 8; j++) {
+        const f32x4_t a = *(const f32x4_t*)(Kt + col * LD + 8 * j + 4 * hh);
+        const f32x4_t c = *(const f32x4_t*)(Vt + col * LD + 8 * j + 4 * hh);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            qreg[4 * j + i] = a[i];
+            oreg[4 * j + i] = c[i];
+        }
+    }
+    const bool q_ok = q0 + col < N;
+    const float lse_q = q_ok ? p.lse[bh * (size_t)N + q0 + col] * kLog2e : 0.0f;
+    const float delta_q = q_ok ? p.delta[bh * (size_t)N + q0 + col] : 0.0f;
+    const float sl2 = p.scale * kLog2e;
+
+    f32x16_t acc_dq[DT];
+#pragma unroll
+    for (int t = 0; t < DT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc_dq[t][i] = 0.0f;
+
+    const int n_kt = (N + kRows - 1) / kRows;
+    for (int kt = wave; kt < n_kt; kt += kNW) {
+        const int kv0 = kt * kRows;
+        stage_tile<DPAD, LD>(Kt, Kg, kv0, N, D, lane, vec);
+        stage_tile<DPAD, LD>(Vt, Vg, kv0, N, D, lane, vec);
+        f32x16_t s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; i++) s[i] = dp[i] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < DPAD / 8; j++) {
+            const f32x4_t a = *(const f32x4_t*)(Kt + col * LD + 8 * j + 4 * hh);
+            const f32x4_t c = *(const f32x4_t*)(Vt + col * LD + 8 * j + 4 * hh);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], qreg[4 * j + i], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x2f32(c[i], oreg[4 * j + i], dp, 0, 0, 0);
+            }
+        }
+        // register i holds key row 8*(i/4) + 4*hh + (i%4) of the tile, query q0 + col
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int kr = 8 * (i >> 2) + 4 * hh + (i & 3);
+            const bool ok = q_ok && (kv0 + kr < N);
+            const float pv = ok ? __builtin_amdgcn_exp2f(s[i] * sl2 - lse_q) : 0.0f;
+            dp[i] = pv * (dp[i] - delta_q) * p.scale;
+        }
+        // dQ^T += K^T . dS^T, two keys per instruction
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int kr = 8 * (i >> 2) + 4 * hh + (i & 3);
+#pragma unroll
+            for (int t = 0; t < DT; t++)
+                acc_dq[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(Kt[kr * LD + t * 32 + col], dp[i], acc_dq[t], 0, 0, 0);
+        }
+    }
+
+    spill_transposed<DT, LD>(Kt, acc_dq, col, hh);
+    __syncthreads();
+    reduce_store<DPAD, LD, 2 * TILE>(lds, 0, p.dq + base, q0, N, D, tid, vec);
+}
+
+}  // namespace
+
+size_t flash_bwd_f32_workspace_floats(int batch, int heads, int seq, int dim) {
+    return (size_t)batch * heads * seq * ((size_t)dim + 2);
+}
+
+hipError_t launch_flash_bwd_f32(hipStream_t stream, const FlashBwdF32Params& p_in, float* workspace, int n_cus) {
+    if (p_in.batch == 0 || p_in.heads == 0 || p_in.seq == 0 || p_in.dim == 0) return hipSuccess;
+    if (p_in.dim > 128) return hipErrorInvalidValue;
+    const size_t rows = (size_t)p_in.batch * p_in.heads * p_in.seq;
+    float* o = workspace;
+    float* lse = workspace + rows * p_in.dim;
+    float* delta = lse + rows;
+
+    // forward once more: O and the row statistic
+    FlashF32Params f{};
+    f.q = p_in.q;
+    f.k = p_in.k;
+    f.v = p_in.v;
+    f.out = o;
+    f.lse = lse;
+    f.batch = p_in.batch;
+    f.heads = f.kv_heads = p_in.heads;
+    f.group = 1;
+    f.seq = p_in.seq;
+    f.dim = p_in.dim;
+    f.mask = kMaskNone;
+    f.ref_bc = 64;
+    f.scale = p_in.scale;
+    f.n_cus = n_cus;
+    f.lq = f.lkv = f.lo = layout_bhnd(p_in.heads, p_in.seq, p_in.dim);
+    hipError_t e = launch_flash_f32(stream, f);
+    if (e != hipSuccess) return e;
+
+    hipLaunchKernelGGL(flash_bwd_delta_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, o, p_in.d_out, delta,
+                       (long long)rows, p_in.dim);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+
+    FlashBwdF32Params p = p_in;
+    p.lse = lse;
+    p.delta = delta;
+    auto aligned = [](const void* ptr) { return (uintptr_t)ptr % 16 == 0; };
+    p.vec = (p.dim % 4 == 0) && aligned(p.q) && aligned(p.k) && aligned(p.v) && aligned(p.d_out) && aligned(p.dq) &&
+            aligned(p.dk) && aligned(p.dv);
+    dim3 grid((p.seq + kRows - 1) / kRows, p.heads, p.batch), block(256);
+    const int dt = (p.dim + 31) / 32;
+    switch (dt) {
+        case 1:
+            hipLaunchKernelGGL(flash_bwd_f32_dkdv_kernel<1>, grid, block, 0, stream, p);
+            hipLaunchKernelGGL(flash_bwd_f32_dq_kernel<1>, grid, block, 0, stream, p);
+            break;
+        case 2:
+            hipLaunchKernelGGL(flash_bwd_f32_dkdv_kernel<2>, grid, block, 0, stream, p);
+            hipLaunchKernelGGL(flash_bwd_f32_dq_kernel<2>, grid, block, 0, stream, p);
+            break;
+        case 3:
+            hipLaunchKernelGGL(flash_bwd_f32_dkdv_kernel<3>, grid, block, 0, stream, p);
+            hipLaunchKernelGGL(flash_bwd_f32_dq_kernel<3>, grid, block, 0, stream, p);
+            break;
+        case 4:
+            hipLaunchKernelGGL(flash_bwd_f32_dkdv_kernel<4>, grid, block, 0, stream, p);
+            hipLaunchKernelGGL(flash_bwd_f32_dq_kernel<4>, grid, block, 0, stream, p);
+            break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace rt

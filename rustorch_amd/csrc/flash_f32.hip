@@ -149,6 +149,7 @@ __global__ __launch_bounds__(64) void flash_fwd_f32_kernel(FlashF32Params p) {
     float l = l_run + other_half(l_run);
     bool good = (l > 0.0f) && (fabsf(l) != __uint_as_float(0x7f800000u)) && (l == l) && !poison;
     float inv_l = 1.0f / l;
+    if (p.lse && hh == 0 && q_row < N) p.lse[((size_t)b * p.heads + h) * (size_t)N + q_row] = m_run + logf(l);
     if (q_row < N) {
 #pragma unroll
         for (int t = 0; t < DT; t++)
@@ -405,6 +406,7 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
     if (wave == 0 && hh == 0) {
         bool good = (l_all > 0.0f) && (fabsf(l_all) != __uint_as_float(0x7f800000u)) && (l_all == l_all) && !poison;
         fin_inv[col] = good ? 1.0f / l_all : quiet_nan();
+        if (p.lse && q0 + col < N) p.lse[((size_t)b * p.heads + h) * (size_t)N + q0 + col] = m_all + logf(l_all);
     }
     // this wave's weighted O, as rows [col][d], into its own K tile
 #pragma unroll

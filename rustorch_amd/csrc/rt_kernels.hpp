@@ -41,9 +41,32 @@ struct FlashF32Params {
     // optional additive score bias, rows of `seq` f32 per query row, added after scaling (zero-initialise to leave off)
     const float* bias;
     long long bias_bh_stride;  // elements between the biases of consecutive (batch, head) pairs; 0 = one for all
+    // optional [batch, heads, seq] output: the row statistic m + ln(l) of the softmax (what a backward pass needs)
+    float* lse;
 };
 // dim <= 128.  Returns hipErrorInvalidValue for an unsupported dim.
 hipError_t launch_flash_f32(hipStream_t stream, const FlashF32Params& p);
+
+// Backward of unmasked f32 attention; every tensor is [batch, heads, seq, dim] row-major and contiguous.
+struct FlashBwdF32Params {
+    const float* q;
+    const float* k;
+    const float* v;
+    const float* d_out;
+    float* dq;
+    float* dk;
+    float* dv;
+    int batch, heads, seq, dim;
+    float scale;
+    // filled by the launcher
+    const float* lse;
+    const float* delta;
+    int vec;
+};
+// Floats of scratch launch_flash_bwd_f32 needs (O, the row statistic and delta).
+size_t flash_bwd_f32_workspace_floats(int batch, int heads, int seq, int dim);
+// dim <= 128.  Runs the forward kernel, then delta, dK/dV and dQ on `stream`.
+hipError_t launch_flash_bwd_f32(hipStream_t stream, const FlashBwdF32Params& p, float* workspace, int n_cus);
 
 struct FlashBf16Params {
     const uint16_t* q;

@@ -146,3 +146,30 @@ def test_prepare_and_cache_argument_errors_before_any_device_use():
     assert lib.rt_buf_zero(None, 16, None, C.byref(err)) == L.RT_ERR_NULL_POINTER
     assert lib.rt_buf_zero(p, 6, None, C.byref(err)) == L.RT_ERR_UNSUPPORTED
     assert L.status_name(L.RT_ERR_ROPE_POSITION_OVERFLOW) == "PositionOverflow"
+
+
+def test_backward_errors_before_any_device_use():
+    """cpu_backward.rs:59-77: q, k, v, "do" lengths in that order, then the three outputs (got = the longest);
+    seq == 0 is Ok; none of this needs a device (cpu_backward.rs:252-278)."""
+    import ctypes as C
+    shape = ra.AttentionShape.new(1, 1, 4, 4)
+    good, bad = np.zeros(16, np.float32), np.zeros(10, np.float32)
+    for pos, name in enumerate(("q", "k", "v", "do")):
+        args = [good] * pos + [bad] * (4 - pos)
+        with pytest.raises(ra.BufferShapeMismatch) as ei:
+            ra.flash_backward(shape, *args, dq=np.zeros(3, np.float32))
+        assert (ei.value.which, ei.value.expected, ei.value.got) == (name, 16, 10)
+    with pytest.raises(ra.OutputShapeMismatch) as ei:
+        ra.flash_backward(shape, good, good, good, good, dq=np.zeros(16, np.float32), dk=np.zeros(20, np.float32),
+                          dv=np.zeros(7, np.float32))
+    assert (ei.value.expected, ei.value.got) == (16, 20)
+    e = np.zeros(0, dtype=np.float32)
+    dq, dk, dv = ra.flash_backward(ra.AttentionShape.new(1, 1, 0, 4), e, e, e, e)
+    assert dq.size == 0 and dk.size == 0 and dv.size == 0
+    # the device entry refuses a workspace that is too small before it looks for a device
+    s = shape._c()
+    need = L.lib().rt_flash_backward_workspace_bytes(C.byref(s))
+    assert need == 1 * 1 * 4 * (4 + 2) * 4
+    err = L.RtErr()
+    rc = L.lib().rt_flash_backward_f32_dev(None, C.byref(s), 16, 16, 16, 16, 16, 16, 16, 16, need - 1, C.byref(err))
+    assert rc == L.RT_ERR_WORKSPACE_TOO_SMALL and (err.expected, err.got) == (need, need - 1)
