@@ -5,9 +5,10 @@ A step is one pass of the bf16 causal prefill kernel over the headline workload
 B=4, H=32, N=4096, D=128 (inputs resident in HBM before the timed region); the same run also
 times the batched GQA decode workload (batch 64, 32 query / 8 kv heads, D=128, context lengths
 uniform in [512, 8192], Lmax 8192) and reports it under "decode", and the f32 causal prefill of
-B=1, H=8, N=2048, D=64 (the reference's own CPU-runnable case) under "f32_prefill".
+B=1, H=8, N=2048, D=64 (the reference's own CPU-runnable case) under "f32_prefill", and the f32
+backward on that shape under "f32_backward".
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only prefill|decode|f32]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only prefill|decode|f32|bwd]
 
 Prints ONE JSON line.  `value` is prefill TFLOP/s with causal-counted FLOPs
 (4*B*H*D*N*(N+1)/2: skipped tiles are not credited); `roofline` prices it against the dense bf16
@@ -149,7 +150,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity sample")
-    ap.add_argument("--only", choices=["prefill", "decode", "f32"], default=None)
+    ap.add_argument("--only", choices=["prefill", "decode", "f32", "bwd"], default=None)
     ap.add_argument("--no-ceiling", action="store_true",
                     help="skip the run of rustorch_amd/lib/mfma_sustained (what a loop of nothing but bf16 MFMA "
                          "sustains on this GPU, reported beside the data-sheet peak)")
@@ -325,6 +326,56 @@ def main():
                 sys.exit(1)
         del dqf, dkf, dvf, dof
 
+    # ------------------------------------------------------------------ f32 backward on the same shape (unmasked, as the reference's)
+    bwd = None
+    if args.only in (None, "bwd"):
+        Bb, Hb, Nb, Db = 1, 8, 2048, 64
+        rng_b = np.random.default_rng(78)
+        n_b = Bb * Hb * Nb * Db
+        host = [rng_b.uniform(-1.0, 1.0, n_b).astype(np.float32) for _ in range(4)]  # q, k, v, dO
+        d_in = [ra.HipStorage.from_numpy(x) for x in host]
+        d_g = [ra.HipStorage(n_b * 4) for _ in range(3)]
+        shape_b = ra.AttentionShape.new(Bb, Hb, Nb, Db)
+        ws_b = ra.flash_backward_workspace_bytes(shape_b)
+        d_ws = ra.HipStorage(ws_b)
+        tm = time_steps(hip, stream, lambda i: ra.flash_backward_f32_dev(shape_b, *d_in, *d_g, d_ws, ws_b, stream=stream),
+                        args.steps, args.warmup)
+        flops_b = 10.0 * Bb * Hb * Db * float(Nb) * Nb
+        bwd = {"metric": "f32 attention backward TFLOP/s", "value": flops_b / (tm.wall_ms / args.steps * 1e-3) / 1e12,
+               "unit": "TFLOP/s", "ms_per_step": tm.wall_ms / args.steps, "kernel_ms_mean": tm.mean_ms, **spread(tm.per),
+               "config": {"workload": "f32 unmasked attention backward (dQ, dK, dV from Q, K, V, dO), B=1 H=8 N=2048 D=64, "
+                                      "U(-1,1) inputs (seed 78), tensors resident in HBM",
+                          "flop_convention": "10*B*H*N*N*D: the five N x N x D products of the backward; the step also "
+                                             "re-runs the forward (2 products) and computes the scores twice (7 products "
+                                             "in the two backward kernels), none of which is counted"},
+               "roofline": {"bound": "mfma", "achieved": flops_b / (tm.mean_ms * 1e-3) / 1e12, "peak": PEAK_F32_TFLOPS,
+                            "unit": "TFLOP/s", "frac": flops_b / (tm.mean_ms * 1e-3) / 1e12 / PEAK_F32_TFLOPS,
+                            "traffic": None,
+                            "kernels": "flash_fwd_f32_splitk_kernel<2> + flash_bwd_delta_kernel + flash_bwd_f32_dkdv_kernel<2> "
+                                       "+ flash_bwd_f32_dq_kernel<2> (one event pair around the timed steps)"}}
+        if not args.no_cpu:
+            n_slab = Bb * Hb  # the reference's backward is a single-threaded loop; the whole workload is a second or two
+            slab = Nb * Db
+            t0 = time.perf_counter()
+            want = oracle.flash_backward(oracle.AttentionShape(1, n_slab, Nb, Db), *[x[:n_slab * slab] for x in host])
+            cpu_s = time.perf_counter() - t0
+            got = [g.download(np.float32)[:n_slab * slab] for g in d_g]
+            err = max(float(np.abs(a - b).max()) for a, b in zip(got, want))
+            bwd["parity_max_abs"] = err
+            bwd["cpu_baseline"] = {"value": flops_b * n_slab / (Bb * Hb) / cpu_s / 1e12, "unit": "TFLOP/s", "cores": 1,
+                                   "kind": "port",
+                                   "sample": f"{n_slab} of the {Bb * Hb} (b,h) slabs once ({cpu_s:.1f} s), the reference's "
+                                             f"single-threaded loops with full N x N matrices; the same slabs are the "
+                                             f"parity sample"}
+            if not err <= 2e-5:
+                print(f"PARITY FAILURE: f32 backward max-abs {err}", file=sys.stderr)
+                sys.exit(1)
+        del d_in, d_g, d_ws
+
+    if prefill is None and decode is None and f32 is None:  # --only bwd
+        print(json.dumps(dict(bwd, n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True,
+                              dtype="f32", data="synthetic", vs_baseline=None)))
+        return
     if prefill is None and decode is None:  # --only f32
         print(json.dumps(dict(f32, n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True,
                               dtype="f32", data="synthetic", vs_baseline=None)))
@@ -358,6 +409,8 @@ def main():
         out["decode"] = decode
     if f32 is not None:
         out["f32_prefill"] = f32
+    if bwd is not None:
+        out["f32_backward"] = bwd
     print(json.dumps(out))
 
 

@@ -6,6 +6,7 @@
 //
 //   rustorch_attn::AttentionShape, AttentionError, flash_forward, flash_forward_masked
 //                                   crates/rustorch-attention/src/cpu_forward.rs:49-242
+//   rustorch_attn::flash_backward   crates/rustorch-attention/src/cpu_backward.rs:46-185
 //   rustorch_attn::Mask             crates/rustorch-attention/src/mask.rs:26-78
 //   rustorch_attn::gqa_forward_f32, GQAError
 //                                   crates/rustorch-nn/src/gqa.rs:36-210
@@ -96,8 +97,8 @@ struct DeviceError : std::runtime_error {
 
 namespace detail {
 inline const char* which_name(int w) {
-    static const char* names[] = {"q", "k", "v", "out", "flash_forward", "mask"};
-    return (w >= 0 && w < 6) ? names[w] : "";
+    static const char* names[] = {"q", "k", "v", "out", "flash_forward", "mask", "do"};
+    return (w >= 0 && w < 7) ? names[w] : "";
 }
 [[noreturn]] inline void throw_device(int rc, const rt_err_detail& e) {
     throw DeviceError(rc, e.hip_error, std::string(rt_status_name(rc)) + ": " + e.message);
@@ -224,6 +225,17 @@ inline void flash_forward_masked(const AttentionShape& shape, const std::vector<
 inline void flash_forward(const AttentionShape& shape, const std::vector<float>& q, const std::vector<float>& k,
                           const std::vector<float>& v, std::vector<float>& out) {
     flash_forward_masked(shape, q, k, v, Mask::none(), out);
+}
+
+// flash_backward (cpu_backward.rs:46-185): (dQ, dK, dV) of unmasked attention; the three outputs are overwritten.
+inline void flash_backward(const AttentionShape& shape, const std::vector<float>& q, const std::vector<float>& k,
+                           const std::vector<float>& v, const std::vector<float>& d_out, std::vector<float>& dq,
+                           std::vector<float>& dk, std::vector<float>& dv) {
+    rt_attention_shape s = shape.c();
+    rt_err_detail e;
+    int rc = rt_flash_backward_f32(&s, q.data(), q.size(), k.data(), k.size(), v.data(), v.size(), d_out.data(),
+                                   d_out.size(), dq.data(), dq.size(), dk.data(), dk.size(), dv.data(), dv.size(), &e);
+    detail::check_attention(rc, e);
 }
 
 // gqa_forward_f32 (gqa.rs:94-210).

@@ -53,6 +53,34 @@ __device__ __forceinline__ void stage_tile(float* dst, const float* __restrict__
     }
 }
 
+// The same copy in two halves, so that a tile can travel from global memory into registers while the previous one is
+// multiplied: 16-byte loads (rows 16-byte aligned, dim a multiple of 4), then 16-byte LDS stores.
+template <int DPAD>
+struct TileRegs {
+    f32x4_t r[kRows * (DPAD / 4) / kWave];
+};
+template <int DPAD>
+__device__ __forceinline__ void load_tile_regs(TileRegs<DPAD>& t, const float* __restrict__ src, int row0, int N, int D,
+                                               int lane) {
+    constexpr int CH = DPAD / 4;
+#pragma unroll
+    for (int n = 0; n < kRows * CH / kWave; n++) {
+        const int idx = kWave * n + lane, r = idx / CH, c = idx % CH;
+        f32x4_t z = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (row0 + r < N && 4 * c < D) z = *(const f32x4_t*)(src + (size_t)(row0 + r) * D + 4 * c);
+        t.r[n] = z;
+    }
+}
+template <int DPAD, int LD>
+__device__ __forceinline__ void store_tile_regs(float* dst, const TileRegs<DPAD>& t, int lane) {
+    constexpr int CH = DPAD / 4;
+#pragma unroll
+    for (int n = 0; n < kRows * CH / kWave; n++) {
+        const int idx = kWave * n + lane, r = idx / CH, c = idx % CH;
+        *(f32x4_t*)(dst + r * LD + 4 * c) = t.r[n];
+    }
+}
+
 // Adds the four waves' 32 x DPAD partial tiles (each at `tile_off` inside its wave's LDS block) and stores rows
 // [row0, row0 + 32) of a [seq, dim] matrix.
 template <int DPAD, int LD, int WAVE_STRIDE>
@@ -152,15 +180,31 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dkdv_ker
         for (int i = 0; i < 16; i++) acc_dv[t][i] = acc_dk[t][i] = 0.0f;
 
     const bool key_ok = kv0 + col < N;
-    const float sl2 = p.scale * kLog2e;
     const int n_qt = (N + kRows - 1) / kRows;
+    // at DT == 2 the registers of a second prefetched tile would cost the second wave per SIMD: dO is staged directly
+    constexpr bool kPrefetchBoth = (DT != 2);
+    TileRegs<DPAD> ra, rb;
+    if (vec && wave < n_qt) {
+        load_tile_regs<DPAD>(ra, Qg, wave * kRows, N, D, lane);
+        if constexpr (kPrefetchBoth) load_tile_regs<DPAD>(rb, dOg, wave * kRows, N, D, lane);
+    }
     for (int qt = wave; qt < n_qt; qt += kNW) {
         const int q0 = qt * kRows;
-        stage_tile<DPAD, LD>(Qt, Qg, q0, N, D, lane, vec);
-        stage_tile<DPAD, LD>(Ot, dOg, q0, N, D, lane, vec);
+        if (vec) {
+            store_tile_regs<DPAD, LD>(Qt, ra, lane);
+            if constexpr (kPrefetchBoth) store_tile_regs<DPAD, LD>(Ot, rb, lane);
+            else stage_tile<DPAD, LD>(Ot, dOg, q0, N, D, lane, true);
+            if (qt + kNW < n_qt) {
+                load_tile_regs<DPAD>(ra, Qg, q0 + kNW * kRows, N, D, lane);
+                if constexpr (kPrefetchBoth) load_tile_regs<DPAD>(rb, dOg, q0 + kNW * kRows, N, D, lane);
+            }
+        } else {
+            stage_tile<DPAD, LD>(Qt, Qg, q0, N, D, lane, false);
+            stage_tile<DPAD, LD>(Ot, dOg, q0, N, D, lane, false);
+        }
         if (hh == 0) {
             const bool ok = q0 + col < N;
-            stat[wave][0][col] = ok ? lse[q0 + col] * kLog2e : 0.0f;
+            stat[wave][0][col] = ok ? lse[q0 + col] : 0.0f;
             stat[wave][1][col] = ok ? delta[q0 + col] : 0.0f;
         }
         f32x16_t s, dp;
@@ -176,12 +220,14 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dkdv_ker
                 dp = __builtin_amdgcn_mfma_f32_32x32x2f32(c[i], vreg[4 * j + i], dp, 0, 0, 0);
             }
         }
-        // register i holds query row 8*(i/4) + 4*hh + (i%4) of the tile, key kv0 + col
+        // register i holds query row 8*(i/4) + 4*hh + (i%4) of the tile, key kv0 + col.  The difference is taken
+        // before the change of base, as in the forward kernel: it is exact where it matters (scores near the row
+        // maximum), so a weight carries one rounding of its exponent
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             const int qr = 8 * (i >> 2) + 4 * hh + (i & 3);
             const bool ok = key_ok && (q0 + qr < N);
-            const float pv = ok ? __builtin_amdgcn_exp2f(s[i] * sl2 - stat[wave][0][qr]) : 0.0f;
+            const float pv = ok ? __builtin_amdgcn_exp2f((s[i] * p.scale - stat[wave][0][qr]) * kLog2e) : 0.0f;
             s[i] = pv;
             dp[i] = pv * (dp[i] - stat[wave][1][qr]) * p.scale;
         }
@@ -240,9 +286,8 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dq_kerne
         }
     }
     const bool q_ok = q0 + col < N;
-    const float lse_q = q_ok ? p.lse[bh * (size_t)N + q0 + col] * kLog2e : 0.0f;
+    const float lse_q = q_ok ? p.lse[bh * (size_t)N + q0 + col] : 0.0f;
     const float delta_q = q_ok ? p.delta[bh * (size_t)N + q0 + col] : 0.0f;
-    const float sl2 = p.scale * kLog2e;
 
     f32x16_t acc_dq[DT];
 #pragma unroll
@@ -251,10 +296,24 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dq_kerne
         for (int i = 0; i < 16; i++) acc_dq[t][i] = 0.0f;
 
     const int n_kt = (N + kRows - 1) / kRows;
+    TileRegs<DPAD> ra, rb;
+    if (vec && wave < n_kt) {
+        load_tile_regs<DPAD>(ra, Kg, wave * kRows, N, D, lane);
+        load_tile_regs<DPAD>(rb, Vg, wave * kRows, N, D, lane);
+    }
     for (int kt = wave; kt < n_kt; kt += kNW) {
         const int kv0 = kt * kRows;
-        stage_tile<DPAD, LD>(Kt, Kg, kv0, N, D, lane, vec);
-        stage_tile<DPAD, LD>(Vt, Vg, kv0, N, D, lane, vec);
+        if (vec) {
+            store_tile_regs<DPAD, LD>(Kt, ra, lane);
+            store_tile_regs<DPAD, LD>(Vt, rb, lane);
+            if (kt + kNW < n_kt) {
+                load_tile_regs<DPAD>(ra, Kg, kv0 + kNW * kRows, N, D, lane);
+                load_tile_regs<DPAD>(rb, Vg, kv0 + kNW * kRows, N, D, lane);
+            }
+        } else {
+            stage_tile<DPAD, LD>(Kt, Kg, kv0, N, D, lane, false);
+            stage_tile<DPAD, LD>(Vt, Vg, kv0, N, D, lane, false);
+        }
         f32x16_t s, dp;
 #pragma unroll
         for (int i = 0; i < 16; i++) s[i] = dp[i] = 0.0f;
@@ -273,7 +332,7 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dq_kerne
         for (int i = 0; i < 16; i++) {
             const int kr = 8 * (i >> 2) + 4 * hh + (i & 3);
             const bool ok = q_ok && (kv0 + kr < N);
-            const float pv = ok ? __builtin_amdgcn_exp2f(s[i] * sl2 - lse_q) : 0.0f;
+            const float pv = ok ? __builtin_amdgcn_exp2f((s[i] * p.scale - lse_q) * kLog2e) : 0.0f;
             dp[i] = pv * (dp[i] - delta_q) * p.scale;
         }
         // dQ^T += K^T . dS^T, two keys per instruction

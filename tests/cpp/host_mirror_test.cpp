@@ -109,6 +109,25 @@ static void test_errors() {
         std::vector<float> e, out;
         flash_forward(AttentionShape::make(2, 4, 0, 16), e, e, e, out);
     }
+    {   // backward: q, k, v, "do" in that order, then the outputs with got = the longest (cpu_backward.rs:59-77)
+        AttentionShape s = AttentionShape::make(1, 1, 4, 4);
+        std::vector<float> good(16), bad(10), g16(16), g20(20), g7(7);
+        const char* which[4] = {"q", "k", "v", "do"};
+        for (int i = 0; i < 4; i++) {
+            const std::vector<float>& a = i > 0 ? good : bad;
+            const std::vector<float>& b = i > 1 ? good : bad;
+            const std::vector<float>& c = i > 2 ? good : bad;
+            AttentionError err(AttentionError::Kind::ZeroDim, "", 0, 0, "");
+            CHECK(throws<AttentionError>([&] { flash_backward(s, a, b, c, bad, g7, g7, g7); }, &err));
+            CHECK(err.kind == AttentionError::Kind::BufferShapeMismatch && err.which == which[i]);
+            CHECK(err.expected == 16 && err.got == 10);
+        }
+        AttentionError err(AttentionError::Kind::ZeroDim, "", 0, 0, "");
+        CHECK(throws<AttentionError>([&] { flash_backward(s, good, good, good, good, g16, g20, g7); }, &err));
+        CHECK(err.kind == AttentionError::Kind::OutputShapeMismatch && err.expected == 16 && err.got == 20);
+        std::vector<float> e;
+        flash_backward(AttentionShape::make(1, 1, 0, 4), e, e, e, e, e, e, e);  // cpu_backward.rs:252-260
+    }
     {   // GQA: head counts first, then q, k, v, out (gqa.rs:106-141)
         std::vector<float> q(20), kv(8), out(20);
         GQAError err(GQAError::Kind::WrongInputLen, "", 0, 0, "");
@@ -191,6 +210,36 @@ static void test_gpu() {
             CHECK(nan_same);
             CHECK(d <= 1e-5f);
         }
+    }
+    {   // backward against central differences of the forward (cpu_backward.rs:230-250) and its closed forms
+        AttentionShape s = AttentionShape::make(1, 2, 6, 4);
+        auto q = lcg(s.buffer_len(), 1), k = lcg(s.buffer_len(), 2), v = lcg(s.buffer_len(), 3), d_out = lcg(s.buffer_len(), 4);
+        std::vector<float> dq(s.buffer_len(), -7.0f), dk(dq), dv(dq);
+        flash_backward(s, q, k, v, d_out, dq, dk, dv);
+        std::vector<float>* ins[3] = {&q, &k, &v};
+        std::vector<float>* grads[3] = {&dq, &dk, &dv};
+        for (int w = 0; w < 3; w++)
+            for (size_t idx : {size_t(0), size_t(5), size_t(10), size_t(29), size_t(47)}) {
+                const float saved = (*ins[w])[idx], eps = 1e-2f;
+                std::vector<float> op(s.buffer_len()), om(s.buffer_len());
+                (*ins[w])[idx] = saved + eps;
+                flash_forward(s, q, k, v, op);
+                (*ins[w])[idx] = saved - eps;
+                flash_forward(s, q, k, v, om);
+                (*ins[w])[idx] = saved;
+                double g = 0.0;
+                for (size_t i = 0; i < op.size(); i++) g += (double)d_out[i] * ((double)op[i] - om[i]) / (2.0 * eps);
+                CHECK(std::fabs((*grads[w])[idx] - g) < 2e-3);
+            }
+        std::vector<float> zero(s.buffer_len(), 0.0f);
+        flash_backward(s, q, k, v, zero, dq, dk, dv);  // cpu_backward.rs:279-299
+        for (size_t i = 0; i < dq.size(); i++) CHECK(dq[i] == 0.0f && dk[i] == 0.0f && dv[i] == 0.0f);
+        // a single key: P == 1, so dV = dO exactly; dQ = dK = 0 up to the rounding of dO.V summed in two orders
+        AttentionShape one = AttentionShape::make(2, 2, 1, 16);
+        auto q1 = lcg(one.buffer_len(), 5), g1 = lcg(one.buffer_len(), 6);
+        std::vector<float> a(one.buffer_len()), b(a), c(a);
+        flash_backward(one, q1, q1, q1, g1, a, b, c);
+        for (size_t i = 0; i < a.size(); i++) CHECK(std::fabs(a[i]) < 1e-6f && std::fabs(b[i]) < 1e-6f && c[i] == g1[i]);
     }
     {   // N == 1: out == v (reference test single_token_returns_v)
         AttentionShape s = AttentionShape::make(1, 1, 1, 4);

@@ -156,3 +156,16 @@ def test_full_size_identities():
     g3 = ra.flash_backward(shape, q, k, v, (2.0 * d1 - 0.5 * d2).astype(np.float32))
     for a, b, c in zip((dq, dk, dv), g2, g3):
         assert max_abs(2.0 * r(a) - 0.5 * r(b), r(c)) < 5e-5
+
+
+def test_large_magnitude_scores(oracle):
+    """Inputs in (-6, 6): scores reach +-70 and most rows are nearly one-hot.  Errors are relative to the size of the
+    gradients (both sides round exp arguments of that size to about 4e-6)."""
+    bhnd = (1, 2, 96, 32)
+    shape = ra.AttentionShape.new(*bhnd)
+    bufs = [lcg_buffer(shape.buffer_len(), s, span=12.0) for s in (51, 52, 53, 54)]
+    got = ra.flash_backward(shape, *bufs)
+    want = oracle.flash_backward(oracle.AttentionShape(*bhnd), *bufs)
+    for name, g, w in zip(("dq", "dk", "dv"), got, want):
+        assert np.isfinite(g).all()
+        assert max_abs(g, w) <= 1e-4 * float(np.abs(w).max()), f"{name}: {max_abs(g, w):.3e} of {np.abs(w).max():.3e}"
