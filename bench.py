@@ -40,6 +40,8 @@ PEAK_F32_TFLOPS = 157.3     # MI355X dense f32 MFMA
 TRAFFIC_PREFILL_BYTES = (270900 * 2.0 + 131100 * 1.0) * 1024
 TRAFFIC_DECODE_BYTES = (623700 * 2.0 + 3224 * 1.0) * 1024
 TRAFFIC_F32_BYTES = (6239 * 2.0 + 4096 * 1.0) * 1024
+# the four kernels of one backward step (forward, delta, dK/dV, dQ): FETCH_SIZE 6242 + 4109 + 8604 + 8335, WRITE_SIZE 4160 + 128 + 8704 + 4096
+TRAFFIC_BWD_BYTES = (27290 * 2.0 + 17088 * 1.0) * 1024
 
 
 class Hip:
@@ -350,7 +352,7 @@ def main():
                                              "in the two backward kernels), none of which is counted"},
                "roofline": {"bound": "mfma", "achieved": flops_b / (tm.mean_ms * 1e-3) / 1e12, "peak": PEAK_F32_TFLOPS,
                             "unit": "TFLOP/s", "frac": flops_b / (tm.mean_ms * 1e-3) / 1e12 / PEAK_F32_TFLOPS,
-                            "traffic": None,
+                            "traffic": TRAFFIC_BWD_BYTES,
                             "kernels": "flash_fwd_f32_splitk_kernel<2> + flash_bwd_delta_kernel + flash_bwd_f32_dkdv_kernel<2> "
                                        "+ flash_bwd_f32_dq_kernel<2> (one event pair around the timed steps)"}}
         if not args.no_cpu:

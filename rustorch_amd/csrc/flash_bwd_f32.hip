@@ -121,6 +121,21 @@ __device__ __forceinline__ void spill_transposed(float* tile, const f32x16_t* ac
         }
 }
 
+// Which (batch*head, owner tile) a workgroup takes.  Workgroups are dealt round-robin to the 8 XCDs, each with its own
+// L2: when the (batch, head) pairs divide evenly, XCD x takes the pairs bh = x (mod 8) one after the other, so that a
+// pair's four input tensors are fetched into one L2 only.
+__device__ __forceinline__ void owner_of_block(int& bh, int& tile) {
+    const int nt = (int)gridDim.x, n_bh = (int)(gridDim.y * gridDim.z);
+    bh = (int)blockIdx.y + (int)gridDim.y * (int)blockIdx.z;
+    tile = (int)blockIdx.x;
+    if ((n_bh & 7) == 0) {
+        const int lin = (int)blockIdx.x + nt * bh;
+        const int xcd = lin & 7, r = lin >> 3;
+        bh = (r / nt) * 8 + xcd;
+        tile = r % nt;
+    }
+}
+
 // one wave per row: delta[row] = sum_d dO[row][d] * O[row][d]
 __global__ __launch_bounds__(256) void flash_bwd_delta_kernel(const float* __restrict__ o, const float* __restrict__ d_out,
                                                               float* __restrict__ delta, long long rows, int D) {
@@ -146,8 +161,10 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dkdv_ker
     const int col = lane & 31, hh = lane >> 5;
     const int N = p.seq, D = p.dim;
     const bool vec = p.vec != 0;
-    const int kv0 = (int)blockIdx.x * kRows;
-    const size_t bh = (size_t)blockIdx.z * gridDim.y + blockIdx.y;
+    int bh_i, tile_i;
+    owner_of_block(bh_i, tile_i);
+    const int kv0 = tile_i * kRows;
+    const size_t bh = (size_t)bh_i;
     const size_t base = bh * (size_t)N * D;
     const float* __restrict__ Qg = p.q + base;
     const float* __restrict__ Kg = p.k + base;
@@ -261,8 +278,10 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dq_kerne
     const int col = lane & 31, hh = lane >> 5;
     const int N = p.seq, D = p.dim;
     const bool vec = p.vec != 0;
-    const int q0 = (int)blockIdx.x * kRows;
-    const size_t bh = (size_t)blockIdx.z * gridDim.y + blockIdx.y;
+    int bh_i, tile_i;
+    owner_of_block(bh_i, tile_i);
+    const int q0 = tile_i * kRows;
+    const size_t bh = (size_t)bh_i;
     const size_t base = bh * (size_t)N * D;
     const float* __restrict__ Qg = p.q + base;
     const float* __restrict__ Kg = p.k + base;
