@@ -107,7 +107,8 @@ int rt_flash_forward_f32(const rt_attention_shape *shape, const float *q, size_t
 /* rustorch_attention::flash_forward_masked -- cpu_forward.rs:193-242.  Check order: ZeroDim,
  * q, k, v lengths, out length, padding length; seq == 0 returns RT_OK without touching `out`.
  * A row with no visible key is NaN (cpu_forward.rs:411-420); with RT_MASK_PADDING, when none of
- * keep[0 .. min(bc, seq)) is set every row is NaN, as the reference's tiled recurrence gives. */
+ * keep[0 .. min(bc, seq)) is set every row is NaN, as the reference's tiled recurrence gives.
+ * dim <= 256 (RT_ERR_UNSUPPORTED beyond). */
 int rt_flash_forward_masked_f32(const rt_attention_shape *shape, const float *q, size_t q_len, const float *k,
                                 size_t k_len, const float *v, size_t v_len, int mask_kind, const uint8_t *keep,
                                 size_t keep_len, float *out, size_t out_len, rt_err_detail *err);

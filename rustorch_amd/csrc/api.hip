@@ -136,7 +136,7 @@ int check_flash_dims(const rt_attention_shape* s, uint64_t n_kv_heads, rt_err_de
 int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n_kv_heads, const float* q,
                      const float* k, const float* v, int mask_kind, const uint8_t* keep, float* out,
                      rt_err_detail* err, bool bnhd = false, const float* bias = nullptr, long long bias_bh_stride = 0) {
-    if (s->dim > 128) return fail(err, RT_ERR_UNSUPPORTED, -1, 128, s->dim, "f32 flash kernel covers dim <= 128");
+    if (s->dim > 256) return fail(err, RT_ERR_UNSUPPORTED, -1, 256, s->dim, "f32 flash kernels cover dim <= 256");
     rt::FlashF32Params p{};
     p.bias = bias;
     p.bias_bh_stride = bias_bh_stride;

@@ -446,7 +446,7 @@ hipError_t launch_flash_f32(hipStream_t stream, const FlashF32Params& p) {
     auto aligned = [](const void* ptr, const TensorLayout& l) {
         return ((uintptr_t)ptr % 16 == 0) && (l.batch_stride % 4 == 0) && (l.head_stride % 4 == 0) && (l.row_pitch % 4 == 0);
     };
-    if (p.dim % 32 == 0 && aligned(p.q, p.lq) && aligned(p.k, p.lkv) && aligned(p.v, p.lkv) && aligned(p.out, p.lo)) {
+    if (p.dim % 32 == 0 && p.dim <= 128 && aligned(p.q, p.lq) && aligned(p.k, p.lkv) && aligned(p.v, p.lkv) && aligned(p.out, p.lo)) {
         dim3 block4(256);
         FlashF32Params pz = p;
         // 8 (dim <= 64) or 4 waves fit on a CU: is every workgroup resident from the start?
@@ -467,6 +467,11 @@ hipError_t launch_flash_f32(hipStream_t stream, const FlashF32Params& p) {
         case 2: hipLaunchKernelGGL(flash_fwd_f32_kernel<2>, grid, block, 0, stream, p); break;
         case 3: hipLaunchKernelGGL(flash_fwd_f32_kernel<3>, grid, block, 0, stream, p); break;
         case 4: hipLaunchKernelGGL(flash_fwd_f32_kernel<4>, grid, block, 0, stream, p); break;
+        // head dims 129..256: the same kernel with a wider tile (about 100 KB of LDS, one workgroup per CU)
+        case 5: hipLaunchKernelGGL(flash_fwd_f32_kernel<5>, grid, block, 0, stream, p); break;
+        case 6: hipLaunchKernelGGL(flash_fwd_f32_kernel<6>, grid, block, 0, stream, p); break;
+        case 7: hipLaunchKernelGGL(flash_fwd_f32_kernel<7>, grid, block, 0, stream, p); break;
+        case 8: hipLaunchKernelGGL(flash_fwd_f32_kernel<8>, grid, block, 0, stream, p); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

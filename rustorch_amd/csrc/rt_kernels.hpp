@@ -44,7 +44,7 @@ struct FlashF32Params {
     // optional [batch, heads, seq] output: the row statistic m + ln(l) of the softmax (what a backward pass needs)
     float* lse;
 };
-// dim <= 128.  Returns hipErrorInvalidValue for an unsupported dim.
+// dim <= 256 (the tiled four-wave kernel up to 128).  Returns hipErrorInvalidValue for an unsupported dim.
 hipError_t launch_flash_f32(hipStream_t stream, const FlashF32Params& p);
 
 // Backward of unmasked f32 attention; every tensor is [batch, heads, seq, dim] row-major and contiguous.

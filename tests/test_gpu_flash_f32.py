@@ -50,6 +50,25 @@ def test_flash_matches_oracle_unit_shapes(oracle, bhnd):
         assert_close_nan(got, want, TOL, str(bhnd))
 
 
+@pytest.mark.parametrize("bhnd", [(1, 2, 70, 129), (1, 1, 100, 192), (2, 1, 65, 256), (1, 1, 33, 200)])
+def test_flash_head_dims_above_128(oracle, bhnd):
+    shape = ra.AttentionShape.new(*bhnd)
+    q, k, v = buffers(shape.buffer_len(), 2.0)
+    keep = np.arange(bhnd[2]) % 3 != 1
+    for mask in (ra.Mask.none(), ra.Mask.causal(), ra.Mask.padding(keep)):
+        got = ra.flash_forward_masked(shape, q, k, v, mask)
+        want = oracle.flash_forward_masked(oracle.AttentionShape(*bhnd), q, k, v, omask(mask))
+        assert_close_nan(got, want, TOL, f"{bhnd} mask={mask.kind}")
+
+
+def test_flash_head_dim_above_256_is_refused():
+    shape = ra.AttentionShape.new(1, 1, 4, 257)
+    z = np.zeros(shape.buffer_len(), np.float32)
+    with pytest.raises(ra.DeviceError) as ei:
+        ra.flash_forward(shape, z, z, z)
+    assert ei.value.status == 21
+
+
 def test_scaling_factor_is_one_over_sqrt_d():
     shape = ra.AttentionShape.new(1, 1, 1, 4)
     e0 = np.array([1.0, 0, 0, 0], dtype=np.float32)
