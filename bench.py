@@ -343,8 +343,18 @@ def main():
         tm = time_steps(hip, stream, lambda i: ra.flash_backward_f32_dev(shape_b, *d_in, *d_g, d_ws, ws_b, stream=stream),
                         args.steps, args.warmup)
         flops_b = 10.0 * Bb * Hb * Db * float(Nb) * Nb
+        # the same gradients from a saved forward (O and m + ln l kept from the forward pass): no recomputation
+        d_o, d_lse = ra.HipStorage(n_b * 4), ra.HipStorage(Bb * Hb * Nb * 4)
+        ra.flash_forward_stats_f32_dev(shape_b, d_in[0], d_in[1], d_in[2], d_o, d_lse, stream=stream)
+        tm_saved = time_steps(hip, stream,
+                              lambda i: ra.flash_backward_saved_f32_dev(shape_b, d_in[0], d_in[1], d_in[2], d_o, d_lse,
+                                                                        d_in[3], *d_g, d_ws, ws_b, stream=stream),
+                              args.steps, args.warmup, spread_steps=0)
         bwd = {"metric": "f32 attention backward TFLOP/s", "value": flops_b / (tm.wall_ms / args.steps * 1e-3) / 1e12,
                "unit": "TFLOP/s", "ms_per_step": tm.wall_ms / args.steps, "kernel_ms_mean": tm.mean_ms, **spread(tm.per),
+               "saved_forward": {"kernel_ms_mean": tm_saved.mean_ms, "tflops": flops_b / (tm_saved.mean_ms * 1e-3) / 1e12,
+                                 "note": "rt_flash_backward_saved_f32_dev: O and the row statistic come from the forward "
+                                         "pass instead of being recomputed (delta + dK/dV + dQ)"},
                "config": {"workload": "f32 unmasked attention backward (dQ, dK, dV from Q, K, V, dO), B=1 H=8 N=2048 D=64, "
                                       "U(-1,1) inputs (seed 78), tensors resident in HBM",
                           "flop_convention": "10*B*H*N*N*D: the five N x N x D products of the backward; the step also "

@@ -148,6 +148,18 @@ int rt_flash_backward_f32_dev(void *stream, const rt_attention_shape *shape, con
                               const float *v, const float *d_out, float *dq, float *dk, float *dv, void *workspace,
                               size_t workspace_bytes, rt_err_detail *err);
 
+/* The saved-forward form of the backward, which the header of cpu_backward.rs describes for a GPU path
+ * (cpu_backward.rs:3-4, :29-35: "from a saved forward pass (Q, K, V, the softmax statistics m and l, and the upstream
+ * gradient dO)"; the reference's CPU function recomputes instead).  rt_flash_forward_stats_f32_dev is the unmasked
+ * forward that also writes the row statistic lse[b,h,i] = m_i + ln(l_i) ([batch,heads,seq] f32);
+ * rt_flash_backward_saved_f32_dev takes that `out` and `lse` back and skips the recomputation.  `workspace`:
+ * batch*heads*seq floats (RT_ERR_WORKSPACE_TOO_SMALL otherwise).  dim <= 128 for the backward. */
+int rt_flash_forward_stats_f32_dev(void *stream, const rt_attention_shape *shape, const float *q, const float *k,
+                                   const float *v, float *out, float *lse, rt_err_detail *err);
+int rt_flash_backward_saved_f32_dev(void *stream, const rt_attention_shape *shape, const float *q, const float *k,
+                                    const float *v, const float *out, const float *lse, const float *d_out, float *dq,
+                                    float *dk, float *dv, void *workspace, size_t workspace_bytes, rt_err_detail *err);
+
 /* flash_forward_masked on device-resident f32 tensors (same semantics; keep is a device
  * pointer to `seq` bytes).  n_kv_heads = 0 means n_kv_heads = heads. */
 int rt_flash_forward_f32_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const float *q,

@@ -378,6 +378,38 @@ inline void flash_forward_varlen_bf16_dev(const AttentionShape& shape, const voi
         e);
 }
 
+// ---- device-resident f32 backward (cpu_backward.rs:46-185; the saved-forward form of its header comment) ----------
+
+inline size_t flash_backward_workspace_bytes(const AttentionShape& shape) {
+    rt_attention_shape s = shape.c();
+    return rt_flash_backward_workspace_bytes(&s);
+}
+inline void flash_backward_f32_dev(const AttentionShape& shape, const float* q, const float* k, const float* v,
+                                   const float* d_out, float* dq, float* dk, float* dv, void* workspace,
+                                   size_t workspace_bytes, void* stream = nullptr) {
+    rt_attention_shape s = shape.c();
+    rt_err_detail e;
+    detail::check_attention(
+        rt_flash_backward_f32_dev(stream, &s, q, k, v, d_out, dq, dk, dv, workspace, workspace_bytes, &e), e);
+}
+// out and lse ([batch, heads, seq], m + ln l) as flash_forward_stats_f32_dev leaves them
+inline void flash_forward_stats_f32_dev(const AttentionShape& shape, const float* q, const float* k, const float* v,
+                                        float* out, float* lse, void* stream = nullptr) {
+    rt_attention_shape s = shape.c();
+    rt_err_detail e;
+    detail::check_attention(rt_flash_forward_stats_f32_dev(stream, &s, q, k, v, out, lse, &e), e);
+}
+// workspace: batch * heads * seq floats
+inline void flash_backward_saved_f32_dev(const AttentionShape& shape, const float* q, const float* k, const float* v,
+                                         const float* out, const float* lse, const float* d_out, float* dq, float* dk,
+                                         float* dv, void* workspace, size_t workspace_bytes, void* stream = nullptr) {
+    rt_attention_shape s = shape.c();
+    rt_err_detail e;
+    detail::check_attention(rt_flash_backward_saved_f32_dev(stream, &s, q, k, v, out, lse, d_out, dq, dk, dv, workspace,
+                                                            workspace_bytes, &e),
+                            e);
+}
+
 // ---- KVCache (crates/rustorch-nn/src/kv_cache.rs:49-256) with its buffers in HBM ---------------------------
 //
 // Same protocol as the reference: append(layer, seq_added, new_k, new_v) for every layer, then advance(seq_added).

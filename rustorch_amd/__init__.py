@@ -5,7 +5,8 @@ librt_attn_hip.so (include/rt_attn.h).  All arithmetic runs in hand-written HIP 
 no CPU fallback.
 """
 from . import _lib
-from .attention import (AttentionShape, Mask, flash_backward, flash_backward_f32_dev,
+from .attention import (AttentionShape, Mask, flash_backward, flash_backward_f32_dev, flash_backward_saved_f32_dev,
+                        flash_forward_stats_f32_dev,
                         flash_backward_workspace_bytes, flash_forward, flash_forward_bf16_dev, flash_forward_bnhd_bf16_dev,
                         flash_forward_bnhd_f32_dev, flash_forward_f32_dev, flash_forward_masked,
                         flash_forward_varlen_bf16_dev, mha_flash_forward_f32, mha_forward_masked_f32)

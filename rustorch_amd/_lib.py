@@ -16,6 +16,7 @@ SYMBOLS = (
     "rt_init", "rt_version", "rt_status_name",
     "rt_flash_forward_f32", "rt_flash_forward_masked_f32", "rt_gqa_forward_f32",
     "rt_flash_backward_f32", "rt_flash_backward_f32_dev", "rt_flash_backward_workspace_bytes",
+    "rt_flash_forward_stats_f32_dev", "rt_flash_backward_saved_f32_dev",
     "rt_flash_forward_f32_dev", "rt_flash_forward_bf16_dev", "rt_flash_forward_varlen_bf16_dev",
     "rt_mha_flash_forward_f32", "rt_mha_forward_masked_f32", "rt_flash_forward_bnhd_f32_dev", "rt_flash_forward_bnhd_bf16_dev",
     "rt_kv_append_bf16", "rt_kv_cache_append_dev", "rt_qk_norm_rope_kv_append_bf16", "rt_gqa_decode_online_bf16", "rt_gqa_decode_batched_bf16",
@@ -83,6 +84,8 @@ def lib():
     L.rt_flash_backward_f32.argtypes = [shp] + [fp, sz] * 7 + [errp]
     L.rt_flash_backward_f32_dev.argtypes = [vp, shp] + [vp] * 8 + [sz, errp]
     L.rt_flash_backward_workspace_bytes.argtypes = [shp]
+    L.rt_flash_forward_stats_f32_dev.argtypes = [vp, shp] + [vp] * 5 + [errp]
+    L.rt_flash_backward_saved_f32_dev.argtypes = [vp, shp] + [vp] * 10 + [sz, errp]
     L.rt_flash_backward_workspace_bytes.restype = sz
     L.rt_flash_forward_f32_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_flash_forward_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]

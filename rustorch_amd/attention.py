@@ -131,6 +131,25 @@ def flash_backward_f32_dev(shape, q, k, v, d_out, dq, dk, dv, workspace, workspa
     raise_for(rc, err)
 
 
+def flash_forward_stats_f32_dev(shape, q, k, v, out, lse, stream=None):
+    """Unmasked f32 forward that also writes lse[b,h,i] = m_i + ln(l_i): what flash_backward_saved_f32_dev takes back."""
+    err = L.RtErr()
+    s = shape._c()
+    rc = L.lib().rt_flash_forward_stats_f32_dev(stream, C.byref(s), dev_ptr(q), dev_ptr(k), dev_ptr(v), dev_ptr(out),
+                                                dev_ptr(lse), C.byref(err))
+    raise_for(rc, err)
+
+
+def flash_backward_saved_f32_dev(shape, q, k, v, out, lse, d_out, dq, dk, dv, workspace, workspace_bytes, stream=None):
+    """The backward from a saved forward (cpu_backward.rs:3-4, :29-35); workspace: batch*heads*seq floats."""
+    err = L.RtErr()
+    s = shape._c()
+    rc = L.lib().rt_flash_backward_saved_f32_dev(stream, C.byref(s), dev_ptr(q), dev_ptr(k), dev_ptr(v), dev_ptr(out),
+                                                 dev_ptr(lse), dev_ptr(d_out), dev_ptr(dq), dev_ptr(dk), dev_ptr(dv),
+                                                 dev_ptr(workspace), workspace_bytes, C.byref(err))
+    raise_for(rc, err)
+
+
 # ---- device-resident tensors (torch GPU tensors, HipStorage, or raw addresses) ---------------------------
 
 

@@ -135,11 +135,13 @@ int check_flash_dims(const rt_attention_shape* s, uint64_t n_kv_heads, rt_err_de
 // bnhd: tensors are [batch, seq, heads, dim] instead of [batch, heads, seq, dim]
 int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n_kv_heads, const float* q,
                      const float* k, const float* v, int mask_kind, const uint8_t* keep, float* out,
-                     rt_err_detail* err, bool bnhd = false, const float* bias = nullptr, long long bias_bh_stride = 0) {
+                     rt_err_detail* err, bool bnhd = false, const float* bias = nullptr, long long bias_bh_stride = 0,
+                     float* lse = nullptr) {
     if (s->dim > 256) return fail(err, RT_ERR_UNSUPPORTED, -1, 256, s->dim, "f32 flash kernels cover dim <= 256");
     rt::FlashF32Params p{};
     p.bias = bias;
     p.bias_bh_stride = bias_bh_stride;
+    p.lse = lse;
     p.q = q;
     p.k = k;
     p.v = v;
@@ -319,8 +321,10 @@ RT_API int rt_gqa_forward_f32(const float* q, size_t q_len, const float* k, size
 
 namespace {
 
+// saved_out / saved_lse non-NULL: the forward is not recomputed and `workspace` holds delta only
 int flash_bwd_device(hipStream_t stream, const rt_attention_shape* s, const float* q, const float* k, const float* v,
-                     const float* d_out, float* dq, float* dk, float* dv, float* workspace, rt_err_detail* err) {
+                     const float* d_out, float* dq, float* dk, float* dv, float* workspace, rt_err_detail* err,
+                     const float* saved_out = nullptr, const float* saved_lse = nullptr) {
     if (s->dim > 128) return fail(err, RT_ERR_UNSUPPORTED, -1, 128, s->dim, "f32 backward kernels cover dim <= 128");
     rt::FlashBwdF32Params p{};
     p.q = q;
@@ -335,7 +339,10 @@ int flash_bwd_device(hipStream_t stream, const rt_attention_shape* s, const floa
     p.seq = (int)s->seq;
     p.dim = (int)s->dim;
     p.scale = 1.0f / sqrtf((float)s->dim);
-    HIP_TRY(rt::launch_flash_bwd_f32(stream, p, workspace, g_num_cus), "flash_bwd_f32 launch");
+    if (saved_out)
+        HIP_TRY(rt::launch_flash_bwd_f32_saved(stream, p, saved_out, saved_lse, workspace), "flash_bwd_f32 launch");
+    else
+        HIP_TRY(rt::launch_flash_bwd_f32(stream, p, workspace, g_num_cus), "flash_bwd_f32 launch");
     return RT_OK;
 }
 
@@ -411,6 +418,40 @@ RT_API int rt_flash_backward_f32_dev(void* stream, const rt_attention_shape* sha
     rc = ensure_device(err);
     if (rc) return rc;
     return flash_bwd_device((hipStream_t)stream, shape, q, k, v, d_out, dq, dk, dv, (float*)workspace, err);
+}
+
+RT_API int rt_flash_forward_stats_f32_dev(void* stream, const rt_attention_shape* shape, const float* q, const float* k,
+                                          const float* v, float* out, float* lse, rt_err_detail* err) {
+    clear_err(err);
+    if (!shape) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "shape is NULL");
+    if (shape->dim == 0) return fail(err, RT_ERR_ZERO_DIM, -1, 0, 0, "dim must be > 0");
+    if (shape->seq == 0 || shape->batch == 0 || shape->heads == 0) return RT_OK;
+    int rc = check_flash_dims(shape, shape->heads, err);
+    if (rc) return rc;
+    if (!q || !k || !v || !out || !lse) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    rc = ensure_device(err);
+    if (rc) return rc;
+    return flash_f32_device((hipStream_t)stream, shape, shape->heads, q, k, v, RT_MASK_NONE, nullptr, out, err, false,
+                            nullptr, 0, lse);
+}
+
+RT_API int rt_flash_backward_saved_f32_dev(void* stream, const rt_attention_shape* shape, const float* q, const float* k,
+                                           const float* v, const float* out, const float* lse, const float* d_out,
+                                           float* dq, float* dk, float* dv, void* workspace, size_t workspace_bytes,
+                                           rt_err_detail* err) {
+    clear_err(err);
+    if (!shape) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "shape is NULL");
+    if (shape->seq == 0 || shape->batch == 0 || shape->heads == 0 || shape->dim == 0) return RT_OK;
+    int rc = check_flash_dims(shape, shape->heads, err);
+    if (rc) return rc;
+    if (!q || !k || !v || !out || !lse || !d_out || !dq || !dk || !dv || !workspace)
+        return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    const size_t need = (size_t)(shape->batch * shape->heads * shape->seq) * sizeof(float);
+    if (workspace_bytes < need)
+        return fail(err, RT_ERR_WORKSPACE_TOO_SMALL, -1, need, workspace_bytes, "backward workspace (delta)");
+    rc = ensure_device(err);
+    if (rc) return rc;
+    return flash_bwd_device((hipStream_t)stream, shape, q, k, v, d_out, dq, dk, dv, (float*)workspace, err, out, lse);
 }
 
 // ---- prefill, device pointers -----------------------------------------------------------------------

@@ -402,10 +402,17 @@ hipError_t launch_flash_bwd_f32(hipStream_t stream, const FlashBwdF32Params& p_i
     f.lq = f.lkv = f.lo = layout_bhnd(p_in.heads, p_in.seq, p_in.dim);
     hipError_t e = launch_flash_f32(stream, f);
     if (e != hipSuccess) return e;
+    return launch_flash_bwd_f32_saved(stream, p_in, o, lse, delta);
+}
 
+hipError_t launch_flash_bwd_f32_saved(hipStream_t stream, const FlashBwdF32Params& p_in, const float* o, const float* lse,
+                                      float* delta) {
+    if (p_in.batch == 0 || p_in.heads == 0 || p_in.seq == 0 || p_in.dim == 0) return hipSuccess;
+    if (p_in.dim > 128) return hipErrorInvalidValue;
+    const size_t rows = (size_t)p_in.batch * p_in.heads * p_in.seq;
     hipLaunchKernelGGL(flash_bwd_delta_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, o, p_in.d_out, delta,
                        (long long)rows, p_in.dim);
-    e = hipGetLastError();
+    hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
 
     FlashBwdF32Params p = p_in;

@@ -67,6 +67,10 @@ struct FlashBwdF32Params {
 size_t flash_bwd_f32_workspace_floats(int batch, int heads, int seq, int dim);
 // dim <= 128.  Runs the forward kernel, then delta, dK/dV and dQ on `stream`.
 hipError_t launch_flash_bwd_f32(hipStream_t stream, const FlashBwdF32Params& p, float* workspace, int n_cus);
+// The same from a saved forward: `o` [B,H,N,D] and `lse` [B,H,N] as launch_flash_f32 leaves them (FlashF32Params::lse);
+// `delta` is B*H*N floats of scratch.  Runs delta, dK/dV and dQ.
+hipError_t launch_flash_bwd_f32_saved(hipStream_t stream, const FlashBwdF32Params& p, const float* o, const float* lse,
+                                      float* delta);
 
 struct FlashBf16Params {
     const uint16_t* q;

@@ -173,3 +173,19 @@ def test_backward_errors_before_any_device_use():
     err = L.RtErr()
     rc = L.lib().rt_flash_backward_f32_dev(None, C.byref(s), 16, 16, 16, 16, 16, 16, 16, 16, need - 1, C.byref(err))
     assert rc == L.RT_ERR_WORKSPACE_TOO_SMALL and (err.expected, err.got) == (need, need - 1)
+
+
+def test_saved_backward_argument_errors_before_any_device_use():
+    import ctypes as C
+    s = ra.AttentionShape.new(2, 3, 5, 8)._c()
+    err = L.RtErr()
+    need = 2 * 3 * 5 * 4
+    rc = L.lib().rt_flash_backward_saved_f32_dev(None, C.byref(s), *([16] * 9), 16, need - 4, C.byref(err))
+    assert rc == L.RT_ERR_WORKSPACE_TOO_SMALL and (err.expected, err.got) == (need, need - 4)
+    rc = L.lib().rt_flash_backward_saved_f32_dev(None, C.byref(s), 16, 16, 16, None, 16, 16, 16, 16, 16, 16, need,
+                                                 C.byref(err))
+    assert rc == L.RT_ERR_NULL_POINTER
+    z = ra.AttentionShape.new(1, 1, 4, 0)._c()
+    assert L.lib().rt_flash_forward_stats_f32_dev(None, C.byref(z), 16, 16, 16, 16, 16, C.byref(err)) == L.RT_ERR_ZERO_DIM
+    e = ra.AttentionShape.new(1, 1, 0, 4)._c()  # nothing to do: Ok without a device
+    assert L.lib().rt_flash_forward_stats_f32_dev(None, C.byref(e), 16, 16, 16, 16, 16, C.byref(err)) == L.RT_OK

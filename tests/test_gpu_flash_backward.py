@@ -169,3 +169,40 @@ def test_large_magnitude_scores(oracle):
     for name, g, w in zip(("dq", "dk", "dv"), got, want):
         assert np.isfinite(g).all()
         assert max_abs(g, w) <= 1e-4 * float(np.abs(w).max()), f"{name}: {max_abs(g, w):.3e} of {np.abs(w).max():.3e}"
+
+
+# ---- the saved-forward form -----------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("bhnd", [(1, 2, 70, 64), (2, 1, 45, 20), (1, 1, 200, 128), (1, 8, 256, 32)])
+def test_saved_forward_form(bhnd):
+    """rt_flash_forward_stats_f32_dev leaves the forward's output and lse = m + ln(l); the backward fed with them gives
+    the bits of the recomputing backward (it runs the same kernels on the same values)."""
+    b, h, n, d = bhnd
+    shape, bufs = inputs(bhnd, seeds=(61, 62, 63, 64))
+    q, k, v, d_out = bufs
+    dq_, dk_, dv_, dg = [dev(x) for x in bufs]
+    d_o, d_lse = ra.HipStorage.zeros(shape.buffer_len() * 4), ra.HipStorage.zeros(b * h * n * 4)
+    ra.flash_forward_stats_f32_dev(shape, dq_, dk_, dv_, d_o, d_lse)
+    ra.synchronize()
+    out, lse = d_o.download(np.float32), d_lse.download(np.float32)
+    assert np.array_equal(out, ra.flash_forward(shape, q, k, v))
+    s = np.einsum("bhid,bhjd->bhij", *[x.astype(np.float64).reshape(bhnd) for x in (q, k)]) / np.sqrt(np.float64(np.float32(d)))
+    m = s.max(axis=-1)
+    want_lse = m + np.log(np.exp(s - m[..., None]).sum(axis=-1))
+    assert max_abs(lse, want_lse.ravel()) <= 1e-5
+    grads = [ra.HipStorage.zeros(shape.buffer_len() * 4) for _ in range(3)]
+    ws = ra.HipStorage.zeros(b * h * n * 4)
+    ra.flash_backward_saved_f32_dev(shape, dq_, dk_, dv_, d_o, d_lse, dg, *grads, ws, ws.byte_len)
+    ra.synchronize()
+    want = ra.flash_backward(shape, *bufs)
+    for name, g, w in zip(("dq", "dk", "dv"), grads, want):
+        assert np.array_equal(g.download(np.float32), w), name
+
+
+def test_saved_forward_form_checks_workspace():
+    shape = ra.AttentionShape.new(1, 2, 8, 8)
+    buf = ra.HipStorage.zeros(4096)
+    with pytest.raises(ra.DeviceError) as ei:
+        ra.flash_backward_saved_f32_dev(shape, *([buf] * 9), buf, 63)
+    assert ei.value.status == L.RT_ERR_WORKSPACE_TOO_SMALL
