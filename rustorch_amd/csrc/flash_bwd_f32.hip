@@ -32,19 +32,22 @@ namespace {
 constexpr int kRows = 32;
 constexpr int kNW = 4;  // waves per workgroup
 
+template <int DPAD>
+struct TileRegs;
+template <int DPAD>
+__device__ __forceinline__ void load_tile_regs(TileRegs<DPAD>& t, const float* __restrict__ src, int row0, int N, int D,
+                                               int lane);
+template <int DPAD, int LD>
+__device__ __forceinline__ void store_tile_regs(float* dst, const TileRegs<DPAD>& t, int lane);
+
 // Copies rows [row0, row0 + 32) x [0, dim) of a [seq, dim] matrix into a 32 x LD LDS tile, zero beyond seq and dim.
 template <int DPAD, int LD>
 __device__ __forceinline__ void stage_tile(float* dst, const float* __restrict__ src, int row0, int N, int D, int lane,
                                            bool vec) {
-    constexpr int CH = DPAD / 4;
     if (vec) {
-#pragma unroll
-        for (int n = 0; n < kRows * CH / kWave; n++) {
-            const int idx = kWave * n + lane, r = idx / CH, c = idx % CH;
-            f32x4_t z = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (row0 + r < N && 4 * c < D) z = *(const f32x4_t*)(src + (size_t)(row0 + r) * D + 4 * c);
-            *(f32x4_t*)(dst + r * LD + 4 * c) = z;
-        }
+        TileRegs<DPAD> t;
+        load_tile_regs<DPAD>(t, src, row0, N, D, lane);
+        store_tile_regs<DPAD, LD>(dst, t, lane);
     } else {
         for (int idx = lane; idx < kRows * DPAD; idx += kWave) {
             const int r = idx / DPAD, d = idx - r * DPAD;
@@ -63,6 +66,14 @@ template <int DPAD>
 __device__ __forceinline__ void load_tile_regs(TileRegs<DPAD>& t, const float* __restrict__ src, int row0, int N, int D,
                                                int lane) {
     constexpr int CH = DPAD / 4;
+    if (D == DPAD && row0 + kRows <= N) {
+        // the whole tile is there and contiguous (row pitch == DPAD): one per-lane address, constant offsets, and no
+        // per-load bounds test (a wave-uniform condition)
+        const f32x4_t* base = (const f32x4_t*)(src + (size_t)row0 * DPAD) + lane;
+#pragma unroll
+        for (int n = 0; n < kRows * CH / kWave; n++) t.r[n] = base[kWave * n];
+        return;
+    }
 #pragma unroll
     for (int n = 0; n < kRows * CH / kWave; n++) {
         const int idx = kWave * n + lane, r = idx / CH, c = idx % CH;
@@ -200,29 +211,44 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dkdv_ker
     const int n_qt = (N + kRows - 1) / kRows;
     // at DT == 2 the registers of a second prefetched tile would cost the second wave per SIMD: dO is staged directly
     constexpr bool kPrefetchBoth = (DT != 2);
+    // A row beyond seq carries the statistic +inf and a key beyond seq the bias -inf: their weights come out of
+    // exp2 as exact zeros and the tile step has no data-dependent branch.
+    const float kbias = key_ok ? 0.0f : neg_inf();
     TileRegs<DPAD> ra, rb;
-    if (vec && wave < n_qt) {
-        load_tile_regs<DPAD>(ra, Qg, wave * kRows, N, D, lane);
-        if constexpr (kPrefetchBoth) load_tile_regs<DPAD>(rb, dOg, wave * kRows, N, D, lane);
+    float nl = 0.0f, nd = 0.0f;  // the next tile's statistic and delta of row `col`
+    auto load_stats = [&](int q0n) {
+        const bool ok = q0n + col < N;
+        nl = ok ? lse[q0n + col] : -neg_inf();
+        nd = ok ? delta[q0n + col] : 0.0f;
+    };
+    if (wave < n_qt) {
+        if (vec) {
+            load_tile_regs<DPAD>(ra, Qg, wave * kRows, N, D, lane);
+            if constexpr (kPrefetchBoth) load_tile_regs<DPAD>(rb, dOg, wave * kRows, N, D, lane);
+        }
+        load_stats(wave * kRows);
     }
     for (int qt = wave; qt < n_qt; qt += kNW) {
         const int q0 = qt * kRows;
+        const bool more = qt + kNW < n_qt;
         if (vec) {
             store_tile_regs<DPAD, LD>(Qt, ra, lane);
             if constexpr (kPrefetchBoth) store_tile_regs<DPAD, LD>(Ot, rb, lane);
             else stage_tile<DPAD, LD>(Ot, dOg, q0, N, D, lane, true);
-            if (qt + kNW < n_qt) {
-                load_tile_regs<DPAD>(ra, Qg, q0 + kNW * kRows, N, D, lane);
-                if constexpr (kPrefetchBoth) load_tile_regs<DPAD>(rb, dOg, q0 + kNW * kRows, N, D, lane);
-            }
         } else {
             stage_tile<DPAD, LD>(Qt, Qg, q0, N, D, lane, false);
             stage_tile<DPAD, LD>(Ot, dOg, q0, N, D, lane, false);
         }
         if (hh == 0) {
-            const bool ok = q0 + col < N;
-            stat[wave][0][col] = ok ? lse[q0 + col] : 0.0f;
-            stat[wave][1][col] = ok ? delta[q0 + col] : 0.0f;
+            stat[wave][0][col] = nl;
+            stat[wave][1][col] = nd;
+        }
+        if (more) {
+            if (vec) {
+                load_tile_regs<DPAD>(ra, Qg, q0 + kNW * kRows, N, D, lane);
+                if constexpr (kPrefetchBoth) load_tile_regs<DPAD>(rb, dOg, q0 + kNW * kRows, N, D, lane);
+            }
+            load_stats(q0 + kNW * kRows);
         }
         f32x16_t s, dp;
 #pragma unroll
@@ -243,8 +269,7 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dkdv_ker
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             const int qr = 8 * (i >> 2) + 4 * hh + (i & 3);
-            const bool ok = key_ok && (q0 + qr < N);
-            const float pv = ok ? __builtin_amdgcn_exp2f((s[i] * p.scale - stat[wave][0][qr]) * kLog2e) : 0.0f;
+            const float pv = __builtin_amdgcn_exp2f(((s[i] * p.scale - stat[wave][0][qr]) + kbias) * kLog2e);
             s[i] = pv;
             dp[i] = pv * (dp[i] - stat[wave][1][qr]) * p.scale;
         }
@@ -305,8 +330,11 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dq_kerne
         }
     }
     const bool q_ok = q0 + col < N;
-    const float lse_q = q_ok ? p.lse[bh * (size_t)N + q0 + col] : 0.0f;
-    const float delta_q = q_ok ? p.delta[bh * (size_t)N + q0 + col] : 0.0f;
+    // a row beyond seq carries the statistic +inf: all its weights come out of exp2 as exact zeros
+    float lse_q = q_ok ? p.lse[bh * (size_t)N + q0 + col] : -neg_inf();
+    float delta_q = q_ok ? p.delta[bh * (size_t)N + q0 + col] : 0.0f;
+    // have the two loads land here: a wait for them inside the loop would also wait for the tile prefetched there
+    asm volatile("" : "+v"(lse_q), "+v"(delta_q));
 
     f32x16_t acc_dq[DT];
 #pragma unroll
@@ -347,11 +375,13 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dq_kerne
             }
         }
         // register i holds key row 8*(i/4) + 4*hh + (i%4) of the tile, query q0 + col
+        const bool edge = kv0 + kRows > N;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             const int kr = 8 * (i >> 2) + 4 * hh + (i & 3);
-            const bool ok = q_ok && (kv0 + kr < N);
-            const float pv = ok ? __builtin_amdgcn_exp2f((s[i] * p.scale - lse_q) * kLog2e) : 0.0f;
+            float arg = s[i] * p.scale - lse_q;
+            if (edge) arg = (kv0 + kr < N) ? arg : neg_inf();  // keys beyond seq, last tile only (uniform branch)
+            const float pv = __builtin_amdgcn_exp2f(arg * kLog2e);
             dp[i] = pv * (dp[i] - delta_q) * p.scale;
         }
         // dQ^T += K^T . dS^T, two keys per instruction

@@ -264,6 +264,19 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
     const uint32_t ld_off = (uint32_t)ld_r * (uint32_t)kv_pitch * 4u + (uint32_t)ld_c * 16u;  // bytes; a few rows: fits
     f32x4_t kreg[NLD], vreg[NLD];
     auto issue_loads = [&](int tile) {
+        if constexpr (kEvenRows) {
+            if (tile * kRows + kRows <= N) {  // whole tile present (wave-uniform): no per-load bounds test
+                const char* kb = (const char*)Kg + (size_t)tile * kRows * kv_pitch * sizeof(float) + ld_off;
+                const char* vb = (const char*)Vg + (size_t)tile * kRows * kv_pitch * sizeof(float) + ld_off;
+#pragma unroll
+                for (int n = 0; n < NLD; n++) {
+                    const size_t step = (size_t)(RPL * n) * kv_pitch * sizeof(float);  // uniform
+                    kreg[n] = *(const f32x4_t*)(kb + step);
+                    vreg[n] = *(const f32x4_t*)(vb + step);
+                }
+                return;
+            }
+        }
 #pragma unroll
         for (int n = 0; n < NLD; n++) {
             f32x4_t zk = {0.0f, 0.0f, 0.0f, 0.0f}, zv = zk;
