@@ -39,9 +39,9 @@ PEAK_F32_TFLOPS = 157.3     # MI355X dense f32 MFMA
 # Counters cannot be read from inside this process; these are the committed measurements, not live values.
 TRAFFIC_PREFILL_BYTES = (270900 * 2.0 + 131100 * 1.0) * 1024
 TRAFFIC_DECODE_BYTES = (623700 * 2.0 + 3224 * 1.0) * 1024
-TRAFFIC_F32_BYTES = (6239 * 2.0 + 4096 * 1.0) * 1024
-# the four kernels of one backward step (forward, delta, dK/dV, dQ): FETCH_SIZE 6242 + 4109 + 8604 + 8335, WRITE_SIZE 4160 + 128 + 8704 + 4096
-TRAFFIC_BWD_BYTES = (27290 * 2.0 + 17088 * 1.0) * 1024
+TRAFFIC_F32_BYTES = (6254 * 2.0 + 4096 * 1.0) * 1024
+# the four kernels of one backward step (forward, delta, dK/dV, dQ): FETCH_SIZE 6248 + 4109 + 8343 + 9359, WRITE_SIZE 4160 + 128 + 8192 + 6144
+TRAFFIC_BWD_BYTES = (28059 * 2.0 + 18624 * 1.0) * 1024
 
 
 class Hip:
