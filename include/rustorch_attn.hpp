@@ -298,6 +298,26 @@ inline std::vector<float> mha_forward_masked_f32(const std::vector<float>& q, co
     return out;
 }
 
+// The branch MultiHeadAttention::forward takes for the attention between its projections, under no_grad on contiguous
+// f32 tensors (attention.rs:325-333, :347-356).
+enum class MhaRoute { Identity, Flash, Composed };
+inline MhaRoute mha_attention_route(size_t t_q, size_t t_kv, bool has_mask) {
+    if (!has_mask && t_q == 1 && t_kv == 1) return MhaRoute::Identity;  // softmax over one position is 1
+    if (!has_mask && t_q == t_kv) return MhaRoute::Flash;
+    return MhaRoute::Composed;
+}
+// Projected q [B,t_q,H*hd], k, v [B,t_kv,H*hd] -> context [B,t_q,H*hd] with that routing.
+inline std::vector<float> mha_attention_f32(const std::vector<float>& q, const std::vector<float>& k,
+                                            const std::vector<float>& v, size_t batch, size_t t_q, size_t t_kv,
+                                            size_t heads, size_t head_dim,
+                                            const std::vector<float>& attn_mask = std::vector<float>()) {
+    switch (mha_attention_route(t_q, t_kv, !attn_mask.empty())) {
+        case MhaRoute::Identity: return v;
+        case MhaRoute::Flash: return mha_flash_forward_f32(q, k, v, batch, t_q, heads, head_dim);
+        default: return mha_forward_masked_f32(q, k, v, batch, t_q, t_kv, heads, head_dim, attn_mask);
+    }
+}
+
 // ---- device memory --------------------------------------------------------------------------------------
 
 class HipStorage {

@@ -225,6 +225,32 @@ def mha_forward_masked_f32(q, k, v, batch: int, t_q: int, t_kv: int, heads: int,
     return out
 
 
+def mha_attention_route(t_q: int, t_kv: int, has_mask: bool) -> str:
+    """Which branch `MultiHeadAttention::forward` takes for the attention between its projections, under no_grad on
+    contiguous f32 tensors (crates/rustorch-nn/src/attention.rs:325-333, :347-356): "identity" for the single-token
+    shortcut (softmax over one position is 1, the context is V), "flash" for unmasked self-attention of equal lengths,
+    "composed" when a mask is given or the lengths differ."""
+    if not has_mask and t_q == 1 and t_kv == 1:
+        return "identity"
+    if not has_mask and t_q == t_kv:
+        return "flash"
+    return "composed"
+
+
+def mha_attention_f32(q, k, v, batch: int, t_q: int, t_kv: int, heads: int, head_dim: int, attn_mask=None):
+    """The attention between the projections of `MultiHeadAttention::forward` with the reference's routing
+    (attention.rs:325-399): projected q [B,t_q,H*hd], k, v [B,t_kv,H*hd] -> context [B,t_q,H*hd], flat f32."""
+    route = mha_attention_route(t_q, t_kv, attn_mask is not None)
+    if route == "identity":
+        v, _ = _f32(v)
+        if v.size != batch * heads * head_dim:
+            raise ValueError(f"v has {v.size} elements, expected {batch * heads * head_dim}")
+        return v.copy()
+    if route == "flash":
+        return mha_flash_forward_f32(q, k, v, batch, t_q, heads, head_dim)
+    return mha_forward_masked_f32(q, k, v, batch, t_q, t_kv, heads, head_dim, attn_mask)
+
+
 def flash_forward_bnhd_f32_dev(shape, q, k, v, out, mask: Mask = None, keep_dev=None, n_kv_heads=0, stream=None):
     """f32 [B,N,H,D] device tensors (k, v: [B,N,Hkv,D]); `shape` is still (batch, heads, seq, dim)."""
     mask = mask or Mask.none()

@@ -128,6 +128,15 @@ static void test_errors() {
         std::vector<float> e;
         flash_backward(AttentionShape::make(1, 1, 0, 4), e, e, e, e, e, e, e);  // cpu_backward.rs:252-260
     }
+    {   // the routing of MultiHeadAttention::forward (attention.rs:325-333, :347-356)
+        CHECK(mha_attention_route(1, 1, false) == MhaRoute::Identity);
+        CHECK(mha_attention_route(1, 1, true) == MhaRoute::Composed);
+        CHECK(mha_attention_route(64, 64, false) == MhaRoute::Flash);
+        CHECK(mha_attention_route(64, 64, true) == MhaRoute::Composed);
+        CHECK(mha_attention_route(1, 64, false) == MhaRoute::Composed);
+        std::vector<float> v = {1, 2, 3, 4, 5, 6, 7, 8};
+        CHECK(mha_attention_f32(v, v, v, 2, 1, 1, 2, 2) == v);  // needs no device
+    }
     {   // GQA: head counts first, then q, k, v, out (gqa.rs:106-141)
         std::vector<float> q(20), kv(8), out(20);
         GQAError err(GQAError::Kind::WrongInputLen, "", 0, 0, "");

@@ -82,3 +82,21 @@ def test_error_order():
     with pytest.raises(ra.WrongInputLen) as e:
         ra.mha_forward_masked_f32(z(nq), z(nk), z(nk), b, tq, tkv, h, d, attn_mask=z(5))
     assert (e.value.which, e.value.expected, e.value.got) == ("mask", tq * tkv, 5)
+
+
+def test_routing_of_multi_head_attention(oracle):
+    """attention.rs:325-399: single token without mask -> the context is V; unmasked equal lengths -> the flash path;
+    a mask or unequal lengths -> the composed path.  All three agree with the oracle's composed core."""
+    rng = np.random.default_rng(11)
+    for b, tq, tkv, h, d, masked in [(3, 1, 1, 2, 8, False), (2, 40, 40, 2, 32, False), (2, 40, 40, 2, 32, True),
+                                     (1, 5, 9, 2, 16, False), (2, 1, 1, 2, 8, True)]:
+        q = rng.standard_normal(b * tq * h * d).astype(np.float32)
+        k = rng.standard_normal(b * tkv * h * d).astype(np.float32)
+        v = rng.standard_normal(b * tkv * h * d).astype(np.float32)
+        mask = ra.causal_mask(tq) if masked and tq == tkv else None
+        route = ra.mha_attention_route(tq, tkv, mask is not None)
+        got = ra.mha_attention_f32(q, k, v, b, tq, tkv, h, d, mask)
+        want = oracle.mha_forward_masked(q, k, v, b, tq, tkv, h, d, mask)
+        assert np.abs(got - want).max() <= 1e-5, route
+        if route == "identity":
+            assert np.array_equal(got, v)

@@ -40,3 +40,16 @@ def test_errors_follow_the_reference():
     y = x.copy()
     ra.RoPE(4, 8).apply_inplace(y, 1, 1, 1, 0)
     assert np.abs(y - x).max() < 1e-6  # position 0 is the identity (rope.rs:247-256)
+
+
+def test_multi_head_attention_routing_rule():
+    """The branch MultiHeadAttention::forward takes (crates/rustorch-nn/src/attention.rs:325-333, :347-356)."""
+    import rustorch_amd as ra
+    assert ra.mha_attention_route(1, 1, False) == "identity"
+    assert ra.mha_attention_route(1, 1, True) == "composed"
+    assert ra.mha_attention_route(128, 128, False) == "flash"
+    assert ra.mha_attention_route(128, 128, True) == "composed"
+    assert ra.mha_attention_route(1, 64, False) == "composed"
+    v = np.arange(2 * 3 * 4, dtype=np.float32)
+    out = ra.mha_attention_f32(v, v, v, 2, 1, 1, 3, 4)  # the identity route needs no device
+    assert np.array_equal(out, v) and out is not v
