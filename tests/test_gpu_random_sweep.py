@@ -107,3 +107,25 @@ def test_random_cases_match_oracle(oracle, seed):
     cases = (_bf16_prefill, _f32_prefill, _decode, _varlen)
     for _ in range(60):
         cases[int(rng.integers(0, len(cases)))](oracle, rng)
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_backward_cases_match_oracle(oracle, seed):
+    """f32 backward on random shapes (every head dim class, ragged tails, single rows), inputs in (-1, 1) or N(0, 0.5);
+    max-abs <= 2e-5 relative to gradients of order one."""
+    rng = np.random.default_rng(seed)
+    for _ in range(40):
+        b, h = int(rng.integers(1, 3)), int(rng.integers(1, 10))
+        n = int(rng.choice([1, 2, 5, 31, 32, 33, 64, 65, 100, 129, 200, 257]))
+        d = int(rng.choice([1, 4, 8, 20, 24, 32, 40, 64, 72, 96, 100, 128]))
+        size = b * h * n * d
+        if rng.integers(0, 2):
+            bufs = [rng.uniform(-1.0, 1.0, size).astype(np.float32) for _ in range(4)]
+        else:
+            bufs = [(rng.standard_normal(size) * 0.5).astype(np.float32) for _ in range(4)]
+        got = ra.flash_backward(ra.AttentionShape.new(b, h, n, d), *bufs)
+        want = oracle.flash_backward(oracle.AttentionShape(b, h, n, d), *bufs)
+        for name, g, w in zip(("dq", "dk", "dv"), got, want):
+            err = float(np.abs(g - w).max())
+            assert np.isfinite(g).all() and err <= 2e-5 * max(1.0, float(np.abs(w).max())), \
+                f"backward B{b} H{h} N{n} D{d} {name}: max-abs {err}"
