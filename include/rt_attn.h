@@ -251,7 +251,11 @@ int rt_qk_norm_rope_kv_append_bf16(void *stream, void *q, const void *k_in, cons
 
 /* LlmKernels::gqa_decode_online_bf16 -- llm_kernels.rs:396-457, :915-958.  q/out
  * [n_heads,head_dim] bf16, caches [n_kv,max_seq,head_dim] bf16 of which [..kv_len] is read;
- * kv head = h*n_kv/n_heads; f32 accumulation, output rounded once. */
+ * kv head = h*n_kv/n_heads; f32 accumulation, output rounded once.  Runs the split-K kernels of the batched entry on
+ * a batch of one (head_dim 64 or 128, at most 16 query heads per kv head; other shapes take a one-workgroup-per-head
+ * kernel).  The reference's signature has no workspace: the partials go to a buffer the library keeps per
+ * (device, stream), allocated by the first call on a stream (so that call must not be under stream capture; later
+ * calls allocate nothing unless max_seq grows). */
 int rt_gqa_decode_online_bf16(void *stream, const void *q, const void *k_cache, const void *v_cache, void *out,
                               int32_t n_heads, int32_t n_kv, int32_t kv_len, int32_t head_dim, int32_t max_seq,
                               rt_err_detail *err);

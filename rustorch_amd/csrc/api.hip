@@ -7,6 +7,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <map>
 #include <mutex>
 
 #include "../../include/rt_attn.h"
@@ -165,6 +166,38 @@ int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n
         p.lkv = rt::layout_bhnd((long long)n_kv_heads, (long long)s->seq, p.dim);
     }
     HIP_TRY(rt::launch_flash_f32(stream, p), "flash_fwd_f32 launch");
+    return RT_OK;
+}
+
+// Scratch the library keeps for entry points whose reference signature has no workspace argument: one buffer per
+// (device, stream), allocated on the first call that needs it, grown when a later call needs more, and kept until
+// the process ends.  Calls on one stream are ordered, so they can share it; calls on different streams get
+// different buffers.  The first call on a stream allocates (hipMalloc): not for use under stream capture.
+struct StreamWs {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+std::mutex g_ws_mutex;
+std::map<std::pair<int, hipStream_t>, StreamWs> g_ws;
+
+int stream_workspace(hipStream_t stream, size_t bytes, float** out, rt_err_detail* err) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev), "hipGetDevice");
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    StreamWs& w = g_ws[{dev, stream}];
+    if (w.bytes < bytes) {
+        if (w.ptr) {
+            // kernels already enqueued on the stream may still use the old buffer
+            HIP_TRY(hipStreamSynchronize(stream), "hipStreamSynchronize");
+            HIP_TRY(hipFree(w.ptr), "hipFree workspace");
+            w.ptr = nullptr;
+            w.bytes = 0;
+        }
+        size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
+        HIP_TRY(hipMalloc(&w.ptr, want), "hipMalloc workspace");
+        w.bytes = want;
+    }
+    *out = (float*)w.ptr;
     return RT_OK;
 }
 
@@ -798,6 +831,35 @@ RT_API int rt_gqa_decode_online_bf16(void* stream, const void* q, const void* k_
     if (!q || !out || (kv_len > 0 && (!k_cache || !v_cache))) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
     rc = ensure_device(err);
     if (rc) return rc;
+    if (rt::decode_split_supported(n_heads, n_kv, head_dim)) {
+        // the split-K kernels of the batched entry, on a batch of one; their partials go to a buffer the library keeps
+        // per stream (the reference's signature has no workspace argument)
+        float* ws = nullptr;
+        rc = stream_workspace((hipStream_t)stream, rt::decode_split_workspace_bytes(1, n_heads, head_dim, max_seq), &ws, err);
+        if (rc) return rc;
+        rt::DecodeSplitParams sp{};
+        sp.q = (const uint16_t*)q;
+        sp.k_cache = (const uint16_t*)k_cache;
+        sp.v_cache = (const uint16_t*)v_cache;
+        sp.out = (uint16_t*)out;
+        sp.kv_lens = nullptr;
+        sp.kv_len = kv_len;
+        sp.ws = ws;
+        sp.batch = 1;
+        sp.heads = n_heads;
+        sp.kv_heads = n_kv;
+        sp.dim = head_dim;
+        sp.max_seq = max_seq;
+        sp.n_part = rt::decode_split_parts(1, max_seq);
+        sp.span_min = rt::decode_split_span_min(1);
+        // no more one-wave workgroups than there are spans of the minimum length (short contexts)
+        const long long steps = (long long)n_kv * ((kv_len + 31) / 32);
+        const long long spans = (steps + sp.span_min - 1) / sp.span_min;
+        sp.n_waves = (int)std::min<long long>(g_decode_waves, std::max<long long>(spans, 1));
+        sp.scale_log2e = (1.0f / sqrtf((float)head_dim)) * rt::kLog2eHost;
+        HIP_TRY(rt::launch_decode_split((hipStream_t)stream, sp), "decode_split launch");
+        return RT_OK;
+    }
     rt::AttnRowsParams p{};
     p.q = q;
     p.k = k_cache;
@@ -840,7 +902,7 @@ RT_API int rt_gqa_decode_batched_bf16(void* stream, const void* q, const void* k
         size_t need = rt::decode_split_workspace_bytes(batch, n_heads, head_dim, max_seq);
         if (!workspace || workspace_bytes < need)
             return fail(err, RT_ERR_WORKSPACE_TOO_SMALL, -1, need, workspace ? workspace_bytes : 0, "workspace too small");
-        rt::DecodeSplitParams p;
+        rt::DecodeSplitParams p{};
         p.q = (const uint16_t*)q;
         p.k_cache = (const uint16_t*)k_cache;
         p.v_cache = (const uint16_t*)v_cache;
@@ -852,7 +914,8 @@ RT_API int rt_gqa_decode_batched_bf16(void* stream, const void* q, const void* k
         p.kv_heads = n_kv;
         p.dim = head_dim;
         p.max_seq = max_seq;
-        p.n_part = rt::decode_split_parts(max_seq);
+        p.n_part = rt::decode_split_parts(batch, max_seq);
+        p.span_min = rt::decode_split_span_min(batch);
         p.n_waves = g_decode_waves;
         p.scale_log2e = (1.0f / sqrtf((float)head_dim)) * rt::kLog2eHost;
         HIP_TRY(rt::launch_decode_split((hipStream_t)stream, p), "decode_split launch");

@@ -164,10 +164,13 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(AttnRowsParams p) {
 // stand are the 8 contraction slots of its B operand for the second product; the V operand is
 // fetched with the same slot -> key map.
 constexpr int kDecRows = 32;     // key rows per step
-constexpr int kDecSpanMin = 8;   // a wave takes at least this many steps (bounds the partials per segment)
+constexpr int kDecSpanMin = 8;   // a wave takes at least this many steps (bounds the partials per segment); batches
+constexpr int kDecSpanMinOne = 2;  // the same for a single sequence, where the latency of one call is what counts
 
 __device__ __forceinline__ int dec_steps(int len) { return (len + kDecRows - 1) / kDecRows; }
-__device__ __forceinline__ int dec_len(const DecodeSplitParams& p, int b) { return min(max(p.kv_lens[b], 0), p.max_seq); }
+__device__ __forceinline__ int dec_len(const DecodeSplitParams& p, int b) {
+    return min(max(p.kv_lens ? p.kv_lens[b] : p.kv_len, 0), p.max_seq);
+}
 
 __device__ __forceinline__ int wave_sum_i(int x) {
 #pragma unroll
@@ -191,7 +194,7 @@ __device__ __forceinline__ void dec_total(const DecodeSplitParams& p, int lane, 
         t += wave_sum_i(i < p.batch ? p.kv_heads * dec_steps(dec_len(p, i)) : 0);
     }
     total = t;
-    span = max((t + p.n_waves - 1) / p.n_waves, kDecSpanMin);
+    span = max((t + p.n_waves - 1) / p.n_waves, p.span_min);
 }
 // First step (in the flat list) of sequence b.
 __device__ __forceinline__ int dec_seq_start(const DecodeSplitParams& p, int lane, int b) {
@@ -423,10 +426,14 @@ __global__ __launch_bounds__(64) void decode_split_kernel(DecodeSplitParams p) {
     }
 }
 
-// grid (heads, batch), 64 * ceil(HD/64) threads: thread d folds element d of the head's partials.
-template <int HD>
-__global__ __launch_bounds__(HD < 64 ? 64 : HD) void decode_merge_kernel(DecodeSplitParams p) {
-    const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+// grid (heads, batch), NS * HD threads: thread (d, j) folds element d of the partials j, j + NS, ... (in groups of
+// eight) of the head, and the NS running states are combined through LDS.  NS = 1 for batches, where a head has a
+// handful of partials; NS = 4 for a single sequence, whose keys are cut into many short spans to keep the latency
+// of the call low and whose heads then have up to a hundred partials each.
+template <int HD, int NS>
+__global__ __launch_bounds__((HD < 64 ? 64 : HD) * NS) void decode_merge_kernel(DecodeSplitParams p) {
+    constexpr int TD = HD < 64 ? 64 : HD;  // threads per sub-state
+    const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x % TD, sub = threadIdx.x / TD;
     const int lane = threadIdx.x & 63;
     const int G = p.heads / p.kv_heads;
     const int kvh = h / G;
@@ -439,19 +446,20 @@ __global__ __launch_bounds__(HD < 64 ? 64 : HD) void decode_merge_kernel(DecodeS
     const float* ws_o = p.ws;
     const float* ws_ml = p.ws + (size_t)p.batch * p.heads * p.n_part * HD;
     const size_t slot0 = ((size_t)b * p.heads + h) * p.n_part;
-    // One pass over the partials, eight at a time: the loads of a group are independent of each other (a head of a
-    // long sequence has a hundred partials, and one dependent load after the other would cost more than the
-    // split kernel), and the running (m, acc, l) is rescaled once per group.
+    const int dd = d < HD ? d : HD - 1;
+    // One pass over the partials, eight at a time: the loads of a group are independent of each other (one dependent
+    // load after the other would cost more than the split kernel), and the running (m, acc, l) is rescaled once
+    // per group.
     constexpr int kGroup = 8;
     float m_all = neg_inf(), acc = 0.0f, l_all = 0.0f;
-    for (int k0 = 0; k0 < n_valid; k0 += kGroup) {
+    for (int k0 = sub * kGroup; k0 < n_valid; k0 += NS * kGroup) {
         float mv[kGroup], lv[kGroup], ov[kGroup];
 #pragma unroll
         for (int j = 0; j < kGroup; j++) {
             const int k = min(k0 + j, n_valid - 1);  // repeats of the last partial are given weight 0 below
             mv[j] = ws_ml[(slot0 + k) * 2];
             lv[j] = ws_ml[(slot0 + k) * 2 + 1];
-            ov[j] = ws_o[(slot0 + k) * HD + d];
+            ov[j] = ws_o[(slot0 + k) * HD + dd];
         }
         float m_new = m_all;
 #pragma unroll
@@ -468,9 +476,31 @@ __global__ __launch_bounds__(HD < 64 ? 64 : HD) void decode_merge_kernel(DecodeS
         }
         m_all = m_new;
     }
+    if constexpr (NS > 1) {
+        __shared__ float sm_acc[NS][TD], sm_m[NS], sm_l[NS];
+        sm_acc[sub][d] = acc;
+        if (d == 0) {
+            sm_m[sub] = m_all;
+            sm_l[sub] = l_all;
+        }
+        __syncthreads();
+        if (sub != 0) return;
+        float m_tot = neg_inf();
+#pragma unroll
+        for (int j = 0; j < NS; j++) m_tot = fmaxf(m_tot, sm_m[j]);
+        const float m_use = (m_tot == neg_inf()) ? 0.0f : m_tot;
+        acc = 0.0f;
+        l_all = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NS; j++) {
+            const float cw = (sm_m[j] == neg_inf()) ? 0.0f : __builtin_amdgcn_exp2f(sm_m[j] - m_use);  // empty state
+            acc += sm_acc[j][d] * cw;
+            l_all += sm_l[j] * cw;
+        }
+    }
     // kv_len == 0: no key contributes, the output row is zero (gqa.rs:261; llm_kernels.rs:456)
     float r = n_valid > 0 ? acc / l_all : 0.0f;
-    p.out[((size_t)b * p.heads + h) * HD + d] = f32_to_bf16_bits(r);
+    if (d < HD) p.out[((size_t)b * p.heads + h) * HD + d] = f32_to_bf16_bits(r);
 }
 
 __global__ void kv_append_kernel(uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache,
@@ -508,7 +538,11 @@ hipError_t launch_split_hd(hipStream_t stream, const DecodeSplitParams& p) {
     hipLaunchKernelGGL(decode_split_kernel<HD>, dim3(p.n_waves), dim3(64), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(decode_merge_kernel<HD>, dim3(p.heads, p.batch), dim3(HD), 0, stream, p);
+    constexpr int TD = HD < 64 ? 64 : HD;
+    if (p.batch == 1)
+        hipLaunchKernelGGL((decode_merge_kernel<HD, 4>), dim3(p.heads, p.batch), dim3(TD * 4), 0, stream, p);
+    else
+        hipLaunchKernelGGL((decode_merge_kernel<HD, 1>), dim3(p.heads, p.batch), dim3(TD), 0, stream, p);
     return hipGetLastError();
 }
 
@@ -520,18 +554,21 @@ bool decode_split_supported(int heads, int kv_heads, int dim) {
     return (dim == 64 || dim == 128) && g <= 16;
 }
 
-int decode_split_parts(int max_seq) {
+int decode_split_span_min(int batch) { return batch == 1 ? kDecSpanMinOne : kDecSpanMin; }
+
+int decode_split_parts(int batch, int max_seq) {
     int steps_max = (max_seq + kDecRows - 1) / kDecRows;
-    return (steps_max + kDecSpanMin - 1) / kDecSpanMin + 1;
+    int span_min = decode_split_span_min(batch);
+    return (steps_max + span_min - 1) / span_min + 1;
 }
 
 size_t decode_split_workspace_bytes(int batch, int heads, int dim, int max_seq) {
-    return (size_t)batch * heads * decode_split_parts(max_seq) * ((size_t)dim + 2) * sizeof(float);
+    return (size_t)batch * heads * decode_split_parts(batch, max_seq) * ((size_t)dim + 2) * sizeof(float);
 }
 
 hipError_t launch_decode_split(hipStream_t stream, const DecodeSplitParams& p) {
     if (p.batch == 0 || p.heads == 0) return hipSuccess;
-    if (p.n_waves <= 0) return hipErrorInvalidValue;
+    if (p.n_waves <= 0 || p.span_min <= 0) return hipErrorInvalidValue;
     if (p.dim == 64) return launch_split_hd<64>(stream, p);
     if (p.dim == 128) return launch_split_hd<128>(stream, p);
     return hipErrorInvalidValue;

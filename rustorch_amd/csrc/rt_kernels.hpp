@@ -117,15 +117,18 @@ struct DecodeSplitParams {
     const uint16_t* k_cache;  // [batch, kv_heads, max_seq, dim]
     const uint16_t* v_cache;
     uint16_t* out;            // [batch, heads, dim]
-    const int32_t* kv_lens;   // device int32[batch]
+    const int32_t* kv_lens;   // device int32[batch], or nullptr: every sequence has kv_len keys
+    int kv_len;
     float* ws;                // partial (o, m, l) per (b, head, chunk)
     int batch, heads, kv_heads, dim, max_seq;
-    int n_part;   // partial slots per (sequence, head): decode_split_parts(max_seq)
+    int n_part;   // partial slots per (sequence, head): decode_split_parts(batch, max_seq)
+    int span_min;  // a wave takes at least this many 32-key steps: decode_split_span_min(batch)
     int n_waves;  // one-wave workgroups launched (all resident at once)
     float scale_log2e;
 };
 bool decode_split_supported(int heads, int kv_heads, int dim);
-int decode_split_parts(int max_seq);
+int decode_split_span_min(int batch);
+int decode_split_parts(int batch, int max_seq);
 size_t decode_split_workspace_bytes(int batch, int heads, int dim, int max_seq);
 hipError_t launch_decode_split(hipStream_t stream, const DecodeSplitParams& p);
 

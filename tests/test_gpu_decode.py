@@ -133,3 +133,30 @@ def test_config_decode_b64_h32_kv8_d128_lmax8192(oracle):
     want = oracle.gqa_decode_batched_bf16(qb, kb, vb, lens, b, hq, hkv, d, max_seq)
     assert np.isfinite(got).all()
     assert max_abs(got, want) <= TOL, f"lens={lens.tolist()}"
+
+
+def test_single_sequence_decode_long_contexts_and_streams(oracle):
+    """The reference call on the split-K path: contexts long enough for a hundred partials per head, a cache that
+    grows between calls (the library's per-stream buffer is re-sized), and two streams used alternately (each has
+    a buffer of its own)."""
+    from _gpu import new_stream
+
+    ra.init(0)
+    hq, hkv, d = 32, 8, 128
+    streams = [None, new_stream(), new_stream()]
+    for max_seq, kv_lens in [(96, [1, 33, 96]), (8192, [8192, 4097, 2048, 65]), (300, [300])]:
+        qb, _ = bf16_round(seeded_normal((hq, d), max_seq))
+        kb, _ = bf16_round(seeded_normal((hkv, max_seq, d), max_seq + 1))
+        vb, _ = bf16_round(seeded_normal((hkv, max_seq, d), max_seq + 2))
+        dq, dk, dv = dev(qb), dev(kb), dev(vb)
+        outs = []
+        for i, kv_len in enumerate(kv_lens):
+            st = streams[i % len(streams)]
+            dout = ra.HipStorage(hq * d * 2)
+            K.gqa_decode_online_bf16(st, dq, dk, dv, dout, hq, hkv, kv_len, d, max_seq)
+            outs.append((kv_len, dout))
+        for st in streams:
+            ra.synchronize(st)
+        for kv_len, dout in outs:
+            want = oracle.gqa_decode_batched_bf16(qb, kb, vb, [kv_len], 1, hq, hkv, d, max_seq)
+            assert max_abs(oracle.bf16_to_f32(dout.download(np.uint16)), want) <= TOL, (max_seq, kv_len)
