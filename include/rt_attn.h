@@ -284,6 +284,10 @@ int rt_buf_zero(void *ptr, size_t bytes, void *stream, rt_err_detail *err);
 int rt_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream, rt_err_detail *err);
 int rt_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream, rt_err_detail *err);
 int rt_stream_synchronize(void *stream, rt_err_detail *err);
+/* A stream at the default priority for the device entry points (the place of the reference's Arc<CudaStream>,
+ * crates/rustorch-cuda/src/llm_kernels.rs:874-880); NULL and err filled on failure. */
+void *rt_stream_create(rt_err_detail *err);
+int rt_stream_destroy(void *stream, rt_err_detail *err);
 
 #ifdef __cplusplus
 }

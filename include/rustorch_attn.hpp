@@ -374,6 +374,27 @@ private:
     size_t bytes_ = 0;
 };
 
+// A stream at the default priority (the place of the reference's Arc<CudaStream>); get() is what the device entry
+// points take.
+class Stream {
+public:
+    Stream() {
+        rt_err_detail e;
+        h_ = rt_stream_create(&e);
+        if (!h_) detail::throw_device(e.hip_error ? RT_ERR_HIP : RT_ERR_NO_DEVICE, e);
+    }
+    Stream(const Stream&) = delete;
+    Stream& operator=(const Stream&) = delete;
+    ~Stream() {
+        rt_err_detail e;
+        if (h_) (void)rt_stream_destroy(h_, &e);
+    }
+    void* get() const { return h_; }
+
+private:
+    void* h_ = nullptr;
+};
+
 inline void synchronize(void* stream = nullptr) {
     rt_err_detail e;
     detail::check_device(rt_stream_synchronize(stream, &e), e);

@@ -22,6 +22,7 @@ SYMBOLS = (
     "rt_kv_append_bf16", "rt_kv_cache_append_dev", "rt_qk_norm_rope_kv_append_bf16", "rt_gqa_decode_online_bf16", "rt_gqa_decode_batched_bf16",
     "rt_gqa_decode_workspace_bytes",
     "rt_buf_alloc", "rt_buf_free", "rt_buf_zero", "rt_memcpy_h2d", "rt_memcpy_d2h", "rt_stream_synchronize",
+    "rt_stream_create", "rt_stream_destroy",
 )
 
 RT_OK = 0
@@ -109,6 +110,9 @@ def lib():
     L.rt_memcpy_h2d.argtypes = [vp, vp, sz, vp, errp]
     L.rt_memcpy_d2h.argtypes = [vp, vp, sz, vp, errp]
     L.rt_stream_synchronize.argtypes = [vp, errp]
+    L.rt_stream_create.argtypes = [errp]
+    L.rt_stream_create.restype = vp
+    L.rt_stream_destroy.argtypes = [vp, errp]
     _lib = L
     return L
 

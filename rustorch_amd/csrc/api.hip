@@ -137,7 +137,7 @@ int check_flash_dims(const rt_attention_shape* s, uint64_t n_kv_heads, rt_err_de
 int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n_kv_heads, const float* q,
                      const float* k, const float* v, int mask_kind, const uint8_t* keep, float* out,
                      rt_err_detail* err, bool bnhd = false, const float* bias = nullptr, long long bias_bh_stride = 0,
-                     float* lse = nullptr) {
+                     float* lse = nullptr, uint64_t seq_kv = 0) {
     if (s->dim > 256) return fail(err, RT_ERR_UNSUPPORTED, -1, 256, s->dim, "f32 flash kernels cover dim <= 256");
     rt::FlashF32Params p{};
     p.bias = bias;
@@ -154,16 +154,18 @@ int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n
     p.group = (int)(s->heads / n_kv_heads);
     p.seq = (int)s->seq;
     p.dim = (int)s->dim;
+    p.seq_kv = (int)seq_kv;
     p.mask = mask_kind;
     p.ref_bc = (int)(s->bc == 0 ? 1 : (s->bc > 0x7fffffffull ? 0x7fffffff : s->bc));
     p.scale = 1.0f / sqrtf((float)s->dim);
     p.n_cus = g_num_cus;
+    const long long kv_rows = (long long)(seq_kv ? seq_kv : s->seq);
     if (bnhd) {
         p.lq = p.lo = rt::layout_bnhd((long long)s->heads, (long long)s->seq, p.dim);
-        p.lkv = rt::layout_bnhd((long long)n_kv_heads, (long long)s->seq, p.dim);
+        p.lkv = rt::layout_bnhd((long long)n_kv_heads, kv_rows, p.dim);
     } else {
         p.lq = p.lo = rt::layout_bhnd((long long)s->heads, (long long)s->seq, p.dim);
-        p.lkv = rt::layout_bhnd((long long)n_kv_heads, (long long)s->seq, p.dim);
+        p.lkv = rt::layout_bhnd((long long)n_kv_heads, kv_rows, p.dim);
     }
     HIP_TRY(rt::launch_flash_f32(stream, p), "flash_fwd_f32 launch");
     return RT_OK;
@@ -670,13 +672,13 @@ RT_API int rt_mha_forward_masked_f32(const float* q, size_t q_len, const float* 
         HIP_TRY(hipMemcpy(dm.p, mask, mask_len * 4, hipMemcpyHostToDevice), "copy mask");
     }
     const long long bias_bh_stride = (mask_len == all_masks && all_masks != one_mask) ? (long long)one_mask : 0;
-    if (t_q == t_kv && head_dim % 32 == 0 && head_dim <= 128) {
-        // self-attention with a head dim the tiled f32 kernel covers: the same kernel as the unmasked path, with
-        // the mask's row added to the scaled scores
+    if (t_kv > 0 && head_dim % 4 == 0 && head_dim <= 128 && fits_int(t_kv)) {
+        // a head dim the tiled f32 kernel covers: the same kernel as the unmasked path, with the mask's row added to
+        // the scaled scores and, for cross-attention, its own number of keys
         rt_attention_shape shape = {batch, heads, t_q, head_dim, 64, 64};
         rc = flash_f32_device(nullptr, &shape, heads, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p,
                               RT_MASK_NONE, nullptr, (float*)dout.p, err, true, mask_len ? (const float*)dm.p : nullptr,
-                              bias_bh_stride);
+                              bias_bh_stride, nullptr, t_kv);
         if (rc) return rc;
         HIP_TRY(hipMemcpy(out, dout.p, q_expected * 4, hipMemcpyDeviceToHost), "copy out");
         return RT_OK;
@@ -1010,5 +1012,37 @@ RT_API int rt_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream,
 RT_API int rt_stream_synchronize(void* stream, rt_err_detail* err) {
     clear_err(err);
     HIP_TRY(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
+    return RT_OK;
+}
+
+RT_API void* rt_stream_create(rt_err_detail* err) {
+    clear_err(err);
+    if (ensure_device(err) != RT_OK) return nullptr;
+    hipStream_t s = nullptr;
+    hipError_t e = hipStreamCreate(&s);
+    if (e != hipSuccess) {
+        fail_hip(err, e, "hipStreamCreate");
+        return nullptr;
+    }
+    return (void*)s;
+}
+
+RT_API int rt_stream_destroy(void* stream, rt_err_detail* err) {
+    clear_err(err);
+    if (!stream) return RT_OK;
+    {
+        // the library's scratch for this stream goes with it
+        std::lock_guard<std::mutex> lock(g_ws_mutex);
+        int dev = 0;
+        if (hipGetDevice(&dev) == hipSuccess) {
+            auto it = g_ws.find({dev, (hipStream_t)stream});
+            if (it != g_ws.end()) {
+                (void)hipStreamSynchronize((hipStream_t)stream);
+                if (it->second.ptr) (void)hipFree(it->second.ptr);
+                g_ws.erase(it);
+            }
+        }
+    }
+    HIP_TRY(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy");
     return RT_OK;
 }

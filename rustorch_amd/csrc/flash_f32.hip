@@ -174,9 +174,9 @@ __global__ __launch_bounds__(64) void flash_fwd_f32_kernel(FlashF32Params p) {
 // The contraction index of the score product is walked in the order d = 8j + 4*half + i (i = 0..3) for both
 // operands, so that a lane fetches its four K values of a chunk with one 16-byte LDS read and Q stays in
 // registers for the whole job.
-template <int DT>
+template <int DT, bool kExactD>  // kExactD: dim == 32 * DT, no column guards anywhere
 __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_kernel(FlashF32Params p) {
-    constexpr int DPAD = 32 * DT;       // == dim
+    constexpr int DPAD = 32 * DT;       // dim rounded up to a multiple of 32 (columns beyond dim are zeros in LDS)
     constexpr int LDK = DPAD + 4;       // row stride of the K tile: 16-byte reads of 16 rows tile all banks
     constexpr int CH = DPAD / 4;        // 16-byte chunks per row
     constexpr int NLD = 32 * CH / 64;   // 16-byte loads per lane, per matrix, per tile
@@ -189,7 +189,8 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, hh = lane >> 5;
-    const int N = p.seq;
+    const int Nq = p.seq, N = p.seq_kv ? p.seq_kv : p.seq;  // N: keys (== queries unless cross-attention)
+    const int D = kExactD ? DPAD : p.dim;
     // Which (batch, head, query tile) this workgroup takes.  Workgroups are dealt round-robin to the 8 XCDs, each
     // with its own L2: when the heads divide evenly, XCD x takes the heads bh = x (mod 8) and walks them one after
     // the other, longest causal rows first, so that a head's K and V are fetched into one L2 only.  When the whole
@@ -234,7 +235,7 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
 #pragma unroll
     for (int j = 0; j < DPAD / 8; j++) {
         f32x4_t z = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (q_row < N) z = *(const f32x4_t*)(Qg + (size_t)q_row * q_pitch + 8 * j + 4 * hh);
+        if (q_row < Nq && 8 * j + 4 * hh < D) z = *(const f32x4_t*)(Qg + (size_t)q_row * q_pitch + 8 * j + 4 * hh);
 #pragma unroll
         for (int i = 0; i < 4; i++) qreg[4 * j + i] = z[i];
     }
@@ -252,7 +253,7 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
     const int n_tiles = (kv_end + kRows - 1) / kRows;
     // additive bias row of this lane's query (MultiHeadAttention's attn_mask, added to the scaled scores)
     const float* __restrict__ bias_row = nullptr;
-    if (p.bias && q_row < N)
+    if (p.bias && q_row < Nq)
         bias_row = p.bias + ((size_t)b * p.heads + h) * (size_t)p.bias_bh_stride + (size_t)q_row * (size_t)N;
     const bool bias_vec = ((N & 3) == 0) && ((((uintptr_t)p.bias) & 15) == 0) && ((p.bias_bh_stride & 3) == 0);
 
@@ -261,11 +262,17 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
     constexpr bool kEvenRows = (64 % CH == 0);
     constexpr int RPL = kEvenRows ? 64 / CH : 0;  // rows per load instruction
     const int ld_r = lane / CH, ld_c = lane % CH;
+    const bool ld_col_ok = kExactD || 4 * ld_c < D;  // this lane's 16-byte column exists
     const uint32_t ld_off = (uint32_t)ld_r * (uint32_t)kv_pitch * 4u + (uint32_t)ld_c * 16u;  // bytes; a few rows: fits
     f32x4_t kreg[NLD], vreg[NLD];
     auto issue_loads = [&](int tile) {
         if constexpr (kEvenRows) {
             if (tile * kRows + kRows <= N) {  // whole tile present (wave-uniform): no per-load bounds test
+                if (!ld_col_ok) {
+#pragma unroll
+                    for (int n = 0; n < NLD; n++) kreg[n] = vreg[n] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                    return;
+                }
                 const char* kb = (const char*)Kg + (size_t)tile * kRows * kv_pitch * sizeof(float) + ld_off;
                 const char* vb = (const char*)Vg + (size_t)tile * kRows * kv_pitch * sizeof(float) + ld_off;
 #pragma unroll
@@ -283,14 +290,14 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
             if constexpr (kEvenRows) {
                 const int row0 = tile * kRows + RPL * n;  // uniform
                 const size_t base = (size_t)row0 * kv_pitch * sizeof(float);
-                if (row0 + ld_r < N) {  // rows past the end are zeros (and masked below)
+                if (row0 + ld_r < N && ld_col_ok) {  // rows past the end are zeros (and masked below)
                     zk = *(const f32x4_t*)((const char*)Kg + base + ld_off);
                     zv = *(const f32x4_t*)((const char*)Vg + base + ld_off);
                 }
             } else {
                 const int idx = 64 * n + lane, r = idx / CH, c = idx % CH;
                 const int kr = tile * kRows + r;
-                if (kr < N) {
+                if (kr < N && 4 * c < D) {
                     zk = *(const f32x4_t*)(Kg + (size_t)kr * kv_pitch + 4 * c);
                     zv = *(const f32x4_t*)(Vg + (size_t)kr * kv_pitch + 4 * c);
                 }
@@ -419,7 +426,7 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
     if (wave == 0 && hh == 0) {
         bool good = (l_all > 0.0f) && (fabsf(l_all) != __uint_as_float(0x7f800000u)) && (l_all == l_all) && !poison;
         fin_inv[col] = good ? 1.0f / l_all : quiet_nan();
-        if (p.lse && q0 + col < N) p.lse[((size_t)b * p.heads + h) * (size_t)N + q0 + col] = m_all + logf(l_all);
+        if (p.lse && q0 + col < Nq) p.lse[((size_t)b * p.heads + h) * (size_t)Nq + q0 + col] = m_all + logf(l_all);
     }
     // this wave's weighted O, as rows [col][d], into its own K tile
 #pragma unroll
@@ -444,7 +451,7 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
             f32x4_t o;
 #pragma unroll
             for (int i = 0; i < 4; i++) o[i] = (inv == inv) ? sum[i] * inv : quiet_nan();
-            if (q0 + r < N) *(f32x4_t*)(Og + (size_t)(q0 + r) * o_pitch + 4 * c) = o;
+            if (q0 + r < Nq && 4 * c < D) *(f32x4_t*)(Og + (size_t)(q0 + r) * o_pitch + 4 * c) = o;
         }
     }
 }
@@ -455,26 +462,39 @@ hipError_t launch_flash_f32(hipStream_t stream, const FlashF32Params& p) {
     if (p.batch == 0 || p.heads == 0 || p.seq == 0) return hipSuccess;
     dim3 grid((p.seq + kRows - 1) / kRows, p.heads, p.batch), block(64);
     int dt = (p.dim + 31) / 32;
-    // the fast kernel reads whole 16-byte chunks: head dim a multiple of 32, rows and bases 16-byte aligned
+    // the fast kernel reads whole 16-byte chunks: head dim a multiple of 4, rows and bases 16-byte aligned
     auto aligned = [](const void* ptr, const TensorLayout& l) {
         return ((uintptr_t)ptr % 16 == 0) && (l.batch_stride % 4 == 0) && (l.head_stride % 4 == 0) && (l.row_pitch % 4 == 0);
     };
-    if (p.dim % 32 == 0 && p.dim <= 128 && aligned(p.q, p.lq) && aligned(p.k, p.lkv) && aligned(p.v, p.lkv) && aligned(p.out, p.lo)) {
+    if (p.dim % 4 == 0 && p.dim <= 128 && aligned(p.q, p.lq) && aligned(p.k, p.lkv) && aligned(p.v, p.lkv) && aligned(p.out, p.lo)) {
         dim3 block4(256);
         FlashF32Params pz = p;
         // 8 (dim <= 64) or 4 waves fit on a CU: is every workgroup resident from the start?
         const long long resident = (long long)p.n_cus * (dt <= 2 ? 2 : 1);
         pz.zigzag = (p.mask == kMaskCausal) && ((long long)grid.x * grid.y * grid.z <= resident) ? 1 : 0;
+        const bool exact = (p.dim % 32 == 0);
         switch (dt) {
-            case 1: hipLaunchKernelGGL(flash_fwd_f32_splitk_kernel<1>, grid, block4, 0, stream, pz); break;
-            case 2: hipLaunchKernelGGL(flash_fwd_f32_splitk_kernel<2>, grid, block4, 0, stream, pz); break;
-            case 3: hipLaunchKernelGGL(flash_fwd_f32_splitk_kernel<3>, grid, block4, 0, stream, pz); break;
-            case 4: hipLaunchKernelGGL(flash_fwd_f32_splitk_kernel<4>, grid, block4, 0, stream, pz); break;
+            case 1:
+                if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<1, true>), grid, block4, 0, stream, pz);
+                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<1, false>), grid, block4, 0, stream, pz);
+                break;
+            case 2:
+                if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<2, true>), grid, block4, 0, stream, pz);
+                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<2, false>), grid, block4, 0, stream, pz);
+                break;
+            case 3:
+                if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<3, true>), grid, block4, 0, stream, pz);
+                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<3, false>), grid, block4, 0, stream, pz);
+                break;
+            case 4:
+                if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<4, true>), grid, block4, 0, stream, pz);
+                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<4, false>), grid, block4, 0, stream, pz);
+                break;
             default: return hipErrorInvalidValue;
         }
         return hipGetLastError();
     }
-    if (p.bias) return hipErrorInvalidValue;  // only the tiled kernel above adds a bias
+    if (p.bias || (p.seq_kv && p.seq_kv != p.seq)) return hipErrorInvalidValue;  // only the tiled kernel above does these
     switch (dt) {
         case 1: hipLaunchKernelGGL(flash_fwd_f32_kernel<1>, grid, block, 0, stream, p); break;
         case 2: hipLaunchKernelGGL(flash_fwd_f32_kernel<2>, grid, block, 0, stream, p); break;

@@ -32,6 +32,7 @@ struct FlashF32Params {
     const uint8_t* keep;  // device, `seq` bytes, for kMaskPadding
     int batch, heads, kv_heads, group;
     int seq, dim;
+    int seq_kv;  // keys per (batch, kv head) when they differ from `seq` (cross-attention; mask none only); 0: == seq
     int mask;
     int ref_bc;  // the reference's key-tile size, for the leading-masked-tile rule
     float scale;

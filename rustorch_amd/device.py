@@ -70,6 +70,35 @@ def synchronize(stream=None):
     raise_for(L.lib().rt_stream_synchronize(stream, C.byref(err)), err)
 
 
+class Stream:
+    """A HIP stream at the default priority; pass `.handle` (or the object) as the `stream` of a device entry."""
+
+    def __init__(self):
+        err = L.RtErr()
+        self.handle = L.lib().rt_stream_create(C.byref(err))
+        if not self.handle:
+            raise_for(L.RT_ERR_HIP if err.hip_error else L.RT_ERR_NO_DEVICE, err)
+
+    @property
+    def _as_parameter_(self):  # lets ctypes take the object where a void* is expected
+        return C.c_void_p(self.handle)
+
+    def synchronize(self):
+        synchronize(self.handle)
+
+    def destroy(self):
+        if getattr(self, "handle", None):
+            err = L.RtErr()
+            L.lib().rt_stream_destroy(self.handle, C.byref(err))
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
 def init(device: int = 0):
     """Select the gfx950 device; raises DeviceError(NoDeviceFound) when there is none."""
     err = L.RtErr()

@@ -11,17 +11,6 @@ def bf16_round(x):
     return bits, oracle.bf16_to_f32(bits)
 
 
-def new_stream():
-    """A HIP stream at the default priority, straight from the runtime the library is linked against."""
-    import ctypes as C
-    hip = C.CDLL("libamdhip64.so")
-    hip.hipStreamCreate.argtypes = [C.POINTER(C.c_void_p)]
-    s = C.c_void_p()
-    rc = hip.hipStreamCreate(C.byref(s))
-    assert rc == 0, f"hipStreamCreate: {rc}"
-    return s
-
-
 def dev(a):
     return ra.HipStorage.from_numpy(np.ascontiguousarray(a))
 

@@ -189,3 +189,17 @@ def test_saved_backward_argument_errors_before_any_device_use():
     assert L.lib().rt_flash_forward_stats_f32_dev(None, C.byref(z), 16, 16, 16, 16, 16, C.byref(err)) == L.RT_ERR_ZERO_DIM
     e = ra.AttentionShape.new(1, 1, 0, 4)._c()  # nothing to do: Ok without a device
     assert L.lib().rt_flash_forward_stats_f32_dev(None, C.byref(e), 16, 16, 16, 16, 16, C.byref(err)) == L.RT_OK
+
+
+def test_stream_create_reports_a_missing_device():
+    import ctypes as C
+    err = L.RtErr()
+    if L.lib().rt_init(0, C.byref(err)) == 0:
+        s = ra.Stream()
+        s.synchronize()
+        s.destroy()
+        return
+    with pytest.raises(ra.DeviceError) as ei:
+        ra.Stream()
+    assert ei.value.status == L.RT_ERR_NO_DEVICE
+    assert L.lib().rt_stream_destroy(None, C.byref(err)) == L.RT_OK

@@ -139,11 +139,8 @@ def test_single_sequence_decode_long_contexts_and_streams(oracle):
     """The reference call on the split-K path: contexts long enough for a hundred partials per head, a cache that
     grows between calls (the library's per-stream buffer is re-sized), and two streams used alternately (each has
     a buffer of its own)."""
-    from _gpu import new_stream
-
-    ra.init(0)
     hq, hkv, d = 32, 8, 128
-    streams = [None, new_stream(), new_stream()]
+    streams = [None, ra.Stream(), ra.Stream()]
     for max_seq, kv_lens in [(96, [1, 33, 96]), (8192, [8192, 4097, 2048, 65]), (300, [300])]:
         qb, _ = bf16_round(seeded_normal((hq, d), max_seq))
         kb, _ = bf16_round(seeded_normal((hkv, max_seq, d), max_seq + 1))

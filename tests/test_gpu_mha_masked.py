@@ -30,7 +30,9 @@ def test_self_attention_with_masks(oracle, b, t, h, d, kind):
     _run(oracle, b, t, t, h, d, mask)
 
 
-@pytest.mark.parametrize("b,tq,tkv,h,d", [(2, 4, 9, 2, 8), (1, 100, 7, 3, 64), (2, 1, 300, 2, 128), (1, 6, 1, 1, 16)])
+@pytest.mark.parametrize("b,tq,tkv,h,d", [(2, 4, 9, 2, 8), (1, 100, 7, 3, 64), (2, 1, 300, 2, 128), (1, 6, 1, 1, 16),
+                                          (2, 70, 333, 3, 80), (1, 257, 64, 2, 20), (1, 33, 1000, 1, 128), (2, 40, 65, 2, 6),
+                                          (1, 31, 97, 2, 132), (8, 16, 512, 8, 64)])
 def test_cross_attention(oracle, b, tq, tkv, h, d):
     rng = np.random.default_rng(9)
     _run(oracle, b, tq, tkv, h, d, None)
