@@ -328,6 +328,13 @@ RT_API int rt_gqa_forward_f32(const float* q, size_t q_len, const float* k, size
         rc = flash_f32_device(nullptr, &s, n_kv_heads, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p,
                               RT_MASK_NONE, nullptr, (float*)dout.p, err);
         if (rc) return rc;
+    } else if (seq_kv > 0 && head_dim % 4 == 0 && head_dim <= 128) {
+        // decode / chunked prefill: every query row attends to all seq_kv keys (gqa.rs:179-208); the tiled kernel
+        // with its own key count
+        rt_attention_shape s = {batch, n_heads, seq_q, head_dim, 64, 64};
+        rc = flash_f32_device(nullptr, &s, n_kv_heads, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p,
+                              RT_MASK_NONE, nullptr, (float*)dout.p, err, false, nullptr, 0, nullptr, seq_kv);
+        if (rc) return rc;
     } else {
         if (head_dim > 512) return fail(err, RT_ERR_UNSUPPORTED, -1, 512, head_dim, "decode rows kernel covers dim <= 512");
         if (seq_q > 65535 * 32ull) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, seq_q, "seq_q too large");

@@ -213,7 +213,8 @@ def test_config_f32_causal_b1_h8_n2048_d64(oracle):
 
 @pytest.mark.parametrize("b,hq,hkv,sq,skv,d", [(1, 4, 4, 3, 3, 4), (1, 8, 2, 4, 4, 8), (2, 6, 3, 1, 37, 16),
                                               (2, 6, 3, 5, 37, 16), (1, 32, 8, 1, 700, 128), (1, 4, 2, 1, 1, 8),
-                                              (2, 8, 2, 130, 130, 64), (1, 3, 1, 2, 9, 200)])
+                                              (2, 8, 2, 130, 130, 64), (1, 3, 1, 2, 9, 200), (1, 8, 2, 100, 333, 64),
+                                              (2, 4, 1, 33, 1000, 128), (1, 6, 2, 65, 31, 20), (1, 2, 1, 7, 70, 5)])
 def test_gqa_forward_matches_oracle(oracle, b, hq, hkv, sq, skv, d):
     q = seeded_normal((b, hq, sq, d), 1)
     k = seeded_normal((b, hkv, skv, d), 2)
