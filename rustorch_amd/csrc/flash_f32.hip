@@ -317,21 +317,8 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
             *(f32x4_t*)(Kw + r * LDK + 4 * c) = kreg[n];
             *(f32x4_t*)(Vw + r * DPAD + 4 * c) = vreg[n];
         }
-        if (tile + NW < n_tiles) issue_loads(tile + NW);
-
-        // S^T = K . Q^T
-        f32x16_t s;
-#pragma unroll
-        for (int i = 0; i < 16; i++) s[i] = 0.0f;
-#pragma unroll
-        for (int j = 0; j < DPAD / 8; j++) {
-            const f32x4_t a = *(const f32x4_t*)(Kw + col * LDK + 8 * j + 4 * hh);
-#pragma unroll
-            for (int i = 0; i < 4; i++) s = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], qreg[4 * j + i], s, 0, 0, 0);
-        }
-        // register i of the accumulator holds key row 8*(i/4) + 4*hh + (i%4), query row `col`
-        float m_tile = neg_inf();
-        const bool edge = (kv0 + kRows > N) || (p.mask == kMaskCausal && kv0 + kRows - 1 > q0) || (p.mask == kMaskPadding);
+        // this tile's bias values are requested ahead of the next tile's rows: a wait for them then leaves the
+        // prefetch in flight (requests complete in order)
         f32x16_t bias;
 #pragma unroll
         for (int i = 0; i < 16; i++) bias[i] = 0.0f;
@@ -350,6 +337,21 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
                 }
             }
         }
+        if (tile + NW < n_tiles) issue_loads(tile + NW);
+
+        // S^T = K . Q^T
+        f32x16_t s;
+#pragma unroll
+        for (int i = 0; i < 16; i++) s[i] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < DPAD / 8; j++) {
+            const f32x4_t a = *(const f32x4_t*)(Kw + col * LDK + 8 * j + 4 * hh);
+#pragma unroll
+            for (int i = 0; i < 4; i++) s = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], qreg[4 * j + i], s, 0, 0, 0);
+        }
+        // register i of the accumulator holds key row 8*(i/4) + 4*hh + (i%4), query row `col`
+        float m_tile = neg_inf();
+        const bool edge = (kv0 + kRows > N) || (p.mask == kMaskCausal && kv0 + kRows - 1 > q0) || (p.mask == kMaskPadding);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             float x = s[i] * p.scale + bias[i];
