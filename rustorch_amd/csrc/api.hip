@@ -9,6 +9,7 @@
 #include <algorithm>
 #include <map>
 #include <mutex>
+#include <vector>
 
 #include "../../include/rt_attn.h"
 #include "rt_kernels.hpp"
@@ -203,11 +204,103 @@ int stream_workspace(hipStream_t stream, size_t bytes, float** out, rt_err_detai
     return RT_OK;
 }
 
+struct DevPtr {  // a device address inside a Stage's block
+    void* p = nullptr;
+};
+
 struct DevBuf {
     void* p = nullptr;
     ~DevBuf() {
         if (p) (void)hipFree(p);
     }
+};
+
+// Staging of one host-slice call: every input, output and scratch buffer of the call sits in ONE device block.
+// Small calls (inputs + outputs within kPinnedBytes) travel through a pinned host buffer the library keeps, as one
+// host-to-device and one device-to-host transfer: a pageable hipMemcpy costs about 60 us whatever its size below
+// a megabyte, and a call has four of them.  One call at a time can hold the pinned buffer; a call that finds it
+// taken (another thread is inside a host-slice entry) or that is larger copies buffer by buffer instead.
+constexpr size_t kPinnedBytes = (size_t)4 << 20;
+std::mutex g_pinned_mutex;
+void* g_pinned = nullptr;
+
+class Stage {
+public:
+    void in(const void* host, size_t bytes, void** dev) { items_.push_back({host, nullptr, bytes, dev, 0, 0}); }
+    void out(void* host, size_t bytes, void** dev) { items_.push_back({nullptr, host, bytes, dev, 0, 1}); }
+    void scratch(size_t bytes, void** dev) { items_.push_back({nullptr, nullptr, bytes, dev, 0, 2}); }
+
+    // Allocates the block, hands out the device pointers and uploads the inputs (register inputs, then outputs,
+    // then scratch).
+    int commit(rt_err_detail* err) {
+        size_t off = 0;
+        for (auto& it : items_) {
+            it.off = off;
+            off += (it.bytes + 255) & ~(size_t)255;
+            if (it.kind == 0) in_end_ = off;
+            if (it.kind == 1) io_end_ = off;
+        }
+        if (io_end_ < in_end_) io_end_ = in_end_;
+        HIP_TRY(hipMalloc(&block_.p, off ? off : 256), "hipMalloc staging block");
+        for (auto& it : items_) *it.dev = (char*)block_.p + it.off;
+        if (io_end_ <= kPinnedBytes) {
+            lock_ = std::unique_lock<std::mutex>(g_pinned_mutex, std::try_to_lock);
+            if (lock_.owns_lock() && !g_pinned && hipHostMalloc(&g_pinned, kPinnedBytes, hipHostMallocDefault) != hipSuccess) {
+                (void)hipGetLastError();
+                g_pinned = nullptr;
+                lock_.unlock();
+            }
+        }
+        if (lock_.owns_lock()) {
+            for (auto& it : items_)
+                if (it.kind == 0 && it.bytes) memcpy((char*)g_pinned + it.off, it.host_in, it.bytes);
+            if (in_end_) HIP_TRY(hipMemcpyAsync(block_.p, g_pinned, in_end_, hipMemcpyHostToDevice, nullptr), "upload");
+        } else {
+            for (auto& it : items_)
+                if (it.kind == 0 && it.bytes)
+                    HIP_TRY(hipMemcpy((char*)block_.p + it.off, it.host_in, it.bytes, hipMemcpyHostToDevice), "copy input");
+        }
+        return RT_OK;
+    }
+
+    // Brings the outputs back; returns after they are in the caller's buffers.
+    int fetch(rt_err_detail* err) {
+        fetched_ = true;  // every path below ends with the stream idle (or reports the failure of the attempt)
+        if (lock_.owns_lock()) {
+            if (io_end_ > in_end_)
+                HIP_TRY(hipMemcpyAsync((char*)g_pinned + in_end_, (char*)block_.p + in_end_, io_end_ - in_end_,
+                                       hipMemcpyDeviceToHost, nullptr),
+                        "download");
+            HIP_TRY(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+            for (auto& it : items_)
+                if (it.kind == 1 && it.bytes) memcpy(it.host_out, (char*)g_pinned + it.off, it.bytes);
+        } else {
+            for (auto& it : items_)
+                if (it.kind == 1 && it.bytes)
+                    HIP_TRY(hipMemcpy(it.host_out, (char*)block_.p + it.off, it.bytes, hipMemcpyDeviceToHost), "copy output");
+        }
+        return RT_OK;
+    }
+
+    ~Stage() {
+        // an early return (a failed launch) may leave work in flight that still reads the block or the pinned buffer
+        if (block_.p && !fetched_) (void)hipStreamSynchronize(nullptr);
+    }
+
+private:
+    struct Item {
+        const void* host_in;
+        void* host_out;
+        size_t bytes;
+        void** dev;
+        size_t off;
+        int kind;  // 0 input, 1 output, 2 scratch
+    };
+    std::vector<Item> items_;
+    size_t in_end_ = 0, io_end_ = 0;
+    bool fetched_ = false;
+    std::unique_lock<std::mutex> lock_;  // declared before block_: the block is freed first, then the pinned buffer released
+    DevBuf block_;
 };
 
 }  // namespace
@@ -261,24 +354,20 @@ RT_API int rt_flash_forward_masked_f32(const rt_attention_shape* shape, const fl
     rc = ensure_device(err);
     if (rc) return rc;
 
-    DevBuf dq, dk, dv, dout, dkeep;
+    Stage st;
+    void *dq, *dk, *dv, *dout, *dkeep = nullptr;
     size_t bytes = n * sizeof(float);
-    HIP_TRY(hipMalloc(&dq.p, bytes), "hipMalloc q");
-    HIP_TRY(hipMalloc(&dk.p, bytes), "hipMalloc k");
-    HIP_TRY(hipMalloc(&dv.p, bytes), "hipMalloc v");
-    HIP_TRY(hipMalloc(&dout.p, bytes), "hipMalloc out");
-    HIP_TRY(hipMemcpy(dq.p, q, bytes, hipMemcpyHostToDevice), "copy q");
-    HIP_TRY(hipMemcpy(dk.p, k, bytes, hipMemcpyHostToDevice), "copy k");
-    HIP_TRY(hipMemcpy(dv.p, v, bytes, hipMemcpyHostToDevice), "copy v");
-    if (mask_kind == RT_MASK_PADDING) {
-        HIP_TRY(hipMalloc(&dkeep.p, keep_len), "hipMalloc keep");
-        HIP_TRY(hipMemcpy(dkeep.p, keep, keep_len, hipMemcpyHostToDevice), "copy keep");
-    }
-    rc = flash_f32_device(nullptr, shape, shape->heads, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p,
-                          mask_kind, (const uint8_t*)dkeep.p, (float*)dout.p, err);
+    st.in(q, bytes, &dq);
+    st.in(k, bytes, &dk);
+    st.in(v, bytes, &dv);
+    if (mask_kind == RT_MASK_PADDING) st.in(keep, keep_len, &dkeep);
+    st.out(out, bytes, &dout);
+    rc = st.commit(err);
     if (rc) return rc;
-    HIP_TRY(hipMemcpy(out, dout.p, bytes, hipMemcpyDeviceToHost), "copy out");
-    return RT_OK;
+    rc = flash_f32_device(nullptr, shape, shape->heads, (const float*)dq, (const float*)dk, (const float*)dv, mask_kind,
+                          (const uint8_t*)dkeep, (float*)dout, err);
+    if (rc) return rc;
+    return st.fetch(err);
 }
 
 RT_API int rt_flash_forward_f32(const rt_attention_shape* shape, const float* q, size_t q_len, const float* k,
@@ -312,16 +401,14 @@ RT_API int rt_gqa_forward_f32(const float* q, size_t q_len, const float* k, size
     int rc = ensure_device(err);
     if (rc) return rc;
 
-    DevBuf dq, dk, dv, dout;
-    HIP_TRY(hipMalloc(&dq.p, q_expected * 4), "hipMalloc q");
-    HIP_TRY(hipMalloc(&dout.p, q_expected * 4), "hipMalloc out");
-    HIP_TRY(hipMalloc(&dk.p, kv_expected ? kv_expected * 4 : 4), "hipMalloc k");
-    HIP_TRY(hipMalloc(&dv.p, kv_expected ? kv_expected * 4 : 4), "hipMalloc v");
-    HIP_TRY(hipMemcpy(dq.p, q, q_expected * 4, hipMemcpyHostToDevice), "copy q");
-    if (kv_expected) {
-        HIP_TRY(hipMemcpy(dk.p, k, kv_expected * 4, hipMemcpyHostToDevice), "copy k");
-        HIP_TRY(hipMemcpy(dv.p, v, kv_expected * 4, hipMemcpyHostToDevice), "copy v");
-    }
+    Stage st;
+    DevPtr dq, dk, dv, dout;
+    st.in(q, q_expected * 4, &dq.p);
+    st.in(k, kv_expected * 4, &dk.p);
+    st.in(v, kv_expected * 4, &dv.p);
+    st.out(out, q_expected * 4, &dout.p);
+    rc = st.commit(err);
+    if (rc) return rc;
     if (seq_q == seq_kv) {
         // prefill: unmasked flash; the kernel maps query head -> kv head itself (no replicated copy)
         rt_attention_shape s = {batch, n_heads, seq_q, head_dim, 64, 64};
@@ -355,8 +442,7 @@ RT_API int rt_gqa_forward_f32(const float* q, size_t q_len, const float* k, size
         p.scale = 1.0f / sqrtf((float)head_dim);
         HIP_TRY(rt::launch_attn_rows_f32(nullptr, p), "attn_rows_f32 launch");
     }
-    HIP_TRY(hipMemcpy(out, dout.p, q_expected * 4, hipMemcpyDeviceToHost), "copy out");
-    return RT_OK;
+    return st.fetch(err);
 }
 
 // ---- backward (cpu_backward.rs:46-185) ----------------------------------------------------------------
@@ -428,20 +514,19 @@ RT_API int rt_flash_backward_f32(const rt_attention_shape* shape, const float* q
     if (rc) return rc;
 
     const size_t bytes = (size_t)expected * sizeof(float);
-    DevBuf in[4], out[3], ws;
+    Stage st;
+    DevPtr in[4], out[3], ws;
     const float* host_in[4] = {q, k, v, d_out};
-    for (int i = 0; i < 4; i++) {
-        HIP_TRY(hipMalloc(&in[i].p, bytes), "hipMalloc input");
-        HIP_TRY(hipMemcpy(in[i].p, host_in[i], bytes, hipMemcpyHostToDevice), "copy input");
-    }
-    for (int i = 0; i < 3; i++) HIP_TRY(hipMalloc(&out[i].p, bytes), "hipMalloc gradient");
-    HIP_TRY(hipMalloc(&ws.p, rt_flash_backward_workspace_bytes(shape)), "hipMalloc workspace");
+    float* host_out[3] = {dq, dk, dv};
+    for (int i = 0; i < 4; i++) st.in(host_in[i], bytes, &in[i].p);
+    for (int i = 0; i < 3; i++) st.out(host_out[i], bytes, &out[i].p);
+    st.scratch(rt_flash_backward_workspace_bytes(shape), &ws.p);
+    rc = st.commit(err);
+    if (rc) return rc;
     rc = flash_bwd_device(nullptr, shape, (const float*)in[0].p, (const float*)in[1].p, (const float*)in[2].p,
                           (const float*)in[3].p, (float*)out[0].p, (float*)out[1].p, (float*)out[2].p, (float*)ws.p, err);
     if (rc) return rc;
-    float* host_out[3] = {dq, dk, dv};
-    for (int i = 0; i < 3; i++) HIP_TRY(hipMemcpy(host_out[i], out[i].p, bytes, hipMemcpyDeviceToHost), "copy gradient");
-    return RT_OK;
+    return st.fetch(err);
 }
 
 RT_API int rt_flash_backward_f32_dev(void* stream, const rt_attention_shape* shape, const float* q, const float* k,
@@ -625,20 +710,19 @@ RT_API int rt_mha_flash_forward_f32(const float* q, size_t q_len, const float* k
     if (rc) return rc;
     rc = ensure_device(err);
     if (rc) return rc;
-    DevBuf dq, dk, dv, dout;
+    Stage st;
+    DevPtr dq, dk, dv, dout;
     size_t bytes = q_len * sizeof(float);
-    HIP_TRY(hipMalloc(&dq.p, bytes), "hipMalloc q");
-    HIP_TRY(hipMalloc(&dk.p, bytes), "hipMalloc k");
-    HIP_TRY(hipMalloc(&dv.p, bytes), "hipMalloc v");
-    HIP_TRY(hipMalloc(&dout.p, bytes), "hipMalloc out");
-    HIP_TRY(hipMemcpy(dq.p, q, bytes, hipMemcpyHostToDevice), "copy q");
-    HIP_TRY(hipMemcpy(dk.p, k, bytes, hipMemcpyHostToDevice), "copy k");
-    HIP_TRY(hipMemcpy(dv.p, v, bytes, hipMemcpyHostToDevice), "copy v");
+    st.in(q, bytes, &dq.p);
+    st.in(k, bytes, &dk.p);
+    st.in(v, bytes, &dv.p);
+    st.out(out, bytes, &dout.p);
+    rc = st.commit(err);
+    if (rc) return rc;
     rc = flash_f32_device(nullptr, &shape, heads, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p,
                           RT_MASK_NONE, nullptr, (float*)dout.p, err, true);
     if (rc) return rc;
-    HIP_TRY(hipMemcpy(out, dout.p, bytes, hipMemcpyDeviceToHost), "copy out");
-    return RT_OK;
+    return st.fetch(err);
 }
 
 RT_API int rt_mha_forward_masked_f32(const float* q, size_t q_len, const float* k, size_t k_len, const float* v,
@@ -664,20 +748,15 @@ RT_API int rt_mha_forward_masked_f32(const float* q, size_t q_len, const float* 
         return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
     int rc = ensure_device(err);
     if (rc) return rc;
-    DevBuf dq, dk, dv, dm, dout;
-    HIP_TRY(hipMalloc(&dq.p, q_expected * 4), "hipMalloc q");
-    HIP_TRY(hipMalloc(&dout.p, q_expected * 4), "hipMalloc out");
-    HIP_TRY(hipMemcpy(dq.p, q, q_expected * 4, hipMemcpyHostToDevice), "copy q");
-    if (kv_expected) {
-        HIP_TRY(hipMalloc(&dk.p, kv_expected * 4), "hipMalloc k");
-        HIP_TRY(hipMalloc(&dv.p, kv_expected * 4), "hipMalloc v");
-        HIP_TRY(hipMemcpy(dk.p, k, kv_expected * 4, hipMemcpyHostToDevice), "copy k");
-        HIP_TRY(hipMemcpy(dv.p, v, kv_expected * 4, hipMemcpyHostToDevice), "copy v");
-    }
-    if (mask_len) {
-        HIP_TRY(hipMalloc(&dm.p, mask_len * 4), "hipMalloc mask");
-        HIP_TRY(hipMemcpy(dm.p, mask, mask_len * 4, hipMemcpyHostToDevice), "copy mask");
-    }
+    Stage st;
+    DevPtr dq, dk, dv, dm, dout;
+    st.in(q, q_expected * 4, &dq.p);
+    st.in(k, kv_expected * 4, &dk.p);
+    st.in(v, kv_expected * 4, &dv.p);
+    st.in(mask, mask_len * 4, &dm.p);
+    st.out(out, q_expected * 4, &dout.p);
+    rc = st.commit(err);
+    if (rc) return rc;
     const long long bias_bh_stride = (mask_len == all_masks && all_masks != one_mask) ? (long long)one_mask : 0;
     if (t_kv > 0 && head_dim % 4 == 0 && head_dim <= 128 && fits_int(t_kv)) {
         // a head dim the tiled f32 kernel covers: the same kernel as the unmasked path, with the mask's row added to
@@ -687,8 +766,7 @@ RT_API int rt_mha_forward_masked_f32(const float* q, size_t q_len, const float* 
                               RT_MASK_NONE, nullptr, (float*)dout.p, err, true, mask_len ? (const float*)dm.p : nullptr,
                               bias_bh_stride, nullptr, t_kv);
         if (rc) return rc;
-        HIP_TRY(hipMemcpy(out, dout.p, q_expected * 4, hipMemcpyDeviceToHost), "copy out");
-        return RT_OK;
+        return st.fetch(err);
     }
     rt::AttnRowsParams p{};
     p.q = dq.p;
@@ -711,8 +789,7 @@ RT_API int rt_mha_forward_masked_f32(const float* q, size_t q_len, const float* 
     p.lq = p.lo = rt::layout_bnhd((long long)heads, (long long)t_q, (int)head_dim);
     p.lkv = rt::layout_bnhd((long long)heads, (long long)t_kv, (int)head_dim);
     HIP_TRY(rt::launch_attn_rows_f32(nullptr, p), "attn_rows_f32 launch");
-    HIP_TRY(hipMemcpy(out, dout.p, q_expected * 4, hipMemcpyDeviceToHost), "copy out");
-    return RT_OK;
+    return st.fetch(err);
 }
 
 RT_API int rt_flash_forward_varlen_bf16_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,
