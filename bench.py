@@ -269,6 +269,19 @@ def main():
                                "unit": "GB/s", "frac": alg_bytes / (ms_kernel * 1e-3) / 1e9 / PEAK_HBM_GBS,
                                "traffic": TRAFFIC_DECODE_BYTES,
                                "kernels": "decode_split + decode_merge (one event pair around the timed steps)"}}
+        # the reference's own call: one sequence per launch (LlmKernels::gqa_decode_online_bf16), back to back on the
+        # stream as a decode loop issues it, on sequence 0's cache
+        single = {}
+        d_o1 = ra.HipStorage(Hq * Dd * 2)
+        for kv_len in (512, 2048, 8192):
+            t1 = time_steps(hip, stream,
+                            lambda i: K.gqa_decode_online_bf16(stream, d_q, sets[i % n_sets][0], sets[i % n_sets][1], d_o1,
+                                                               Hq, Hkv, kv_len, Dd, Lmax),
+                            args.steps, args.warmup, spread_steps=0)
+            single[str(kv_len)] = {"us_per_call": t1.mean_ms * 1e3,
+                                   "GB/s": (2 * Hkv * kv_len * Dd * 2 + 2 * Hq * Dd * 2) / (t1.mean_ms * 1e-3) / 1e9}
+        decode["single_sequence"] = dict(single, note="rt_gqa_decode_online_bf16, 32 q / 8 kv heads, D=128: two launches "
+                                                      "per call, issued back to back from the host")
         if not args.no_cpu:
             threads = min(oracle.max_threads(), 16)
             got = oracle.bf16_to_f32(d_o.download(np.uint16))
