@@ -250,6 +250,30 @@ static void test_gpu() {
         flash_backward(one, q1, q1, q1, g1, a, b, c);
         for (size_t i = 0; i < a.size(); i++) CHECK(std::fabs(a[i]) < 1e-6f && std::fabs(b[i]) < 1e-6f && c[i] == g1[i]);
     }
+    {   // the device-resident backward on a stream of its own, recomputing and from a saved forward: the host entry's bits
+        AttentionShape s = AttentionShape::make(2, 2, 70, 32);
+        const size_t n = s.buffer_len(), bytes = n * sizeof(float);
+        auto q = lcg(n, 11), k = lcg(n, 12), v = lcg(n, 13), g = lcg(n, 14);
+        std::vector<float> dq(n), dk(n), dv(n);
+        flash_backward(s, q, k, v, g, dq, dk, dv);
+        Stream st;
+        HipStorage hq(bytes), hk(bytes), hv(bytes), hg(bytes), ho(bytes), hl(2 * 2 * 70 * sizeof(float));
+        HipStorage gq(bytes), gk(bytes), gv(bytes), ws(flash_backward_workspace_bytes(s));
+        hq.upload(q.data(), bytes, st.get());
+        hk.upload(k.data(), bytes, st.get());
+        hv.upload(v.data(), bytes, st.get());
+        hg.upload(g.data(), bytes, st.get());
+        auto f = [](const HipStorage& h) { return (float*)h.ptr(); };
+        flash_backward_f32_dev(s, f(hq), f(hk), f(hv), f(hg), f(gq), f(gk), f(gv), ws.ptr(), ws.byte_len(), st.get());
+        synchronize(st.get());
+        CHECK(gq.to_host<float>() == dq && gk.to_host<float>() == dk && gv.to_host<float>() == dv);
+        HipStorage sq(bytes), sk(bytes), sv(bytes);
+        flash_forward_stats_f32_dev(s, f(hq), f(hk), f(hv), f(ho), f(hl), st.get());
+        flash_backward_saved_f32_dev(s, f(hq), f(hk), f(hv), f(ho), f(hl), f(hg), f(sq), f(sk), f(sv), ws.ptr(),
+                                     ws.byte_len(), st.get());
+        synchronize(st.get());
+        CHECK(sq.to_host<float>() == dq && sk.to_host<float>() == dk && sv.to_host<float>() == dv);
+    }
     {   // N == 1: out == v (reference test single_token_returns_v)
         AttentionShape s = AttentionShape::make(1, 1, 1, 4);
         std::vector<float> q = {1, 2, 3, 4}, k = {4, 3, 2, 1}, v = {0.5f, -1.5f, 2.5f, 7.0f}, out(4);
