@@ -222,11 +222,27 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
 
     // leading-masked-tile rule of the reference's recurrence (cpu_forward.rs:364-384), as in the kernel above
     bool poison = false;
+    // The keep vector as one bit per key in LDS (up to 32 * kKeepWords keys; longer ones are read byte by byte in the
+    // loop): a tile step then reads one word, and a tile without a hidden key is not masked at all.
+    constexpr int kKeepWords = 1024;
+    __shared__ uint32_t keep_bits[kKeepWords];
+    const bool keep_in_lds = (p.mask == kMaskPadding) && N <= 32 * kKeepWords;
     if (p.mask == kMaskPadding) {
         int lim = p.ref_bc < N ? p.ref_bc : N;
         bool any = false;
         for (int j = lane; j < lim; j += kWave) any |= (p.keep[j] != 0);
         poison = !__any(any);
+        if (keep_in_lds) {
+            for (int base = wave * kWave; base < N; base += NW * kWave) {
+                const int key = base + lane;
+                const unsigned long long bal = __ballot(key < N && p.keep[key] != 0);
+                if (lane == 0) {
+                    keep_bits[base >> 5] = (uint32_t)bal;
+                    keep_bits[(base >> 5) + 1] = (uint32_t)(bal >> 32);
+                }
+            }
+            __syncthreads();
+        }
     }
 
     // Q as B operand, in registers: qreg[4j + i] = Q[q0 + col][8j + 4hh + i]
@@ -351,7 +367,9 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
         }
         // register i of the accumulator holds key row 8*(i/4) + 4*hh + (i%4), query row `col`
         float m_tile = neg_inf();
-        const bool edge = (kv0 + kRows > N) || (p.mask == kMaskCausal && kv0 + kRows - 1 > q0) || (p.mask == kMaskPadding);
+        const uint32_t keep_word = keep_in_lds ? keep_bits[kv0 >> 5] : 0u;  // bit r: key kv0 + r is visible
+        const bool edge = (kv0 + kRows > N) || (p.mask == kMaskCausal && kv0 + kRows - 1 > q0) ||
+                          (p.mask == kMaskPadding && keep_word != 0xffffffffu);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             float x = s[i] * p.scale + bias[i];
@@ -359,7 +377,10 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
                 int kr = kv0 + 8 * (i >> 2) + 4 * hh + (i & 3);
                 bool masked = kr >= N;
                 if (p.mask == kMaskCausal) masked |= kr > q_row;
-                if (p.mask == kMaskPadding) masked |= (kr < N) && (p.keep[kr] == 0);
+                if (p.mask == kMaskPadding) {
+                    if (keep_in_lds) masked |= ((keep_word >> (8 * (i >> 2) + 4 * hh + (i & 3))) & 1u) == 0;
+                    else masked |= (kr < N) && (p.keep[kr] == 0);
+                }
                 x = masked ? neg_inf() : x;
             }
             s[i] = x;
