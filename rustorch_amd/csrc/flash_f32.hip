@@ -174,7 +174,9 @@ __global__ __launch_bounds__(64) void flash_fwd_f32_kernel(FlashF32Params p) {
 // The contraction index of the score product is walked in the order d = 8j + 4*half + i (i = 0..3) for both
 // operands, so that a lane fetches its four K values of a chunk with one 16-byte LDS read and Q stays in
 // registers for the whole job.
-template <int DT, bool kExactD>  // kExactD: dim == 32 * DT, no column guards anywhere
+// kExactD: dim == 32 * DT, no column guards anywhere.  kPad: the instantiation for Mask::Padding (the only one that
+// carries the keep bits in LDS and looks at p.keep).
+template <int DT, bool kExactD, bool kPad>
 __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_kernel(FlashF32Params p) {
     constexpr int DPAD = 32 * DT;       // dim rounded up to a multiple of 32 (columns beyond dim are zeros in LDS)
     constexpr int LDK = DPAD + 4;       // row stride of the K tile: 16-byte reads of 16 rows tile all banks
@@ -225,9 +227,9 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
     // The keep vector as one bit per key in LDS (up to 32 * kKeepWords keys; longer ones are read byte by byte in the
     // loop): a tile step then reads one word, and a tile without a hidden key is not masked at all.
     constexpr int kKeepWords = 1024;
-    __shared__ uint32_t keep_bits[kKeepWords];
-    const bool keep_in_lds = (p.mask == kMaskPadding) && N <= 32 * kKeepWords;
-    if (p.mask == kMaskPadding) {
+    __shared__ uint32_t keep_bits[kPad ? kKeepWords : 2];
+    const bool keep_in_lds = kPad && N <= 32 * kKeepWords;
+    if constexpr (kPad) {
         int lim = p.ref_bc < N ? p.ref_bc : N;
         bool any = false;
         for (int j = lane; j < lim; j += kWave) any |= (p.keep[j] != 0);
@@ -369,7 +371,7 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
         float m_tile = neg_inf();
         const uint32_t keep_word = keep_in_lds ? keep_bits[kv0 >> 5] : 0u;  // bit r: key kv0 + r is visible
         const bool edge = (kv0 + kRows > N) || (p.mask == kMaskCausal && kv0 + kRows - 1 > q0) ||
-                          (p.mask == kMaskPadding && keep_word != 0xffffffffu);
+                          (kPad && keep_word != 0xffffffffu);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             float x = s[i] * p.scale + bias[i];
@@ -377,7 +379,7 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
                 int kr = kv0 + 8 * (i >> 2) + 4 * hh + (i & 3);
                 bool masked = kr >= N;
                 if (p.mask == kMaskCausal) masked |= kr > q_row;
-                if (p.mask == kMaskPadding) {
+                if constexpr (kPad) {
                     if (keep_in_lds) masked |= ((keep_word >> (8 * (i >> 2) + 4 * hh + (i & 3))) & 1u) == 0;
                     else masked |= (kr < N) && (p.keep[kr] == 0);
                 }
@@ -495,23 +497,31 @@ hipError_t launch_flash_f32(hipStream_t stream, const FlashF32Params& p) {
         // 8 (dim <= 64) or 4 waves fit on a CU: is every workgroup resident from the start?
         const long long resident = (long long)p.n_cus * (dt <= 2 ? 2 : 1);
         pz.zigzag = (p.mask == kMaskCausal) && ((long long)grid.x * grid.y * grid.z <= resident) ? 1 : 0;
-        const bool exact = (p.dim % 32 == 0);
+        const bool exact = (p.dim % 32 == 0), pad = (p.mask == kMaskPadding);
         switch (dt) {
             case 1:
-                if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<1, true>), grid, block4, 0, stream, pz);
-                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<1, false>), grid, block4, 0, stream, pz);
+                if (pad && exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<1, true, true>), grid, block4, 0, stream, pz);
+                else if (pad) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<1, false, true>), grid, block4, 0, stream, pz);
+                else if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<1, true, false>), grid, block4, 0, stream, pz);
+                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<1, false, false>), grid, block4, 0, stream, pz);
                 break;
             case 2:
-                if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<2, true>), grid, block4, 0, stream, pz);
-                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<2, false>), grid, block4, 0, stream, pz);
+                if (pad && exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<2, true, true>), grid, block4, 0, stream, pz);
+                else if (pad) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<2, false, true>), grid, block4, 0, stream, pz);
+                else if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<2, true, false>), grid, block4, 0, stream, pz);
+                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<2, false, false>), grid, block4, 0, stream, pz);
                 break;
             case 3:
-                if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<3, true>), grid, block4, 0, stream, pz);
-                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<3, false>), grid, block4, 0, stream, pz);
+                if (pad && exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<3, true, true>), grid, block4, 0, stream, pz);
+                else if (pad) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<3, false, true>), grid, block4, 0, stream, pz);
+                else if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<3, true, false>), grid, block4, 0, stream, pz);
+                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<3, false, false>), grid, block4, 0, stream, pz);
                 break;
             case 4:
-                if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<4, true>), grid, block4, 0, stream, pz);
-                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<4, false>), grid, block4, 0, stream, pz);
+                if (pad && exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<4, true, true>), grid, block4, 0, stream, pz);
+                else if (pad) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<4, false, true>), grid, block4, 0, stream, pz);
+                else if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<4, true, false>), grid, block4, 0, stream, pz);
+                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<4, false, false>), grid, block4, 0, stream, pz);
                 break;
             default: return hipErrorInvalidValue;
         }
