@@ -16,6 +16,8 @@
 // Semantics kept from the reference: scale applied to the finished dot product, mask -> -inf
 // after scaling, row without a visible key -> NaN row, `out = O * (1/l)`.  Tiles a causal mask
 // empties are skipped, not computed.
+#include <type_traits>
+
 #include "rt_common.hpp"
 #include "rt_kernels.hpp"
 
@@ -174,10 +176,12 @@ __global__ __launch_bounds__(64) void flash_fwd_f32_kernel(FlashF32Params p) {
 // The contraction index of the score product is walked in the order d = 8j + 4*half + i (i = 0..3) for both
 // operands, so that a lane fetches its four K values of a chunk with one 16-byte LDS read and Q stays in
 // registers for the whole job.
-// kExactD: dim == 32 * DT, no column guards anywhere.  kPad: the instantiation for Mask::Padding (the only one that
-// carries the keep bits in LDS and looks at p.keep).
-template <int DT, bool kExactD, bool kPad>
+// kExactD: dim == 32 * DT, no column guards anywhere.  kMode: one instantiation per way of masking, so that the tile
+// step of each holds only its own tests -- 0 none, 1 causal, 2 Mask::Padding (the only one that carries the keep
+// bits in LDS and looks at p.keep), 3 none plus an additive score bias.
+template <int DT, bool kExactD, int kMode>
 __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_kernel(FlashF32Params p) {
+    constexpr bool kCausal = kMode == 1, kPad = kMode == 2, kBias = kMode == 3;
     constexpr int DPAD = 32 * DT;       // dim rounded up to a multiple of 32 (columns beyond dim are zeros in LDS)
     constexpr int LDK = DPAD + 4;       // row stride of the K tile: 16-byte reads of 16 rows tile all banks
     constexpr int CH = DPAD / 4;        // 16-byte chunks per row
@@ -267,11 +271,11 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
     float l_run = 0.0f;  // this lane's share of the row sum
 
     int kv_end = N;
-    if (p.mask == kMaskCausal) kv_end = min(N, q0 + kRows);
+    if (kCausal) kv_end = min(N, q0 + kRows);
     const int n_tiles = (kv_end + kRows - 1) / kRows;
     // additive bias row of this lane's query (MultiHeadAttention's attn_mask, added to the scaled scores)
     const float* __restrict__ bias_row = nullptr;
-    if (p.bias && q_row < Nq)
+    if (kBias && q_row < Nq)
         bias_row = p.bias + ((size_t)b * p.heads + h) * (size_t)p.bias_bh_stride + (size_t)q_row * (size_t)N;
     const bool bias_vec = ((N & 3) == 0) && ((((uintptr_t)p.bias) & 15) == 0) && ((p.bias_bh_stride & 3) == 0);
 
@@ -340,7 +344,7 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
         f32x16_t bias;
 #pragma unroll
         for (int i = 0; i < 16; i++) bias[i] = 0.0f;
-        if (bias_row) {
+        if (kBias && bias_row) {
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int kr0 = kv0 + 8 * g + 4 * hh;
@@ -370,15 +374,15 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
         // register i of the accumulator holds key row 8*(i/4) + 4*hh + (i%4), query row `col`
         float m_tile = neg_inf();
         const uint32_t keep_word = keep_in_lds ? keep_bits[kv0 >> 5] : 0u;  // bit r: key kv0 + r is visible
-        const bool edge = (kv0 + kRows > N) || (p.mask == kMaskCausal && kv0 + kRows - 1 > q0) ||
+        const bool edge = (kv0 + kRows > N) || (kCausal && kv0 + kRows - 1 > q0) ||
                           (kPad && keep_word != 0xffffffffu);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            float x = s[i] * p.scale + bias[i];
+            float x = kBias ? s[i] * p.scale + bias[i] : s[i] * p.scale;
             if (edge) {
                 int kr = kv0 + 8 * (i >> 2) + 4 * hh + (i & 3);
                 bool masked = kr >= N;
-                if (p.mask == kMaskCausal) masked |= kr > q_row;
+                if (kCausal) masked |= kr > q_row;
                 if constexpr (kPad) {
                     if (keep_in_lds) masked |= ((keep_word >> (8 * (i >> 2) + 4 * hh + (i & 3))) & 1u) == 0;
                     else masked |= (kr < N) && (p.keep[kr] == 0);
@@ -498,31 +502,27 @@ hipError_t launch_flash_f32(hipStream_t stream, const FlashF32Params& p) {
         const long long resident = (long long)p.n_cus * (dt <= 2 ? 2 : 1);
         pz.zigzag = (p.mask == kMaskCausal) && ((long long)grid.x * grid.y * grid.z <= resident) ? 1 : 0;
         const bool exact = (p.dim % 32 == 0), pad = (p.mask == kMaskPadding);
+        if (p.bias && p.mask != kMaskNone) return hipErrorInvalidValue;  // a bias comes without a mask kind
+        const int mode = pad ? 2 : (p.mask == kMaskCausal ? 1 : (p.bias ? 3 : 0));
+        auto launch = [&](auto dt_c, auto exact_c) {
+            constexpr int kDT = decltype(dt_c)::value;
+            constexpr bool kEx = decltype(exact_c)::value;
+            switch (mode) {
+                case 0: hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<kDT, kEx, 0>), grid, block4, 0, stream, pz); break;
+                case 1: hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<kDT, kEx, 1>), grid, block4, 0, stream, pz); break;
+                case 2: hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<kDT, kEx, 2>), grid, block4, 0, stream, pz); break;
+                default: hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<kDT, kEx, 3>), grid, block4, 0, stream, pz); break;
+            }
+        };
+        auto launch_dt = [&](auto dt_c) {
+            if (exact) launch(dt_c, std::true_type{});
+            else launch(dt_c, std::false_type{});
+        };
         switch (dt) {
-            case 1:
-                if (pad && exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<1, true, true>), grid, block4, 0, stream, pz);
-                else if (pad) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<1, false, true>), grid, block4, 0, stream, pz);
-                else if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<1, true, false>), grid, block4, 0, stream, pz);
-                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<1, false, false>), grid, block4, 0, stream, pz);
-                break;
-            case 2:
-                if (pad && exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<2, true, true>), grid, block4, 0, stream, pz);
-                else if (pad) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<2, false, true>), grid, block4, 0, stream, pz);
-                else if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<2, true, false>), grid, block4, 0, stream, pz);
-                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<2, false, false>), grid, block4, 0, stream, pz);
-                break;
-            case 3:
-                if (pad && exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<3, true, true>), grid, block4, 0, stream, pz);
-                else if (pad) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<3, false, true>), grid, block4, 0, stream, pz);
-                else if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<3, true, false>), grid, block4, 0, stream, pz);
-                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<3, false, false>), grid, block4, 0, stream, pz);
-                break;
-            case 4:
-                if (pad && exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<4, true, true>), grid, block4, 0, stream, pz);
-                else if (pad) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<4, false, true>), grid, block4, 0, stream, pz);
-                else if (exact) hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<4, true, false>), grid, block4, 0, stream, pz);
-                else hipLaunchKernelGGL((flash_fwd_f32_splitk_kernel<4, false, false>), grid, block4, 0, stream, pz);
-                break;
+            case 1: launch_dt(std::integral_constant<int, 1>{}); break;
+            case 2: launch_dt(std::integral_constant<int, 2>{}); break;
+            case 3: launch_dt(std::integral_constant<int, 3>{}); break;
+            case 4: launch_dt(std::integral_constant<int, 4>{}); break;
             default: return hipErrorInvalidValue;
         }
         return hipGetLastError();
