@@ -393,12 +393,15 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_fwd_f32_splitk_k
             m_tile = (x > m_tile) ? x : m_tile;  // NaN never wins, as in the reference's `if x > m`
         }
         {
-            float o = other_half(m_tile);
-            m_tile = (o > m_tile) ? o : m_tile;
+            // the two halves of the wave hold the same query rows: v_permlane32_swap leaves the lower halves' values
+            // in one register and the upper halves' in the other, without a trip through LDS (neither is NaN)
+            auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(m_tile), __float_as_uint(m_tile), false, false);
+            const float lo = __uint_as_float(r[0]), hi = __uint_as_float(r[1]);
+            m_tile = (hi > lo) ? hi : lo;
         }
         float m_new = (m_tile > m_run) ? m_tile : m_run;
         float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
-        float alpha = (m_run == neg_inf()) ? 0.0f : expf(m_run - m_use);
+        float alpha = (m_run == neg_inf()) ? 0.0f : __builtin_amdgcn_exp2f((m_run - m_use) * kLog2e);
         m_run = m_new;
         // exp(x) as exp2(x * log2 e) on the hardware exp2: the difference is taken first (exact for the terms
         // that matter), so the argument carries one rounding, about 1e-7 relative on each weight
