@@ -39,7 +39,7 @@ PEAK_F32_TFLOPS = 157.3     # MI355X dense f32 MFMA
 # Counters cannot be read from inside this process; these are the committed measurements, not live values.
 TRAFFIC_PREFILL_BYTES = (270900 * 2.0 + 131100 * 1.0) * 1024
 TRAFFIC_DECODE_BYTES = (623700 * 2.0 + 3224 * 1.0) * 1024
-TRAFFIC_F32_BYTES = (6254 * 2.0 + 4096 * 1.0) * 1024
+TRAFFIC_F32_BYTES = (6229 * 2.0 + 4096 * 1.0) * 1024
 # the four kernels of one backward step (forward, delta, dK/dV, dQ): FETCH_SIZE 6248 + 4109 + 8343 + 9359, WRITE_SIZE 4160 + 128 + 8192 + 6144
 TRAFFIC_BWD_BYTES = (28059 * 2.0 + 18624 * 1.0) * 1024
 
@@ -318,7 +318,7 @@ def main():
                                       "tensors resident in HBM", "flop_convention": "4*B*H*D*N*(N+1)/2 (causal-counted)"},
                "roofline": {"bound": "mfma", "achieved": flops_f / (tm.mean_ms * 1e-3) / 1e12, "peak": PEAK_F32_TFLOPS,
                             "unit": "TFLOP/s", "frac": flops_f / (tm.mean_ms * 1e-3) / 1e12 / PEAK_F32_TFLOPS,
-                            "traffic": TRAFFIC_F32_BYTES, "kernel": "flash_fwd_f32_splitk_kernel<2>"}}
+                            "traffic": TRAFFIC_F32_BYTES, "kernel": "flash_fwd_f32_splitk_kernel<2, exact, causal>"}}
         if not args.no_cpu:
             threads = min(oracle.max_threads(), 16)
             got = dof.download(np.float32)
