@@ -252,7 +252,7 @@ int rt_qk_norm_rope_kv_append_bf16(void *stream, void *q, const void *k_in, cons
 /* LlmKernels::gqa_decode_online_bf16 -- llm_kernels.rs:396-457, :915-958.  q/out
  * [n_heads,head_dim] bf16, caches [n_kv,max_seq,head_dim] bf16 of which [..kv_len] is read;
  * kv head = h*n_kv/n_heads; f32 accumulation, output rounded once.  Runs the split-K kernels of the batched entry on
- * a batch of one (head_dim 64 or 128, at most 16 query heads per kv head; other shapes take a one-workgroup-per-head
+ * a batch of one (head_dim 64, 128 or 256, at most 16 query heads per kv head; other shapes take a one-workgroup-per-head
  * kernel).  The reference's signature has no workspace: the partials go to a buffer the library keeps per
  * (device, stream), allocated by the first call on a stream (so that call must not be under stream capture; later
  * calls allocate nothing unless max_seq grows). */
@@ -263,7 +263,9 @@ int rt_gqa_decode_online_bf16(void *stream, const void *q, const void *k_cache, 
 /* The batched, ragged form of the same call: q/out [batch,n_heads,head_dim], caches
  * [batch,n_kv,max_seq,head_dim], kv_lens device int32[batch] (sequence b reads [..kv_lens[b]]).
  * Split-K over the context with a second-pass (m, l, o) merge; `workspace` (device, at least
- * rt_gqa_decode_workspace_bytes(...) bytes, 256-byte aligned) holds the partial results.
+ * rt_gqa_decode_workspace_bytes(...) bytes, 256-byte aligned) holds the partial results.  The split-K kernels cover
+ * head_dim 64, 128 and 256 with at most 16 query heads per kv head; other shapes take a one-workgroup-per-head kernel
+ * (head_dim <= 512) that needs no workspace (rt_gqa_decode_workspace_bytes returns 0 for them).
  * batch = 1 with kv_lens = [kv_len] is the reference call.  A sequence with kv_lens[b] == 0
  * gives rows of +0.0 (the reference kernel ends with o / fmaxf(l, 1e-12f) = 0, llm_kernels.rs:456;
  * crates/rustorch-nn/src/gqa.rs:260-261 fills the row with 0 before an empty key loop). */

@@ -551,7 +551,7 @@ hipError_t launch_split_hd(hipStream_t stream, const DecodeSplitParams& p) {
 bool decode_split_supported(int heads, int kv_heads, int dim) {
     if (kv_heads <= 0 || heads % kv_heads != 0) return false;
     int g = heads / kv_heads;
-    return (dim == 64 || dim == 128) && g <= 16;
+    return (dim == 64 || dim == 128 || dim == 256) && g <= 16;
 }
 
 int decode_split_span_min(int batch) { return batch == 1 ? kDecSpanMinOne : kDecSpanMin; }
@@ -571,6 +571,7 @@ hipError_t launch_decode_split(hipStream_t stream, const DecodeSplitParams& p) {
     if (p.n_waves <= 0 || p.span_min <= 0) return hipErrorInvalidValue;
     if (p.dim == 64) return launch_split_hd<64>(stream, p);
     if (p.dim == 128) return launch_split_hd<128>(stream, p);
+    if (p.dim == 256) return launch_split_hd<256>(stream, p);
     return hipErrorInvalidValue;
 }
 

@@ -30,7 +30,8 @@ def test_kv_append_bf16_matches_oracle(oracle):
 
 
 @pytest.mark.parametrize("hq,hkv,d,max_seq,kv_len", [(8, 2, 32, 320, 1), (8, 2, 32, 320, 77), (32, 8, 128, 600, 600),
-                                                     (6, 3, 96, 50, 49), (4, 4, 256, 40, 40), (8, 2, 64, 10, 0)])
+                                                     (6, 3, 96, 50, 49), (4, 4, 256, 40, 40), (8, 2, 64, 10, 0),
+                                                     (16, 2, 256, 4096, 4096), (16, 2, 256, 100, 64), (8, 8, 256, 300, 257)])
 def test_gqa_decode_online_bf16_matches_oracle(oracle, hq, hkv, d, max_seq, kv_len):
     """The reference call (batch 1): compared with the restated device kernel (bf16 out) and with
     the CPU path in f32."""
@@ -71,6 +72,8 @@ def run_batched(oracle, qb, kb, vb, lens, b, hq, hkv, d, max_seq):
     (2, 16, 8, 64, 300, [300, 17]),
     (2, 6, 2, 128, 100, [100, 50]),   # group of 3: outside the split-K kernel, generic path
     (2, 4, 2, 96, 100, [100, 50]),    # head dim 96: generic path
+    (3, 16, 2, 256, 600, [600, 1, 333]),
+    (2, 8, 8, 256, 130, [0, 130]),
 ])
 def test_gqa_decode_batched_matches_oracle(oracle, b, hq, hkv, d, max_seq, lens):
     qb, qf = bf16_round(seeded_normal((b, hq, d), 1))
