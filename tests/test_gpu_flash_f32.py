@@ -243,3 +243,34 @@ def test_gqa_errors():
     with pytest.raises(ra.WrongInputLen) as ei:
         ra.gqa_forward_f32(z(16), z(8), z(8), z(15), 1, 4, 2, 1, 1, 4)
     assert ei.value.which == "out"
+
+
+def test_host_slice_calls_from_several_threads(oracle):
+    """flash_forward is re-entrant in the reference (rayon's global pool, no state of its own).  Here small calls share
+    one pinned staging buffer: one call at a time holds it, a concurrent one copies buffer by buffer.  Four threads
+    call at once (ctypes releases the interpreter lock during the call) and every result must be its own."""
+    import threading
+
+    shapes = [(1, 2, 40, 16), (2, 1, 65, 32), (1, 1, 130, 64), (1, 3, 33, 8)]
+    work = []
+    for t, bhnd in enumerate(shapes):
+        shape = ra.AttentionShape.new(*bhnd)
+        bufs = [lcg_buffer(shape.buffer_len(), 100 * t + i, 2.0) for i in range(3)]
+        want = oracle.flash_forward_masked(oracle.AttentionShape(*bhnd), *bufs, "causal")
+        work.append((shape, bufs, want))
+    errors = []
+
+    def run(idx):
+        shape, bufs, want = work[idx]
+        for _ in range(25):
+            got = ra.flash_forward_masked(shape, *bufs, ra.Mask.causal())
+            d = max_abs(got, want)
+            if not d <= TOL:
+                errors.append((idx, d))
+
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(len(work))]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors[:3]
