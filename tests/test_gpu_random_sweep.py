@@ -129,3 +129,36 @@ def test_random_backward_cases_match_oracle(oracle, seed):
             err = float(np.abs(g - w).max())
             assert np.isfinite(g).all() and err <= 2e-5 * max(1.0, float(np.abs(w).max())), \
                 f"backward B{b} H{h} N{n} D{d} {name}: max-abs {err}"
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_random_mha_and_gqa_cases_match_oracle(oracle, seed):
+    """The masked / cross-attention core and gqa_forward_f32 on random shapes: self and cross lengths, head dims that
+    are and are not multiples of 4 or 32 (the tiled kernel, its zero-padded form and the row kernel), shared and
+    per-head additive masks, every grouping of query heads."""
+    rng = np.random.default_rng(seed)
+    for _ in range(100):
+        b, h = int(rng.integers(1, 4)), int(rng.integers(1, 5))
+        tq = int(rng.choice([1, 2, 7, 31, 32, 33, 64, 100, 129, 257]))
+        tkv = tq if rng.random() < 0.4 else int(rng.choice([1, 3, 32, 33, 65, 128, 200, 300, 513]))
+        d = int(rng.choice([1, 3, 4, 8, 12, 16, 20, 32, 40, 64, 80, 96, 100, 128, 132, 160]))
+        q = rng.standard_normal(b * tq * h * d).astype(np.float32)
+        k = rng.standard_normal(b * tkv * h * d).astype(np.float32)
+        v = rng.standard_normal(b * tkv * h * d).astype(np.float32)
+        kind = int(rng.integers(0, 4))
+        mask = None
+        if kind == 1:
+            mask = np.where(rng.random((tq, tkv)) > 0.3, 0.0, -1.0e4).astype(np.float32)
+        elif kind == 2:
+            mask = rng.standard_normal((b * h, tq, tkv)).astype(np.float32)
+        elif kind == 3 and tq == tkv:
+            mask = ra.causal_mask(tq)
+        got = ra.mha_forward_masked_f32(q, k, v, b, tq, tkv, h, d, mask)
+        want = oracle.mha_forward_masked(q, k, v, b, tq, tkv, h, d, mask)
+        _compare(f"mha B{b} Tq{tq} Tkv{tkv} H{h} D{d} mask{kind}", got, want, 1e-5)
+        hkv = int(rng.choice([x for x in (1, 2, 4) if h % x == 0]))
+        kk = rng.standard_normal(b * hkv * tkv * d).astype(np.float32)
+        vv = rng.standard_normal(b * hkv * tkv * d).astype(np.float32)
+        out = np.zeros(b * h * tq * d, dtype=np.float32)
+        ra.gqa_forward_f32(q, kk, vv, out, b, h, hkv, tq, tkv, d)
+        _compare(f"gqa B{b} H{h}/{hkv} Sq{tq} Skv{tkv} D{d}", out, oracle.gqa_forward_f32(q, kk, vv, b, h, hkv, tq, tkv, d), 1e-5)
