@@ -209,6 +209,12 @@ int rt_mha_forward_masked_f32(const float *q, size_t q_len, const float *k, size
                               const float *mask, size_t mask_len, float *out, size_t out_len, size_t batch,
                               size_t t_q, size_t t_kv, size_t heads, size_t head_dim, rt_err_detail *err);
 
+/* The same attention on device-resident tensors, enqueued on `stream` (no host checks of the tensor lengths are
+ * possible; the mask length is checked as above). */
+int rt_mha_forward_masked_f32_dev(void *stream, const float *q, const float *k, const float *v, const float *mask,
+                                  size_t mask_len, float *out, size_t batch, size_t t_q, size_t t_kv, size_t heads,
+                                  size_t head_dim, rt_err_detail *err);
+
 /* ---- decode, device pointers ------------------------------------------------------------------ */
 
 /* LlmKernels::kv_append_bf16 -- crates/rustorch-cuda/src/llm_kernels.rs:353-372, :874-910.

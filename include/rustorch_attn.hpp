@@ -298,6 +298,17 @@ inline std::vector<float> mha_forward_masked_f32(const std::vector<float>& q, co
     return out;
 }
 
+// mha_forward_masked_f32 on device-resident tensors, enqueued on `stream`; `mask` is a device buffer of mask_len
+// elements (t_q*t_kv or batch*heads*t_q*t_kv) or nullptr.
+inline void mha_forward_masked_f32_dev(const float* q, const float* k, const float* v, float* out, size_t batch,
+                                       size_t t_q, size_t t_kv, size_t heads, size_t head_dim,
+                                       const float* mask = nullptr, size_t mask_len = 0, void* stream = nullptr) {
+    rt_err_detail e;
+    int rc = rt_mha_forward_masked_f32_dev(stream, q, k, v, mask, mask_len, out, batch, t_q, t_kv, heads, head_dim, &e);
+    if (rc == RT_ERR_WRONG_INPUT_LEN) detail::check_gqa(rc, e);  // which = "mask"
+    detail::check_attention(rc, e);
+}
+
 // The branch MultiHeadAttention::forward takes for the attention between its projections, under no_grad on contiguous
 // f32 tensors (attention.rs:325-333, :347-356).
 enum class MhaRoute { Identity, Flash, Composed };

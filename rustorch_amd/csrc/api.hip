@@ -725,6 +725,51 @@ RT_API int rt_mha_flash_forward_f32(const float* q, size_t q_len, const float* k
     return st.fetch(err);
 }
 
+namespace {
+
+// The attention of rt_mha_forward_masked_f32 on device-resident tensors (arguments already checked).
+int mha_masked_device(hipStream_t stream, const float* q, const float* k, const float* v, const float* mask,
+                      size_t mask_len, float* out, size_t batch, size_t t_q, size_t t_kv, size_t heads,
+                      size_t head_dim, rt_err_detail* err) {
+    const size_t one_mask = t_q * t_kv, all_masks = batch * heads * one_mask;
+    int rc = RT_OK;
+    const long long bias_bh_stride = (mask_len == all_masks && all_masks != one_mask) ? (long long)one_mask : 0;
+    auto aligned16 = [](const void* ptr) { return ((uintptr_t)ptr & 15) == 0; };
+    if (t_kv > 0 && head_dim % 4 == 0 && head_dim <= 128 && fits_int(t_kv) && aligned16(q) && aligned16(k) &&
+        aligned16(v) && aligned16(out)) {
+        // a head dim the tiled f32 kernel covers (and 16-byte aligned tensors): the same kernel as the unmasked path,
+        // with the mask's row added to the scaled scores and, for cross-attention, its own number of keys
+        rt_attention_shape shape = {batch, heads, t_q, head_dim, 64, 64};
+        rc = flash_f32_device(stream, &shape, heads, q, k, v, RT_MASK_NONE, nullptr, out, err, true,
+                              mask_len ? mask : nullptr, bias_bh_stride, nullptr, t_kv);
+        return rc;
+    }
+    rt::AttnRowsParams p{};
+    p.q = q;
+    p.k = k;
+    p.v = v;
+    p.out = out;
+    p.kv_lens = nullptr;
+    p.batch = (int)batch;
+    p.heads = (int)heads;
+    p.kv_heads = (int)heads;
+    p.seq_q = (int)t_q;
+    p.kv_len = (int)t_kv;
+    p.kv_stride = (int)t_kv;
+    p.dim = (int)head_dim;
+    p.head_map = 0;
+    p.scale = 1.0f / sqrtf((float)head_dim);
+    p.bias = mask_len ? mask : nullptr;
+    p.bias_bh_stride = bias_bh_stride;
+    p.use_layout = 1;
+    p.lq = p.lo = rt::layout_bnhd((long long)heads, (long long)t_q, (int)head_dim);
+    p.lkv = rt::layout_bnhd((long long)heads, (long long)t_kv, (int)head_dim);
+    HIP_TRY(rt::launch_attn_rows_f32(stream, p), "attn_rows_f32 launch");
+    return RT_OK;
+}
+
+}  // namespace
+
 RT_API int rt_mha_forward_masked_f32(const float* q, size_t q_len, const float* k, size_t k_len, const float* v,
                                      size_t v_len, const float* mask, size_t mask_len, float* out, size_t out_len,
                                      size_t batch, size_t t_q, size_t t_kv, size_t heads, size_t head_dim,
@@ -757,39 +802,33 @@ RT_API int rt_mha_forward_masked_f32(const float* q, size_t q_len, const float* 
     st.out(out, q_expected * 4, &dout.p);
     rc = st.commit(err);
     if (rc) return rc;
-    const long long bias_bh_stride = (mask_len == all_masks && all_masks != one_mask) ? (long long)one_mask : 0;
-    if (t_kv > 0 && head_dim % 4 == 0 && head_dim <= 128 && fits_int(t_kv)) {
-        // a head dim the tiled f32 kernel covers: the same kernel as the unmasked path, with the mask's row added to
-        // the scaled scores and, for cross-attention, its own number of keys
-        rt_attention_shape shape = {batch, heads, t_q, head_dim, 64, 64};
-        rc = flash_f32_device(nullptr, &shape, heads, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p,
-                              RT_MASK_NONE, nullptr, (float*)dout.p, err, true, mask_len ? (const float*)dm.p : nullptr,
-                              bias_bh_stride, nullptr, t_kv);
-        if (rc) return rc;
-        return st.fetch(err);
-    }
-    rt::AttnRowsParams p{};
-    p.q = dq.p;
-    p.k = dk.p;
-    p.v = dv.p;
-    p.out = dout.p;
-    p.kv_lens = nullptr;
-    p.batch = (int)batch;
-    p.heads = (int)heads;
-    p.kv_heads = (int)heads;
-    p.seq_q = (int)t_q;
-    p.kv_len = (int)t_kv;
-    p.kv_stride = (int)t_kv;
-    p.dim = (int)head_dim;
-    p.head_map = 0;
-    p.scale = 1.0f / sqrtf((float)head_dim);
-    p.bias = mask_len ? (const float*)dm.p : nullptr;
-    p.bias_bh_stride = bias_bh_stride;
-    p.use_layout = 1;
-    p.lq = p.lo = rt::layout_bnhd((long long)heads, (long long)t_q, (int)head_dim);
-    p.lkv = rt::layout_bnhd((long long)heads, (long long)t_kv, (int)head_dim);
-    HIP_TRY(rt::launch_attn_rows_f32(nullptr, p), "attn_rows_f32 launch");
+    rc = mha_masked_device(nullptr, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p,
+                           mask_len ? (const float*)dm.p : nullptr, mask_len, (float*)dout.p, batch, t_q, t_kv, heads,
+                           head_dim, err);
+    if (rc) return rc;
     return st.fetch(err);
+}
+
+RT_API int rt_mha_forward_masked_f32_dev(void* stream, const float* q, const float* k, const float* v, const float* mask,
+                                         size_t mask_len, float* out, size_t batch, size_t t_q, size_t t_kv,
+                                         size_t heads, size_t head_dim, rt_err_detail* err) {
+    clear_err(err);
+    if (head_dim == 0) return fail(err, RT_ERR_ZERO_DIM, -1, 0, 0, "dim must be > 0");
+    const size_t embed = heads * head_dim;
+    const size_t q_expected = batch * t_q * embed, kv_expected = batch * t_kv * embed;
+    const size_t one_mask = t_q * t_kv, all_masks = batch * heads * one_mask;
+    if (!mask) mask_len = 0;
+    if (mask_len != 0 && mask_len != one_mask && mask_len != all_masks)
+        return fail(err, RT_ERR_WRONG_INPUT_LEN, RT_WHICH_MASK, one_mask, mask_len, "mask length");
+    if (q_expected == 0) return RT_OK;
+    if (!q || !out || (kv_expected && (!k || !v))) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    if (head_dim > 512) return fail(err, RT_ERR_UNSUPPORTED, -1, 512, head_dim, "rows kernel covers dim <= 512");
+    if (heads > 65535 || batch > 65535 || t_q > 0x7fffffffull || t_kv > 0x7fffffffull || embed > 0x7fffffffull)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    int rc = ensure_device(err);
+    if (rc) return rc;
+    return mha_masked_device((hipStream_t)stream, q, k, v, mask_len ? mask : nullptr, mask_len, out, batch, t_q, t_kv,
+                             heads, head_dim, err);
 }
 
 RT_API int rt_flash_forward_varlen_bf16_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,

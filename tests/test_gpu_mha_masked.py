@@ -102,3 +102,26 @@ def test_routing_of_multi_head_attention(oracle):
         assert np.abs(got - want).max() <= 1e-5, route
         if route == "identity":
             assert np.array_equal(got, v)
+
+
+@pytest.mark.parametrize("b,tq,tkv,h,d,kind", [(2, 40, 40, 2, 32, "causal"), (1, 70, 333, 3, 80, "per_head"),
+                                                (2, 33, 9, 2, 6, "none"), (1, 5, 64, 2, 130, "shared")])
+def test_device_entry_matches_host_entry(b, tq, tkv, h, d, kind):
+    """rt_mha_forward_masked_f32_dev on a stream of its own gives the bits of the host-slice entry (same kernels)."""
+    from _gpu import dev
+
+    rng = np.random.default_rng(13)
+    q = rng.standard_normal(b * tq * h * d).astype(np.float32)
+    k = rng.standard_normal(b * tkv * h * d).astype(np.float32)
+    v = rng.standard_normal(b * tkv * h * d).astype(np.float32)
+    mask = {"none": None, "causal": ra.causal_mask(tq) if tq == tkv else None,
+            "shared": np.where(rng.random((tq, tkv)) > 0.3, 0.0, -1.0e4).astype(np.float32),
+            "per_head": rng.standard_normal((b * h, tq, tkv)).astype(np.float32)}[kind]
+    want = ra.mha_forward_masked_f32(q, k, v, b, tq, tkv, h, d, mask)
+    st = ra.Stream()
+    dq, dk, dv = dev(q), dev(k), dev(v)
+    dm = dev(mask.ravel()) if mask is not None else None
+    dout = ra.HipStorage.zeros(q.nbytes)
+    ra.mha_forward_masked_f32_dev(dq, dk, dv, dout, b, tq, tkv, h, d, dm, 0 if mask is None else mask.size, stream=st)
+    st.synchronize()
+    assert np.array_equal(dout.download(np.float32), want)
