@@ -122,6 +122,12 @@ int rt_gqa_forward_f32(const float *q, size_t q_len, const float *k, size_t k_le
                        float *out, size_t out_len, size_t batch, size_t n_heads, size_t n_kv_heads, size_t seq_q,
                        size_t seq_kv, size_t head_dim, rt_err_detail *err);
 
+/* gqa_forward_f32 (gqa.rs:94-210) on device-resident f32 tensors, enqueued on `stream`: the head-count check and the
+ * same kernels; the tensor lengths cannot be checked. */
+int rt_gqa_forward_f32_dev(void *stream, const float *q, const float *k, const float *v, float *out, size_t batch,
+                           size_t n_heads, size_t n_kv_heads, size_t seq_q, size_t seq_kv, size_t head_dim,
+                           rt_err_detail *err);
+
 /* rustorch_nn::attention::mha_flash_forward_f32 -- crates/rustorch-nn/src/attention.rs:452-495.  q, k, v
  * [batch, seq, heads, head_dim] host slices, out [batch, seq, heads*head_dim]; unmasked attention per
  * (batch, head) with the checks of flash_forward on the shape (batch, heads, seq, head_dim), in its order. */

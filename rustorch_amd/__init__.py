@@ -16,7 +16,7 @@ from .errors import (AttentionError, BufferShapeMismatch, DeviceError, GQAError,
                      KVWrongInputLen, LayerOutOfRange,
                      MaskError, OutputShapeMismatch, Overflow, PaddingLengthMismatch, PositionOverflow, RoPEError,
                      RopeWrongInputLen, WrongInputLen, ZeroDim)
-from .gqa import gqa_forward_f32
+from .gqa import gqa_forward_f32, gqa_forward_f32_dev
 from .kv_cache import KVCache
 from .llm_kernels import LlmKernels
 from .masks import MASK_NEG, bool_to_additive, causal_mask, sliding_window_mask

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "librt_attn_hip.so")
 # every symbol include/rt_attn.h declares
 SYMBOLS = (
     "rt_init", "rt_version", "rt_status_name",
-    "rt_flash_forward_f32", "rt_flash_forward_masked_f32", "rt_gqa_forward_f32",
+    "rt_flash_forward_f32", "rt_flash_forward_masked_f32", "rt_gqa_forward_f32", "rt_gqa_forward_f32_dev",
     "rt_flash_backward_f32", "rt_flash_backward_f32_dev", "rt_flash_backward_workspace_bytes",
     "rt_flash_forward_stats_f32_dev", "rt_flash_backward_saved_f32_dev",
     "rt_flash_forward_f32_dev", "rt_flash_forward_bf16_dev", "rt_flash_forward_varlen_bf16_dev",
@@ -82,6 +82,7 @@ def lib():
     L.rt_flash_forward_f32.argtypes = [shp, fp, sz, fp, sz, fp, sz, fp, sz, errp]
     L.rt_flash_forward_masked_f32.argtypes = [shp, fp, sz, fp, sz, fp, sz, C.c_int, u8p, sz, fp, sz, errp]
     L.rt_gqa_forward_f32.argtypes = [fp, sz, fp, sz, fp, sz, fp, sz, sz, sz, sz, sz, sz, sz, errp]
+    L.rt_gqa_forward_f32_dev.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, errp]
     L.rt_flash_backward_f32.argtypes = [shp] + [fp, sz] * 7 + [errp]
     L.rt_flash_backward_f32_dev.argtypes = [vp, shp] + [vp] * 8 + [sz, errp]
     L.rt_flash_backward_workspace_bytes.argtypes = [shp]

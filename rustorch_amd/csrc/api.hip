@@ -377,6 +377,48 @@ RT_API int rt_flash_forward_f32(const rt_attention_shape* shape, const float* q,
                                        err);
 }
 
+namespace {
+
+// The attention of rt_gqa_forward_f32 on device-resident tensors (arguments already checked).
+int gqa_device(hipStream_t stream, const float* q, const float* k, const float* v, float* out, size_t batch,
+               size_t n_heads, size_t n_kv_heads, size_t seq_q, size_t seq_kv, size_t head_dim, rt_err_detail* err) {
+    auto aligned16 = [](const void* ptr) { return ((uintptr_t)ptr & 15) == 0; };
+    if (seq_q == seq_kv) {
+        // prefill: unmasked flash; the kernel maps query head -> kv head itself (no replicated copy)
+        rt_attention_shape s = {batch, n_heads, seq_q, head_dim, 64, 64};
+        return flash_f32_device(stream, &s, n_kv_heads, q, k, v, RT_MASK_NONE, nullptr, out, err);
+    }
+    if (seq_kv > 0 && head_dim % 4 == 0 && head_dim <= 128 && aligned16(q) && aligned16(k) && aligned16(v) &&
+        aligned16(out)) {
+        // decode / chunked prefill: every query row attends to all seq_kv keys (gqa.rs:179-208); the tiled kernel
+        // with its own key count
+        rt_attention_shape s = {batch, n_heads, seq_q, head_dim, 64, 64};
+        return flash_f32_device(stream, &s, n_kv_heads, q, k, v, RT_MASK_NONE, nullptr, out, err, false, nullptr, 0,
+                                nullptr, seq_kv);
+    }
+    if (head_dim > 512) return fail(err, RT_ERR_UNSUPPORTED, -1, 512, head_dim, "decode rows kernel covers dim <= 512");
+    if (seq_q > 65535 * 32ull) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, seq_q, "seq_q too large");
+    rt::AttnRowsParams p{};
+    p.q = q;
+    p.k = k;
+    p.v = v;
+    p.out = out;
+    p.kv_lens = nullptr;
+    p.batch = (int)batch;
+    p.heads = (int)n_heads;
+    p.kv_heads = (int)n_kv_heads;
+    p.seq_q = (int)seq_q;
+    p.kv_len = (int)seq_kv;
+    p.kv_stride = (int)seq_kv;
+    p.dim = (int)head_dim;
+    p.head_map = 0;
+    p.scale = 1.0f / sqrtf((float)head_dim);
+    HIP_TRY(rt::launch_attn_rows_f32(stream, p), "attn_rows_f32 launch");
+    return RT_OK;
+}
+
+}  // namespace
+
 RT_API int rt_gqa_forward_f32(const float* q, size_t q_len, const float* k, size_t k_len, const float* v,
                               size_t v_len, float* out, size_t out_len, size_t batch, size_t n_heads,
                               size_t n_kv_heads, size_t seq_q, size_t seq_kv, size_t head_dim, rt_err_detail* err) {
@@ -409,40 +451,28 @@ RT_API int rt_gqa_forward_f32(const float* q, size_t q_len, const float* k, size
     st.out(out, q_expected * 4, &dout.p);
     rc = st.commit(err);
     if (rc) return rc;
-    if (seq_q == seq_kv) {
-        // prefill: unmasked flash; the kernel maps query head -> kv head itself (no replicated copy)
-        rt_attention_shape s = {batch, n_heads, seq_q, head_dim, 64, 64};
-        rc = flash_f32_device(nullptr, &s, n_kv_heads, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p,
-                              RT_MASK_NONE, nullptr, (float*)dout.p, err);
-        if (rc) return rc;
-    } else if (seq_kv > 0 && head_dim % 4 == 0 && head_dim <= 128) {
-        // decode / chunked prefill: every query row attends to all seq_kv keys (gqa.rs:179-208); the tiled kernel
-        // with its own key count
-        rt_attention_shape s = {batch, n_heads, seq_q, head_dim, 64, 64};
-        rc = flash_f32_device(nullptr, &s, n_kv_heads, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p,
-                              RT_MASK_NONE, nullptr, (float*)dout.p, err, false, nullptr, 0, nullptr, seq_kv);
-        if (rc) return rc;
-    } else {
-        if (head_dim > 512) return fail(err, RT_ERR_UNSUPPORTED, -1, 512, head_dim, "decode rows kernel covers dim <= 512");
-        if (seq_q > 65535 * 32ull) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, seq_q, "seq_q too large");
-        rt::AttnRowsParams p{};
-        p.q = dq.p;
-        p.k = dk.p;
-        p.v = dv.p;
-        p.out = dout.p;
-        p.kv_lens = nullptr;
-        p.batch = (int)batch;
-        p.heads = (int)n_heads;
-        p.kv_heads = (int)n_kv_heads;
-        p.seq_q = (int)seq_q;
-        p.kv_len = (int)seq_kv;
-        p.kv_stride = (int)seq_kv;
-        p.dim = (int)head_dim;
-        p.head_map = 0;
-        p.scale = 1.0f / sqrtf((float)head_dim);
-        HIP_TRY(rt::launch_attn_rows_f32(nullptr, p), "attn_rows_f32 launch");
-    }
+    rc = gqa_device(nullptr, (const float*)dq.p, (const float*)dk.p, (const float*)dv.p, (float*)dout.p, batch, n_heads,
+                    n_kv_heads, seq_q, seq_kv, head_dim, err);
+    if (rc) return rc;
     return st.fetch(err);
+}
+
+RT_API int rt_gqa_forward_f32_dev(void* stream, const float* q, const float* k, const float* v, float* out, size_t batch,
+                                  size_t n_heads, size_t n_kv_heads, size_t seq_q, size_t seq_kv, size_t head_dim,
+                                  rt_err_detail* err) {
+    clear_err(err);
+    if (n_kv_heads == 0 || n_heads % n_kv_heads != 0)
+        return fail(err, RT_ERR_HEAD_COUNT_MISMATCH, -1, n_heads, n_kv_heads, "n_heads not divisible by n_kv_heads");
+    if (seq_q == seq_kv && head_dim == 0) return fail(err, RT_ERR_WRONG_INPUT_LEN, RT_WHICH_FLASH, 0, 0, "flash_forward");
+    const size_t q_expected = batch * n_heads * seq_q * head_dim, kv_expected = batch * n_kv_heads * seq_kv * head_dim;
+    if (q_expected == 0) return RT_OK;
+    if (!q || !out || (kv_expected && (!k || !v))) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    if (!fits_int(batch) || !fits_int(n_heads) || !fits_int(seq_q) || !fits_int(seq_kv) || !fits_int(head_dim) ||
+        batch > 65535 || n_heads > 65535)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    int rc = ensure_device(err);
+    if (rc) return rc;
+    return gqa_device((hipStream_t)stream, q, k, v, out, batch, n_heads, n_kv_heads, seq_q, seq_kv, head_dim, err);
 }
 
 // ---- backward (cpu_backward.rs:46-185) ----------------------------------------------------------------

@@ -25,3 +25,13 @@ def gqa_forward_f32(q, k, v, out, batch, n_heads, n_kv_heads, seq_q, seq_kv, hea
                                     out.size, batch, n_heads, n_kv_heads, seq_q, seq_kv, head_dim, C.byref(err))
     raise_for(rc, err)
     return out
+
+
+def gqa_forward_f32_dev(q, k, v, out, batch, n_heads, n_kv_heads, seq_q, seq_kv, head_dim, stream=None):
+    """The same on device-resident f32 tensors; enqueues on `stream` and returns."""
+    from .device import dev_ptr
+
+    err = L.RtErr()
+    rc = L.lib().rt_gqa_forward_f32_dev(stream, dev_ptr(q), dev_ptr(k), dev_ptr(v), dev_ptr(out), batch, n_heads,
+                                        n_kv_heads, seq_q, seq_kv, head_dim, C.byref(err))
+    raise_for(rc, err)

@@ -231,6 +231,25 @@ def test_gqa_forward_matches_oracle(oracle, b, hq, hkv, sq, skv, d):
         assert (o[:, h].max(axis=1) <= vv[:, h // g].max(axis=1) + 1e-5).all()
 
 
+@pytest.mark.parametrize("b,hq,hkv,sq,skv,d", [(2, 8, 2, 130, 130, 64), (1, 8, 2, 100, 333, 64), (1, 6, 2, 65, 31, 20),
+                                              (1, 2, 1, 7, 70, 5), (1, 32, 8, 1, 700, 128)])
+def test_gqa_device_entry_matches_host_entry(b, hq, hkv, sq, skv, d):
+    from _gpu import dev
+
+    q = seeded_normal((b, hq, sq, d), 4)
+    k = seeded_normal((b, hkv, skv, d), 5)
+    v = seeded_normal((b, hkv, skv, d), 6)
+    want = np.zeros(b * hq * sq * d, dtype=np.float32)
+    ra.gqa_forward_f32(q, k, v, want, b, hq, hkv, sq, skv, d)
+    st = ra.Stream()
+    dout = ra.HipStorage.zeros(want.nbytes)
+    ra.gqa_forward_f32_dev(dev(q), dev(k), dev(v), dout, b, hq, hkv, sq, skv, d, stream=st)
+    st.synchronize()
+    assert np.array_equal(dout.download(np.float32), want)
+    with pytest.raises(ra.HeadCountMismatch):
+        ra.gqa_forward_f32_dev(dout, dout, dout, dout, 1, 5, 2, 1, 1, 4)
+
+
 def test_gqa_errors():
     z = lambda n: np.zeros(n, dtype=np.float32)
     with pytest.raises(ra.HeadCountMismatch):
