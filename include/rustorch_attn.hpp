@@ -298,6 +298,15 @@ inline std::vector<float> mha_forward_masked_f32(const std::vector<float>& q, co
     return out;
 }
 
+// gqa_forward_f32 on device-resident tensors, enqueued on `stream`.
+inline void gqa_forward_f32_dev(const float* q, const float* k, const float* v, float* out, size_t batch,
+                                size_t n_heads, size_t n_kv_heads, size_t seq_q, size_t seq_kv, size_t head_dim,
+                                void* stream = nullptr) {
+    rt_err_detail e;
+    detail::check_gqa(rt_gqa_forward_f32_dev(stream, q, k, v, out, batch, n_heads, n_kv_heads, seq_q, seq_kv, head_dim, &e),
+                      e);
+}
+
 // mha_forward_masked_f32 on device-resident tensors, enqueued on `stream`; `mask` is a device buffer of mask_len
 // elements (t_q*t_kv or batch*heads*t_q*t_kv) or nullptr.
 inline void mha_forward_masked_f32_dev(const float* q, const float* k, const float* v, float* out, size_t batch,
