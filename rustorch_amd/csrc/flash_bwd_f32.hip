@@ -343,19 +343,21 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dq_kerne
         for (int i = 0; i < 16; i++) acc_dq[t][i] = 0.0f;
 
     const int n_kt = (N + kRows - 1) / kRows;
+    constexpr bool kPrefetchBoth = (DT != 2);
     TileRegs<DPAD> ra, rb;
     if (vec && wave < n_kt) {
         load_tile_regs<DPAD>(ra, Kg, wave * kRows, N, D, lane);
-        load_tile_regs<DPAD>(rb, Vg, wave * kRows, N, D, lane);
+        if constexpr (kPrefetchBoth) load_tile_regs<DPAD>(rb, Vg, wave * kRows, N, D, lane);
     }
     for (int kt = wave; kt < n_kt; kt += kNW) {
         const int kv0 = kt * kRows;
         if (vec) {
             store_tile_regs<DPAD, LD>(Kt, ra, lane);
-            store_tile_regs<DPAD, LD>(Vt, rb, lane);
+            if constexpr (kPrefetchBoth) store_tile_regs<DPAD, LD>(Vt, rb, lane);
+            else stage_tile<DPAD, LD>(Vt, Vg, kv0, N, D, lane, true);
             if (kt + kNW < n_kt) {
                 load_tile_regs<DPAD>(ra, Kg, kv0 + kNW * kRows, N, D, lane);
-                load_tile_regs<DPAD>(rb, Vg, kv0 + kNW * kRows, N, D, lane);
+                if constexpr (kPrefetchBoth) load_tile_regs<DPAD>(rb, Vg, kv0 + kNW * kRows, N, D, lane);
             }
         } else {
             stage_tile<DPAD, LD>(Kt, Kg, kv0, N, D, lane, false);
