@@ -94,6 +94,10 @@ typedef struct rt_err_detail {
  * compute entry point does the same lazily on first use (the reference compiles its kernels
  * lazily behind a OnceLock, crates/rustorch-cuda/src/llm_kernels.rs:578-641). */
 int rt_init(int device, rt_err_detail *err);
+/* Frees what the library keeps between calls (the per-stream scratch of rt_gqa_decode_online_bf16, the pinned
+ * staging buffer of the host-slice entries).  Optional; no call may be in flight.  The library stays usable: the
+ * buffers come back on demand. */
+int rt_shutdown(rt_err_detail *err);
 const char *rt_version(void);
 const char *rt_status_name(int status);
 

@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "librt_attn_hip.so")
 
 # every symbol include/rt_attn.h declares
 SYMBOLS = (
-    "rt_init", "rt_version", "rt_status_name",
+    "rt_init", "rt_shutdown", "rt_version", "rt_status_name",
     "rt_flash_forward_f32", "rt_flash_forward_masked_f32", "rt_gqa_forward_f32", "rt_gqa_forward_f32_dev",
     "rt_flash_backward_f32", "rt_flash_backward_f32_dev", "rt_flash_backward_workspace_bytes",
     "rt_flash_forward_stats_f32_dev", "rt_flash_backward_saved_f32_dev",
@@ -112,6 +112,7 @@ def lib():
     L.rt_memcpy_h2d.argtypes = [vp, vp, sz, vp, errp]
     L.rt_memcpy_d2h.argtypes = [vp, vp, sz, vp, errp]
     L.rt_stream_synchronize.argtypes = [vp, errp]
+    L.rt_shutdown.argtypes = [errp]
     L.rt_stream_create.argtypes = [errp]
     L.rt_stream_create.restype = vp
     L.rt_stream_destroy.argtypes = [vp, errp]

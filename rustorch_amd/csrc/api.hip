@@ -1199,3 +1199,25 @@ RT_API int rt_stream_destroy(void* stream, rt_err_detail* err) {
     HIP_TRY(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy");
     return RT_OK;
 }
+
+RT_API int rt_shutdown(rt_err_detail* err) {
+    clear_err(err);
+    // what the library keeps between calls: the per-stream scratch of rt_gqa_decode_online_bf16 and the pinned staging
+    // buffer of the host-slice entries.  The caller makes sure no call is in flight.
+    {
+        std::lock_guard<std::mutex> lock(g_ws_mutex);
+        for (auto& kv : g_ws)
+            if (kv.second.ptr) {
+                (void)hipStreamSynchronize(kv.first.second);
+                (void)hipFree(kv.second.ptr);
+            }
+        g_ws.clear();
+    }
+    {
+        std::lock_guard<std::mutex> lock(g_pinned_mutex);
+        if (g_pinned) (void)hipHostFree(g_pinned);
+        g_pinned = nullptr;
+    }
+    (void)hipGetLastError();
+    return RT_OK;
+}

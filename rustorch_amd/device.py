@@ -105,6 +105,12 @@ def init(device: int = 0):
     raise_for(L.lib().rt_init(device, C.byref(err)), err)
 
 
+def shutdown():
+    """Free the buffers the library keeps between calls (it stays usable; they come back on demand)."""
+    err = L.RtErr()
+    raise_for(L.lib().rt_shutdown(C.byref(err)), err)
+
+
 def dev_ptr(x) -> int:
     """Raw device address of a HipStorage, a torch tensor on the GPU, or an int."""
     if x is None:

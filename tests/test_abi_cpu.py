@@ -203,3 +203,8 @@ def test_stream_create_reports_a_missing_device():
         ra.Stream()
     assert ei.value.status == L.RT_ERR_NO_DEVICE
     assert L.lib().rt_stream_destroy(None, C.byref(err)) == L.RT_OK
+
+
+def test_shutdown_without_a_device_is_a_no_op():
+    ra.shutdown()
+    ra.shutdown()

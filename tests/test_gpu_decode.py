@@ -160,3 +160,19 @@ def test_single_sequence_decode_long_contexts_and_streams(oracle):
         for kv_len, dout in outs:
             want = oracle.gqa_decode_batched_bf16(qb, kb, vb, [kv_len], 1, hq, hkv, d, max_seq)
             assert max_abs(oracle.bf16_to_f32(dout.download(np.uint16)), want) <= TOL, (max_seq, kv_len)
+
+
+def test_shutdown_frees_and_the_library_stays_usable(oracle):
+    hq, hkv, d, max_seq, kv_len = 8, 2, 64, 300, 257
+    qb, _ = bf16_round(seeded_normal((hq, d), 1))
+    kb, _ = bf16_round(seeded_normal((hkv, max_seq, d), 2))
+    vb, _ = bf16_round(seeded_normal((hkv, max_seq, d), 3))
+    want = oracle.gqa_decode_batched_bf16(qb, kb, vb, [kv_len], 1, hq, hkv, d, max_seq)
+    for _ in range(2):
+        dout = ra.HipStorage(hq * d * 2)
+        K.gqa_decode_online_bf16(None, dev(qb), dev(kb), dev(vb), dout, hq, hkv, kv_len, d, max_seq)
+        ra.synchronize()
+        assert max_abs(oracle.bf16_to_f32(dout.download(np.uint16)), want) <= TOL
+        small = ra.flash_forward(ra.AttentionShape.new(1, 1, 4, 4), *[np.ones(16, np.float32)] * 3)  # pinned staging
+        assert np.allclose(small, 1.0)
+        ra.shutdown()
