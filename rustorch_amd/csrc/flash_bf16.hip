@@ -42,13 +42,6 @@
 
 #include <type_traits>
 
-// Phase marker for a timing harness that includes this file with its own definition; nothing here.
-#ifndef RT_PHASE
-#define RT_PHASE(id)
-#define RT_PHASE_DECL
-#define RT_PHASE_DUMP
-#endif
-
 namespace rt {
 
 namespace {
@@ -163,7 +156,6 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: branches on it are scalar
     const int grp = wave >> 2;                                  // 0: waves 0-3, 1: waves 4-7 (one of each per SIMD)
     const int col = lane & 31, hh = lane >> 5;
-    RT_PHASE_DECL;
 
     // slot swizzles (see the header): K rows are read 16 at a time at one slot (b128), V rows 4 at a
     // time over 4 adjacent slots (transposing b64 reads)
@@ -453,7 +445,6 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         // ---- C: the products, and right after each the read that refills its operand for the next C.
         // Score and P.V instructions alternate: a score instruction accumulates onto the one before it,
         // and back-to-back dependent matrix instructions would wait for each other.
-        RT_PHASE(0);
         __builtin_amdgcn_s_setprio(3);  // the multiplying wave goes first: its next instruction frees the matrix pipe
         lds_operands_ready();
         __builtin_amdgcn_sched_barrier(0);  // no matrix instruction may be moved ahead of that wait
@@ -481,10 +472,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         }
         if (i == 2) __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wave's share has landed
         if (i == NITEMS - 1) __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): stage st may be refilled
-        RT_PHASE(1);
         __builtin_amdgcn_s_setprio(0);
         cluster_barrier();
-        RT_PHASE(2);
         // ---- S
         if (MODE == kMaskPadding) {
             if (keep_in_lds) {
@@ -502,9 +491,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         // conversions that make it down to that use, past the barrier and in between the matrix
         // instructions; pinning the values here keeps the work in this cluster
         asm volatile("" : "+v"(pB[0]), "+v"(pB[1]), "+v"(l_run));
-        RT_PHASE(3);
         cluster_barrier();
-        RT_PHASE(9);
     };
     auto run_step = [&](int kv0, int kv_next, int st, int mask_from) {
         static_assert(NITEMS == 4, "items per step");
@@ -537,7 +524,6 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         settle_queries();
         __syncthreads();
-        RT_PHASE(10);
 
         // an item needs masking when its last key lies past the last existing key or past the wave's first row
         const int mask_from = kCausal ? min(n_keys - 1, qw) : n_keys - 1;
@@ -583,9 +569,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         uint16_t* __restrict__ og_out = Og;
         const bool padded_row = (MODE == kMaskVarlenCausal) && (q_row >= n_keys);
         job = job_of_round(++round);
-        RT_PHASE(4);
         if (job >= 0) begin_job(job);  // its loads travel while the output is normalised and stored
-        RT_PHASE(5);
 
         // acc_o[dt][i] = O^T[d = 32dt + 8(i/4) + 4hh + i%4][row col of the wave]
         float l = sum_with_other_half(l_run);
@@ -614,7 +598,6 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
                 u32x2_t wv = {cvt_pk_bf16(o[0], o[1]), cvt_pk_bf16(o[2], o[3])};
                 *(u32x2_t __attribute__((address_space(3)))*)(uintptr_t)(park ^ (uint32_t)(16 * (4 * dt + j))) = wv;
             }
-        RT_PHASE(6);
         // (the same wave wrote and now reads: no barrier needed, the LDS queue is in order)
         {
             const int r0 = lane_e / SPR, pos = lane_e % SPR;  // instruction n covers rows n*RPI + r0
@@ -630,9 +613,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
                     *(u32x4_t*)(gp + (size_t)n * RPI * o_pitch_b + (slot_off ^ (uint32_t)(swz_o(n * RPI) * 16))) = v;
             }
         }
-        RT_PHASE(11);
     }
-    RT_PHASE_DUMP;
 }
 
 template <int HD>
