@@ -6,9 +6,16 @@ B=4, H=32, N=4096, D=128 (inputs resident in HBM before the timed region); the s
 times the batched GQA decode workload (batch 64, 32 query / 8 kv heads, D=128, context lengths
 uniform in [512, 8192], Lmax 8192) and reports it under "decode", and the f32 causal prefill of
 B=1, H=8, N=2048, D=64 (the reference's own CPU-runnable case) under "f32_prefill", and the f32
-backward on that shape under "f32_backward".
+backward on that shape under "f32_backward", the padded-batch prefill (B=16, H=16, D=64, lengths in [128, 1024])
+under "padded_prefill" and the long-context prefill (B=1, H=32, N=16384, D=128, Q scaled by 2) under
+"long_prefill".
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only prefill|decode|f32|bwd]
+Every leg first runs a settle phase: launches of the leg's own step until SETTLE_MS of device time have passed
+(after an idle period the clocks first drop and then recover over some tens of milliseconds); the phase is
+reported as settle_ms / settle_launches and is followed by the counted warm-up (--warmup) and the timed region
+(--steps), which is the only part that enters value, ms_per_step and roofline.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only prefill|decode|f32|bwd|padded|long]
 
 Prints ONE JSON line.  `value` is prefill TFLOP/s with causal-counted FLOPs
 (4*B*H*D*N*(N+1)/2: skipped tiles are not credited); `roofline` prices it against the dense bf16
@@ -34,14 +41,35 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 PEAK_F32_TFLOPS = 157.3     # MI355X dense f32 MFMA
-# HBM bytes per launch of the dominant kernels on the bench workloads, from the rocprofv3 --pmc runs
-# summarised under profiles/ (FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB, the factors a 256 MiB copy reads).
-# Counters cannot be read from inside this process; these are the committed measurements, not live values.
-TRAFFIC_PREFILL_BYTES = (270900 * 2.0 + 131100 * 1.0) * 1024
-TRAFFIC_DECODE_BYTES = (623700 * 2.0 + 3224 * 1.0) * 1024
-TRAFFIC_F32_BYTES = (6229 * 2.0 + 4096 * 1.0) * 1024
-# the four kernels of one backward step (forward, delta, dK/dV, dQ): FETCH_SIZE 6248 + 4109 + 8343 + 9359, WRITE_SIZE 4160 + 128 + 8192 + 6144
-TRAFFIC_BWD_BYTES = (28059 * 2.0 + 18624 * 1.0) * 1024
+SETTLE_MS = 100.0           # device time of the settle phase that precedes every leg's warm-up
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def profile_traffic(md_name, entry):
+    """HBM bytes per launch of a kernel (or a step of several kernels) as measured with rocprofv3 --pmc and
+    written down in profiles/<md_name>: the file carries a fenced block
+
+        ```json traffic
+        {"<entry>": {"fetch_size": F, "write_size": W}, ..., "scale": {"fetch_kib": 2.0, "write_kib": 1.0}}
+        ```
+
+    with the FETCH_SIZE / WRITE_SIZE readings per launch and the factors that a copy of known size gave for them.
+    Counters cannot be read from inside this process: the figure is the committed measurement, and it is None
+    when the file or the entry is not there."""
+    import re
+    try:
+        text = open(os.path.join(PROFILES, md_name)).read()
+    except OSError:
+        return None
+    m = re.search(r"```json traffic\n(.*?)```", text, re.S)
+    if not m:
+        return None
+    try:
+        block = json.loads(m.group(1))
+        e, sc = block[entry], block["scale"]
+        return (float(e["fetch_size"]) * float(sc["fetch_kib"]) + float(e["write_size"]) * float(sc["write_kib"])) * 1024
+    except (ValueError, KeyError, TypeError):
+        return None
 
 
 class Hip:
@@ -87,21 +115,44 @@ class Timing:
     pair of HIP events on `stream` around the K steps (nothing is recorded between launches, so the stream runs
     them back to back as a serving loop would).  per: per-step durations of 100 further steps run after the timed
     region, each between its own pair of events (the spread; each reads a few microseconds longer than a
-    back-to-back step)."""
+    back-to-back step).  settle_ms / settle_launches: the settle phase that ran before the warm-up."""
 
-    def __init__(self, wall_ms, region_ms, steps, per):
+    def __init__(self, wall_ms, region_ms, steps, per, settle_ms, settle_launches):
         self.wall_ms, self.mean_ms, self.per = wall_ms, region_ms / steps, per
+        self.settle_ms, self.settle_launches = settle_ms, settle_launches
+
+    def settle(self):
+        return {"settle_ms": self.settle_ms, "settle_launches": self.settle_launches}
 
 
-def time_steps(hip, stream, launch, steps, warmup, spread_steps=100):
+def settle(hip, stream, launch, min_ms=SETTLE_MS):
+    """Launches the step back to back until `min_ms` of device time have passed (event pairs around growing
+    batches).  Returns (device ms, launches).  Not part of any reported rate."""
+    done_ms, n, batch = 0.0, 0, 4
+    e0, e1 = hip.event(), hip.event()
+    while done_ms < min_ms and n < 100000:
+        hip.record(e0, stream)
+        for i in range(batch):
+            launch(n + i)
+        hip.record(e1, stream)
+        ms = hip.elapsed_ms(e0, e1)
+        done_ms += ms
+        n += batch
+        per = max(ms / batch, 1e-3)
+        batch = int(min(max((min_ms - done_ms) / per, 1), 4096))
+    return done_ms, n
+
+
+def time_steps(hip, stream, launch, steps, warmup, spread_steps=100, settle_ms=SETTLE_MS):
+    s_ms, s_n = settle(hip, stream, launch, settle_ms) if settle_ms > 0 else (0.0, 0)
     for i in range(warmup):
-        launch(i)
+        launch(s_n + i)
     hip.sync()
     e0, e1 = hip.event(), hip.event()
     t0 = time.perf_counter()
     hip.record(e0, stream)
     for i in range(steps):
-        launch(warmup + i)
+        launch(s_n + warmup + i)
     hip.record(e1, stream)
     hip.sync()
     wall_ms = (time.perf_counter() - t0) * 1e3
@@ -109,11 +160,11 @@ def time_steps(hip, stream, launch, steps, warmup, spread_steps=100):
     evs = [(hip.event(), hip.event()) for _ in range(spread_steps)]
     for j, (a, b) in enumerate(evs):
         hip.record(a, stream)
-        launch(warmup + steps + j)
+        launch(s_n + warmup + steps + j)
         hip.record(b, stream)
     hip.sync()
     per = np.array([hip.elapsed_ms(a, b) for a, b in evs]) if evs else np.zeros(0)
-    return Timing(wall_ms, region_ms, steps, per)
+    return Timing(wall_ms, region_ms, steps, per, s_ms, s_n)
 
 
 def spread(per):
@@ -147,12 +198,11 @@ def sustained_mfma():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # defaults long enough to leave the first ~15 ms after an idle period, in which the clocks first drop and
-    # then recover (launches of the same kernel take 540, 730, then 530 us): 250 launches are 0.15 s
+    # whatever --steps and --warmup are, every leg is preceded by its settle phase (see the module docstring)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity sample")
-    ap.add_argument("--only", choices=["prefill", "decode", "f32", "bwd"], default=None)
+    ap.add_argument("--only", choices=["prefill", "decode", "f32", "bwd", "padded", "long"], default=None)
     ap.add_argument("--no-ceiling", action="store_true",
                     help="skip the run of rustorch_amd/lib/mfma_sustained (what a loop of nothing but bf16 MFMA "
                          "sustains on this GPU, reported beside the data-sheet peak)")
@@ -182,12 +232,15 @@ def main():
     rng = np.random.default_rng(1234)
     out = {}
 
-    # ------------------------------------------------------------------ prefill (the step)
-    B, H, N, D = 4, 32, 4096, 128
-    prefill = None
-    if args.only in (None, "prefill"):
+    threads = min(oracle.max_threads(), 16)
+
+    def causal_prefill(B, H, N, D, seed, q_scale, cpu_slabs, kernel_name, traffic):
+        """bf16 causal prefill on [B,H,N,D]: timing, and (unless --no-cpu) parity and the CPU baseline on the first
+        `cpu_slabs` (b,h) slabs."""
+        rng_p = np.random.default_rng(seed)
         n_el = B * H * N * D
-        qb, kb, vb = (oracle.f32_to_bf16(rng.standard_normal(n_el, dtype=np.float32)) for _ in range(3))
+        qb = oracle.f32_to_bf16(rng_p.standard_normal(n_el, dtype=np.float32) * np.float32(q_scale))
+        kb, vb = (oracle.f32_to_bf16(rng_p.standard_normal(n_el, dtype=np.float32)) for _ in range(2))
         dq, dk, dv = (ra.HipStorage.from_numpy(x) for x in (qb, kb, vb))
         dout = ra.HipStorage(n_el * 2)
         shape = ra.AttentionShape.new(B, H, N, D)
@@ -199,34 +252,112 @@ def main():
         flops_full = 4.0 * B * H * D * float(N) * N
         ms_step = tm.wall_ms / args.steps
         ms_kernel = tm.mean_ms
-        prefill = {"ms_per_step": ms_step, "kernel_ms_mean": ms_kernel, **spread(tm.per),
-                   "tflops": flops_causal / (ms_step * 1e-3) / 1e12,
-                   "tflops_kernel": flops_causal / (ms_kernel * 1e-3) / 1e12,
-                   "tflops_unmasked_convention": flops_full / (ms_kernel * 1e-3) / 1e12}
+        achieved = flops_causal / (ms_kernel * 1e-3) / 1e12
+        leg = {"ms_per_step": ms_step, "kernel_ms_mean": ms_kernel, **spread(tm.per), **tm.settle(),
+               "tflops": flops_causal / (ms_step * 1e-3) / 1e12,
+               "tflops_unmasked_convention": flops_full / (ms_kernel * 1e-3) / 1e12,
+               "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                            "frac": achieved / PEAK_BF16_TFLOPS, "traffic": traffic, "kernel": kernel_name,
+                            "kernel_ms_mean": ms_kernel, **spread(tm.per)}}
         if not args.no_cpu:
-            # parity + CPU baseline on a sample of (b,h) slabs: the oracle computes every tile, like the reference
-            threads = min(oracle.max_threads(), 16)
-            slabs = list(range(B * H))  # the whole workload: every (b,h) slab is checked
+            # parity + CPU baseline on (b,h) slabs: the oracle computes every tile, like the reference
+            slabs = list(range(min(cpu_slabs, B * H)))
             got = oracle.bf16_to_f32(dout.download(np.uint16)).reshape(B * H, N * D)
-            qs = np.stack([oracle.bf16_to_f32(qb.reshape(B * H, -1)[s]) for s in slabs])
-            ks = np.stack([oracle.bf16_to_f32(kb.reshape(B * H, -1)[s]) for s in slabs])
-            vs = np.stack([oracle.bf16_to_f32(vb.reshape(B * H, -1)[s]) for s in slabs])
+            qs, ks, vs = (np.stack([oracle.bf16_to_f32(x.reshape(B * H, -1)[s]) for s in slabs]) for x in (qb, kb, vb))
             t0 = time.perf_counter()
             want = oracle.flash_forward_masked(oracle.AttentionShape(1, len(slabs), N, D), qs, ks, vs, "causal",
                                                threads=threads).reshape(len(slabs), N * D)
             cpu_s = time.perf_counter() - t0
             err = float(np.abs(got[slabs] - want).max())
-            prefill["parity_max_abs"] = err
-            prefill["cpu"] = {"value": flops_causal * len(slabs) / (B * H) / cpu_s / 1e12, "unit": "TFLOP/s",
-                              "cores": threads, "kind": "port",
-                              "sample": f"all {len(slabs)} (b,h) slabs of the workload once, one task per slab as "
-                                        f"rayon does, {cpu_s:.1f} s wall on {threads} threads; f32 on the bf16-rounded "
-                                        f"inputs; causal-counted FLOPs although every tile is computed, as in the "
-                                        f"reference"}
-            if err > 2e-2:
-                print(f"PARITY FAILURE: prefill max-abs {err}", file=sys.stderr)
+            leg["parity_max_abs"] = err
+            which = "all" if len(slabs) == B * H else "the first"
+            leg["cpu_baseline"] = {"value": flops_causal * len(slabs) / (B * H) / cpu_s / 1e12, "unit": "TFLOP/s",
+                                   "cores": min(threads, len(slabs)), "kind": "port",
+                                   "sample": f"{which} {len(slabs)} of the {B * H} (b,h) slabs once, one task per slab "
+                                             f"as rayon does, {cpu_s:.1f} s wall on {min(threads, len(slabs))} threads; "
+                                             f"f32 on the bf16-rounded inputs; causal-counted FLOPs although every tile "
+                                             f"is computed, as in the reference; the same slabs are the parity sample"}
+            if not err <= 2e-2:
+                print(f"PARITY FAILURE: prefill B={B} H={H} N={N} D={D} max-abs {err}", file=sys.stderr)
                 sys.exit(1)
-        del dq, dk, dv, dout
+        return leg
+
+    # ------------------------------------------------------------------ prefill (the step)
+    B, H, N, D = 4, 32, 4096, 128
+    prefill = None
+    if args.only in (None, "prefill"):
+        prefill = causal_prefill(B, H, N, D, 1234, 1.0, B * H, "flash_fwd_bf16_kernel<128, causal>",
+                                 profile_traffic("flash_fwd_bf16_b4_h32_n4096_d128.md", "flash_fwd_bf16_kernel<128,causal>"))
+
+    # ------------------------------------------------------------------ long-context prefill (Q scaled by 2)
+    long_p = None
+    if args.only in (None, "long"):
+        Bl, Hl, Nl, Dl = 1, 32, 16384, 128
+        # the CPU port needs ~5 s per slab per thread at this length: half of the 32 slabs, one per thread
+        long_p = causal_prefill(Bl, Hl, Nl, Dl, 55, 2.0, 16, "flash_fwd_bf16_kernel<128, causal>",
+                                profile_traffic("flash_fwd_bf16_b1_h32_n16384_d128.md", "flash_fwd_bf16_kernel<128,causal>"))
+        long_p = {"metric": "prefill attn TFLOP/s", "value": long_p.pop("tflops"), "unit": "TFLOP/s", **long_p,
+                  "config": {"workload": "bf16 long-context causal prefill, B=1 H=32 N=16384 D=128, N(0,1) inputs with Q "
+                                         "scaled by 2.0 before rounding (seed 55), f32 accumulation",
+                             "flop_convention": "4*B*H*D*N*(N+1)/2 (causal-counted)"}}
+
+    # ------------------------------------------------------------------ padded-batch prefill (per-sequence lengths + causal)
+    padded = None
+    if args.only in (None, "padded"):
+        Bp, Hp, Np, Dp = 16, 16, 1024, 64
+        rng_v = np.random.default_rng(33)
+        lens_p = rng_v.integers(128, 1025, size=Bp).astype(np.int32)
+        n_el = Bp * Hp * Np * Dp
+        qb, kb, vb = (oracle.f32_to_bf16(rng_v.standard_normal(n_el, dtype=np.float32)) for _ in range(3))
+        dq, dk, dv = (ra.HipStorage.from_numpy(x) for x in (qb, kb, vb))
+        dout = ra.HipStorage(n_el * 2)
+        dlens = ra.HipStorage.from_numpy(lens_p)
+        shape_p = ra.AttentionShape.new(Bp, Hp, Np, Dp)
+        tm = time_steps(hip, stream, lambda i: ra.flash_forward_varlen_bf16_dev(shape_p, dq, dk, dv, dlens, dout, True,
+                                                                                stream=stream),
+                        args.steps, args.warmup)
+        ll = lens_p.astype(np.float64)
+        flops_p = float(4.0 * Hp * Dp * (ll * (ll + 1) / 2.0).sum())  # valid (query, key) pairs only
+        achieved = flops_p / (tm.mean_ms * 1e-3) / 1e12
+        padded = {"metric": "prefill attn TFLOP/s", "value": flops_p / (tm.wall_ms / args.steps * 1e-3) / 1e12,
+                  "unit": "TFLOP/s", "ms_per_step": tm.wall_ms / args.steps, "kernel_ms_mean": tm.mean_ms,
+                  **spread(tm.per), **tm.settle(),
+                  "config": {"workload": "bf16 padded-batch prefill, B=16 H=16 D=64, max N=1024, valid lengths U[128,1024] "
+                                         "(seed 33), key padding + causal, padded query rows written as zeros",
+                             "seq_lens": [int(x) for x in lens_p],
+                             "flop_convention": "4*H*D*sum_b len_b*(len_b+1)/2 (valid pairs only)"},
+                  "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                               "frac": achieved / PEAK_BF16_TFLOPS,
+                               "traffic": profile_traffic("flash_fwd_bf16_varlen_b16_h16_n1024_d64.md",
+                                                          "flash_fwd_bf16_kernel<64,varlen>"),
+                               "kernel": "flash_fwd_bf16_kernel<64, varlen>", "kernel_ms_mean": tm.mean_ms}}
+        if not args.no_cpu:
+            # the oracle of a sequence is the reference's causal forward on the problem truncated to its length
+            got = oracle.bf16_to_f32(dout.download(np.uint16)).reshape(Bp, Hp, Np, Dp)
+            q4, k4, v4 = (oracle.bf16_to_f32(x).reshape(Bp, Hp, Np, Dp) for x in (qb, kb, vb))
+            err, cpu_s = 0.0, 0.0
+            zeros_ok = True
+            for b in range(Bp):
+                L = int(lens_p[b])
+                qs, ks, vs = (np.ascontiguousarray(x[b, :, :L, :]).ravel() for x in (q4, k4, v4))
+                t0 = time.perf_counter()
+                want = oracle.flash_forward_masked(oracle.AttentionShape(1, Hp, L, Dp), qs, ks, vs, "causal",
+                                                   threads=threads).reshape(Hp, L, Dp)
+                cpu_s += time.perf_counter() - t0
+                err = max(err, float(np.abs(got[b, :, :L, :] - want).max()))
+                pad = got[b, :, L:, :]
+                zeros_ok &= bool((pad.view(np.uint32) == 0).all())  # exact +0.0
+            padded["parity_max_abs"] = err
+            padded["padded_rows_exact_zero"] = zeros_ok
+            padded["cpu_baseline"] = {"value": flops_p / cpu_s / 1e12, "unit": "TFLOP/s", "cores": min(threads, Hp),
+                                      "kind": "port",
+                                      "sample": f"the whole workload once ({cpu_s:.2f} s): per sequence the reference's "
+                                                f"causal forward on the problem truncated to its length, one task per "
+                                                f"head; every tile computed, valid-pair FLOPs counted"}
+            if not (err <= 2e-2 and zeros_ok):
+                print(f"PARITY FAILURE: padded prefill max-abs {err}, zero rows {zeros_ok}", file=sys.stderr)
+                sys.exit(1)
+        del dq, dk, dv, dout, dlens
 
     # ------------------------------------------------------------------ decode
     decode = None
@@ -260,14 +391,14 @@ def main():
         ms_kernel = tm.mean_ms
         decode = {"metric": "decode attn HBM GB/s", "value": alg_bytes / (tm.wall_ms / args.steps * 1e-3) / 1e9,
                   "unit": "GB/s", "ms_per_step": tm.wall_ms / args.steps, "kernel_ms_mean": ms_kernel,
-                  **spread(tm.per),
+                  **spread(tm.per), **tm.settle(),
                   "algorithmic_bytes": alg_bytes,
                   "config": {"workload": "bf16 GQA decode, batch 64, 32 q / 8 kv heads, D=128, ctx U[512,8192] "
                                          "(seed 4), cache (B,Hkv,Lmax=8192,D)", "sum_len": int(lens.sum()),
                              "cache_sets_rotated": n_sets},
                   "roofline": {"bound": "hbm", "achieved": alg_bytes / (ms_kernel * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                                "unit": "GB/s", "frac": alg_bytes / (ms_kernel * 1e-3) / 1e9 / PEAK_HBM_GBS,
-                               "traffic": TRAFFIC_DECODE_BYTES,
+                               "traffic": profile_traffic("decode_split_b64_hq32_hkv8_d128_ctx512-8192.md", "decode_step"),
                                "kernels": "decode_split + decode_merge (one event pair around the timed steps)"}}
         # the reference's own call: one sequence per launch (LlmKernels::gqa_decode_online_bf16), back to back on the
         # stream as a decode loop issues it, on sequence 0's cache
@@ -283,7 +414,6 @@ def main():
         decode["single_sequence"] = dict(single, note="rt_gqa_decode_online_bf16, 32 q / 8 kv heads, D=128: two launches "
                                                       "per call, issued back to back from the host")
         if not args.no_cpu:
-            threads = min(oracle.max_threads(), 16)
             got = oracle.bf16_to_f32(d_o.download(np.uint16))
             t0 = time.perf_counter()
             want = oracle.gqa_decode_batched_bf16(qd, kc, vc, lens, Bd, Hq, Hkv, Dd, Lmax, threads=threads)
@@ -314,13 +444,13 @@ def main():
         flops_f = 4.0 * Bf * Hf * Df * (Nf * (Nf + 1) / 2.0)
         f32 = {"metric": "f32 prefill attn TFLOP/s", "value": flops_f / (tm.wall_ms / args.steps * 1e-3) / 1e12,
                "unit": "TFLOP/s", "ms_per_step": tm.wall_ms / args.steps, "kernel_ms_mean": tm.mean_ms, **spread(tm.per),
+               **tm.settle(),
                "config": {"workload": "f32 causal flash-attention forward, B=1 H=8 N=2048 D=64, N(0,1) inputs (seed 77), "
                                       "tensors resident in HBM", "flop_convention": "4*B*H*D*N*(N+1)/2 (causal-counted)"},
                "roofline": {"bound": "mfma", "achieved": flops_f / (tm.mean_ms * 1e-3) / 1e12, "peak": PEAK_F32_TFLOPS,
                             "unit": "TFLOP/s", "frac": flops_f / (tm.mean_ms * 1e-3) / 1e12 / PEAK_F32_TFLOPS,
-                            "traffic": TRAFFIC_F32_BYTES, "kernel": "flash_fwd_f32_splitk_kernel<2, exact, causal>"}}
+                            "traffic": profile_traffic("flash_fwd_f32_b1_h8_n2048_d64.md", "flash_fwd_f32_splitk_kernel<2,exact,causal>"), "kernel": "flash_fwd_f32_splitk_kernel<2, exact, causal>"}}
         if not args.no_cpu:
-            threads = min(oracle.max_threads(), 16)
             got = dof.download(np.float32)
             oracle.flash_forward_masked(oracle.AttentionShape(Bf, Hf, Nf, Df), qf, kf, vf, "causal", threads=threads)  # warm
             reps = 5
@@ -365,6 +495,7 @@ def main():
                               args.steps, args.warmup, spread_steps=0)
         bwd = {"metric": "f32 attention backward TFLOP/s", "value": flops_b / (tm.wall_ms / args.steps * 1e-3) / 1e12,
                "unit": "TFLOP/s", "ms_per_step": tm.wall_ms / args.steps, "kernel_ms_mean": tm.mean_ms, **spread(tm.per),
+               **tm.settle(),
                "saved_forward": {"kernel_ms_mean": tm_saved.mean_ms, "tflops": flops_b / (tm_saved.mean_ms * 1e-3) / 1e12,
                                  "note": "rt_flash_backward_saved_f32_dev: O and the row statistic come from the forward "
                                          "pass instead of being recomputed (delta + dK/dV + dQ)"},
@@ -375,7 +506,7 @@ def main():
                                              "in the two backward kernels), none of which is counted"},
                "roofline": {"bound": "mfma", "achieved": flops_b / (tm.mean_ms * 1e-3) / 1e12, "peak": PEAK_F32_TFLOPS,
                             "unit": "TFLOP/s", "frac": flops_b / (tm.mean_ms * 1e-3) / 1e12 / PEAK_F32_TFLOPS,
-                            "traffic": TRAFFIC_BWD_BYTES,
+                            "traffic": profile_traffic("flash_bwd_f32_b1_h8_n2048_d64.md", "backward_step"),
                             "kernels": "flash_fwd_f32_splitk_kernel<2> + flash_bwd_delta_kernel + flash_bwd_f32_dkdv_kernel<2> "
                                        "+ flash_bwd_f32_dq_kernel<2> (one event pair around the timed steps)"}}
         if not args.no_cpu:
@@ -397,45 +528,38 @@ def main():
                 sys.exit(1)
         del d_in, d_g, d_ws
 
-    if prefill is None and decode is None and f32 is None:  # --only bwd
-        print(json.dumps(dict(bwd, n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True,
-                              dtype="f32", data="synthetic", vs_baseline=None)))
+    tail = dict(n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True, data="synthetic",
+                vs_baseline=None, scaling="weak")
+    if prefill is None:  # --only <one of the other legs>: that leg is the line
+        leg, dtype = next((x, t) for x, t in ((decode, "bf16"), (long_p, "bf16"), (padded, "bf16"), (f32, "f32"),
+                                              (bwd, "f32")) if x is not None)
+        print(json.dumps(dict(leg, dtype=dtype, **tail)))
         return
-    if prefill is None and decode is None:  # --only f32
-        print(json.dumps(dict(f32, n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True,
-                              dtype="f32", data="synthetic", vs_baseline=None)))
-        return
-    if prefill is None:  # --only decode: report the decode line as the main one
-        print(json.dumps(dict(decode, n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True,
-                              dtype="bf16", data="synthetic", vs_baseline=None)))
-        return
-    achieved = prefill["tflops_kernel"]
     sustained = None if args.no_ceiling else sustained_mfma()
     out = {
         "metric": "prefill attn TFLOP/s (% bf16 MFMA peak); decode attn HBM GB/s (% peak)",
         "value": prefill["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": prefill["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
+        "settle_ms": prefill["settle_ms"], "settle_launches": prefill["settle_launches"],
         "config": {"workload": "bf16 causal prefill attention, B=4 H=32 N=4096 D=128, N(0,1) inputs (seed 1234), "
                                "f32 accumulation", "flop_convention": "4*B*H*D*N*(N+1)/2 (causal-counted)",
-                   "tflops_unmasked_convention_4BHN2D": prefill["tflops_unmasked_convention"]},
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_PREFILL_BYTES, "kernel": "flash_fwd_bf16_kernel<128>",
-                     "kernel_ms_mean": prefill["kernel_ms_mean"],
-                     **{k: prefill[k] for k in ("kernel_ms_median", "kernel_ms_p99", "kernel_ms_min") if k in prefill}},
+                   "tflops_unmasked_convention_4BHN2D": prefill["tflops_unmasked_convention"],
+                   "settle": f"every leg first launches its own step until {SETTLE_MS:.0f} ms of device time have "
+                             f"passed (settle_ms, settle_launches), then runs the counted warm-up and the timed steps"},
+        "roofline": prefill["roofline"],
     }
     if sustained is not None:
         # context for `frac`: under load the power limit, not the 2.4 GHz of the data sheet, sets the clock
-        out["roofline"]["sustained_mfma"] = dict(sustained, frac_of_sustained=achieved / sustained["tflops"])
-    if "cpu" in prefill:
-        out["cpu_baseline"] = prefill["cpu"]
+        out["roofline"]["sustained_mfma"] = dict(sustained,
+                                                 frac_of_sustained=prefill["roofline"]["achieved"] / sustained["tflops"])
+    if "cpu_baseline" in prefill:
+        out["cpu_baseline"] = prefill["cpu_baseline"]
         out["parity_max_abs"] = prefill["parity_max_abs"]
-    if decode is not None:
-        out["decode"] = decode
-    if f32 is not None:
-        out["f32_prefill"] = f32
-    if bwd is not None:
-        out["f32_backward"] = bwd
+    for key, leg in (("decode", decode), ("padded_prefill", padded), ("long_prefill", long_p), ("f32_prefill", f32),
+                     ("f32_backward", bwd)):
+        if leg is not None:
+            out[key] = leg
     print(json.dumps(out))
 
 

@@ -171,7 +171,14 @@ int rt_flash_backward_saved_f32_dev(void *stream, const rt_attention_shape *shap
                                     float *dk, float *dv, void *workspace, size_t workspace_bytes, rt_err_detail *err);
 
 /* flash_forward_masked on device-resident f32 tensors (same semantics; keep is a device
- * pointer to `seq` bytes).  n_kv_heads = 0 means n_kv_heads = heads. */
+ * pointer to `seq` bytes).  n_kv_heads = 0 means n_kv_heads = heads.
+ *
+ * One divergence from the reference, for non-finite V under the causal mask (it holds for every prefill entry of
+ * this library, host-slice or device, f32 or bf16): the reference walks every key tile and multiplies the hidden
+ * probabilities (exact zeros) into V, so a NaN or Inf in V row j makes EVERY query row NaN in that column
+ * (0 * NaN; cpu_forward.rs:268-425 skips no tile).  The kernels skip key tiles that lie wholly past a query tile
+ * and never read those rows: query rows i >= j are NaN as in the reference, rows i <= j - 256 are finite (the value
+ * the reference gives with V row j zeroed), rows in between may be either.  Finite inputs are unaffected. */
 int rt_flash_forward_f32_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const float *q,
                              const float *k, const float *v, int mask_kind, const uint8_t *keep, float *out,
                              rt_err_detail *err);
@@ -271,7 +278,10 @@ int rt_qk_norm_rope_kv_append_bf16(void *stream, void *q, const void *k_in, cons
  * a batch of one (head_dim 64, 128 or 256, at most 16 query heads per kv head; other shapes take a one-workgroup-per-head
  * kernel).  The reference's signature has no workspace: the partials go to a buffer the library keeps per
  * (device, stream), allocated by the first call on a stream (so that call must not be under stream capture; later
- * calls allocate nothing unless max_seq grows). */
+ * calls allocate nothing unless max_seq grows; a grown buffer replaces the old one, which is kept until
+ * rt_stream_destroy / rt_shutdown, so concurrent callers never see freed memory).  q and the caches should be
+ * 16-byte aligned: the split-K kernels move 16 bytes per lane, and tensors that are not aligned take the
+ * one-workgroup-per-head kernel instead (same results, slower). */
 int rt_gqa_decode_online_bf16(void *stream, const void *q, const void *k_cache, const void *v_cache, void *out,
                               int32_t n_heads, int32_t n_kv, int32_t kv_len, int32_t head_dim, int32_t max_seq,
                               rt_err_detail *err);
@@ -279,7 +289,9 @@ int rt_gqa_decode_online_bf16(void *stream, const void *q, const void *k_cache, 
 /* The batched, ragged form of the same call: q/out [batch,n_heads,head_dim], caches
  * [batch,n_kv,max_seq,head_dim], kv_lens device int32[batch] (sequence b reads [..kv_lens[b]]).
  * Split-K over the context with a second-pass (m, l, o) merge; `workspace` (device, at least
- * rt_gqa_decode_workspace_bytes(...) bytes, 256-byte aligned) holds the partial results.  The split-K kernels cover
+ * rt_gqa_decode_workspace_bytes(...) bytes, 16-byte aligned or the call fails with RT_ERR_WORKSPACE_TOO_SMALL)
+ * holds the partial results.  q and the caches should be 16-byte aligned too (tensors that are not take the
+ * one-workgroup-per-head kernel: same results, slower, no workspace).  The split-K kernels cover
  * head_dim 64, 128 and 256 with at most 16 query heads per kv head; other shapes take a one-workgroup-per-head kernel
  * (head_dim <= 512) that needs no workspace (rt_gqa_decode_workspace_bytes returns 0 for them).
  * batch = 1 with kv_lens = [kv_len] is the reference call.  A sequence with kv_lens[b] == 0

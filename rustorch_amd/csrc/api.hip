@@ -173,12 +173,16 @@ int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n
 }
 
 // Scratch the library keeps for entry points whose reference signature has no workspace argument: one buffer per
-// (device, stream), allocated on the first call that needs it, grown when a later call needs more, and kept until
-// the process ends.  Calls on one stream are ordered, so they can share it; calls on different streams get
-// different buffers.  The first call on a stream allocates (hipMalloc): not for use under stream capture.
+// (device, stream), allocated on the first call that needs it and kept until rt_stream_destroy / rt_shutdown.
+// Calls on one stream are ordered, so they can share it; calls on different streams get different buffers.  When a
+// later call needs more, a larger block is allocated and the old one is RETIRED, not freed: another thread may have
+// been handed the old pointer and not yet enqueued its kernels (the lock below covers the bookkeeping only, not
+// the caller's launches), and kernels already enqueued may still use it.  Retired blocks are freed with the
+// stream's entry.  The first call on a stream allocates (hipMalloc): not for use under stream capture.
 struct StreamWs {
     void* ptr = nullptr;
     size_t bytes = 0;
+    std::vector<void*> retired;
 };
 std::mutex g_ws_mutex;
 std::map<std::pair<int, hipStream_t>, StreamWs> g_ws;
@@ -189,19 +193,25 @@ int stream_workspace(hipStream_t stream, size_t bytes, float** out, rt_err_detai
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     StreamWs& w = g_ws[{dev, stream}];
     if (w.bytes < bytes) {
-        if (w.ptr) {
-            // kernels already enqueued on the stream may still use the old buffer
-            HIP_TRY(hipStreamSynchronize(stream), "hipStreamSynchronize");
-            HIP_TRY(hipFree(w.ptr), "hipFree workspace");
-            w.ptr = nullptr;
-            w.bytes = 0;
-        }
-        size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
-        HIP_TRY(hipMalloc(&w.ptr, want), "hipMalloc workspace");
+        // grow geometrically, so that a context that lengthens token by token retires a handful of blocks at most
+        size_t want = std::max<size_t>(std::max<size_t>(bytes, (size_t)1 << 20), 2 * w.bytes);
+        void* fresh = nullptr;
+        HIP_TRY(hipMalloc(&fresh, want), "hipMalloc workspace");
+        if (w.ptr) w.retired.push_back(w.ptr);
+        w.ptr = fresh;
         w.bytes = want;
     }
     *out = (float*)w.ptr;
     return RT_OK;
+}
+
+// frees what a stream's entry holds; the caller holds g_ws_mutex and has made sure the stream is idle
+void release_stream_ws(StreamWs& w) {
+    if (w.ptr) (void)hipFree(w.ptr);
+    for (void* r : w.retired) (void)hipFree(r);
+    w.ptr = nullptr;
+    w.bytes = 0;
+    w.retired.clear();
 }
 
 struct DevPtr {  // a device address inside a Stage's block
@@ -986,7 +996,10 @@ RT_API int rt_gqa_decode_online_bf16(void* stream, const void* q, const void* k_
     if (!q || !out || (kv_len > 0 && (!k_cache || !v_cache))) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
     rc = ensure_device(err);
     if (rc) return rc;
-    if (rt::decode_split_supported(n_heads, n_kv, head_dim)) {
+    // the split-K kernels move q, K and V 16 bytes at a time; tensors that are not 16-byte aligned take the
+    // element-wise kernel below
+    const bool aligned = ((((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0);
+    if (aligned && rt::decode_split_supported(n_heads, n_kv, head_dim)) {
         // the split-K kernels of the batched entry, on a batch of one; their partials go to a buffer the library keeps
         // per stream (the reference's signature has no workspace argument)
         float* ws = nullptr;
@@ -1053,10 +1066,16 @@ RT_API int rt_gqa_decode_batched_bf16(void* stream, const void* q, const void* k
         return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
     rc = ensure_device(err);
     if (rc) return rc;
-    if (rt::decode_split_supported(n_heads, n_kv, head_dim)) {
+    // the split-K kernels move q, K, V and the partials 16 bytes at a time; tensors that are not 16-byte aligned
+    // take the element-wise kernel below, which needs no workspace
+    const bool aligned = ((((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0);
+    if (aligned && rt::decode_split_supported(n_heads, n_kv, head_dim)) {
         size_t need = rt::decode_split_workspace_bytes(batch, n_heads, head_dim, max_seq);
         if (!workspace || workspace_bytes < need)
             return fail(err, RT_ERR_WORKSPACE_TOO_SMALL, -1, need, workspace ? workspace_bytes : 0, "workspace too small");
+        if ((uintptr_t)workspace & 15)
+            return fail(err, RT_ERR_WORKSPACE_TOO_SMALL, -1, 16, (uint64_t)((uintptr_t)workspace & 15),
+                        "workspace must be 16-byte aligned");
         rt::DecodeSplitParams p{};
         p.q = (const uint16_t*)q;
         p.k_cache = (const uint16_t*)k_cache;
@@ -1191,7 +1210,7 @@ RT_API int rt_stream_destroy(void* stream, rt_err_detail* err) {
             auto it = g_ws.find({dev, (hipStream_t)stream});
             if (it != g_ws.end()) {
                 (void)hipStreamSynchronize((hipStream_t)stream);
-                if (it->second.ptr) (void)hipFree(it->second.ptr);
+                release_stream_ws(it->second);
                 g_ws.erase(it);
             }
         }
@@ -1206,11 +1225,10 @@ RT_API int rt_shutdown(rt_err_detail* err) {
     // buffer of the host-slice entries.  The caller makes sure no call is in flight.
     {
         std::lock_guard<std::mutex> lock(g_ws_mutex);
-        for (auto& kv : g_ws)
-            if (kv.second.ptr) {
-                (void)hipStreamSynchronize(kv.first.second);
-                (void)hipFree(kv.second.ptr);
-            }
+        for (auto& kv : g_ws) {
+            if (kv.second.ptr) (void)hipStreamSynchronize(kv.first.second);
+            release_stream_ws(kv.second);
+        }
         g_ws.clear();
     }
     {

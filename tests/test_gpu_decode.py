@@ -176,3 +176,38 @@ def test_shutdown_frees_and_the_library_stays_usable(oracle):
         small = ra.flash_forward(ra.AttentionShape.new(1, 1, 4, 4), *[np.ones(16, np.float32)] * 3)  # pinned staging
         assert np.allclose(small, 1.0)
         ra.shutdown()
+
+
+def test_decode_unaligned_tensors_take_the_elementwise_kernel(oracle):
+    """q and caches that start 2 bytes past a 16-byte boundary: the 16-byte loads of the split-K kernels do not apply,
+    the call routes to the one-workgroup-per-head kernel and gives the same result; a misaligned workspace is an
+    error."""
+    b, hq, hkv, d, max_seq = 2, 8, 2, 128, 300
+    lens = [300, 77]
+    qb, _ = bf16_round(seeded_normal((b, hq, d), 1))
+    kb, _ = bf16_round(seeded_normal((b, hkv, max_seq, d), 2))
+    vb, _ = bf16_round(seeded_normal((b, hkv, max_seq, d), 3))
+    want = oracle.gqa_decode_batched_bf16(qb, kb, vb, lens, b, hq, hkv, d, max_seq)
+
+    def shifted(bits):  # a device buffer whose payload starts at byte 2
+        host = np.concatenate([np.zeros(1, np.uint16), bits.ravel()])
+        store = dev(host)
+        return store, store.ptr + 2
+
+    (sq, pq), (sk, pk), (sv, pv) = shifted(qb), shifted(kb), shifted(vb)
+    dlens = dev(np.asarray(lens, dtype=np.int32))
+    ws = ra.HipStorage(max(K.gqa_decode_workspace_bytes(b, hq, hkv, d, max_seq), 256))
+    dout = ra.HipStorage(b * hq * d * 2)
+    K.gqa_decode_batched_bf16(None, pq, pk, pv, dout, dlens, b, hq, hkv, d, max_seq, ws, ws.byte_len)
+    ra.synchronize()
+    assert max_abs(oracle.bf16_to_f32(dout.download(np.uint16)), want) <= TOL
+    # the single-sequence call on sequence 1's slabs
+    dout1 = ra.HipStorage(hq * d * 2)
+    K.gqa_decode_online_bf16(None, pq + hq * d * 2, pk + hkv * max_seq * d * 2, pv + hkv * max_seq * d * 2, dout1, hq, hkv,
+                             lens[1], d, max_seq)
+    ra.synchronize()
+    assert max_abs(oracle.bf16_to_f32(dout1.download(np.uint16)), want.reshape(b, hq * d)[1]) <= TOL
+    with pytest.raises(ra.DeviceError) as ei:
+        K.gqa_decode_batched_bf16(None, dev(qb), dev(kb), dev(vb), dout, dlens, b, hq, hkv, d, max_seq, ws.ptr + 4,
+                                  ws.byte_len - 4)
+    assert ei.value.status == 22

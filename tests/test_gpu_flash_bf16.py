@@ -176,3 +176,33 @@ def test_unsupported_dim_is_an_error():
     with pytest.raises(ra.DeviceError) as ei:
         ra.flash_forward_bf16_dev(shape, z, z, z, z)
     assert ei.value.status == 21
+
+
+@pytest.mark.parametrize("bad", [np.nan, np.inf])
+def test_non_finite_v_row_at_a_causally_hidden_position(oracle, bad):
+    """A non-finite V row j under the causal mask.  The reference walks every key tile and multiplies the hidden
+    probabilities (exact zeros) into V, so 0 * NaN poisons EVERY query row (cpu_forward.rs:268-425: no tile is
+    skipped).  The kernels skip key tiles that lie wholly past a query tile and never read those V rows: rows that
+    see key j (i >= j) are NaN as in the reference; rows at least 256 positions before j are finite and equal the
+    result with that V row replaced by zeros; rows in between are NaN or that finite value."""
+    b, h, n, d, j = 1, 2, 1024, 128, 700
+    (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d), (51, 52, 53))
+    vbad = vf.copy().reshape(b, h, n, d)
+    vbad[:, :, j, 5] = bad
+    vbad = vbad.ravel()
+    vzero = vf.copy().reshape(b, h, n, d)
+    vzero[:, :, j, :] = 0.0
+    vzero = vzero.ravel()
+    shape, osh = ra.AttentionShape.new(b, h, n, d), oracle.AttentionShape(b, h, n, d)
+    want_ref = oracle.flash_forward_masked(osh, qf, kf, vbad, "causal").reshape(b, h, n, d)
+    assert np.isnan(want_ref[..., 5]).all()  # the reference: every row, hidden or not
+    got = flash_bf16(shape, qb, kb, oracle.f32_to_bf16(vbad), ra.Mask.causal()).reshape(b, h, n, d)
+    clean = oracle.flash_forward_masked(osh, qf, kf, vzero, "causal").reshape(b, h, n, d)
+    assert np.isnan(got[:, :, j:, 5]).all()
+    early = got[:, :, :j - 255]
+    assert np.isfinite(early).all() and max_abs(early, clean[:, :, :j - 255]) <= TOL
+    mid = got[:, :, j - 255:j]
+    ok = np.isnan(mid) | (np.abs(mid - clean[:, :, j - 255:j]) <= TOL)
+    assert ok.all()
+    # the other columns of the poisoned rows stay finite in both (only column 5 of V is bad)
+    assert np.isfinite(got[..., :5]).all() and np.isfinite(want_ref[..., :5]).all()

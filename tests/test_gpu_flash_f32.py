@@ -293,3 +293,27 @@ def test_host_slice_calls_from_several_threads(oracle):
     for th in threads:
         th.join()
     assert not errors, errors[:3]
+
+
+@pytest.mark.parametrize("bad", [np.nan, -np.inf])
+def test_non_finite_v_row_at_a_causally_hidden_position(oracle, bad):
+    """A non-finite V row j under the causal mask.  The reference multiplies the hidden probabilities (exact zeros)
+    into V on every key tile, so 0 * NaN poisons every query row; the kernels skip key tiles that lie wholly past a
+    query tile.  Rows that see key j are NaN as in the reference; rows at least 256 positions before j are finite
+    and equal the result with that V row zeroed; rows in between are NaN or that finite value."""
+    b, h, n, d, j = 1, 2, 600, 64, 400
+    q, k, v = (seeded_normal(b * h * n * d, s) for s in (61, 62, 63))
+    vbad = v.copy().reshape(b, h, n, d)
+    vbad[:, :, j, 3] = bad
+    vzero = v.copy().reshape(b, h, n, d)
+    vzero[:, :, j, :] = 0.0
+    shape, osh = ra.AttentionShape.new(b, h, n, d), oracle.AttentionShape(b, h, n, d)
+    want_ref = oracle.flash_forward_masked(osh, q, k, vbad.ravel(), "causal").reshape(b, h, n, d)
+    assert np.isnan(want_ref[..., 3]).all()
+    got = ra.flash_forward_masked(shape, q, k, vbad.ravel(), ra.Mask.causal()).reshape(b, h, n, d)
+    clean = oracle.flash_forward_masked(osh, q, k, vzero.ravel(), "causal").reshape(b, h, n, d)
+    assert np.isnan(got[:, :, j:, 3]).all()
+    early = got[:, :, :j - 255]
+    assert np.isfinite(early).all() and max_abs(early, clean[:, :, :j - 255]) <= TOL
+    mid = got[:, :, j - 255:j]
+    assert (np.isnan(mid) | (np.abs(mid - clean[:, :, j - 255:j]) <= TOL)).all()

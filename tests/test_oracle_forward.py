@@ -308,3 +308,17 @@ def test_varlen_causal_matches_f64_on_valid_rows(oracle):
         assert np.abs(out[b, :, :n] - ref).max() < 5e-6
         assert (out[b, :, n:] == 0.0).all()
         assert np.isnan(nan_out[b, :, n:]).all()
+
+
+def test_non_finite_v_row_poisons_every_row_even_where_hidden(oracle):
+    """cpu_forward.rs:268-425 multiplies P (exact zeros where masked) into every V tile: 0 * NaN = NaN reaches every
+    query row in that column, hidden or not, in the tiled form; the scalar and naive forms agree."""
+    b, h, n, d, j = 1, 1, 130, 8, 100
+    q, k, v = (lcg_buffer(b * h * n * d, s, 2.0) for s in (5, 6, 7))
+    v = v.copy()
+    v[j * d + 2] = np.nan
+    sh = oracle.AttentionShape(b, h, n, d)
+    out = oracle.flash_forward_masked(sh, q, k, v, "causal").reshape(n, d)
+    assert np.isnan(out[:, 2]).all() and np.isfinite(np.delete(out, 2, axis=1)).all()
+    naive = oracle.naive_forward_masked(sh, q, k, v, "causal").reshape(n, d)
+    assert np.array_equal(np.isnan(naive), np.isnan(out))
