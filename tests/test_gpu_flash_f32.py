@@ -309,11 +309,12 @@ def test_non_finite_v_row_at_a_causally_hidden_position(oracle, bad):
     vzero[:, :, j, :] = 0.0
     shape, osh = ra.AttentionShape.new(b, h, n, d), oracle.AttentionShape(b, h, n, d)
     want_ref = oracle.flash_forward_masked(osh, q, k, vbad.ravel(), "causal").reshape(b, h, n, d)
-    assert np.isnan(want_ref[..., 3]).all()
+    assert (~np.isfinite(want_ref[..., 3])).all()
     got = ra.flash_forward_masked(shape, q, k, vbad.ravel(), ra.Mask.causal()).reshape(b, h, n, d)
     clean = oracle.flash_forward_masked(osh, q, k, vzero.ravel(), "causal").reshape(b, h, n, d)
-    assert np.isnan(got[:, :, j:, 3]).all()
+    assert (~np.isfinite(got[:, :, j:, 3])).all()  # NaN, or +-Inf where the row's weight on key j is positive
     early = got[:, :, :j - 255]
     assert np.isfinite(early).all() and max_abs(early, clean[:, :, :j - 255]) <= TOL
     mid = got[:, :, j - 255:j]
-    assert (np.isnan(mid) | (np.abs(mid - clean[:, :, j - 255:j]) <= TOL)).all()
+    with np.errstate(invalid="ignore"):
+        assert (~np.isfinite(mid) | (np.abs(mid - clean[:, :, j - 255:j]) <= TOL)).all()
