@@ -301,6 +301,23 @@ int rt_gqa_decode_batched_bf16(void *stream, const void *q, const void *k_cache,
                                const int32_t *kv_lens, int32_t batch, int32_t n_heads, int32_t n_kv,
                                int32_t head_dim, int32_t max_seq, void *workspace, size_t workspace_bytes,
                                rt_err_detail *err);
+
+/* No counterpart in the reference.  rt_gqa_decode_batched_bf16 for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): same arguments without
+ * the workspace, same kernels, same results bit for bit.  The split-K partials go to a fixed 8 MiB block of device
+ * memory inside the library (one per GPU, there from the moment the library's code is loaded on that GPU until the
+ * process ends); the call allocates and frees nothing.  rt_init(device) looks the block's address up; without it
+ * the first call on a device does.
+ *   - Limit: (4 * CUs + batch * n_kv) * (n_heads / n_kv) * (head_dim + 2) * 4 bytes must fit in 8 MiB (the headline
+ *     decode workload, batch 64, 32 / 8 heads, head_dim 128, needs 3.2 MB); beyond it RT_ERR_WORKSPACE_TOO_SMALL
+ *     (expected = bytes needed, got = 8 MiB).  Only the split-K shapes (head_dim 64 / 128 / 256, at most 16 query
+ *     heads per kv head, 16-byte aligned q and caches); others RT_ERR_UNSUPPORTED.
+ *   - Every call on a GPU uses that GPU's one block: calls that overlap on one GPU (two streams, two threads) race
+ *     and give wrong results.  Calls on one stream are ordered and safe.  Nothing needs clearing between calls:
+ *     every partial a call reads was written by the same call. */
+int rt_gqa_decode_batched_bf16_noalloc(void *stream, const void *q, const void *k_cache, const void *v_cache, void *out,
+                                       const int32_t *kv_lens, int32_t batch, int32_t n_heads, int32_t n_kv,
+                                       int32_t head_dim, int32_t max_seq, rt_err_detail *err);
 size_t rt_gqa_decode_workspace_bytes(int32_t batch, int32_t n_heads, int32_t n_kv, int32_t head_dim,
                                      int32_t max_seq);
 

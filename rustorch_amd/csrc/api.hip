@@ -341,7 +341,14 @@ RT_API const char* rt_status_name(int status) {
 
 RT_API int rt_init(int device, rt_err_detail* err) {
     clear_err(err);
-    return ensure_device(err, device < 0 ? 0 : device);
+    int rc = ensure_device(err, device < 0 ? 0 : device);
+    if (rc) return rc;
+    // the address of the library's fixed scratch block on this device, looked up here so that the first call of
+    // rt_gqa_decode_batched_bf16_noalloc has nothing left to set up
+    float* scratch = nullptr;
+    size_t scratch_bytes = 0;
+    HIP_TRY(rt::decode_static_scratch(&scratch, &scratch_bytes), "hipGetSymbolAddress(static scratch)");
+    return RT_OK;
 }
 
 // ---- prefill, host slices -------------------------------------------------------------------------
@@ -1113,6 +1120,53 @@ RT_API int rt_gqa_decode_batched_bf16(void* stream, const void* q, const void* k
     p.head_map = 1;
     p.scale = 1.0f / sqrtf((float)head_dim);
     HIP_TRY(rt::launch_attn_rows_bf16((hipStream_t)stream, p), "attn_rows_bf16 launch");
+    return RT_OK;
+}
+
+// The batched decode for callers that cannot allocate (under HIP graph capture, in serving loops or harnesses that
+// forbid hipMalloc): the partials go to the library's fixed scratch block in device memory instead of a workspace
+// argument.  Calls nothing that allocates or frees.
+RT_API int rt_gqa_decode_batched_bf16_noalloc(void* stream, const void* q, const void* k_cache, const void* v_cache,
+                                              void* out, const int32_t* kv_lens, int32_t batch, int32_t n_heads,
+                                              int32_t n_kv, int32_t head_dim, int32_t max_seq, rt_err_detail* err) {
+    clear_err(err);
+    int rc = check_decode_dims(batch, n_heads, n_kv, head_dim, max_seq, err);
+    if (rc) return rc;
+    if (batch == 0 || n_heads == 0) return RT_OK;
+    if (!q || !out || !kv_lens || (max_seq > 0 && (!k_cache || !v_cache)))
+        return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    rc = ensure_device(err);
+    if (rc) return rc;
+    if (!rt::decode_split_supported(n_heads, n_kv, head_dim))
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, (uint64_t)head_dim,
+                    "the no-allocation decode covers head_dim 64, 128, 256 with at most 16 query heads per kv head");
+    if ((((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) != 0)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 16, 0, "the no-allocation decode needs 16-byte aligned q and caches");
+    float* scratch = nullptr;
+    size_t scratch_bytes = 0;
+    HIP_TRY(rt::decode_static_scratch(&scratch, &scratch_bytes), "hipGetSymbolAddress(static scratch)");
+    const size_t need = rt::decode_split_compact_bytes(batch, n_heads, n_kv, head_dim, g_decode_waves);
+    if (need > scratch_bytes)
+        return fail(err, RT_ERR_WORKSPACE_TOO_SMALL, -1, (uint64_t)need, (uint64_t)scratch_bytes,
+                    "batch too large for the library's fixed scratch block; use rt_gqa_decode_batched_bf16 with a workspace");
+    rt::DecodeSplitParams p{};
+    p.q = (const uint16_t*)q;
+    p.k_cache = (const uint16_t*)k_cache;
+    p.v_cache = (const uint16_t*)v_cache;
+    p.out = (uint16_t*)out;
+    p.kv_lens = kv_lens;
+    p.ws = scratch;
+    p.batch = batch;
+    p.heads = n_heads;
+    p.kv_heads = n_kv;
+    p.dim = head_dim;
+    p.max_seq = max_seq;
+    p.n_part = rt::decode_split_parts(batch, max_seq);
+    p.span_min = rt::decode_split_span_min(batch);
+    p.n_waves = g_decode_waves;
+    p.scale_log2e = (1.0f / sqrtf((float)head_dim)) * rt::kLog2eHost;
+    p.compact = 1;
+    HIP_TRY(rt::launch_decode_split((hipStream_t)stream, p), "decode_split launch");
     return RT_OK;
 }
 

@@ -12,6 +12,7 @@
 //   kv_append_kernel      llm_kernels.rs:353-372.
 //   kv_block_append_kernel  KVLayerCache::append, crates/rustorch-nn/src/kv_cache.rs:77-112 (seq_added rows per head).
 #include <algorithm>
+#include <mutex>
 
 #include "rt_common.hpp"
 #include "rt_kernels.hpp"
@@ -170,6 +171,12 @@ constexpr int kDecSpanMinOne = 2;  // the same for a single sequence, where the 
 __device__ __forceinline__ int dec_steps(int len) { return (len + kDecRows - 1) / kDecRows; }
 __device__ __forceinline__ int dec_len(const DecodeSplitParams& p, int b) {
     return min(max(p.kv_lens ? p.kv_lens[b] : p.kv_len, 0), p.max_seq);
+}
+
+// slots of `ws` (the (m, l) pairs follow the slots' o vectors)
+__device__ __forceinline__ size_t dec_slots(const DecodeSplitParams& p) {
+    return p.compact ? ((size_t)p.n_waves + (size_t)p.batch * p.kv_heads) * (size_t)(p.heads / p.kv_heads)
+                     : (size_t)p.batch * p.heads * p.n_part;
 }
 
 __device__ __forceinline__ int wave_sum_i(int x) {
@@ -405,8 +412,9 @@ __global__ __launch_bounds__(64) void decode_split_kernel(DecodeSplitParams p) {
             const int part = w - seg_first / span;
             if (hcol < G) {
                 float* ws_o = p.ws;
-                float* ws_ml = p.ws + (size_t)p.batch * p.heads * p.n_part * HD;
-                const size_t slot = ((size_t)cur.b * p.heads + (size_t)cur.kvh * G + hcol) * p.n_part + part;
+                float* ws_ml = p.ws + dec_slots(p) * HD;
+                const size_t slot = p.compact ? ((size_t)w + (size_t)cur.b * Hkv + cur.kvh) * G + hcol
+                                              : ((size_t)cur.b * p.heads + (size_t)cur.kvh * G + hcol) * p.n_part + part;
                 // acc_o[dt][i] = O^T[d = 16dt + 4g + i][h]
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++) *(f32x4_t*)(ws_o + slot * HD + 16 * dt + 4 * g4) = acc_o[dt];
@@ -444,8 +452,11 @@ __global__ __launch_bounds__((HD < 64 ? 64 : HD) * NS) void decode_merge_kernel(
     const int w_first = seg_first / span;
     const int n_valid = steps_b > 0 ? (seg_first + steps_b - 1) / span - w_first + 1 : 0;
     const float* ws_o = p.ws;
-    const float* ws_ml = p.ws + (size_t)p.batch * p.heads * p.n_part * HD;
-    const size_t slot0 = ((size_t)b * p.heads + h) * p.n_part;
+    const float* ws_ml = p.ws + dec_slots(p) * HD;
+    // partial k of the head sits at slot0 + k * slot_step
+    const size_t slot0 = p.compact ? ((size_t)w_first + (size_t)b * p.kv_heads + kvh) * G + (h - kvh * G)
+                                   : ((size_t)b * p.heads + h) * p.n_part;
+    const size_t slot_step = p.compact ? (size_t)G : 1;
     const int dd = d < HD ? d : HD - 1;
     // One pass over the partials, eight at a time: the loads of a group are independent of each other (one dependent
     // load after the other would cost more than the split kernel), and the running (m, acc, l) is rescaled once
@@ -457,9 +468,10 @@ __global__ __launch_bounds__((HD < 64 ? 64 : HD) * NS) void decode_merge_kernel(
 #pragma unroll
         for (int j = 0; j < kGroup; j++) {
             const int k = min(k0 + j, n_valid - 1);  // repeats of the last partial are given weight 0 below
-            mv[j] = ws_ml[(slot0 + k) * 2];
-            lv[j] = ws_ml[(slot0 + k) * 2 + 1];
-            ov[j] = ws_o[(slot0 + k) * HD + dd];
+            const size_t slot = slot0 + (size_t)k * slot_step;
+            mv[j] = ws_ml[slot * 2];
+            lv[j] = ws_ml[slot * 2 + 1];
+            ov[j] = ws_o[slot * HD + dd];
         }
         float m_new = m_all;
 #pragma unroll
@@ -564,6 +576,41 @@ int decode_split_parts(int batch, int max_seq) {
 
 size_t decode_split_workspace_bytes(int batch, int heads, int dim, int max_seq) {
     return (size_t)batch * heads * decode_split_parts(batch, max_seq) * ((size_t)dim + 2) * sizeof(float);
+}
+
+size_t decode_split_compact_bytes(int batch, int heads, int kv_heads, int dim, int n_waves) {
+    return ((size_t)n_waves + (size_t)batch * kv_heads) * (size_t)(heads / kv_heads) * ((size_t)dim + 2) * sizeof(float);
+}
+
+// ---- the library's own scratch, for callers that cannot allocate ----------------------------------------------
+// A fixed block of device memory that exists from the moment the code object is loaded on a GPU until the process
+// ends; every GPU holds its own copy at its own address.  The name `static_scratch` is only a handle for
+// hipGetSymbolAddress on the host side: kernels are given the address that call returns, never the name.
+constexpr size_t kStaticScratchBytes = (size_t)8 << 20;
+static __device__ __align__(256) unsigned char static_scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+}  // namespace
+
+hipError_t decode_static_scratch(float** ptr, size_t* bytes) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* addr = nullptr;
+        e = hipGetSymbolAddress(&addr, HIP_SYMBOL(static_scratch));
+        if (e != hipSuccess) return e;
+        if (!addr) return hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = addr;
+    }
+    *ptr = (float*)g_scratch_ptr[dev];
+    *bytes = kStaticScratchBytes;
+    return hipSuccess;
 }
 
 hipError_t launch_decode_split(hipStream_t stream, const DecodeSplitParams& p) {

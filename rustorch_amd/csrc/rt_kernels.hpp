@@ -126,11 +126,22 @@ struct DecodeSplitParams {
     int span_min;  // a wave takes at least this many 32-key steps: decode_split_span_min(batch)
     int n_waves;  // one-wave workgroups launched (all resident at once)
     float scale_log2e;
+    // Where a partial sits in `ws`.  0: slot (sequence, head, k-th wave on the segment), n_part slots per head --
+    // sized for the worst case of every segment at max_seq.  1: slot (wave index + segment index, head of the
+    // group): along the flat step list every partial advances the wave, the segment or both, so the sum numbers
+    // them without collisions, and (n_waves + batch * kv_heads) * group slots hold any batch whatever its lengths.
+    int compact;
 };
 bool decode_split_supported(int heads, int kv_heads, int dim);
 int decode_split_span_min(int batch);
 int decode_split_parts(int batch, int max_seq);
 size_t decode_split_workspace_bytes(int batch, int heads, int dim, int max_seq);
+// bytes of `ws` in the compact layout
+size_t decode_split_compact_bytes(int batch, int heads, int kv_heads, int dim, int n_waves);
+// The library's own scratch block for callers that cannot allocate: a fixed array in device memory (one per GPU,
+// held until the process ends).  Looks its address up once per device (the device must be current) and returns it
+// with its size.
+hipError_t decode_static_scratch(float** ptr, size_t* bytes);
 hipError_t launch_decode_split(hipStream_t stream, const DecodeSplitParams& p);
 
 // KVLayerCache::append on device buffers of 2- or 4-byte elements: [batch_heads, seq_added, head_dim] into

@@ -66,3 +66,14 @@ class LlmKernels:
                                                      dev_ptr(out), dev_ptr(kv_lens), batch, n_heads, n_kv,
                                                      head_dim, max_seq, dev_ptr(workspace), workspace_bytes,
                                                      C.byref(err)), err)
+
+    @staticmethod
+    def gqa_decode_batched_bf16_noalloc(stream, q, k_cache, v_cache, out, kv_lens, batch, n_heads, n_kv, head_dim,
+                                        max_seq):
+        """gqa_decode_batched_bf16 without a workspace argument: the partials go to a fixed block of device memory
+        inside the library, and the call allocates nothing (for callers under graph capture or in loops that must
+        not call hipMalloc).  Calls that overlap on one GPU race."""
+        err = L.RtErr()
+        raise_for(L.lib().rt_gqa_decode_batched_bf16_noalloc(stream, dev_ptr(q), dev_ptr(k_cache), dev_ptr(v_cache),
+                                                             dev_ptr(out), dev_ptr(kv_lens), batch, n_heads, n_kv,
+                                                             head_dim, max_seq, C.byref(err)), err)
