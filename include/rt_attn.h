@@ -184,8 +184,12 @@ int rt_flash_forward_f32_dev(void *stream, const rt_attention_shape *shape, uint
                              rt_err_detail *err);
 
 /* The bf16 counterpart (bf16 in, f32 accumulate, bf16 out rounded once, to nearest even):
- * q/out [batch,heads,seq,dim], k/v [batch,n_kv_heads,seq,dim].  MFMA kernels cover dim 64 and
- * 128; other dims return RT_ERR_UNSUPPORTED. */
+ * q/out [batch,heads,seq,dim], k/v [batch,n_kv_heads,seq,dim].  Any dim up to 256 that is a multiple of 8 (the
+ * reference's forward takes any dim != 0, cpu_forward.rs:142-169; other dims return RT_ERR_UNSUPPORTED here and
+ * are served by the f32 entries); tensors 16-byte aligned.  Two MFMA kernels stand behind it: a persistent
+ * 8-wave kernel for dim 64 / 128 on unpadded batches of at least 512 rows per sequence and 256 jobs of 256 rows,
+ * and a 4-wave tile kernel for everything else (short or few sequences, padded batches, other dims).  RT_ATTN_BF16_PREFILL=tile or =persistent in the environment forces one
+ * of them where both apply. */
 int rt_flash_forward_bf16_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const void *q,
                               const void *k, const void *v, int mask_kind, const uint8_t *keep, void *out,
                               rt_err_detail *err);
@@ -201,6 +205,17 @@ int rt_flash_forward_bnhd_f32_dev(void *stream, const rt_attention_shape *shape,
 int rt_flash_forward_bnhd_bf16_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const void *q,
                                    const void *k, const void *v, int mask_kind, const uint8_t *keep, void *out,
                                    rt_err_detail *err);
+
+/* bf16 counterpart of rt_mha_forward_masked_f32_dev -- steps 2-8 of MultiHeadAttention::forward's composed path
+ * (crates/rustorch-nn/src/attention.rs:371-399; masks crates/rustorch-nn/src/masks.rs:22-80): q/out bf16
+ * [batch,t_q,heads*head_dim], k/v bf16 [batch,t_kv,heads*head_dim] (t_q != t_kv is cross-attention), `mask` an
+ * additive f32 bias on the device with t_q*t_kv ([T,T] / [1,T,T]) or batch*heads*t_q*t_kv ([B*H,T,T]) elements,
+ * or NULL.  scores = (q.k)/sqrt(head_dim) + mask in f32, softmax, .V; bf16 out rounded once.  A row masked with
+ * -1e4 everywhere comes out uniform, a row of -inf as NaN, as in the f32 entry.  head_dim up to 256, a multiple
+ * of 8; tensors 16-byte aligned.  Asynchronous on `stream`. */
+int rt_mha_forward_masked_bf16_dev(void *stream, const void *q, const void *k, const void *v, const float *mask,
+                                   size_t mask_len, void *out, size_t batch, size_t t_q, size_t t_kv, size_t heads,
+                                   size_t head_dim, rt_err_detail *err);
 
 /* Padded-batch causal prefill: sequence b has seq_lens[b] <= seq valid positions (device
  * int32[batch]); key j of sequence b is masked iff j > i or j >= seq_lens[b].  Valid rows equal
@@ -301,6 +316,20 @@ int rt_gqa_decode_batched_bf16(void *stream, const void *q, const void *k_cache,
                                const int32_t *kv_lens, int32_t batch, int32_t n_heads, int32_t n_kv,
                                int32_t head_dim, int32_t max_seq, void *workspace, size_t workspace_bytes,
                                rt_err_detail *err);
+
+/* gqa_decode_batched_f32 -- crates/rustorch-metal/src/kernels.rs:14432-14516 (launcher :14522-14570) in bf16 and over
+ * a batch of sequences: `seq_new` consecutive new positions per sequence attend to the cache, each up to and
+ * including itself.  q/out bf16 [batch,seq_new,n_heads,head_dim] (position-major, as the reference's
+ * [B,n_heads,head_dim]); caches bf16 [batch,n_kv,max_seq,head_dim], already holding the new positions' keys and
+ * values (rt_qk_norm_rope_kv_append_bf16 with seq = seq_new puts them there); kv_lens device int32[batch] = keys in
+ * the cache INCLUDING the new ones, or NULL: every sequence has `kv_len`.  Position s of sequence b sees keys
+ * [0, kv_lens[b] - seq_new + s]: pos_base of the reference is kv_lens[b] - seq_new.  batch = 1, kv_lens = NULL,
+ * kv_len = pos_base + B is the reference call; seq_new = 1 is rt_gqa_decode_batched_bf16.  kv head = h / (n_heads /
+ * n_kv).  A position that sees no key (kv_lens[b] < seq_new - s) gives a NaN row.  head_dim up to 256, a multiple of 8;
+ * tensors 16-byte aligned; no workspace.  Asynchronous on `stream`. */
+int rt_gqa_decode_chunk_bf16(void *stream, const void *q, const void *k_cache, const void *v_cache, void *out,
+                             const int32_t *kv_lens, int32_t kv_len, int32_t batch, int32_t seq_new, int32_t n_heads,
+                             int32_t n_kv, int32_t head_dim, int32_t max_seq, rt_err_detail *err);
 
 /* No counterpart in the reference.  rt_gqa_decode_batched_bf16 for callers that cannot allocate device memory
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): same arguments without

@@ -19,6 +19,9 @@
  *   ro_kv_trim                crates/rustorch-llm/src/model.rs:638-650
  *   ro_gqa_decode_online_bf16 crates/rustorch-cuda/src/llm_kernels.rs:396-457
  *   ro_kv_append_bf16         crates/rustorch-cuda/src/llm_kernels.rs:353-372
+ *   ro_gqa_decode_chunk_bf16  crates/rustorch-metal/src/kernels.rs:14432-14516 (gqa_decode_batched_f32: several
+ *                             consecutive query positions over one cache, each causal to itself), per sequence,
+ *                             f32 on bf16-rounded inputs
  *   ro_rope_tables            crates/rustorch-nn/src/rope.rs:63-90 (RoPE::new)
  *   ro_rope_half_split        crates/rustorch-nn/src/rope.rs:162-205 (apply_inplace_half_split)
  *   ro_rope_interleaved       crates/rustorch-nn/src/rope.rs:96-142 (apply_inplace)
@@ -629,6 +632,61 @@ RO_EXPORT void ro_gqa_decode_batched_bf16(const uint16_t *q, const uint16_t *k_c
         free(kf);
         free(vf);
         free(qf);
+    }
+}
+
+/* ---- gqa_decode_batched_f32 (crates/rustorch-metal/src/kernels.rs:14432-14516), per sequence of a batch.
+ * Query position s (0 <= s < seq_new) of sequence b sits at absolute position pos_base_b + s with
+ * pos_base_b = kv_lens[b] - seq_new and attends to keys [0, pos_base_b + s] (kv_len = pos_base + b + 1 in the
+ * shader).  Phases as in the shader: scores = dot * inv_sqrt_d; max; e = exp(score - max); sum; weights =
+ * e * (1 / sum); out[d] = sum_p weights[p] * v[p][d] in ascending p.  q/out [B,seq_new,Hq,D] (position-major, the
+ * shader's q + b * n_heads * head_dim + q_h * head_dim), caches [B,Hkv,max_seq,D]; kv head = q_h / (Hq / Hkv).
+ * bf16 bit patterns in, f32 out.  A position with no visible key (kv_lens[b] - seq_new + s < 0) has an empty
+ * softmax: the shader would divide 0 by 0; the row is NaN here. */
+RO_EXPORT void ro_gqa_decode_chunk_bf16(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache,
+                                        const int32_t *kv_lens, float *out, int batch, int seq_new, int n_heads,
+                                        int n_kv, int head_dim, int max_seq, int threads) {
+    const size_t D = (size_t)head_dim, group = (size_t)n_heads / n_kv;
+    const float inv_sqrt_d = 1.0f / sqrtf((float)head_dim);
+    if (threads < 1) threads = 1;
+    long n_tasks = (long)batch * n_heads;
+#pragma omp parallel for schedule(dynamic, 1) num_threads(threads)
+    for (long task = 0; task < n_tasks; task++) {
+        const size_t b = (size_t)task / n_heads, q_h = (size_t)task % n_heads, kv_h = q_h / group;
+        const long pos_base = (long)kv_lens[b] - seq_new;
+        const uint16_t *kb = k_cache + (b * n_kv + kv_h) * (size_t)max_seq * D;
+        const uint16_t *vb = v_cache + (b * n_kv + kv_h) * (size_t)max_seq * D;
+        float *shared = (float *)malloc(sizeof(float) * ((size_t)max_seq + 1));
+        for (int s = 0; s < seq_new; s++) {
+            const uint16_t *qp = q + ((b * seq_new + s) * n_heads + q_h) * D;
+            float *op = out + ((b * seq_new + s) * n_heads + q_h) * D;
+            long kv_len = pos_base + s + 1;
+            if (kv_len > max_seq) kv_len = max_seq;
+            if (kv_len <= 0) {
+                for (size_t d = 0; d < D; d++) op[d] = NAN;
+                continue;
+            }
+            float max_score = -INFINITY;
+            for (long p = 0; p < kv_len; p++) {
+                float dot = 0.0f;
+                for (size_t d = 0; d < D; d++) dot += ro_bf16_to_f32(qp[d]) * ro_bf16_to_f32(kb[(size_t)p * D + d]);
+                shared[p] = dot * inv_sqrt_d;
+                if (shared[p] > max_score) max_score = shared[p];
+            }
+            float sum = 0.0f;
+            for (long p = 0; p < kv_len; p++) {
+                shared[p] = expf(shared[p] - max_score);
+                sum += shared[p];
+            }
+            const float inv_sum = 1.0f / sum;
+            for (long p = 0; p < kv_len; p++) shared[p] *= inv_sum;
+            for (size_t d = 0; d < D; d++) {
+                float acc = 0.0f;
+                for (long p = 0; p < kv_len; p++) acc += shared[p] * ro_bf16_to_f32(vb[(size_t)p * D + d]);
+                op[d] = acc;
+            }
+        }
+        free(shared);
     }
 }
 

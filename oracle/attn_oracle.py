@@ -100,6 +100,8 @@ def lib():
         L.ro_gqa_decode_online_bf16.restype = None
         L.ro_gqa_decode_batched_bf16.argtypes = [u16p, u16p, u16p, i32p, fp] + [C.c_int] * 6
         L.ro_gqa_decode_batched_bf16.restype = None
+        L.ro_gqa_decode_chunk_bf16.argtypes = [u16p, u16p, u16p, i32p, fp] + [C.c_int] * 7
+        L.ro_gqa_decode_chunk_bf16.restype = None
         for name in ("ro_osm_empty",):
             getattr(L, name).argtypes = [C.POINTER(_Osm)]
             getattr(L, name).restype = None
@@ -326,6 +328,22 @@ def gqa_decode_batched_bf16(q, k_cache, v_cache, kv_lens, batch, n_heads, n_kv, 
     lib().ro_gqa_decode_batched_bf16(qp, kp, vp, lens.ctypes.data_as(C.POINTER(C.c_int32)),
                                      out.ctypes.data_as(C.POINTER(C.c_float)), batch, n_heads, n_kv, head_dim,
                                      max_seq, t)
+    return out
+
+
+def gqa_decode_chunk_bf16(q, k_cache, v_cache, kv_lens, batch, seq_new, n_heads, n_kv, head_dim, max_seq, threads=None):
+    """gqa_decode_batched_f32 (crates/rustorch-metal/src/kernels.rs:14432-14516) per sequence: `seq_new` consecutive
+    query positions, position s of sequence b seeing keys [0, kv_lens[b] - seq_new + s].  q bf16 bits
+    [B,seq_new,Hq,D], caches bf16 bits [B,Hkv,max_seq,D]; returns float32 [B*seq_new*Hq*D]."""
+    q, qp = _u16(q)
+    kc, kp = _u16(k_cache)
+    vc, vp = _u16(v_cache)
+    lens = np.ascontiguousarray(kv_lens, dtype=np.int32)
+    out = np.zeros(batch * seq_new * n_heads * head_dim, dtype=np.float32)
+    t = lib().ro_max_threads() if threads is None else threads
+    lib().ro_gqa_decode_chunk_bf16(qp, kp, vp, lens.ctypes.data_as(C.POINTER(C.c_int32)),
+                                   out.ctypes.data_as(C.POINTER(C.c_float)), batch, seq_new, n_heads, n_kv, head_dim,
+                                   max_seq, t)
     return out
 
 

@@ -236,6 +236,17 @@ def mha_forward_masked_f32_dev(q, k, v, out, batch: int, t_q: int, t_kv: int, he
     raise_for(rc, err)
 
 
+def mha_forward_masked_bf16_dev(q, k, v, out, batch: int, t_q: int, t_kv: int, heads: int, head_dim: int, attn_mask=None,
+                                mask_len: int = 0, stream=None):
+    """The same composed path on bf16 device tensors ([B,t,H*hd] bit patterns) with an f32 device mask of `mask_len`
+    elements (t_q*t_kv or B*H*t_q*t_kv) or None; bf16 out.  Enqueues on `stream` and returns."""
+    err = L.RtErr()
+    rc = L.lib().rt_mha_forward_masked_bf16_dev(stream, dev_ptr(q), dev_ptr(k), dev_ptr(v), dev_ptr(attn_mask),
+                                                mask_len if attn_mask is not None else 0, dev_ptr(out), batch, t_q, t_kv,
+                                                heads, head_dim, C.byref(err))
+    raise_for(rc, err)
+
+
 def mha_attention_route(t_q: int, t_kv: int, has_mask: bool) -> str:
     """Which branch `MultiHeadAttention::forward` takes for the attention between its projections, under no_grad on
     contiguous f32 tensors (crates/rustorch-nn/src/attention.rs:325-333, :347-356): "identity" for the single-token

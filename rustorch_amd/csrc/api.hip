@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <algorithm>
@@ -649,6 +650,19 @@ RT_API int rt_flash_forward_f32_dev(void* stream, const rt_attention_shape* shap
     return flash_f32_device((hipStream_t)stream, shape, n_kv_heads, q, k, v, mask_kind, keep, out, err);
 }
 
+// Which bf16 prefill kernel serves a call.  RT_ATTN_BF16_PREFILL=tile|persistent in the environment forces one
+// where both apply (for measurements and tests); otherwise the persistent 8-wave kernel takes head dims 64 and 128
+// on unpadded batches with at least 512 rows per sequence and a job for every CU, and the 4-wave tile kernel
+// everything else.
+enum class PrefillKernel { kAuto, kTile, kPersistent };
+static PrefillKernel prefill_kernel_override() {
+    const char* e = getenv("RT_ATTN_BF16_PREFILL");
+    if (!e) return PrefillKernel::kAuto;
+    if (strcmp(e, "tile") == 0) return PrefillKernel::kTile;
+    if (strcmp(e, "persistent") == 0) return PrefillKernel::kPersistent;
+    return PrefillKernel::kAuto;
+}
+
 static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads, const void* q,
                              const void* k, const void* v, int mask, const uint8_t* keep, const int32_t* seq_lens,
                              int zero_padded_rows, void* out, rt_err_detail* err, bool bnhd = false) {
@@ -659,15 +673,23 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
     if (shape->seq == 0 || shape->batch == 0 || shape->heads == 0) return RT_OK;
     int rc = check_flash_dims(shape, n_kv_heads, err);
     if (rc) return rc;
-    if (shape->dim != 64 && shape->dim != 128)
-        return fail(err, RT_ERR_UNSUPPORTED, -1, 128, shape->dim, "bf16 flash kernels cover dim 64 and 128");
+    if (shape->dim > 256 || shape->dim % 8 != 0)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 256, shape->dim,
+                    "bf16 flash kernels cover head dims up to 256 that are a multiple of 8");
     if ((shape->seq + 127) / 128 * shape->batch * shape->heads > 0x7fffffffull)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
-    {   // the kernel addresses the rows of one (batch, head) slab with 32-bit byte offsets
+    // the persistent kernel needs a job (256 query rows of one head) for every CU and gains on the tile kernel as the
+    // rows get longer; a padded batch is a set of jobs of very different lengths, which the tile kernel's
+    // dispatcher-balanced workgroups handle better
+    const bool persistent_dim = shape->dim == 64 || shape->dim == 128;
+    const uint64_t jobs256 = (shape->seq + 255) / 256 * shape->batch * shape->heads;
+    bool persistent = persistent_dim && shape->seq >= 512 && jobs256 >= 256 && mask != rt::kMaskVarlenCausal;
+    const PrefillKernel forced = prefill_kernel_override();
+    if (forced == PrefillKernel::kTile) persistent = false;
+    if (forced == PrefillKernel::kPersistent && persistent_dim) persistent = true;
+    if (persistent) {  // that kernel addresses the rows of one (batch, head) slab with 32-bit byte offsets
         const uint64_t pitch_b = (bnhd ? shape->heads : 1) * shape->dim * 2;
-        if (shape->seq * pitch_b >= (1ull << 32))
-            return fail(err, RT_ERR_UNSUPPORTED, -1, (1ull << 32) / pitch_b, shape->seq,
-                        "bf16 flash kernels need seq * row pitch below 4 GiB");
+        if (shape->seq * pitch_b >= (1ull << 32)) persistent = false;
     }
     if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 16, 0, "bf16 flash kernels need 16-byte aligned tensors");
@@ -675,6 +697,44 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
         return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
     rc = ensure_device(err);
     if (rc) return rc;
+    const int dim = (int)shape->dim;
+    rt::TensorLayout lq, lkv;
+    if (bnhd) {
+        lq = rt::layout_bnhd((long long)shape->heads, (long long)shape->seq, dim);
+        lkv = rt::layout_bnhd((long long)n_kv_heads, (long long)shape->seq, dim);
+    } else {
+        lq = rt::layout_bhnd((long long)shape->heads, (long long)shape->seq, dim);
+        lkv = rt::layout_bhnd((long long)n_kv_heads, (long long)shape->seq, dim);
+    }
+    const int ref_bc = (int)(shape->bc == 0 ? 1 : (shape->bc > 0x7fffffffull ? 0x7fffffff : shape->bc));
+    const float scale = 1.0f / sqrtf((float)shape->dim);
+    if (!persistent) {
+        rt::FlashTileParams t{};
+        t.q = (const uint16_t*)q;
+        t.k = (const uint16_t*)k;
+        t.v = (const uint16_t*)v;
+        t.out = (uint16_t*)out;
+        t.keep = keep;
+        // a padded batch: sequence b has seq_lens[b] query positions and as many keys, masked causally
+        t.q_lens = mask == rt::kMaskVarlenCausal ? seq_lens : nullptr;
+        t.kv_lens = t.q_lens;
+        t.batch = (int)shape->batch;
+        t.heads = (int)shape->heads;
+        t.kv_heads = (int)n_kv_heads;
+        t.group = (int)(shape->heads / n_kv_heads);
+        t.pack = 1;
+        t.seq_q = t.seq_kv = (int)shape->seq;
+        t.dim = dim;
+        t.mask = mask == rt::kMaskVarlenCausal ? rt::kMaskCausal : mask;
+        t.ref_bc = ref_bc;
+        t.zero_padded_rows = zero_padded_rows;
+        t.scale = scale;
+        t.scale_log2e = scale * rt::kLog2eHost;
+        t.lq = t.lo = lq;
+        t.lkv = lkv;
+        HIP_TRY(rt::launch_flash_tile_bf16((hipStream_t)stream, t), "flash_tile_bf16 launch");
+        return RT_OK;
+    }
     rt::FlashBf16Params p;
     p.q = (const uint16_t*)q;
     p.k = (const uint16_t*)k;
@@ -687,19 +747,14 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
     p.kv_heads = (int)n_kv_heads;
     p.group = (int)(shape->heads / n_kv_heads);
     p.seq = (int)shape->seq;
-    p.dim = (int)shape->dim;
+    p.dim = dim;
     p.mask = mask;
-    p.ref_bc = (int)(shape->bc == 0 ? 1 : (shape->bc > 0x7fffffffull ? 0x7fffffff : shape->bc));
+    p.ref_bc = ref_bc;
     p.zero_padded_rows = zero_padded_rows;
-    p.scale_log2e = (1.0f / sqrtf((float)shape->dim)) * rt::kLog2eHost;
+    p.scale_log2e = scale * rt::kLog2eHost;
     p.n_workers = g_num_cus;
-    if (bnhd) {
-        p.lq = p.lo = rt::layout_bnhd((long long)shape->heads, (long long)shape->seq, p.dim);
-        p.lkv = rt::layout_bnhd((long long)n_kv_heads, (long long)shape->seq, p.dim);
-    } else {
-        p.lq = p.lo = rt::layout_bhnd((long long)shape->heads, (long long)shape->seq, p.dim);
-        p.lkv = rt::layout_bhnd((long long)n_kv_heads, (long long)shape->seq, p.dim);
-    }
+    p.lq = p.lo = lq;
+    p.lkv = lkv;
     HIP_TRY(rt::launch_flash_bf16((hipStream_t)stream, p), "flash_fwd_bf16 launch");
     return RT_OK;
 }
@@ -878,6 +933,58 @@ RT_API int rt_mha_forward_masked_f32_dev(void* stream, const float* q, const flo
                              heads, head_dim, err);
 }
 
+// bf16 counterpart of rt_mha_forward_masked_f32_dev: steps 2-8 of MultiHeadAttention::forward's composed path
+// (crates/rustorch-nn/src/attention.rs:371-399) on bf16 [B,T,H*hd] tensors with an f32 additive mask.
+RT_API int rt_mha_forward_masked_bf16_dev(void* stream, const void* q, const void* k, const void* v, const float* mask,
+                                          size_t mask_len, void* out, size_t batch, size_t t_q, size_t t_kv,
+                                          size_t heads, size_t head_dim, rt_err_detail* err) {
+    clear_err(err);
+    if (head_dim == 0) return fail(err, RT_ERR_ZERO_DIM, -1, 0, 0, "dim must be > 0");
+    const size_t embed = heads * head_dim;
+    const size_t q_expected = batch * t_q * embed, kv_expected = batch * t_kv * embed;
+    const size_t one_mask = t_q * t_kv, all_masks = batch * heads * one_mask;
+    if (!mask) mask_len = 0;
+    if (mask_len != 0 && mask_len != one_mask && mask_len != all_masks)
+        return fail(err, RT_ERR_WRONG_INPUT_LEN, RT_WHICH_MASK, one_mask, mask_len, "mask length");
+    if (q_expected == 0) return RT_OK;
+    if (!q || !out || (kv_expected && (!k || !v))) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    if (!rt::flash_tile_bf16_supported((int)std::min<size_t>(head_dim, 1 << 20)))
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 256, head_dim, "bf16 kernels cover head dims up to 256 that are a multiple of 8");
+    if (heads > 65535 || batch > 65535 || t_q > 0x7fffffffull || t_kv > 0x7fffffffull || embed > 0x7fffffffull ||
+        (t_q + 127) / 128 * batch * heads > 0x7fffffffull)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0 || ((uintptr_t)mask & 3) != 0)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 16, 0, "bf16 kernels need 16-byte aligned tensors");
+    int rc = ensure_device(err);
+    if (rc) return rc;
+    rt::FlashTileParams t{};
+    t.q = (const uint16_t*)q;
+    t.k = (const uint16_t*)k;
+    t.v = (const uint16_t*)v;
+    t.out = (uint16_t*)out;
+    t.bias = mask_len ? mask : nullptr;
+    t.bias_bh_stride = (mask_len == all_masks && all_masks != one_mask) ? (long long)one_mask : 0;
+    t.bias_vec4 = (((uintptr_t)mask & 15) == 0 && t_kv % 4 == 0) ? 1 : 0;
+    t.batch = (int)batch;
+    t.heads = t.kv_heads = (int)heads;
+    t.group = 1;
+    t.pack = 1;
+    t.seq_q = (int)t_q;
+    t.seq_kv = (int)t_kv;
+    t.dim = (int)head_dim;
+    t.mask = rt::kMaskNone;
+    t.ref_bc = 64;
+    t.zero_padded_rows = 0;
+    t.scale = 1.0f / sqrtf((float)head_dim);
+    t.scale_log2e = t.scale * rt::kLog2eHost;
+    t.lq = t.lo = rt::layout_bnhd((long long)heads, (long long)t_q, (int)head_dim);
+    t.lkv = rt::layout_bnhd((long long)heads, (long long)t_kv, (int)head_dim);
+    if (t_kv == 0)  // no key to weigh: the reference's products over an empty axis leave rows of zeros
+        return rt_buf_zero(out, q_expected * 2, stream, err);
+    HIP_TRY(rt::launch_flash_tile_bf16((hipStream_t)stream, t), "flash_tile_bf16 launch");
+    return RT_OK;
+}
+
 RT_API int rt_flash_forward_varlen_bf16_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,
                                             const void* q, const void* k, const void* v, const int32_t* seq_lens,
                                             int zero_padded_rows, void* out, rt_err_detail* err) {
@@ -1051,6 +1158,55 @@ RT_API int rt_gqa_decode_online_bf16(void* stream, const void* q, const void* k_
     p.head_map = 1;
     p.scale = 1.0f / sqrtf((float)head_dim);
     HIP_TRY(rt::launch_attn_rows_bf16((hipStream_t)stream, p), "attn_rows_bf16 launch");
+    return RT_OK;
+}
+
+// Several new positions per sequence against the cache, causally masked: the bf16 form of gqa_decode_batched_f32
+// (crates/rustorch-metal/src/kernels.rs:14432-14516), batched over sequences with their own context lengths.
+RT_API int rt_gqa_decode_chunk_bf16(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out,
+                                    const int32_t* kv_lens, int32_t kv_len, int32_t batch, int32_t seq_new,
+                                    int32_t n_heads, int32_t n_kv, int32_t head_dim, int32_t max_seq,
+                                    rt_err_detail* err) {
+    clear_err(err);
+    int rc = check_decode_dims(batch, n_heads, n_kv, head_dim, max_seq, err);
+    if (rc) return rc;
+    if (seq_new < 0) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "negative dimension");
+    if (!kv_lens && (kv_len < seq_new || kv_len > max_seq))
+        return fail(err, RT_ERR_KV_OVERFLOW, -1, (uint64_t)max_seq, (uint64_t)(int64_t)kv_len,
+                    "kv_len must cover the new positions and fit the cache");
+    if (batch == 0 || n_heads == 0 || seq_new == 0) return RT_OK;
+    if (!q || !out || !k_cache || !v_cache) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    if (!rt::flash_tile_bf16_supported(head_dim))
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 256, (uint64_t)head_dim,
+                    "bf16 kernels cover head dims up to 256 that are a multiple of 8");
+    if ((((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)out) & 15) != 0)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 16, 0, "bf16 kernels need 16-byte aligned tensors");
+    const int group = n_heads / n_kv;
+    if ((int64_t)seq_new * group > 0x7fffffffll) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    rc = ensure_device(err);
+    if (rc) return rc;
+    rt::FlashTileParams t{};
+    t.q = (const uint16_t*)q;
+    t.k = (const uint16_t*)k_cache;
+    t.v = (const uint16_t*)v_cache;
+    t.out = (uint16_t*)out;
+    t.kv_lens = kv_lens;
+    t.batch = batch;
+    t.heads = n_heads;
+    t.kv_heads = n_kv;
+    t.group = group;
+    t.pack = group;  // rows of a tile run over (position, head of the group): one pass over a kv head's keys serves them all
+    t.seq_q = seq_new;
+    t.seq_kv = kv_lens ? max_seq : kv_len;
+    t.dim = head_dim;
+    t.mask = rt::kMaskCausal;  // position s sees keys [0, kv_len - seq_new + s]
+    t.ref_bc = 64;
+    t.zero_padded_rows = 0;
+    t.scale = 1.0f / sqrtf((float)head_dim);
+    t.scale_log2e = t.scale * rt::kLog2eHost;
+    t.lq = t.lo = rt::layout_bnhd((long long)n_heads, (long long)seq_new, head_dim);
+    t.lkv = rt::layout_bhnd((long long)n_kv, (long long)max_seq, head_dim);
+    HIP_TRY(rt::launch_flash_tile_bf16((hipStream_t)stream, t), "flash_tile_bf16 launch");
     return RT_OK;
 }
 

@@ -92,6 +92,34 @@ struct FlashBf16Params {
 // dim in {64, 128}.
 hipError_t launch_flash_bf16(hipStream_t stream, const FlashBf16Params& p);
 
+// The general bf16 forward (flash_bf16_tile.hip): any dim <= 256 that is a multiple of 8, own key count, per-sequence
+// query / key counts, causal mask aligned to the last key, key-padding vector, additive f32 bias, packed GQA rows.
+struct FlashTileParams {
+    const uint16_t* q;
+    const uint16_t* k;
+    const uint16_t* v;
+    uint16_t* out;
+    const uint8_t* keep;      // kMaskPadding: device, seq_kv bytes
+    const int32_t* q_lens;    // optional device int32[batch]: valid query positions (rows past them are padding)
+    const int32_t* kv_lens;   // optional device int32[batch]: keys that exist
+    const float* bias;        // optional additive score bias, f32 rows of seq_kv per query position, added after scaling
+    long long bias_bh_stride; // elements between the biases of consecutive (batch, head) pairs; 0 = one for all
+    int bias_vec4;            // bias rows may be read 16 bytes at a time (base and seq_kv * 4 bytes both 16-byte aligned)
+    int batch, heads, kv_heads, group;
+    // 1: a tile's rows are positions of one head.  group: rows run over (position, head of the GQA group), row
+    // r = position * group + head-in-group, so that all heads of a kv head share one pass over its keys.
+    int pack;
+    int seq_q, seq_kv, dim;
+    int mask;   // kMaskNone, kMaskCausal (key j visible to position i iff j <= i + (keys - valid queries)), kMaskPadding
+    int ref_bc;
+    int zero_padded_rows;  // rows past q_lens[b]: +0.0 (else NaN)
+    float scale_log2e;     // (1/sqrt(dim)) * log2(e)
+    float scale;           // 1/sqrt(dim)
+    TensorLayout lq, lkv, lo;
+};
+bool flash_tile_bf16_supported(int dim);
+hipError_t launch_flash_tile_bf16(hipStream_t stream, const FlashTileParams& p);
+
 // Unmasked attention of every query row over all keys; generic in dim (<= 512), head
 // grouping, kv_len and query count.  T is float or uint16_t (bf16 bits).
 struct AttnRowsParams {

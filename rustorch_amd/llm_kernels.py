@@ -77,3 +77,19 @@ class LlmKernels:
         raise_for(L.lib().rt_gqa_decode_batched_bf16_noalloc(stream, dev_ptr(q), dev_ptr(k_cache), dev_ptr(v_cache),
                                                              dev_ptr(out), dev_ptr(kv_lens), batch, n_heads, n_kv,
                                                              head_dim, max_seq, C.byref(err)), err)
+
+    @staticmethod
+    def gqa_decode_chunk_bf16(stream, q, k_cache, v_cache, out, kv_lens, batch, seq_new, n_heads, n_kv, head_dim,
+                              max_seq):
+        """`seq_new` consecutive new positions per sequence against the cache, causally masked (the bf16, batched form
+        of gqa_decode_batched_f32, crates/rustorch-metal/src/kernels.rs:14432-14516): q/out [B,seq_new,Hq,D], caches
+        [B,Hkv,max_seq,D] already holding the new positions; `kv_lens` a device int32[B] buffer of key counts that
+        include the new positions, or an int used for every sequence."""
+        err = L.RtErr()
+        if isinstance(kv_lens, (int,)):
+            lens_ptr, kv_len = None, int(kv_lens)
+        else:
+            lens_ptr, kv_len = dev_ptr(kv_lens), 0
+        raise_for(L.lib().rt_gqa_decode_chunk_bf16(stream, dev_ptr(q), dev_ptr(k_cache), dev_ptr(v_cache), dev_ptr(out),
+                                                   lens_ptr, kv_len, batch, seq_new, n_heads, n_kv, head_dim, max_seq,
+                                                   C.byref(err)), err)

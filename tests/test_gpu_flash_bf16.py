@@ -19,9 +19,23 @@ def inputs(shape_q, shape_kv, seeds=(1, 2, 3), q_mul=1.0):
     return bf16_round(q), bf16_round(k), bf16_round(v)
 
 
-@pytest.mark.parametrize("d", [64, 128])
+# (kernel forced through RT_ATTN_BF16_PREFILL, head dim): the persistent 8-wave kernel covers 64 and 128, the
+# 4-wave tile kernel every multiple of 8 up to 256 (zero-padded to 32 / 64 / 96 / 128 / 256 in LDS)
+KERNEL_DIMS = [("persistent", 64), ("persistent", 128), ("tile", 32), ("tile", 64), ("tile", 80), ("tile", 96),
+               ("tile", 128), ("tile", 8), ("tile", 200), ("tile", 256)]
+
+
+@pytest.fixture
+def force_kernel(monkeypatch):
+    def force(name):
+        monkeypatch.setenv("RT_ATTN_BF16_PREFILL", name)
+    return force
+
+
+@pytest.mark.parametrize("kernel,d", KERNEL_DIMS)
 @pytest.mark.parametrize("n", [1, 2, 31, 63, 64, 65, 127, 128, 129, 200, 513])
-def test_flash_bf16_matches_oracle(oracle, n, d):
+def test_flash_bf16_matches_oracle(oracle, force_kernel, n, kernel, d):
+    force_kernel(kernel)
     b, h = 2, 3
     (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d), (n, n + 1, n + 2))
     shape = ra.AttentionShape.new(b, h, n, d)
@@ -31,7 +45,24 @@ def test_flash_bf16_matches_oracle(oracle, n, d):
     for mask, om in ((ra.Mask.none(), None), (ra.Mask.causal(), "causal"), (ra.Mask.padding(keep), ("padding", keep))):
         got = flash_bf16(shape, qb, kb, vb, mask)
         want = oracle.flash_forward_masked(oracle.AttentionShape(b, h, n, d), qf, kf, vf, om)
-        assert_close_nan(got, want, TOL, f"n={n} d={d} mask={mask.kind}")
+        assert_close_nan(got, want, TOL, f"n={n} d={d} mask={mask.kind} kernel={kernel}")
+
+
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("n", [300, 2048 + 77])
+def test_both_prefill_kernels_agree(oracle, force_kernel, n, d):
+    """The two kernels behind rt_flash_forward_bf16_dev on one input: each within the bar of the oracle, and of
+    each other (they round P to bf16 at the same point, so they differ by accumulation order only)."""
+    b, h = 1, 8
+    (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d), (71, 72, 73))
+    shape = ra.AttentionShape.new(b, h, n, d)
+    want = oracle.flash_forward_masked(oracle.AttentionShape(b, h, n, d), qf, kf, vf, "causal")
+    outs = {}
+    for kernel in ("persistent", "tile"):
+        force_kernel(kernel)
+        outs[kernel] = flash_bf16(shape, qb, kb, vb, ra.Mask.causal())
+        assert_close_nan(outs[kernel], want, TOL, kernel)
+    assert max_abs(outs["persistent"], outs["tile"]) <= TOL
 
 
 def test_flash_bf16_closed_forms():
@@ -49,7 +80,9 @@ def test_flash_bf16_closed_forms():
     assert max_abs(out, cf) <= 2 ** -7 * 2.0  # weights sum to 1 up to P's bf16 rounding
 
 
-def test_flash_bf16_masks_nan_rules(oracle):
+@pytest.mark.parametrize("kernel", ["persistent", "tile"])
+def test_flash_bf16_masks_nan_rules(oracle, force_kernel, kernel):
+    force_kernel(kernel)
     b, h, n, d = 1, 2, 150, 64
     (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d))
     shape = ra.AttentionShape.new(b, h, n, d)
@@ -70,9 +103,11 @@ def test_flash_bf16_masks_nan_rules(oracle):
         assert_close_nan(got, want, TOL)
 
 
+@pytest.mark.parametrize("kernel", ["persistent", "tile"])
 @pytest.mark.parametrize("hq,hkv", [(8, 2), (4, 1), (6, 6)])
-def test_flash_bf16_gqa_head_mapping(oracle, hq, hkv):
+def test_flash_bf16_gqa_head_mapping(oracle, force_kernel, kernel, hq, hkv):
     """kv head = h / (Hq/Hkv): equals the oracle on explicitly replicated K/V (gqa.rs:151-177)."""
+    force_kernel(kernel)
     b, n, d = 2, 130, 128
     (qb, qf), (kb, kf), (vb, vf) = inputs((b, hq, n, d), (b, hkv, n, d))
     got = flash_bf16(ra.AttentionShape.new(b, hq, n, d), qb, kb, vb, ra.Mask.causal(), n_kv_heads=hkv)
@@ -95,8 +130,10 @@ def run_varlen(shape, qb, kb, vb, lens, zero=True):
     return attn_oracle.bf16_to_f32(dout.download(np.uint16, n_out))
 
 
-def test_varlen_small(oracle):
-    b, h, n, d = 4, 2, 200, 64
+@pytest.mark.parametrize("kernel,d", [("persistent", 64), ("tile", 64), ("tile", 96), ("persistent", 128)])
+def test_varlen_small(oracle, force_kernel, kernel, d):
+    force_kernel(kernel)
+    b, h, n = 4, 2, 200
     lens = [200, 1, 129, 0]
     (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d))
     shape = ra.AttentionShape.new(b, h, n, d)
@@ -110,9 +147,11 @@ def test_varlen_small(oracle):
                 assert (g[i, :, L:] == 0.0).all() and not np.signbit(g[i, :, L:]).any()
 
 
-def test_config_padded_batch_b16_h16_n1024_d64(oracle):
+@pytest.mark.parametrize("kernel", ["auto", "persistent", "tile"])
+def test_config_padded_batch_b16_h16_n1024_d64(oracle, force_kernel, kernel):
     """The variable-length workload of the benchmark set: lengths uniform in [128, 1024] from a seed, key padding + causal,
     padded query rows exactly 0."""
+    force_kernel(kernel)
     b, h, n, d = 16, 16, 1024, 64
     lens = np.random.default_rng(2026).integers(128, 1025, size=b).astype(np.int32)
     (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d), (21, 22, 23))
@@ -170,21 +209,25 @@ def test_config_long_context_b1_h32_n16384_d128(oracle):
             assert max_abs(got[hi, i], want) <= TOL, (hi, i)
 
 
-def test_unsupported_dim_is_an_error():
-    shape = ra.AttentionShape.new(1, 1, 8, 96)
-    z = dev(np.zeros(8 * 96, dtype=np.uint16))
+@pytest.mark.parametrize("d", [257, 264, 100, 4])
+def test_unsupported_dim_is_an_error(d):
+    """Head dims above 256, or not a multiple of 8 (rows would not be 16-byte aligned), are refused."""
+    shape = ra.AttentionShape.new(1, 1, 8, d)
+    z = dev(np.zeros(8 * d, dtype=np.uint16))
     with pytest.raises(ra.DeviceError) as ei:
         ra.flash_forward_bf16_dev(shape, z, z, z, z)
     assert ei.value.status == 21
 
 
+@pytest.mark.parametrize("kernel", ["persistent", "tile"])
 @pytest.mark.parametrize("bad", [np.nan, np.inf])
-def test_non_finite_v_row_at_a_causally_hidden_position(oracle, bad):
+def test_non_finite_v_row_at_a_causally_hidden_position(oracle, force_kernel, kernel, bad):
     """A non-finite V row j under the causal mask.  The reference walks every key tile and multiplies the hidden
     probabilities (exact zeros) into V, so 0 * NaN (or 0 * Inf) makes EVERY query row non-finite in that column (cpu_forward.rs:268-425: no tile is
     skipped).  The kernels skip key tiles that lie wholly past a query tile and never read those V rows: rows that
     see key j (i >= j) are NaN as in the reference; rows at least 256 positions before j are finite and equal the
     result with that V row replaced by zeros; rows in between are NaN or that finite value."""
+    force_kernel(kernel)
     b, h, n, d, j = 1, 2, 1024, 128, 700
     (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d), (51, 52, 53))
     vbad = vf.copy().reshape(b, h, n, d)
@@ -207,3 +250,22 @@ def test_non_finite_v_row_at_a_causally_hidden_position(oracle, bad):
     assert ok.all()
     # the other columns of the poisoned rows stay finite in both (only column 5 of V is bad)
     assert np.isfinite(got[..., :5]).all() and np.isfinite(want_ref[..., :5]).all()
+
+
+@pytest.mark.parametrize("kernel,d", [("persistent", 64), ("persistent", 128), ("tile", 64), ("tile", 128), ("tile", 96)])
+def test_two_launches_give_the_same_bits(force_kernel, kernel, d):
+    """No atomics, no order that depends on timing: the same inputs give the same output bits on every launch.
+    (A vector instruction that reads a matrix result too early, for one, shows up here as last-bit differences.)"""
+    force_kernel(kernel)
+    b, h, n = 1, 2, 300
+    (qb, _), (kb, _), (vb, _) = inputs((b, h, n, d), (b, h, n, d), (81, 82, 83))
+    shape = ra.AttentionShape.new(b, h, n, d)
+    dq, dk, dv = dev(qb), dev(kb), dev(vb)
+    for mask in (ra.Mask.none(), ra.Mask.causal()):
+        outs = []
+        for _ in range(4):
+            dout = ra.HipStorage(qb.size * 2)
+            ra.flash_forward_bf16_dev(shape, dq, dk, dv, dout, mask)
+            ra.synchronize()
+            outs.append(dout.download(np.uint16))
+        assert all(np.array_equal(outs[0], o) for o in outs[1:])

@@ -291,3 +291,68 @@ def test_gqa_decode_batched_matches_per_sequence_reference_call(oracle):
         ref = attention_f64(qf[b].reshape(1, hq, 1, d), np.repeat(kf[b, :, :n], g, axis=0)[None],
                             np.repeat(vf[b, :, :n], g, axis=0)[None])[0, :, 0]
         assert np.abs(out[b] - ref).max() < 5e-6
+
+
+# ---- ro_gqa_decode_chunk_bf16: gqa_decode_batched_f32 (crates/rustorch-metal/src/kernels.rs:14432-14516) ------
+
+
+def _chunk_inputs(oracle, b, s, hq, hkv, d, max_seq, seed):
+    rng = np.random.default_rng(seed)
+    q = oracle.f32_to_bf16(rng.standard_normal((b, s, hq, d), dtype=np.float32))
+    k = oracle.f32_to_bf16(rng.standard_normal((b, hkv, max_seq, d), dtype=np.float32))
+    v = oracle.f32_to_bf16(rng.standard_normal((b, hkv, max_seq, d), dtype=np.float32))
+    return q, k, v
+
+
+def test_chunk_decode_against_float64_brute_force(oracle):
+    """Every (sequence, position, head) row against softmax(q.K^T / sqrt(d)) V in float64 over the keys
+    [0, kv_len - seq_new + s]: a wrong causal offset, head map or layout fails here."""
+    b, s, hq, hkv, d, max_seq = 2, 5, 6, 2, 16, 40
+    lens = [40, 9]
+    q, k, v = _chunk_inputs(oracle, b, s, hq, hkv, d, max_seq, 3)
+    got = oracle.gqa_decode_chunk_bf16(q, k, v, lens, b, s, hq, hkv, d, max_seq).reshape(b, s, hq, d)
+    qf = oracle.bf16_to_f32(q).astype(np.float64).reshape(b, s, hq, d)
+    kf = oracle.bf16_to_f32(k).astype(np.float64).reshape(b, hkv, max_seq, d)
+    vf = oracle.bf16_to_f32(v).astype(np.float64).reshape(b, hkv, max_seq, d)
+    for bi in range(b):
+        for si in range(s):
+            n = lens[bi] - s + si + 1
+            for h in range(hq):
+                kv = h // (hq // hkv)
+                sc = kf[bi, kv, :n] @ qf[bi, si, h] / np.sqrt(np.float64(np.float32(d)))
+                w = np.exp(sc - sc.max())
+                want = (w / w.sum()) @ vf[bi, kv, :n]
+                assert np.abs(got[bi, si, h] - want).max() <= 5e-6, (bi, si, h)
+
+
+def test_chunk_of_one_position_is_the_single_row_decode(oracle):
+    """seq_new = 1 reduces to decode_attn_row on the prefix (gqa.rs:216-270), the function the batched decode oracle
+    applies: same phases in the same order."""
+    b, hq, hkv, d, max_seq = 3, 8, 2, 32, 70
+    lens = [70, 1, 33]
+    q, k, v = _chunk_inputs(oracle, b, 1, hq, hkv, d, max_seq, 5)
+    a = oracle.gqa_decode_chunk_bf16(q, k, v, lens, b, 1, hq, hkv, d, max_seq)
+    w = oracle.gqa_decode_batched_bf16(q, k, v, lens, b, hq, hkv, d, max_seq)
+    assert np.abs(a - w).max() <= 1e-6
+
+
+def test_chunk_from_position_zero_is_causal_attention(oracle):
+    """kv_len = seq_new (pos_base 0): row s sees keys [0, s], which is the causal forward of
+    cpu_forward.rs:193-425 on the same tensors (closed form: row 0 equals V[0])."""
+    b, s, hq, hkv, d = 1, 37, 4, 2, 16
+    q, k, v = _chunk_inputs(oracle, b, s, hq, hkv, d, s, 8)
+    got = oracle.gqa_decode_chunk_bf16(q, k, v, [s], b, s, hq, hkv, d, s).reshape(b, s, hq, d)
+    vf = oracle.bf16_to_f32(v).reshape(b, hkv, s, d)
+    kf = oracle.bf16_to_f32(k).reshape(b, hkv, s, d)
+    qf = oracle.bf16_to_f32(q).reshape(b, s, hq, d).transpose(0, 2, 1, 3)
+    g = hq // hkv
+    assert np.array_equal(got[0, 0], np.repeat(vf[0, :, 0], g, axis=0))
+    want = oracle.flash_forward_masked(oracle.AttentionShape(b, hq, s, d), np.ascontiguousarray(qf),
+                                       np.repeat(kf, g, axis=1), np.repeat(vf, g, axis=1), "causal")
+    assert np.abs(got - want.reshape(b, hq, s, d).transpose(0, 2, 1, 3)).max() <= 1e-5
+
+
+def test_chunk_position_without_keys_is_nan(oracle):
+    q, k, v = _chunk_inputs(oracle, 1, 3, 2, 1, 8, 10, 1)
+    got = oracle.gqa_decode_chunk_bf16(q, k, v, [1], 1, 3, 2, 1, 8, 10).reshape(3, 2, 8)
+    assert np.isnan(got[:2]).all() and np.isfinite(got[2]).all()
