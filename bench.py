@@ -328,9 +328,10 @@ def main():
                              "flop_convention": "4*H*D*sum_b len_b*(len_b+1)/2 (valid pairs only)"},
                   "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                                "frac": achieved / PEAK_BF16_TFLOPS,
-                               "traffic": profile_traffic("flash_fwd_bf16_varlen_b16_h16_n1024_d64.md",
-                                                          "flash_fwd_bf16_kernel<64,varlen>"),
-                               "kernel": "flash_fwd_bf16_kernel<64, varlen>", "kernel_ms_mean": tm.mean_ms}}
+                               "traffic": profile_traffic("flash_tile_bf16_varlen_b16_h16_n1024_d64.md",
+                                                          "flash_tile_bf16_kernel<64,causal>"),
+                               "kernel": "flash_tile_bf16_kernel<64, causal> (per-sequence lengths)",
+                               "kernel_ms_mean": tm.mean_ms}}
         if not args.no_cpu:
             # the oracle of a sequence is the reference's causal forward on the problem truncated to its length
             got = oracle.bf16_to_f32(dout.download(np.uint16)).reshape(Bp, Hp, Np, Dp)

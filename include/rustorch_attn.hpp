@@ -318,6 +318,16 @@ inline void mha_forward_masked_f32_dev(const float* q, const float* k, const flo
     detail::check_attention(rc, e);
 }
 
+// The same composed path on bf16 device tensors (bit patterns, [B,t,H*hd]) with an f32 device mask; bf16 out.
+inline void mha_forward_masked_bf16_dev(const void* q, const void* k, const void* v, void* out, size_t batch, size_t t_q,
+                                        size_t t_kv, size_t heads, size_t head_dim, const float* mask = nullptr,
+                                        size_t mask_len = 0, void* stream = nullptr) {
+    rt_err_detail e;
+    int rc = rt_mha_forward_masked_bf16_dev(stream, q, k, v, mask, mask_len, out, batch, t_q, t_kv, heads, head_dim, &e);
+    if (rc == RT_ERR_WRONG_INPUT_LEN) detail::check_gqa(rc, e);  // which = "mask"
+    detail::check_attention(rc, e);
+}
+
 // The branch MultiHeadAttention::forward takes for the attention between its projections, under no_grad on contiguous
 // f32 tensors (attention.rs:325-333, :347-356).
 enum class MhaRoute { Identity, Flash, Composed };
@@ -600,6 +610,27 @@ struct LlmKernels {
         rt_err_detail e;
         detail::check_gqa(rt_gqa_decode_batched_bf16(stream, q, k_cache, v_cache, out, kv_lens, batch, n_heads, n_kv,
                                                      head_dim, max_seq, workspace, workspace_bytes, &e),
+                          e);
+    }
+    // The same without a workspace: the partials go to a fixed block of device memory inside the library, and the call
+    // allocates nothing (for callers under graph capture or in loops that must not allocate).
+    static void gqa_decode_batched_bf16_noalloc(void* stream, const void* q, const void* k_cache, const void* v_cache,
+                                                void* out, const int32_t* kv_lens, int32_t batch, int32_t n_heads,
+                                                int32_t n_kv, int32_t head_dim, int32_t max_seq) {
+        rt_err_detail e;
+        detail::check_gqa(rt_gqa_decode_batched_bf16_noalloc(stream, q, k_cache, v_cache, out, kv_lens, batch, n_heads,
+                                                             n_kv, head_dim, max_seq, &e),
+                          e);
+    }
+    // gqa_decode_batched_f32 (crates/rustorch-metal/src/kernels.rs:14432-14516) in bf16 over a batch: seq_new consecutive
+    // new positions per sequence, position s seeing keys [0, kv_lens[b] - seq_new + s]; q/out [B,seq_new,Hq,D].
+    // kv_lens == nullptr: every sequence has kv_len keys.
+    static void gqa_decode_chunk_bf16(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out,
+                                      const int32_t* kv_lens, int32_t kv_len, int32_t batch, int32_t seq_new,
+                                      int32_t n_heads, int32_t n_kv, int32_t head_dim, int32_t max_seq) {
+        rt_err_detail e;
+        detail::check_gqa(rt_gqa_decode_chunk_bf16(stream, q, k_cache, v_cache, out, kv_lens, kv_len, batch, seq_new,
+                                                   n_heads, n_kv, head_dim, max_seq, &e),
                           e);
     }
 };

@@ -92,7 +92,7 @@ def test_no_device_is_reported_not_hidden():
 
 
 def test_bf16_prefill_argument_errors_before_any_device_use():
-    """Unsupported head dim, misaligned tensors and rows beyond 32-bit offsets are refused by the host checks."""
+    """Unsupported head dims and misaligned tensors are refused by the host checks."""
     import ctypes as C
     lib = L.lib()
 
@@ -101,14 +101,13 @@ def test_bf16_prefill_argument_errors_before_any_device_use():
         s = ra.AttentionShape.new(b, h, n, d)._c()
         return fn(None, C.byref(s), 0, q, k, v, 1, None, o, C.byref(err)), err
 
-    rc, err = call(lib.rt_flash_forward_bf16_dev, 1, 1, 8, 96)
-    assert rc == L.RT_ERR_UNSUPPORTED and b"64 and 128" in err.message
+    for d in (100, 264, 4):  # not a multiple of 8 (rows would not be 16-byte aligned), or above 256
+        rc, err = call(lib.rt_flash_forward_bf16_dev, 1, 1, 8, d)
+        assert rc == L.RT_ERR_UNSUPPORTED and b"multiple of 8" in err.message
     rc, err = call(lib.rt_flash_forward_bf16_dev, 1, 1, 8, 128, q=0x1008)
     assert rc == L.RT_ERR_UNSUPPORTED and b"aligned" in err.message
-    rc, err = call(lib.rt_flash_forward_bf16_dev, 1, 1, 1 << 24, 128)  # 2^24 rows x 256 B = 4 GiB
-    assert rc == L.RT_ERR_UNSUPPORTED and b"4 GiB" in err.message
-    rc, err = call(lib.rt_flash_forward_bnhd_bf16_dev, 1, 64, 1 << 18, 128)  # row pitch 16 KiB in [B,N,H,D]
-    assert rc == L.RT_ERR_UNSUPPORTED and b"4 GiB" in err.message
+    rc, err = call(lib.rt_flash_forward_bnhd_bf16_dev, 1, 1, 8, 96, v=0x3004)
+    assert rc == L.RT_ERR_UNSUPPORTED and b"aligned" in err.message
     rc, err = call(lib.rt_flash_forward_bf16_dev, 1, 1, 8, 0)
     assert rc == L.RT_ERR_ZERO_DIM
     rc, err = call(lib.rt_flash_forward_bf16_dev, 1, 1, 0, 128, q=None)  # seq == 0: Ok, nothing touched
@@ -208,3 +207,39 @@ def test_stream_create_reports_a_missing_device():
 def test_shutdown_without_a_device_is_a_no_op():
     ra.shutdown()
     ra.shutdown()
+
+
+def test_general_bf16_entries_argument_errors_before_any_device_use():
+    """rt_mha_forward_masked_bf16_dev, rt_gqa_decode_chunk_bf16 and rt_gqa_decode_batched_bf16_noalloc refuse bad
+    arguments in the host checks (the pointers below are never dereferenced)."""
+    import ctypes as C
+    lib = L.lib()
+    err = L.RtErr()
+    p = 0x1000
+    assert lib.rt_mha_forward_masked_bf16_dev(None, p, p, p, None, 0, p, 1, 4, 4, 2, 0, C.byref(err)) == L.RT_ERR_ZERO_DIM
+    rc = lib.rt_mha_forward_masked_bf16_dev(None, p, p, p, p, 15, p, 1, 4, 4, 2, 16, C.byref(err))
+    assert rc == L.RT_ERR_WRONG_INPUT_LEN and err.which == 5 and (err.expected, err.got) == (16, 15)
+    assert lib.rt_mha_forward_masked_bf16_dev(None, p, p, p, None, 0, p, 1, 4, 4, 2, 20, C.byref(err)) == L.RT_ERR_UNSUPPORTED
+    assert lib.rt_mha_forward_masked_bf16_dev(None, p + 2, p, p, None, 0, p, 1, 4, 4, 2, 16, C.byref(err)) == L.RT_ERR_UNSUPPORTED
+    assert lib.rt_mha_forward_masked_bf16_dev(None, None, p, p, None, 0, p, 1, 4, 4, 2, 16, C.byref(err)) == L.RT_ERR_NULL_POINTER
+    assert lib.rt_mha_forward_masked_bf16_dev(None, None, None, None, None, 0, None, 0, 4, 4, 2, 16, C.byref(err)) == L.RT_OK
+
+    def chunk(kv_lens, kv_len, batch, s, hq, hkv, d, max_seq, q=p):
+        return lib.rt_gqa_decode_chunk_bf16(None, q, p, p, p, kv_lens, kv_len, batch, s, hq, hkv, d, max_seq, C.byref(err))
+
+    assert chunk(None, 8, 1, 4, 8, 3, 64, 16) == L.RT_ERR_HEAD_COUNT_MISMATCH
+    assert chunk(None, 8, 1, 4, 8, 2, 0, 16) == L.RT_ERR_ZERO_DIM
+    assert chunk(None, 3, 1, 4, 8, 2, 64, 16) == L.RT_ERR_KV_OVERFLOW   # fewer keys than new positions
+    assert chunk(None, 17, 1, 4, 8, 2, 64, 16) == L.RT_ERR_KV_OVERFLOW  # more keys than the cache holds
+    assert chunk(None, 8, 1, 4, 8, 2, 20, 16) == L.RT_ERR_UNSUPPORTED
+    assert chunk(None, 8, 1, 4, 8, 2, 64, 16, q=p + 2) == L.RT_ERR_UNSUPPORTED
+    assert chunk(None, 8, 1, 0, 8, 2, 64, 16) == L.RT_OK  # no new position: nothing to do
+    assert chunk(None, 8, 1, 4, 8, 2, 64, 16, q=None) == L.RT_ERR_NULL_POINTER
+
+    def noalloc(batch, hq, hkv, d, max_seq, lens=p, q=p):
+        return lib.rt_gqa_decode_batched_bf16_noalloc(None, q, p, p, p, lens, batch, hq, hkv, d, max_seq, C.byref(err))
+
+    assert noalloc(2, 8, 3, 128, 16) == L.RT_ERR_HEAD_COUNT_MISMATCH
+    assert noalloc(2, 8, 2, 0, 16) == L.RT_ERR_ZERO_DIM
+    assert noalloc(2, 8, 2, 128, 16, lens=None) == L.RT_ERR_NULL_POINTER
+    assert noalloc(0, 8, 2, 128, 16) == L.RT_OK
