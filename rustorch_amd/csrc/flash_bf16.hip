@@ -407,25 +407,31 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
                 for (int i = 0; i < 16; i++) acc_o[t][i] *= alpha;
         }
     };
-    // p = exp2(s*c - m*c), row-sum share, and the two B operands of the item
+    // p = exp2(s*c - m*c), the two B operands of the item, and the row-sum share, taken from the ROUNDED values with
+    // v_dot2_f32_bf16 against ones: the weights that are summed are the weights the second product applies, and
+    // eight instructions do what sixteen additions did
     auto exp_item = [&]() {
         const float mc = ((m_run == neg_inf()) ? 0.0f : m_run) * c;
-        float part[4];
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c, -mc));
-            s[i] = e;
-            if (i < 4) part[i] = e;
-            else part[i & 3] += e;
-        }
-        l_run += (part[0] + part[1]) + (part[2] + part[3]);
+        for (int i = 0; i < 16; i++) s[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c, -mc));
+        const bf16x2_t ones = __builtin_bit_cast(bf16x2_t, 0x3f803f80u);
+        float part0 = 0.0f, part1 = 0.0f;
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             u32x4_t pb;
 #pragma unroll
-            for (int e = 0; e < 4; e++) pb[e] = cvt_pk_bf16(s[8 * u + 2 * e], s[8 * u + 2 * e + 1]);
+            for (int e = 0; e < 4; e++) {
+                // (the packed pair stays in a scalar: a bit cast of a vector ELEMENT to bf16x2 as the operand of the
+                // dot instruction has been seen to read the wrong element)
+                const f32x2_t pair = {s[8 * u + 2 * e], s[8 * u + 2 * e + 1]};
+                const bf16x2_t w = __builtin_convertvector(pair, bf16x2_t);  // v_cvt_pk_bf16_f32, RNE
+                pb[e] = __builtin_bit_cast(uint32_t, w);
+                if (e & 1) part1 = __builtin_amdgcn_fdot2_f32_bf16(w, ones, part1, false);
+                else part0 = __builtin_amdgcn_fdot2_f32_bf16(w, ones, part0, false);
+            }
             pB[u] = __builtin_bit_cast(bf16x8_t, pb);
         }
+        l_run += part0 + part1;
     };
     // one barrier per cluster; nothing may be scheduled across it
     auto cluster_barrier = [&]() {

@@ -84,7 +84,7 @@ __device__ __forceinline__ int t_wave_min_i(int x) {
 
 template <int DP>
 struct TileCfg {
-    static constexpr int KT = (DP <= 64 || DP > 128) ? 32 : 64;  // keys per LDS tile
+    static constexpr int KT = DP <= 128 ? 64 : 32;  // keys per LDS tile
     // wave groups: group g takes the g-th share of every tile's 32-key items.  Two groups (eight waves) where the
     // registers allow two such workgroups per CU: the walk over the keys of a query tile is then half as long,
     // which is what a launch of many short sequences waits for at its end.
@@ -94,9 +94,9 @@ struct TileCfg {
     static constexpr int THREADS = 64 * NWAVES;
     static constexpr int LDK = DP + 8;                        // +16 B: 16 rows x 16 B tile all 64 banks
     static constexpr int LDV = DP + (DP % 64 == 0 ? 32 : 0);  // row pitch = 16 or 48 (mod 64) words: 4 rows x 64 B tile all banks
-    static constexpr int OCC = DP <= 64 ? 4 : (DP <= 128 ? 2 : 1);  // workgroups per CU the register budget is set for
+    static constexpr int OCC = DP <= 64 ? 3 : (DP <= 128 ? 2 : 1);  // workgroups per CU the register budget is set for
     static constexpr int DT = DP / 32;
-    static constexpr int PF = DP <= 64 ? 3 : 1;  // register sets of tiles in flight (wider rows take too many registers for more)
+    static constexpr int PF = DP <= 64 ? 2 : 1;  // register sets of tiles in flight (wider rows take too many registers for more)
     static constexpr int TILE_BYTES = 2 * KT * (LDK + LDV) * 2;           // two stages of K and V
     // one region per query-row wave: the partner group's (O, m, l) when the keys are split two ways, and the
     // staged output rows
@@ -309,113 +309,155 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, TileCfg<DP>::OCC) void flash_
 
         // one tile: this wave's item, then the next tile is parked from register set SET (= (t + 1) % PF) and the
         // set is refilled with tile t + 1 + PF
-        auto walk_tile = [&](int t, auto set_c) {
-            const int st = t & 1;
+        // ---- pieces of an item (32 keys against the wave's 32 query rows)
+        // bias values of an item: requested ahead of the matrix instructions that hide their latency
+        auto bias_fetch = [&](int k0, f32x4_t (&bv)[4]) {
 #pragma unroll
-            for (int it = 0; it < NI; it++) {
-            const int k0 = t * KT + 32 * (NI * grp + it);  // first key of the item
-            if (k0 <= wave_lim_max) {  // else every row of this wave has all of these keys hidden (wave-uniform)
-                // bias values of the item: requested ahead of the matrix instructions that hide their latency
-                f32x4_t bv[4];
-                if (BIAS) {
+            for (int j = 0; j < 4; j++) {
+                const int kb = k0 + 8 * j + 4 * hh;
+                f32x4_t x = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (valid) {
+                    if (p.bias_vec4 && kb + 3 < n_keys) {
+                        x = *(const f32x4_t*)(bias_row + kb);
+                    } else {
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const int kb = k0 + 8 * j + 4 * hh;
-                        f32x4_t x = {0.0f, 0.0f, 0.0f, 0.0f};
-                        if (valid) {
-                            if (p.bias_vec4 && kb + 3 < n_keys) {
-                                x = *(const f32x4_t*)(bias_row + kb);
-                            } else {
-#pragma unroll
-                                for (int e = 0; e < 4; e++)
-                                    if (kb + e < n_keys) x[e] = bias_row[kb + e];
-                            }
-                        }
-                        bv[j] = x;
+                        for (int e = 0; e < 4; e++)
+                            if (kb + e < n_keys) x[e] = bias_row[kb + e];
                     }
                 }
-                // ---- S^T = K . Q^T
-                f32x16_t s;
+                bv[j] = x;
+            }
+        };
+        auto k_operand = [&](int st, int it, int ks) {
+            return *(const bf16x8_t*)(Ks + st * KT * LDK + 32 * it * LDK + k_off + 16 * ks);
+        };
+        // bias (scores = (q . k) * scale + bias, crates/rustorch-nn/src/attention.rs:378-392, kept in the natural domain
+        // so that a bias of -1e4 weighs as it does in the reference), then the masks
+        auto mask_item = [&](int it, int k0, f32x16_t& sc, const f32x4_t (&bv)[4]) {
+            if (BIAS) {
 #pragma unroll
-                for (int i = 0; i < 16; i++) s[i] = 0.0f;
+                for (int i = 0; i < 16; i++) sc[i] = __builtin_fmaf(sc[i], p.scale, bv[i >> 2][i & 3]);
+            }
+            if (k0 + 31 > wave_lim_min) {
 #pragma unroll
-                for (int ks = 0; ks < KS; ks++) {
-                    const bf16x8_t a = *(const bf16x8_t*)(Ks + st * KT * LDK + 32 * it * LDK + k_off + 16 * ks);
-                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[ks], s, 0, 0, 0);
+                for (int i = 0; i < 16; i++) {
+                    const int kr = k0 + 8 * (i >> 2) + 4 * hh + (i & 3);
+                    sc[i] = (kr > lim) ? neg_inf() : sc[i];
                 }
-                if (BIAS) {
-                    // scores = (q . k) * scale + bias (crates/rustorch-nn/src/attention.rs:378-392), kept in the natural
-                    // domain so that a bias of -1e4 weighs as it does in the reference
-#pragma unroll
-                    for (int i = 0; i < 16; i++) s[i] = __builtin_fmaf(s[i], p.scale, bv[i >> 2][i & 3]);
-                }
-                // ---- mask
-                if (k0 + 31 > wave_lim_min) {
+            }
+            if (MODE == kMaskPadding) {
+                const uint32_t keep_word = (uint32_t)(keep_bits >> (32 * it));
+                if (keep_word != 0xffffffffu) {
+                    const uint32_t mine = keep_word >> (4 * hh);  // bit 8(i/4) + i%4 of `mine` is key 8(i/4) + 4hh + i%4
 #pragma unroll
                     for (int i = 0; i < 16; i++) {
-                        const int kr = k0 + 8 * (i >> 2) + 4 * hh + (i & 3);
-                        s[i] = (kr > lim) ? neg_inf() : s[i];
+                        const bool kept = (mine >> (8 * (i >> 2) + (i & 3))) & 1u;
+                        sc[i] = kept ? sc[i] : neg_inf();
                     }
                 }
-                if (MODE == kMaskPadding) {
-                    const uint32_t keep_word = (uint32_t)(keep_bits >> (32 * it));
-                    if (keep_word != 0xffffffffu) {
-                        const uint32_t mine = keep_word >> (4 * hh);  // bit 8(i/4) + i%4 of `mine` is key 8(i/4) + 4hh + i%4
-#pragma unroll
-                        for (int i = 0; i < 16; i++) {
-                            const bool kept = (mine >> (8 * (i >> 2) + (i & 3))) & 1u;
-                            s[i] = kept ? s[i] : neg_inf();
-                        }
-                    }
-                }
-                // ---- online softmax; the running max is raised lazily (only when some row's item max exceeds it by
-                // 2^8 in the exp2 domain), so the rescale of O leaves the steady state
-                const float m_item = t_max_with_other_half(t_max16(s));
-                if (__builtin_expect(__any(m_item > m_run + lazy), 0)) {
-                    const float m_new = t_vmax(m_run, m_item);
-                    const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
-                    const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * cc);  // m_run = -inf -> 0
-                    m_run = m_new;
-                    l_run *= alpha;
-#pragma unroll
-                    for (int tt = 0; tt < DT; tt++)
-#pragma unroll
-                        for (int i = 0; i < 16; i++) acc_o[tt][i] *= alpha;
-                }
-                const float mc = ((m_run == neg_inf()) ? 0.0f : m_run) * cc;
-#pragma unroll
-                for (int i = 0; i < 16; i++) s[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], cc, -mc));
-                // P as the two B operands of the item, and the row sum taken from the rounded values (the weights the
-                // second product applies are then exactly the ones that are summed): v_dot2_f32_bf16 against ones
-                bf16x8_t pB[2];
-                float part0 = 0.0f, part1 = 0.0f;
-                const bf16x2t ones = __builtin_bit_cast(bf16x2t, 0x3f803f80u);
-#pragma unroll
-                for (int u = 0; u < 2; u++) {
-                    u32x4_t pb;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const f32x2t pair = {s[8 * u + 2 * e], s[8 * u + 2 * e + 1]};
-                        const bf16x2t w = __builtin_convertvector(pair, bf16x2t);  // v_cvt_pk_bf16_f32, RNE
-                        pb[e] = __builtin_bit_cast(uint32_t, w);
-                        if (e & 1) part1 = __builtin_amdgcn_fdot2_f32_bf16(w, ones, part1, false);
-                        else part0 = __builtin_amdgcn_fdot2_f32_bf16(w, ones, part0, false);
-                    }
-                    pB[u] = __builtin_bit_cast(bf16x8_t, pb);
-                }
-                l_run += part0 + part1;
-                // ---- O^T += V^T . P^T: contraction slots 0-3 of a lane are keys 16u + 4hh + 0..3, slots 4-7 keys 16u + 8 + 4hh + 0..3
-#pragma unroll
-                for (int u = 0; u < 2; u++)
-#pragma unroll
-                    for (int dt = 0; dt < DT; dt++) {
-                        const uint16_t* vp = Vs + st * KT * LDV + (32 * it + 16 * u) * LDV + v_off + 32 * dt;
-                        const u32x2_t lo = t_lds_read_tr16(vp);
-                        const u32x2_t hi = t_lds_read_tr16(vp + 8 * LDV);
-                        const u32x4_t av = {lo[0], lo[1], hi[0], hi[1]};
-                        acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), pB[u], acc_o[dt], 0, 0, 0);
-                    }
             }
+        };
+        // the running max is raised lazily (only when some row's new max exceeds it by 2^8 in the exp2 domain), so the
+        // rescale of O leaves the steady state; returns m * cc for the exponentials
+        auto raise_max = [&](float m_item) {
+            if (__builtin_expect(__any(m_item > m_run + lazy), 0)) {
+                const float m_new = t_vmax(m_run, m_item);
+                const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+                const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * cc);  // m_run = -inf -> 0
+                m_run = m_new;
+                l_run *= alpha;
+#pragma unroll
+                for (int tt = 0; tt < DT; tt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) acc_o[tt][i] *= alpha;
+            }
+            return ((m_run == neg_inf()) ? 0.0f : m_run) * cc;
+        };
+        // p = exp2(s * cc - mc) in place, P as the two B operands of the item, and the row sum taken from the rounded
+        // values (the weights the second product applies are then exactly the ones that are summed): v_dot2_f32_bf16
+        // against ones.  (The packed pair stays in a scalar: a bit cast of a vector ELEMENT to bf16x2 as the operand of
+        // the dot instruction has been seen to read the wrong element.)
+        auto exp_item = [&](f32x16_t& sc, float mc, bf16x8_t (&pB)[2]) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) sc[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], cc, -mc));
+            float part0 = 0.0f, part1 = 0.0f;
+            const bf16x2t ones = __builtin_bit_cast(bf16x2t, 0x3f803f80u);
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                u32x4_t pb;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const f32x2t pair = {sc[8 * u + 2 * e], sc[8 * u + 2 * e + 1]};
+                    const bf16x2t w = __builtin_convertvector(pair, bf16x2t);  // v_cvt_pk_bf16_f32, RNE
+                    pb[e] = __builtin_bit_cast(uint32_t, w);
+                    if (e & 1) part1 = __builtin_amdgcn_fdot2_f32_bf16(w, ones, part1, false);
+                    else part0 = __builtin_amdgcn_fdot2_f32_bf16(w, ones, part0, false);
+                }
+                pB[u] = __builtin_bit_cast(bf16x8_t, pb);
+            }
+            l_run += part0 + part1;
+        };
+        // O^T += V^T . P^T: contraction slots 0-3 of a lane are keys 16u + 4hh + 0..3, slots 4-7 keys 16u + 8 + 4hh + 0..3
+        auto pv_item = [&](int st, int it, const bf16x8_t (&pB)[2]) {
+#pragma unroll
+            for (int u = 0; u < 2; u++)
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++) {
+                    const uint16_t* vp = Vs + st * KT * LDV + (32 * it + 16 * u) * LDV + v_off + 32 * dt;
+                    const u32x2_t lo = t_lds_read_tr16(vp);
+                    const u32x2_t hi = t_lds_read_tr16(vp + 8 * LDV);
+                    const u32x4_t av = {lo[0], lo[1], hi[0], hi[1]};
+                    acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), pB[u], acc_o[dt], 0, 0, 0);
+                }
+        };
+        auto one_item = [&](int st, int it, int k0) {
+            f32x4_t bv[4];
+            if (BIAS) bias_fetch(k0, bv);
+            f32x16_t sc;
+#pragma unroll
+            for (int i = 0; i < 16; i++) sc[i] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_operand(st, it, ks), qreg[ks], sc, 0, 0, 0);
+            mask_item(it, k0, sc, bv);
+            const float mc = raise_max(t_max_with_other_half(t_max16(sc)));
+            bf16x8_t pB[2];
+            exp_item(sc, mc, pB);
+            pv_item(st, it, pB);
+        };
+        // Two items of a tile as one: their score products are two independent chains of matrix instructions, issued
+        // alternately (a chain on one accumulator waits for itself), and one softmax step covers the 64 keys -- one max,
+        // one rescale test.  Without it a wave alone on its SIMD spends most of a tile waiting on its own latencies,
+        // which is what the last, long query tiles of a launch do.
+        auto two_items = [&](int st, int k0) {
+            f32x16_t s0, s1;
+#pragma unroll
+            for (int i = 0; i < 16; i++) s0[i] = s1[i] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_operand(st, 0, ks), qreg[ks], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_operand(st, 1, ks), qreg[ks], s1, 0, 0, 0);
+            }
+            const f32x4_t no_bias[4] = {};
+            mask_item(0, k0, s0, no_bias);
+            mask_item(1, k0 + 32, s1, no_bias);
+            const float mc = raise_max(t_max_with_other_half(t_vmax(t_max16(s0), t_max16(s1))));
+            bf16x8_t pA[2], pC[2];
+            exp_item(s0, mc, pA);
+            exp_item(s1, mc, pC);
+            pv_item(st, 0, pA);
+            pv_item(st, 1, pC);
+        };
+
+        auto walk_tile = [&](int t, auto set_c) {
+            const int st = t & 1;
+            const int k0 = t * KT + 32 * NI * grp;  // first key of this wave's items
+            if (NI == 2 && !BIAS && DP <= 64 && k0 + 32 <= wave_lim_max) {
+                two_items(st, k0);
+            } else {
+#pragma unroll
+                for (int it = 0; it < NI; it++)
+                    // else every row of this wave has all of these keys hidden (wave-uniform)
+                    if (k0 + 32 * it <= wave_lim_max) one_item(st, it, k0 + 32 * it);
             }
             // ---- the next tile: its registers have been in flight during the last PF tiles' work
             if (t + 1 < n_tiles) {
