@@ -687,6 +687,7 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
     const PrefillKernel forced = prefill_kernel_override();
     if (forced == PrefillKernel::kTile) persistent = false;
     if (forced == PrefillKernel::kPersistent && persistent_dim) persistent = true;
+    if (mask == rt::kMaskPadding && shape->seq > (uint64_t)rt::kFlashBf16MaxPaddingKeys) persistent = false;
     if (persistent) {  // that kernel addresses the rows of one (batch, head) slab with 32-bit byte offsets
         const uint64_t pitch_b = (bnhd ? shape->heads : 1) * shape->dim * 2;
         if (shape->seq * pitch_b >= (1ull << 32)) persistent = false;

@@ -181,11 +181,12 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
 
     bool poison = false;  // a padding mask hiding the reference's whole first key tile: every row NaN
     // The keep vector as one bit per key, a word per 32-key item, built once per workgroup (masks of up to
-    // kKeepWords * 32 keys; longer ones are read byte by byte where they are applied).  A word of ones is the
-    // common case -- padding sits at the tail -- and costs the softmax cluster nothing.
-    constexpr int kKeepWords = 2048;
+    // kFlashBf16MaxPaddingKeys keys; the launcher refuses longer ones, which go to the tile kernel).  A word of ones
+    // is the common case -- padding sits at the tail -- and costs the softmax cluster nothing.
+    constexpr int kKeepWords = kFlashBf16MaxPaddingKeys / 32;
     __shared__ uint32_t keep_bits[MODE == kMaskPadding ? kKeepWords : 1];
-    const bool keep_in_lds = (MODE == kMaskPadding) && (N <= 32 * kKeepWords);
+    // (the launcher sends longer padding masks to the tile kernel, so the bits are always in LDS here)
+    constexpr bool keep_in_lds = (MODE == kMaskPadding);
     if (MODE == kMaskPadding) {
         int lim = p.ref_bc < N ? p.ref_bc : N;
         bool any = false;
@@ -376,7 +377,6 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             int kr = kv_base + 8 * (i >> 2) + 4 * hh + (i & 3);
             bool masked = kr >= n_keys;
             if (kCausal) masked |= kr > q_row;
-            if (MODE == kMaskPadding) masked |= (kr < N) && (p.keep[kr] == 0);
             s[i] = masked ? neg_inf() : s[i];
         }
     };
@@ -640,6 +640,7 @@ hipError_t launch_hd(hipStream_t stream, const FlashBf16Params& p, dim3 grid, di
 
 hipError_t launch_flash_bf16(hipStream_t stream, const FlashBf16Params& p) {
     if (p.batch == 0 || p.heads == 0 || p.seq == 0) return hipSuccess;
+    if (p.mask == kMaskPadding && p.seq > kFlashBf16MaxPaddingKeys) return hipErrorInvalidValue;
     int n_qtiles = (p.seq + BR - 1) / BR;
     size_t n_jobs = (size_t)n_qtiles * p.batch * p.heads;
     size_t workers = p.n_workers > 0 ? (size_t)p.n_workers : 256;

@@ -89,7 +89,8 @@ struct FlashBf16Params {
     int n_workers;      // persistent workgroups to launch: the number of CUs
     TensorLayout lq, lkv, lo;  // layouts of q, of k and v, of out; seq * row_pitch * 2 bytes must stay below 2^32
 };
-// dim in {64, 128}.
+// dim in {64, 128}; a padding mask (kMaskPadding) of at most kFlashBf16MaxPaddingKeys keys.
+constexpr int kFlashBf16MaxPaddingKeys = 65536;
 hipError_t launch_flash_bf16(hipStream_t stream, const FlashBf16Params& p);
 
 // The general bf16 forward (flash_bf16_tile.hip): any dim <= 256 that is a multiple of 8, own key count, per-sequence

@@ -269,3 +269,21 @@ def test_two_launches_give_the_same_bits(force_kernel, kernel, d):
             ra.synchronize()
             outs.append(dout.download(np.uint16))
         assert all(np.array_equal(outs[0], o) for o in outs[1:])
+
+
+def test_padding_mask_longer_than_the_persistent_kernel_holds(oracle):
+    """A key-padding vector of more than 65536 keys: the persistent kernel keeps the mask as bits in LDS and stops
+    there, so the call goes to the tile kernel whatever the head dim.  Sampled rows are checked through the reference's
+    single-row attention over the kept keys (a padding mask hides the same keys from every query)."""
+    b, h, n, d = 1, 1, 66000, 64
+    (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d), (91, 92, 93))
+    keep = np.ones(n, bool)
+    keep[500:40000] = False
+    keep[65990:] = False
+    got = flash_bf16(ra.AttentionShape.new(b, h, n, d), qb, kb, vb, ra.Mask.padding(keep)).reshape(n, d)
+    assert np.isfinite(got).all()
+    k2, v2 = kf.reshape(n, d)[keep], vf.reshape(n, d)[keep]
+    q2 = qf.reshape(n, d)
+    for i in (0, 1, 499, 500, 39999, 40000, 65535, 65536, 65999):
+        want = oracle.gqa_forward_f32(q2[i], k2, v2, 1, 1, 1, 1, k2.shape[0], d)
+        assert max_abs(got[i], want) <= TOL, i
