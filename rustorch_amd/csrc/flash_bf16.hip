@@ -21,22 +21,30 @@
 // Schedule.  A wave can start one instruction every four to five cycles whatever its kind, and a
 // matrix instruction keeps the matrix pipe busy for 32 cycles, so a wave that only multiplies leaves
 // most issue slots free while a wave that only does softmax needs all of them.  The two waves of a SIMD
-// therefore alternate, one cluster apart, with one workgroup barrier per cluster:
+// therefore alternate, one cluster apart:
 //
 //   C(k): S^T(k) = K(k).Q^T and O^T += V(k-1)^T.P(k-1)^T (16 matrix instructions, operands in registers),
-//         with the LDS reads of the NEXT cluster's operands (V(k), K(k+1)) and the global->LDS requests
-//         of the next tile slotted in between;
-//   S(k): row max, rescale check, P(k) = exp2(..), row sums, conversion to bf16: vector work only.
+//         with the LDS reads of the NEXT cluster's operands (V(k), K(k+1)) slotted in between and the
+//         global->LDS requests of the next tile behind them;
+//   S(k): P(k) = exp2(..), row sums, conversion to bf16, overflow check: vector work only.
 //
-// Waves 0-3 run C(k) while waves 4-7 run S(k-1), then they swap.
+// Waves 0-3 run C(k) while waves 4-7 run S(k-1), then they swap.  The alternation is not enforced cluster
+// by cluster: the matrix pipe is the shared resource, a wave in its matrix cluster runs at raised priority
+// (waves 0-3 above waves 4-7, which settles the tie at the start of a job), and a wave whose partner holds
+// the pipe gets the gaps.  The workgroup meets at two barriers per step only, the two the LDS tile needs:
+// "the next tile has landed" before its first read (the matrix cluster of item 3) and "this tile has been
+// read" before the requests that overwrite it (item 0 of the next step).  Waves 0-3 pass them behind their
+// softmax clusters of items 2 and 3, waves 4-7 behind their matrix clusters of the same items, which also
+// puts the two groups one cluster apart again twice per step.
 //
 // LDS tiles are unpadded; bank conflicts are avoided by an XOR swizzle of the 16-byte slots of a row,
 // applied on the global side of the load (lane l of a load instruction always lands at LDS byte 16*l
 // of its 1 KB block, so it fetches the slot that belongs there).
 //
-// The running max is only raised (and O, l rescaled) when some row's item max exceeds it by more
-// than 2^8 in the exp2 domain: P then stays below 2^8, harmless in f32/bf16, and the rescale of the
-// 64 O registers leaves the steady-state loop.
+// The steady-state softmax takes no row max at all: P is formed against the running max as it stands (a
+// stale max scales a row's P, O and l by one common factor), and the lane's share of the row sum, which is
+// needed anyway, bounds every P of the lane.  Only when a share passes 2^16, or is not a number, or the row
+// has no max yet, does the wave compute the item max, rescale O and l and redo P from the scores.
 #include "rt_common.hpp"
 #include "rt_kernels.hpp"
 
@@ -51,7 +59,7 @@ constexpr int NTHREADS = 64 * NWAVES;
 constexpr int BR = 32 * NWAVES;  // query rows per job
 constexpr int BC = 128;          // key rows per step (one barrier per step)
 constexpr int NITEMS = BC / 32;  // 32-key items per step
-constexpr float kLazyLog2 = 8.0f;
+constexpr float kTrigSum = 65536.0f;  // a lane's 16-key share of a row sum above this sends the wave to the slow path
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
@@ -145,6 +153,11 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     constexpr int KS = HD / 16;              // contraction steps of the score product
     constexpr int DT = HD / 32;              // 32-row tiles of O^T
     constexpr bool kCausal = (MODE == kMaskCausal) || (MODE == kMaskVarlenCausal);
+    // Two barriers per step (see the header) at head dim 128.  At head dim 64 a matrix cluster is half as long as a
+    // softmax cluster, the pipe is no longer what paces the waves, and the older scheme measures 2-3 % faster: a
+    // barrier behind every cluster, waves 4-7 held one cluster behind waves 0-3 by one extra barrier at either end
+    // of a job.
+    constexpr bool kLockstep = (HD == 64);
     static_assert(NLD >= 1 && NLD <= NITEMS && BC % (RPI * NWAVES) == 0, "tile load split");
 
     // [K stage 0][K stage 1][V stage 0][V stage 1]: with this order every operand read of the steady state
@@ -177,7 +190,6 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     // bytes between consecutive rows of a (batch, head) slab: ROWB when the slab is contiguous
     const uint32_t q_pitch_b = (uint32_t)p.lq.row_pitch * 2u, kv_pitch_b = (uint32_t)p.lkv.row_pitch * 2u;
     const uint32_t o_pitch_b = (uint32_t)p.lo.row_pitch * 2u;
-    const float lazy_raw = kLazyLog2 / c;  // the rescale threshold in raw-score units
 
     bool poison = false;  // a padding mask hiding the reference's whole first key tile: every row NaN
     // The keep vector as one bit per key, a word per 32-key item, built once per workgroup (masks of up to
@@ -213,6 +225,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     const int ld_row0 = wave * RPI + lane / SPR;
     const uint32_t ld_k0 = (uint32_t)(((lane % SPR) ^ swz_k(ld_row0)) * 16);  // byte offset inside a global row
     const uint32_t ld_v0 = (uint32_t)(((lane % SPR) ^ swz_v(ld_row0)) * 16);
+    const uint32_t ld_off_k = (uint32_t)ld_row0 * kv_pitch_b + ld_k0, ld_off_v = (uint32_t)ld_row0 * kv_pitch_b + ld_v0;
     // ---- per-lane bases of the operand reads.  The swizzles only permute address bits that the operand
     // index also occupies, so operand ks (dt) of a lane sits at base ^ 32*ks (base ^ 64*dt): one register
     // per matrix, one XOR per read.  The stage bit is toggled into the bases once per step; item and
@@ -238,6 +251,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     bf16x8_t qreg[KS];  // Q as B operand, in registers for the whole job
     f32x16_t acc_o[DT];
     float m_run, l_run;
+    float neg_mc;  // -m_run * c, or +inf while the row has no max yet
     // operands of the next matrix cluster, and the scores / probabilities that travel between clusters
     bf16x8_t a[KS];      // K(k)
     u32x4_t vreg[2][DT]; // V(k-1): [16-key half][32-row tile of O^T]
@@ -252,6 +266,15 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
     auto load_part = [&](int n, int kv0, int st) {
         const uint32_t kdst = lds_base + (uint32_t)(st * TILE_B + (wave + NWAVES * n) * 1024);
+        // A tile that lies wholly inside the keys (every tile but a ragged last one) needs no per-lane arithmetic:
+        // the rows of instruction n start at a wave-uniform offset, which goes into the scalar base, and the lane's
+        // own offset is a constant of the kernel.
+        if (__builtin_expect(kv0 + BC <= n_keys, 1)) {
+            const size_t blk = (size_t)((uint32_t)(kv0 + NWAVES * RPI * n) * kv_pitch_b);
+            load_to_lds(Kg + blk, ld_off_k, kdst);
+            load_to_lds(Vg + blk, ld_off_v, kdst + 2 * TILE_B);
+            return;
+        }
         int r = kv0 + ld_row0 + NWAVES * RPI * n;
         asm volatile("" : "+v"(r));  // recompute per call: hoisted copies of these offsets only cost registers
         r = min(r, n_keys - 1);
@@ -361,7 +384,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         u32x2_t hi = lds_read_tr16(ptr + 8 * ROWB);
         vreg[u][dt] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
     };
-    auto mfma_qk = [&](int ks) { s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], qreg[ks], s, 0, 0, 0); };
+    auto mfma_qk = [&](int ks) {
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], qreg[ks], s, 0, 0, 0); };
     auto mfma_pv = [&](int j) {
         const int u = j / DT, dt = j % DT;
         acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vreg[u][dt]), pB[u],
@@ -392,66 +416,121 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             s[i] = __uint_as_float(x);
         }
     };
-    // raise the running max when it pays (wave-uniform branch)
-    auto update_max = [&]() {
-        float m_item = max_with_other_half(max16(s));
-        if (__builtin_expect(__any(m_item > m_run + lazy_raw), 0)) {
-            float m_new = vmax(m_run, m_item);
-            float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
-            float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);  // m_run = -inf -> 0
+    // The softmax of one item.  Fast path: P = exp2(s*c - m*c) with the running max AS IT STANDS, rounded to
+    // bf16 (the two B operands of the item), and the lane's share of the row sum.  No row max is taken: a stale
+    // max only scales a row's P, O and l by one common factor, which is harmless until it overflows, and the
+    // share of the row sum that falls out anyway bounds every P of the lane from above.  Only when some lane's
+    // share is above kTrigSum -- or is NaN, or the row has no max yet (neg_mc = +inf makes the share inf or
+    // NaN) -- does the wave take the slow path: the true item max, the rescale of O and l, and P again from
+    // the scores, which are still in their registers.
+    auto exp_with = [&](float nmc, float& part) {
+        float part0 = 0.0f, part1 = 0.0f;
+        // Issue order is fixed by hand, eight scores at a time: the exponent arguments, then the exponentials, then the
+        // sums and conversions, so that no instruction reads the result of the one or two before it (a dependent
+        // instruction waits out the producer's latency, and v_exp_f32's is long).  The empty assembly statements are
+        // what holds the order: each takes the values of a stage as read-write arguments, so the stage before it
+        // cannot sink below and the one after cannot rise.
+        float t[8];
+        uint32_t w[8];
+        auto pin8 = [&]() {
+            asm volatile("" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]), "+v"(t[7]));
+        };
+        auto args = [&](int u) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) t[i] = __builtin_fmaf(s[8 * u + i], c, nmc);
+            pin8();
+        };
+        auto exps = [&]() {
+#pragma unroll
+            for (int i = 0; i < 8; i++) t[i] = __builtin_amdgcn_exp2f(t[i]);
+            pin8();
+        };
+        auto convert = [&](int u) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) w[4 * u + e] = cvt_pk_bf16(t[2 * e], t[2 * e + 1]);
+            asm volatile("" : "+v"(w[4 * u]), "+v"(w[4 * u + 1]), "+v"(w[4 * u + 2]), "+v"(w[4 * u + 3]));
+        };
+        // The lane's share of the row sum is added up with plain v_add_f32 in two chains.  (v_dot2c_f32_bf16 against
+        // ones would sum the rounded values in half the instructions, but it runs on the matrix pipe: while the
+        // SIMD's other wave is in its matrix cluster each one waits for a gap there, and eight of them cost
+        // more than the sixteen additions.)
+        auto sum8 = [&]() {
+#pragma unroll
+            for (int i = 0; i < 8; i += 2) {
+                part0 += t[i];
+                part1 += t[i + 1];
+            }
+        };
+        args(0);
+        exps();
+        sum8();
+        convert(0);
+        asm volatile("" : "+v"(part0), "+v"(part1));
+        args(1);
+        exps();
+        sum8();
+        convert(1);
+        pB[0] = __builtin_bit_cast(bf16x8_t, u32x4_t{w[0], w[1], w[2], w[3]});
+        pB[1] = __builtin_bit_cast(bf16x8_t, u32x4_t{w[4], w[5], w[6], w[7]});
+        part = part0 + part1;
+    };
+    auto softmax_item = [&]() {
+        float part;
+        exp_with(neg_mc, part);
+        if (__builtin_expect(__any(!(part <= kTrigSum)), 0)) {
+            const float m_item = max_with_other_half(max16(s));
+            const float m_new = vmax(m_run, m_item);
+            const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);  // m_run = -inf -> 0
             m_run = m_new;
             l_run *= alpha;
 #pragma unroll
             for (int t = 0; t < DT; t++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) acc_o[t][i] *= alpha;
+            const float mc = m_use * c;
+            // a row that has seen no key yet keeps taking this path (and gets P = 0 from it: exp2(-inf - 0))
+            neg_mc = (m_new == neg_inf()) ? __uint_as_float(0x7f800000u) : -mc;
+            exp_with(-mc, part);
         }
+        l_run += part;
     };
-    // p = exp2(s*c - m*c), the two B operands of the item, and the row-sum share, taken from the ROUNDED values with
-    // v_dot2_f32_bf16 against ones: the weights that are summed are the weights the second product applies, and
-    // eight instructions do what sixteen additions did
-    auto exp_item = [&]() {
-        const float mc = ((m_run == neg_inf()) ? 0.0f : m_run) * c;
-#pragma unroll
-        for (int i = 0; i < 16; i++) s[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c, -mc));
-        const bf16x2_t ones = __builtin_bit_cast(bf16x2_t, 0x3f803f80u);
-        float part0 = 0.0f, part1 = 0.0f;
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-            u32x4_t pb;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                // (the packed pair stays in a scalar: a bit cast of a vector ELEMENT to bf16x2 as the operand of the
-                // dot instruction has been seen to read the wrong element)
-                const f32x2_t pair = {s[8 * u + 2 * e], s[8 * u + 2 * e + 1]};
-                const bf16x2_t w = __builtin_convertvector(pair, bf16x2_t);  // v_cvt_pk_bf16_f32, RNE
-                pb[e] = __builtin_bit_cast(uint32_t, w);
-                if (e & 1) part1 = __builtin_amdgcn_fdot2_f32_bf16(w, ones, part1, false);
-                else part0 = __builtin_amdgcn_fdot2_f32_bf16(w, ones, part0, false);
-            }
-            pB[u] = __builtin_bit_cast(bf16x8_t, pb);
-        }
-        l_run += part0 + part1;
-    };
-    // one barrier per cluster; nothing may be scheduled across it
+    // a workgroup barrier that nothing may be scheduled across
     auto cluster_barrier = [&]() {
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // The end of cluster C (after_c) or S of item i: nothing is scheduled across it.  Of the step's two workgroup
+    // barriers the first publishes this wave's share of the next tile (vmcnt(0) before it).
+    auto cluster_edge = [&](bool after_c, int i) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (kLockstep) {
+            if (after_c && i == 2) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share has landed
+            __builtin_amdgcn_s_barrier();
+        } else if (i >= 2 && (grp == 1) == after_c) {
+            if (i == 2) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+            __builtin_amdgcn_s_barrier();
+        }
         __builtin_amdgcn_sched_barrier(0);
     };
     static_assert(KS == 2 * DT, "one P.V matrix instruction per score matrix instruction");
 
     // One step = one 128-key tile = four items, each a C cluster and an S cluster.  A wave runs every item of
     // a step it takes part in (an item hidden from all of its rows by the causal mask is scored, masked to
-    // -inf and contributes exact zeros): all eight waves then meet the same barriers.  The one exception is
-    // taken a whole step at a time, in the job loop: a last key tile that lies wholly past a wave's rows.
+    // -inf and contributes exact zeros): the two waves of a SIMD then stay one cluster apart.  The one exception
+    // is taken a whole step at a time, in the job loop: a last key tile that lies wholly past a wave's rows.
+    // Barriers: waves 4-7 behind C of items 2 and 3, waves 0-3 behind S of the same items (see the header).
     auto run_item = [&](auto i_c, int kv0, int kv_next, int st, int mask_from) {
         constexpr int i = decltype(i_c)::value;
         constexpr int item_off = 32 * i * ROWB;
         // ---- C: the products, and right after each the read that refills its operand for the next C.
         // Score and P.V instructions alternate: a score instruction accumulates onto the one before it,
         // and back-to-back dependent matrix instructions would wait for each other.
-        __builtin_amdgcn_s_setprio(3);  // the multiplying wave goes first: its next instruction frees the matrix pipe
+        // the multiplying wave goes first (its next instruction frees the matrix pipe); when both waves of a SIMD
+        // multiply, waves 0-3 win and waves 4-7 fill the gaps
+        if (kLockstep || grp == 0) __builtin_amdgcn_s_setprio(3);
+        else __builtin_amdgcn_s_setprio(2);
         lds_operands_ready();
         __builtin_amdgcn_sched_barrier(0);  // no matrix instruction may be moved ahead of that wait
         zero_s();
@@ -467,7 +546,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             __builtin_amdgcn_sched_barrier(0);
         }
         // the next tile (or, with none left, this tile again: served from cache into the idle stage,
-        // which keeps the cluster free of branches): requested with items 0 and 1, awaited with item 2
+        // which keeps the cluster free of branches): requested with items 0 and 1, awaited at the first barrier
         if (NLD >= 2) {
             if (i < 2) {
 #pragma unroll
@@ -476,10 +555,9 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         } else if (i == 0) {
             load_part(0, kv_next, st ^ 1);
         }
-        if (i == 2) __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wave's share has landed
         if (i == NITEMS - 1) __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): stage st may be refilled
         __builtin_amdgcn_s_setprio(0);
-        cluster_barrier();
+        cluster_edge(true, i);
         // ---- S
         if (MODE == kMaskPadding) {
             if (keep_in_lds) {
@@ -491,13 +569,12 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         } else if (__builtin_expect(kv0 + 32 * i + 31 > mask_from, 0)) {
             mask_item(kv0 + 32 * i);
         }
-        update_max();
-        exp_item();
+        softmax_item();
         // P is only used by the next matrix cluster, and the compiler would sink the exponentials and
         // conversions that make it down to that use, past the barrier and in between the matrix
         // instructions; pinning the values here keeps the work in this cluster
         asm volatile("" : "+v"(pB[0]), "+v"(pB[1]), "+v"(l_run));
-        cluster_barrier();
+        cluster_edge(false, i);
     };
     auto run_step = [&](int kv0, int kv_next, int st, int mask_from) {
         static_assert(NITEMS == 4, "items per step");
@@ -518,6 +595,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
 #pragma unroll
             for (int i = 0; i < 16; i++) acc_o[t][i] = 0.0f;
         m_run = neg_inf();
+        neg_mc = __uint_as_float(0x7f800000u);
         l_run = 0.0f;
         // the first C of a job has no previous item: it multiplies zeros into O
 #pragma unroll
@@ -533,15 +611,16 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
 
         // an item needs masking when its last key lies past the last existing key or past the wave's first row
         const int mask_from = kCausal ? min(n_keys - 1, qw) : n_keys - 1;
-        if (grp == 1) cluster_barrier();  // the second group runs one cluster behind the first
+        if (kLockstep && grp == 1) cluster_barrier();  // the second group runs one cluster behind the first
         if (n_steps > 0) {
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) k_read_one(std::integral_constant<int, 0>{}, 0, ks);  // K(0)
         }
-        cluster_barrier();
+        if (kLockstep) cluster_barrier();
+        __builtin_amdgcn_sched_barrier(0);
         // With a causal mask the job's last key tile starts past the last row of the waves that own the upper
         // half of the query tile: for them every score of that step would be masked.  Such a wave finishes its
-        // last live item and then only keeps the barriers company for a step (no matrix, LDS or vector work: on a
+        // last live item and then only meets that step's two barriers (no matrix, LDS or vector work: on a
         // part whose clock is set by power the idle wave is worth more than its cycles).
         const bool dead_last = kCausal && n_steps > 0 && (n_steps - 1) * BC > qw + 31;
         const int n_run = n_steps - (dead_last ? 1 : 0);
@@ -558,7 +637,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         }
         if (dead_last) {
 #pragma unroll 1
-            for (int cl = 0; cl < 2 * NITEMS; cl++) cluster_barrier();
+            for (int cl = 0; cl < (kLockstep ? 2 * NITEMS : 2); cl++) cluster_barrier();
             k_base ^= (uint32_t)TILE_B;
             v_base ^= (uint32_t)TILE_B;
         }
@@ -566,8 +645,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
             k_base ^= (uint32_t)TILE_B;
             v_base ^= (uint32_t)TILE_B;
         }
-        cluster_barrier();
-        if (grp == 0) cluster_barrier();  // the first group waits for the second to finish
+        cluster_barrier();  // every wave has read its last operands: LDS is free for the output and the next job
+        if (kLockstep && grp == 0) cluster_barrier();  // (the first group waits for the second to finish)
 
         // ---- this job's output.  Stage 1 of LDS is free (the next job's first tile goes to stage 0): each
         // wave parks its 32 normalised rows there, swizzled, and streams them out as whole rows.

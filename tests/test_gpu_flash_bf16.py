@@ -65,6 +65,32 @@ def test_both_prefill_kernels_agree(oracle, force_kernel, n, d):
     assert max_abs(outs["persistent"], outs["tile"]) <= TOL
 
 
+@pytest.mark.parametrize("kernel,d", [("persistent", 64), ("persistent", 128), ("tile", 64), ("tile", 128)])
+def test_row_max_that_keeps_rising_along_the_keys(oracle, force_kernel, kernel, d):
+    """Scores that grow with the key index: a ramp that lifts the row max by tens of units from one 32-key item to
+    the next, one key hundreds of units above everything before it (an exponential taken against the old max
+    overflows f32), then keys far below the max.  Whatever rule a kernel uses to decide when to raise its running
+    max, the result is the plain softmax of the oracle."""
+    force_kernel(kernel)
+    b, h, n = 1, 2, 700
+    rng = np.random.default_rng(5)
+    u = np.full(d, 1.0 / np.sqrt(d), dtype=np.float32) * np.float32(d ** 0.25)  # (a u).(b u) / sqrt(d) = a b
+    a_row = rng.uniform(1.0, 3.0, size=(b, h, n, 1)).astype(np.float32)
+    prof = np.concatenate([np.linspace(-50.0, 50.0, 400), np.full(50, 20.0), [400.0], np.full(149, 100.0),
+                           np.full(100, -300.0)]).astype(np.float32)
+    assert prof.size == n
+    q = a_row * u + 0.3 * rng.standard_normal((b, h, n, d), dtype=np.float32)
+    k = prof[None, None, :, None] * u + 0.3 * rng.standard_normal((b, h, n, d), dtype=np.float32)
+    v = rng.standard_normal((b, h, n, d), dtype=np.float32)
+    (qb, qf), (kb, kf), (vb, vf) = bf16_round(q), bf16_round(k), bf16_round(v)
+    shape = ra.AttentionShape.new(b, h, n, d)
+    for mask, om in ((ra.Mask.causal(), "causal"), (ra.Mask.none(), None)):
+        got = flash_bf16(shape, qb, kb, vb, mask)
+        want = oracle.flash_forward_masked(oracle.AttentionShape(b, h, n, d), qf, kf, vf, om)
+        assert np.isfinite(want).all()
+        assert_close_nan(got, want, TOL, f"kernel={kernel} d={d} mask={mask.kind}")
+
+
 def test_flash_bf16_closed_forms():
     """N=1 => out == v exactly; causal row 0 == V[0] exactly; constant V => constant output."""
     d = 128
