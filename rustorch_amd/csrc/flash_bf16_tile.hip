@@ -31,7 +31,7 @@ namespace rt {
 namespace {
 
 constexpr int TROWS = 128;  // query rows per workgroup: four waves' worth, each wave 32
-constexpr float kTileLazyLog2 = 8.0f;
+constexpr float kTileTrigSum = 65536.0f;  // a lane's 16-key share of a row sum above this sends the wave to the slow path
 
 typedef short s16x4t __attribute__((ext_vector_type(4)));
 typedef float f32x2t __attribute__((ext_vector_type(2)));
@@ -71,52 +71,53 @@ __device__ __forceinline__ float t_max16(const f32x16_t& s) {
     t2 = t_max3(t2, s[13], s[14]);
     return __builtin_fmaxf(t_max3(t0, t1, t2), s[15]);
 }
-__device__ __forceinline__ int t_wave_max_i(int x) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) x = max(x, __shfl_xor(x, off, 64));
-    return x;
-}
-__device__ __forceinline__ int t_wave_min_i(int x) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) x = min(x, __shfl_xor(x, off, 64));
-    return x;
-}
 
 template <int DP>
 struct TileCfg {
     static constexpr int KT = DP <= 128 ? 64 : 32;  // keys per LDS tile
-    // wave groups: group g takes the g-th share of every tile's 32-key items.  Two groups (eight waves) where the
-    // registers allow two such workgroups per CU: the walk over the keys of a query tile is then half as long,
-    // which is what a launch of many short sequences waits for at its end.
-    static constexpr int NG = 1;
-    static constexpr int NI = KT / 32 / NG;                   // items a wave takes per tile
-    static constexpr int NWAVES = 4 * NG;
-    static constexpr int THREADS = 64 * NWAVES;
+    static constexpr int NI = KT / 32;              // 32-key items per tile
+    static constexpr int THREADS = 256;
     static constexpr int LDK = DP + 8;                        // +16 B: 16 rows x 16 B tile all 64 banks
     static constexpr int LDV = DP + (DP % 64 == 0 ? 32 : 0);  // row pitch = 16 or 48 (mod 64) words: 4 rows x 64 B tile all banks
     static constexpr int OCC = DP <= 64 ? 3 : (DP <= 128 ? 2 : 1);  // workgroups per CU the register budget is set for
     static constexpr int DT = DP / 32;
-    static constexpr int PF = DP <= 64 ? 2 : 1;  // register sets of tiles in flight (wider rows take too many registers for more)
+    static constexpr int PF = DP <= 32 ? 2 : 1;  // register sets of tiles in flight (wider rows take too many registers for more)
     static constexpr int TILE_BYTES = 2 * KT * (LDK + LDV) * 2;           // two stages of K and V
-    // one region per query-row wave: the partner group's (O, m, l) when the keys are split two ways, and the
-    // staged output rows
-    static constexpr int REGION = NG == 2 ? (4 * DT + 1) * 1024 : 32 * LDK * 2;
+    static constexpr int REGION = 32 * LDK * 2;                           // a wave's staged output rows
     static constexpr int LDS_BYTES = TILE_BYTES > 4 * REGION ? TILE_BYTES : 4 * REGION;
-    static_assert(REGION >= 32 * LDK * 2, "a region holds a wave's output rows");
 };
 
 // MODE: kMaskNone, kMaskCausal, kMaskPadding.  BIAS: an additive f32 score bias is applied (then MODE is kMaskNone).
-template <int DP, int MODE, bool BIAS>
-__global__ __launch_bounds__(TileCfg<DP>::THREADS, TileCfg<DP>::OCC) void flash_tile_bf16_kernel(FlashTileParams p) {
+// PACKED: query rows run over (position, head of the GQA group) (then MODE is kMaskCausal and there is no bias).
+// The grid is (heads or kv heads, batch, query tiles): no division stands between a workgroup and its first load.
+//
+// The key walk of a wave is a software pipeline over 32-key items, one step per item j:
+//
+//   S(j+1) = K(j+1).Q^T           KS matrix instructions   | both independent of the vector work, issued in between
+//   O^T   += V(j-1)^T.P(j-1)^T    2 DT matrix instructions | it so that the wave never waits on the matrix pipe
+//   P(j)   = softmax step on S(j)  ~60 vector instructions
+//
+// so a wave that is alone on its SIMD (the long query tiles at the end of a launch of short sequences) keeps the
+// matrix pipe and the vector pipe busy at once instead of running the three phases of an item back to back.
+// K therefore sits in LDS one tile ahead of V: during tile t the waves read K(t+1) and V(t-1), and after the
+// tile's one barrier (behind the step of its first item) K(t+2) and V(t+1) are parked over K(t) and V(t-1).
+template <int DP, int MODE, bool BIAS, bool PACKED>
+__global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : TileCfg<DP>::OCC) void flash_tile_bf16_kernel(FlashTileParams p) {
     using Cfg = TileCfg<DP>;
-    constexpr int KT = Cfg::KT, LDK = Cfg::LDK, LDV = Cfg::LDV, NG = Cfg::NG, NI = Cfg::NI, TTHREADS = Cfg::THREADS;
+    constexpr int KT = Cfg::KT, LDK = Cfg::LDK, LDV = Cfg::LDV, NI = Cfg::NI, TTHREADS = Cfg::THREADS;
     constexpr int KS = DP / 16;        // contraction steps of the score product
     constexpr int DT = DP / 32;        // 32-row tiles of O^T
+    constexpr int NM = 2 * KS;         // matrix instructions of a step: KS for S(j+1), 2 DT = KS for P(j-1).V(j-1)
     constexpr int CH = DP / 8;         // 16-byte chunks per (padded) row
     constexpr int CHUNKS = KT * CH;    // chunks of one matrix's tile
     constexpr int NL = (CHUNKS + TTHREADS - 1) / TTHREADS;  // chunks a thread moves per matrix per tile
     constexpr bool kCausal = MODE == kMaskCausal;
     constexpr int PF = Cfg::PF;        // register sets of tiles in flight behind the two LDS stages
+    static_assert(2 * DT == KS, "one P.V matrix instruction per score matrix instruction");
+    // Head dims above 128 do not have the registers for two score tiles and their operands in flight (O alone is 128
+    // registers), nor does head dim 128 with a bias (two items' bias values): there an item runs its three phases
+    // one after the other, and K is parked with V.
+    constexpr bool PIPE = DP <= 128 && !(BIAS && DP == 128);
 
     __shared__ __attribute__((aligned(16))) unsigned char lds[Cfg::LDS_BYTES];
     uint16_t* const Ks = (uint16_t*)lds;                      // [2][KT * LDK]
@@ -125,42 +126,26 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, TileCfg<DP>::OCC) void flash_
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int grp = wave >> 2;   // which share of a tile's items this wave takes
-    // which 32 query rows of the tile it owns.  Wave w runs on SIMD w % 4, and under a causal mask the rows at the
-    // end of a tile see more keys than those at its start: the assignment rotates from workgroup to workgroup so
-    // that no SIMD collects the long rows of every tile.
-    const int wq = (wave + (int)blockIdx.x) & 3;
     const int col = lane & 31, hh = lane >> 5;
 
-    // ---- which tile.  Workgroups are dealt round-robin to the 8 XCDs (each with its own L2): when the units
-    // ((batch, head) pairs, or (batch, kv head) when rows are packed) divide by 8, XCD x gets the units
-    // u = x (mod 8), so that all query tiles of a unit share K and V through one L2.  Within an XCD the tiles go
-    // out last query tile first: the longest causal rows of every unit, then the next longest, ... -- the
-    // dispatcher hands a free slot the next tile in that order, so the long ones start first and the short ones
-    // fill the gaps at the end.
-    const int G = p.pack;  // heads per packed row block (1: rows are positions of one head)
+    // ---- which tile.  The grid is (unit within the batch, batch, rank of the query tile), dispatched x first: all
+    // units' tiles of rank 0 (the last query tile, the longest causal rows), then rank 1, ... -- the dispatcher hands a
+    // free slot the next tile in that order, so the long ones start first and the short ones fill the gaps at the
+    // end.  Workgroups go round-robin to the 8 XCDs (each with its own L2) in the same order: when the units
+    // ((batch, head) pairs, or (batch, kv head) when rows are packed) divide by 8, all query tiles of a unit land on
+    // one XCD and share K and V through its L2.
+    const int G = PACKED ? p.pack : 1;  // heads per packed row block (1: rows are positions of one head)
     const int rows_total = p.seq_q * G;
-    const int n_qtiles = (rows_total + TROWS - 1) / TROWS;
-    const int heads_u = G > 1 ? p.kv_heads : p.heads;
-    const int n_units = p.batch * heads_u;
-    int unit, rank;
-    {
-        const int id = blockIdx.x;
-        if ((n_units & 7) == 0) {
-            const int x = id & 7, k = id >> 3;
-            const int upx = n_units >> 3;
-            rank = k / upx;
-            unit = (k - rank * upx) * 8 + x;
-        } else {
-            rank = id / n_units;
-            unit = id - rank * n_units;
-        }
-    }
-    const int qtile = n_qtiles - 1 - rank;
+    const int hx = blockIdx.x, b = blockIdx.y;
+    const int qtile = (int)gridDim.z - 1 - (int)blockIdx.z;
     const int q0 = qtile * TROWS;
-    const int b = unit / heads_u, hx = unit - b * heads_u;
-    const int kvh = G > 1 ? hx : hx / p.group;
-    const int h0 = G > 1 ? hx * G : hx;  // head of a row with g = 0
+    // kv head: hx itself when rows are packed, else hx / group (group_magic = 2^32 / group + 1, exact below 2^16 heads)
+    const int kvh = (PACKED || p.group_magic == 0) ? hx : (int)__umulhi((uint32_t)hx, p.group_magic);
+    const int h0 = PACKED ? hx * G : hx;  // head of a row with g = 0
+    // which 32 query rows of the tile a wave owns.  Wave w runs on SIMD w % 4, and under a causal mask the rows at
+    // the end of a tile see more keys than those at its start: the assignment rotates from workgroup to workgroup
+    // so that no SIMD collects the long rows of every tile.
+    const int wq = (wave + hx + b + (int)blockIdx.z) & 3;
 
     const int n_q = p.q_lens ? min(max(p.q_lens[b], 0), p.seq_q) : p.seq_q;          // valid query positions
     const int n_keys = p.kv_lens ? min(max(p.kv_lens[b], 0), p.seq_kv) : p.seq_kv;  // keys that exist
@@ -189,6 +174,87 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, TileCfg<DP>::OCC) void flash_
     const float cc = BIAS ? kLog2e : p.scale_log2e;  // exp2 argument per unit of score
 
     if (n_tiles > 0) {
+        const uint16_t* __restrict__ Kg = p.k + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+        const uint16_t* __restrict__ Vg = p.v + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+
+        // ---- tile movement: chunk c = tid + TTHREADS n of a tile is (row c / CH, 16-byte chunk c % CH).  A tile
+        // travels global -> registers -> LDS.  LDS holds two stages of each matrix; PF register sets per matrix hold
+        // the tiles behind them, so that a load has PF tile-times to arrive.
+        u32x4_t kreg[PF][NL], vreg[PF][NL];
+        uint32_t keep_raw[PF];
+#pragma unroll
+        for (int i = 0; i < PF; i++) {
+            keep_raw[i] = 1;
+#pragma unroll
+            for (int n = 0; n < NL; n++) kreg[i][n] = vreg[i][n] = u32x4_t{0u, 0u, 0u, 0u};
+        }
+        // per-thread constants of the movement (hoisted: the loop then spends a handful of instructions per tile on it)
+        int ld_row[NL];       // row of the tile this thread moves
+        uint32_t ld_col[NL];  // element offset inside a row; the same in K and V
+        uint32_t st_k[NL], st_v[NL];  // byte offsets of the chunk in an LDS stage
+        bool ld_on[NL];
+#pragma unroll
+        for (int n = 0; n < NL; n++) {
+            const int c = tid + TTHREADS * n;
+            const int row = c / CH, ch = c - row * CH;
+            ld_row[n] = row;
+            st_k[n] = (uint32_t)((row * LDK + 8 * ch) * 2);
+            st_v[n] = (uint32_t)((2 * KT * LDK + row * LDV + 8 * ch) * 2);
+            ld_on[n] = 8 * ch < D;
+            ld_col[n] = ld_on[n] ? (uint32_t)(8 * ch) : 0u;  // a chunk past the head dim is requested (from column 0) but never parked
+        }
+        static_assert(CHUNKS % TTHREADS == 0, "every thread moves NL chunks of every tile");
+        // Every request below is unconditional -- a tile index past the last tile is clamped to it, a chunk past the
+        // head dim reads column 0 -- and only the LDS write is predicated.  With no branch around a load the compiler
+        // counts the loads in flight exactly and waits at a park for the oldest register set only; with one it
+        // falls back to waiting for all of them, which empties the prefetch queue at every tile.
+        if (D < DP) {  // the columns that are never parked are zero in both stages
+            for (int i = tid; i < Cfg::TILE_BYTES / 16; i += TTHREADS) ((u32x4_t*)lds)[i] = u32x4_t{0u, 0u, 0u, 0u};
+            __syncthreads();
+        }
+        const int last_kv0 = (n_tiles - 1) * KT;
+        const uint32_t kv_pitch = (uint32_t)p.lkv.row_pitch;
+        // rows past the end re-read the last key; they are masked in the score tile
+        auto chunk_at = [&](int n, int kv0) __attribute__((always_inline)) { return (size_t)(uint32_t)min(kv0 + ld_row[n], n_keys - 1) * kv_pitch + ld_col[n]; };
+        auto issue_k = [&](u32x4_t (&dst)[NL], int kv0) __attribute__((always_inline)) {
+            kv0 = min(kv0, last_kv0);
+#pragma unroll
+            for (int n = 0; n < NL; n++) dst[n] = *(const u32x4_t*)(Kg + chunk_at(n, kv0));
+        };
+        auto issue_v = [&](auto set_c, int kv0) __attribute__((always_inline)) {
+            constexpr int SET = decltype(set_c)::value;
+            kv0 = min(kv0, last_kv0);
+#pragma unroll
+            for (int n = 0; n < NL; n++) vreg[SET][n] = *(const u32x4_t*)(Vg + chunk_at(n, kv0));
+            // key-padding vector of the tile: one byte per lane, turned into bits with a ballot when the tile is parked
+            if (MODE == kMaskPadding) {
+                const int j = kv0 + (lane & (KT - 1));
+                const uint32_t kb = p.keep[min(j, n_keys - 1)];
+                keep_raw[SET] = (j < n_keys) ? kb : 1u;  // keys past the end are masked by `lim`
+            }
+        };
+        auto park_k = [&](const u32x4_t (&src)[NL], int st) __attribute__((always_inline)) {
+#pragma unroll
+            for (int n = 0; n < NL; n++)
+                if (D == DP || ld_on[n]) *(u32x4_t*)(lds + st * (KT * LDK * 2) + st_k[n]) = src[n];
+        };
+        uint64_t keep_cur = ~0ull, keep_next = ~0ull;  // keep bits of the tile whose items are in their softmax step, and of the next
+        auto park_v = [&](auto set_c, int st) __attribute__((always_inline)) {
+            constexpr int SET = decltype(set_c)::value;
+#pragma unroll
+            for (int n = 0; n < NL; n++)
+                if (D == DP || ld_on[n]) *(u32x4_t*)(lds + st * (KT * LDV * 2) + st_v[n]) = vreg[SET][n];
+            if (MODE == kMaskPadding) keep_next = __ballot(keep_raw[SET] != 0);
+        };
+
+        // tiles 0 (K and V) and 1 (K) are requested before anything else of the set-up: their latency covers it
+        u32x4_t k1[NL];
+#pragma unroll
+        for (int n = 0; n < NL; n++) k1[n] = u32x4_t{0u, 0u, 0u, 0u};
+        issue_k(kreg[0], 0);
+        issue_v(std::integral_constant<int, 0>{}, 0);
+        if (PIPE) issue_k(k1, KT);
+
         // ---- this lane's query row
         const int r = q0 + 32 * wq + col;
         const int s_pos = G > 1 ? r / G : r;
@@ -198,12 +264,21 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, TileCfg<DP>::OCC) void flash_
         int lim = n_keys - 1;  // last key this row sees
         if (kCausal) lim = min(lim, s_pos + off);
         if (!valid) lim = -1;
-        const int wave_lim_max = __builtin_amdgcn_readfirstlane(t_wave_max_i(lim));  // scalar: the tests on them are wave-uniform
-        const int wave_lim_min = __builtin_amdgcn_readfirstlane(t_wave_min_i(lim));
+        // the largest and smallest `lim` of the wave, as scalars (the tests on them are wave-uniform): lim grows with
+        // the row, and the rows that are not valid are the last ones
+        int wave_lim_max, wave_lim_min;
+        {
+            const int r_first = q0 + 32 * wq, r_last = r_first + 31;
+            const int r_lim = min(rows_total, n_q * G);  // rows below it are valid
+            const int r_top = min(r_last, r_lim - 1);
+            const int s_top = G > 1 ? r_top / G : r_top, s_bot = G > 1 ? r_first / G : r_first;
+            wave_lim_max = r_first < r_lim ? (kCausal ? min(n_keys - 1, s_top + off) : n_keys - 1) : -1;
+            wave_lim_min = r_last < r_lim ? (kCausal ? min(n_keys - 1, s_bot + off) : n_keys - 1) : -1;
+        }
+        // items this wave walks: the ones that hold a key some row of it sees (a prefix of the workgroup's items)
+        const int n_it = wave_lim_max < 0 ? 0 : min(n_tiles * NI, (wave_lim_max >> 5) + 1);
 
         const size_t q_off = (size_t)b * p.lq.batch_stride + (size_t)(h0 + g) * p.lq.head_stride + (size_t)s_pos * p.lq.row_pitch;
-        const uint16_t* __restrict__ Kg = p.k + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
-        const uint16_t* __restrict__ Vg = p.v + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
 
         // Mask::Padding hiding the reference's whole first key tile: every row NaN (the tiled recurrence of
         // cpu_forward.rs:268-425 takes exp(-inf - (-inf)) on that tile and never recovers)
@@ -224,94 +299,38 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, TileCfg<DP>::OCC) void flash_
             qreg[ks] = __builtin_bit_cast(bf16x8_t, z);
         }
 
-        // ---- tile movement: chunk c = tid + TTHREADS n of a tile is (row c / CH, 16-byte chunk c % CH).  A tile
-        // travels global -> registers -> LDS.  LDS holds two stages; PF register sets hold the tiles behind them, so
-        // that a load has PF tile-times to arrive (a workgroup alone on its CU walks a tile in well under the
-        // memory latency, and a short sequence is exactly that case at the end of a launch).
-        u32x4_t kreg[PF][NL], vreg[PF][NL];
-        uint32_t keep_raw[PF];
-#pragma unroll
-        for (int i = 0; i < PF; i++) {
-            keep_raw[i] = 1;
-#pragma unroll
-            for (int n = 0; n < NL; n++) kreg[i][n] = vreg[i][n] = u32x4_t{0u, 0u, 0u, 0u};
-        }
-        // per-thread constants of the movement (hoisted: the loop then spends a handful of instructions per tile on it)
-        int ld_row[NL];       // row of the tile this thread moves
-        uint32_t ld_col[NL];  // element offset inside a row; the same in K and V
-        uint32_t st_k[NL], st_v[NL];  // byte offsets of the chunk in an LDS stage
-        bool ld_on[NL];
-#pragma unroll
-        for (int n = 0; n < NL; n++) {
-            const int c = tid + TTHREADS * n;
-            const int row = c / CH, ch = c - row * CH;
-            ld_row[n] = row;
-            ld_col[n] = (uint32_t)(8 * ch);
-            st_k[n] = (uint32_t)((row * LDK + 8 * ch) * 2);
-            st_v[n] = (uint32_t)((2 * KT * LDK + row * LDV + 8 * ch) * 2);
-            ld_on[n] = (CHUNKS % TTHREADS == 0 || c < CHUNKS) && 8 * ch < D;
-        }
-        const uint32_t kv_pitch = (uint32_t)p.lkv.row_pitch;
-        auto issue_loads = [&](auto set_c, int kv0) {
-            constexpr int SET = decltype(set_c)::value;
-#pragma unroll
-            for (int n = 0; n < NL; n++) {
-                const int key = min(kv0 + ld_row[n], n_keys - 1);  // rows past the end re-read the last key; masked below
-                if (ld_on[n]) {  // (the registers of chunks that are never loaded stay at their initial zero)
-                    const size_t e = (size_t)(uint32_t)key * kv_pitch + ld_col[n];
-                    kreg[SET][n] = *(const u32x4_t*)(Kg + e);
-                    vreg[SET][n] = *(const u32x4_t*)(Vg + e);
-                }
-            }
-            // key-padding vector of the tile: one byte per lane, turned into bits with a ballot when the tile is parked
-            if (MODE == kMaskPadding) {
-                const int j = kv0 + 32 * NI * grp + (lane & (32 * NI - 1));
-                keep_raw[SET] = (j < n_keys) ? p.keep[j] : 1u;  // keys past the end are masked by `lim`
-            }
-        };
-        uint64_t keep_bits = ~0ull;  // keep bits of this wave's items of the tile in LDS
-        auto park = [&](auto set_c, int st) {
-            constexpr int SET = decltype(set_c)::value;
-#pragma unroll
-            for (int n = 0; n < NL; n++) {
-                if (CHUNKS % TTHREADS == 0 || tid + TTHREADS * n < CHUNKS) {
-                    *(u32x4_t*)(lds + st * (KT * LDK * 2) + st_k[n]) = kreg[SET][n];
-                    *(u32x4_t*)(lds + st * (KT * LDV * 2) + st_v[n]) = vreg[SET][n];
-                }
-            }
-            if (MODE == kMaskPadding) keep_bits = __ballot(keep_raw[SET] != 0);
-        };
-
-        const float lazy = kTileLazyLog2 / cc;  // the rescale threshold in score units
-
         // per-lane LDS offsets (elements): K operand row `col`, slots 8 hh; V operand row (j >> 2) + 4 hh, columns 16 g16 + 4 (j & 3)
-        const int k_off = (32 * NI * grp + col) * LDK + 8 * hh;
-        const int v_off = (32 * NI * grp + ((lane & 15) >> 2) + 4 * hh) * LDV + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+        const int k_off = col * LDK + 8 * hh;
+        const int v_off = (((lane & 15) >> 2) + 4 * hh) * LDV + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
         // bias rows of this lane's query: f32 [seq_q, seq_kv] per (batch, head) or one for all
         const float* bias_row = nullptr;
         if (BIAS) bias_row = p.bias + ((size_t)b * p.heads + (h0 + g)) * (size_t)p.bias_bh_stride + (size_t)s_pos * (size_t)p.seq_kv;
 
-        // tile 0 goes straight to LDS; tiles 1 .. PF wait in the register sets (tile i in set i % PF)
-        issue_loads(std::integral_constant<int, 0>{}, 0);
-        park(std::integral_constant<int, 0>{}, 0);
+        // K(0), V(0) -> stage 0, K(1) -> stage 1; then the register sets take K(2) .. K(1 + PF) and V(1) .. V(PF)
+        // (K(j) travels in set j % PF, and so does V(j))
+        park_k(kreg[0], 0);
+        park_v(std::integral_constant<int, 0>{}, 0);
+        keep_cur = keep_next;
+        if (PIPE) park_k(k1, 1);
         {
-            auto prefetch = [&](auto i_c) {
-                constexpr int I = decltype(i_c)::value;
-                if (I < n_tiles) issue_loads(std::integral_constant<int, I % PF>{}, I * KT);
+            auto prefetch = [&](auto i_c) __attribute__((always_inline)) {
+                constexpr int I = decltype(i_c)::value;  // 0 .. PF - 1
+                constexpr int KA = PIPE ? 2 : 1;         // K runs a tile ahead of V in the pipelined walk only
+                issue_k(kreg[(KA + I) % PF], (KA + I) * KT);
+                issue_v(std::integral_constant<int, (1 + I) % PF>{}, (1 + I) * KT);
             };
-            prefetch(std::integral_constant<int, 1>{});
-            if (PF >= 2) prefetch(std::integral_constant<int, 2>{});
-            if (PF >= 3) prefetch(std::integral_constant<int, 3>{});
+            prefetch(std::integral_constant<int, 0>{});
+            if (PF >= 2) prefetch(std::integral_constant<int, 1>{});
+            if (PF >= 3) prefetch(std::integral_constant<int, 2>{});
             static_assert(PF <= 3, "prologue covers up to three sets");
         }
         __syncthreads();
 
-        // one tile: this wave's item, then the next tile is parked from register set SET (= (t + 1) % PF) and the
-        // set is refilled with tile t + 1 + PF
-        // ---- pieces of an item (32 keys against the wave's 32 query rows)
-        // bias values of an item: requested ahead of the matrix instructions that hide their latency
-        auto bias_fetch = [&](int k0, f32x4_t (&bv)[4]) {
+        // ---- pieces of a step
+        // bias values of an item (scores = (q . k) * scale + bias, crates/rustorch-nn/src/attention.rs:378-392, kept in
+        // the natural domain so that a bias of -1e4 weighs as it does in the reference): requested a step ahead
+        auto bias_fetch = [&](int k0, f32x4_t (&bv)[4]) __attribute__((always_inline)) {
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const int kb = k0 + 8 * j + 4 * hh;
@@ -328,12 +347,8 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, TileCfg<DP>::OCC) void flash_
                 bv[j] = x;
             }
         };
-        auto k_operand = [&](int st, int it, int ks) {
-            return *(const bf16x8_t*)(Ks + st * KT * LDK + 32 * it * LDK + k_off + 16 * ks);
-        };
-        // bias (scores = (q . k) * scale + bias, crates/rustorch-nn/src/attention.rs:378-392, kept in the natural domain
-        // so that a bias of -1e4 weighs as it does in the reference), then the masks
-        auto mask_item = [&](int it, int k0, f32x16_t& sc, const f32x4_t (&bv)[4]) {
+        // the bias, then the masks, on the scores of the item whose keys start at k0 (item `it` of its tile)
+        auto mask_item = [&](int it, int k0, f32x16_t& sc, const f32x4_t (&bv)[4]) __attribute__((always_inline)) {
             if (BIAS) {
 #pragma unroll
                 for (int i = 0; i < 16; i++) sc[i] = __builtin_fmaf(sc[i], p.scale, bv[i >> 2][i & 3]);
@@ -346,7 +361,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, TileCfg<DP>::OCC) void flash_
                 }
             }
             if (MODE == kMaskPadding) {
-                const uint32_t keep_word = (uint32_t)(keep_bits >> (32 * it));
+                const uint32_t keep_word = (uint32_t)(keep_cur >> (32 * it));
                 if (keep_word != 0xffffffffu) {
                     const uint32_t mine = keep_word >> (4 * hh);  // bit 8(i/4) + i%4 of `mine` is key 8(i/4) + 4hh + i%4
 #pragma unroll
@@ -357,155 +372,295 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, TileCfg<DP>::OCC) void flash_
                 }
             }
         };
-        // the running max is raised lazily (only when some row's new max exceeds it by 2^8 in the exp2 domain), so the
-        // rescale of O leaves the steady state; returns m * cc for the exponentials
-        auto raise_max = [&](float m_item) {
-            if (__builtin_expect(__any(m_item > m_run + lazy), 0)) {
-                const float m_new = t_vmax(m_run, m_item);
-                const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
-                const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * cc);  // m_run = -inf -> 0
-                m_run = m_new;
-                l_run *= alpha;
-#pragma unroll
-                for (int tt = 0; tt < DT; tt++)
-#pragma unroll
-                    for (int i = 0; i < 16; i++) acc_o[tt][i] *= alpha;
-            }
-            return ((m_run == neg_inf()) ? 0.0f : m_run) * cc;
+        // operand m of a step: even m = K rows of the next item (A operand of score instruction m / 2), odd m = V of
+        // the previous item (contraction slots 0-3 of a lane are keys 16u + 4hh + 0..3, slots 4-7 keys 16u + 8 + 4hh + 0..3)
+        auto load_op = [&](int m, const uint16_t* kp, const uint16_t* vp) __attribute__((always_inline)) {
+            if ((m & 1) == 0) return *(const u32x4_t*)(kp + 16 * (m >> 1));
+            const int i = m >> 1, u = i / DT, dt = i - u * DT;
+            const u32x2_t lo = t_lds_read_tr16(vp + 16 * u * LDV + 32 * dt);
+            const u32x2_t hi = t_lds_read_tr16(vp + 16 * u * LDV + 32 * dt + 8 * LDV);
+            return u32x4_t{lo[0], lo[1], hi[0], hi[1]};
         };
-        // p = exp2(s * cc - mc) in place, P as the two B operands of the item, and the row sum taken from the rounded
-        // values (the weights the second product applies are then exactly the ones that are summed): v_dot2_f32_bf16
-        // against ones.  (The packed pair stays in a scalar: a bit cast of a vector ELEMENT to bf16x2 as the operand of
-        // the dot instruction has been seen to read the wrong element.)
-        auto exp_item = [&](f32x16_t& sc, float mc, bf16x8_t (&pB)[2]) {
+        // An empty assembly statement that takes x as a read-write argument: whatever makes x stays above it, whatever
+        // uses x stays below.  A run of them is a fence for exactly the values named.
+        auto pin_f = [](float& x) __attribute__((always_inline)) { asm volatile("" : "+v"(x)); };
+        auto pin_u = [](uint32_t& x) __attribute__((always_inline)) { asm volatile("" : "+v"(x)); };
+        auto pin_b = [](bf16x8_t& x) __attribute__((always_inline)) { asm volatile("" : "+v"(x)); };
+
+        float neg_mc = valid ? __uint_as_float(0x7f800000u) : 0.0f;  // -m_run * cc; +inf while a valid row has no max yet
+        // The values that travel from step to step come in pairs: a step reads one of a pair and writes the other, and
+        // the next step has them the other way round, so nothing is copied.
+        f32x16_t s_a, s_b;        // S(j), made in step j - 1, and S(j + 1)
+        bf16x8_t p_a[2], p_b[2];  // P(j - 1) and P(j)
+        p_a[0] = p_a[1] = p_b[0] = p_b[1] = __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u});
+        f32x4_t bv_a[4] = {}, bv_b[4] = {};  // bias values of item j and of item j + 1
+
+        // S(0), before the pipeline starts
+        {
 #pragma unroll
-            for (int i = 0; i < 16; i++) sc[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], cc, -mc));
+            for (int i = 0; i < 16; i++) s_a[i] = s_b[i] = 0.0f;
+            if (BIAS) bias_fetch(0, bv_a);
+            if (PIPE && n_it > 0) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++)
+                    s_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)(Ks + k_off + 16 * ks), qreg[ks], s_a, 0, 0, 0);
+            }
+        }
+
+        // O^T += V(j-1)^T . P(j-1)^T alone: behind the wave's last item
+        auto drain = [&](const uint16_t* vp) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < KS; i++) {
+                const int u = i / DT, dt = i - u * DT;
+                const u32x4_t av = load_op(2 * i + 1, nullptr, vp);
+                acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), p_a[u], acc_o[dt], 0, 0, 0);
+            }
+        };
+        // P = exp2(s * cc + nmc) of the 16 scores a lane holds as the item's two B operands, and the lane's share of
+        // the row sum (plain additions: v_dot2c_f32_bf16 would halve their number but runs on the matrix pipe, where
+        // it queues behind the matrix instructions of every wave of the SIMD)
+        auto exp_plain = [&](const f32x16_t& sc, float nmc, uint32_t (&w)[8], float& part) __attribute__((always_inline)) {
             float part0 = 0.0f, part1 = 0.0f;
-            const bf16x2t ones = __builtin_bit_cast(bf16x2t, 0x3f803f80u);
 #pragma unroll
-            for (int u = 0; u < 2; u++) {
-                u32x4_t pb;
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const f32x2t pair = {sc[8 * u + 2 * e], sc[8 * u + 2 * e + 1]};
-                    const bf16x2t w = __builtin_convertvector(pair, bf16x2t);  // v_cvt_pk_bf16_f32, RNE
-                    pb[e] = __builtin_bit_cast(uint32_t, w);
-                    if (e & 1) part1 = __builtin_amdgcn_fdot2_f32_bf16(w, ones, part1, false);
-                    else part0 = __builtin_amdgcn_fdot2_f32_bf16(w, ones, part0, false);
-                }
-                pB[u] = __builtin_bit_cast(bf16x8_t, pb);
+            for (int e = 0; e < 8; e++) {
+                const float x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[2 * e], cc, nmc));
+                const float x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[2 * e + 1], cc, nmc));
+                part0 += x0;
+                part1 += x1;
+                w[e] = t_cvt_pk_bf16(x0, x1);
             }
-            l_run += part0 + part1;
-        };
-        // O^T += V^T . P^T: contraction slots 0-3 of a lane are keys 16u + 4hh + 0..3, slots 4-7 keys 16u + 8 + 4hh + 0..3
-        auto pv_item = [&](int st, int it, const bf16x8_t (&pB)[2]) {
-#pragma unroll
-            for (int u = 0; u < 2; u++)
-#pragma unroll
-                for (int dt = 0; dt < DT; dt++) {
-                    const uint16_t* vp = Vs + st * KT * LDV + (32 * it + 16 * u) * LDV + v_off + 32 * dt;
-                    const u32x2_t lo = t_lds_read_tr16(vp);
-                    const u32x2_t hi = t_lds_read_tr16(vp + 8 * LDV);
-                    const u32x4_t av = {lo[0], lo[1], hi[0], hi[1]};
-                    acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), pB[u], acc_o[dt], 0, 0, 0);
-                }
-        };
-        auto one_item = [&](int st, int it, int k0) {
-            f32x4_t bv[4];
-            if (BIAS) bias_fetch(k0, bv);
-            f32x16_t sc;
-#pragma unroll
-            for (int i = 0; i < 16; i++) sc[i] = 0.0f;
-#pragma unroll
-            for (int ks = 0; ks < KS; ks++) sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_operand(st, it, ks), qreg[ks], sc, 0, 0, 0);
-            mask_item(it, k0, sc, bv);
-            const float mc = raise_max(t_max_with_other_half(t_max16(sc)));
-            bf16x8_t pB[2];
-            exp_item(sc, mc, pB);
-            pv_item(st, it, pB);
-        };
-        // Two items of a tile as one: their score products are two independent chains of matrix instructions, issued
-        // alternately (a chain on one accumulator waits for itself), and one softmax step covers the 64 keys -- one max,
-        // one rescale test.  Without it a wave alone on its SIMD spends most of a tile waiting on its own latencies,
-        // which is what the last, long query tiles of a launch do.
-        auto two_items = [&](int st, int k0) {
-            f32x16_t s0, s1;
-#pragma unroll
-            for (int i = 0; i < 16; i++) s0[i] = s1[i] = 0.0f;
-#pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_operand(st, 0, ks), qreg[ks], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_operand(st, 1, ks), qreg[ks], s1, 0, 0, 0);
-            }
-            const f32x4_t no_bias[4] = {};
-            mask_item(0, k0, s0, no_bias);
-            mask_item(1, k0 + 32, s1, no_bias);
-            const float mc = raise_max(t_max_with_other_half(t_vmax(t_max16(s0), t_max16(s1))));
-            bf16x8_t pA[2], pC[2];
-            exp_item(s0, mc, pA);
-            exp_item(s1, mc, pC);
-            pv_item(st, 0, pA);
-            pv_item(st, 1, pC);
+            part = part0 + part1;
         };
 
-        auto walk_tile = [&](int t, auto set_c) {
+        // the slow path of a softmax step: the item max, O and l rescaled to it, P again from the scores
+        auto raise_max_and_redo = [&](const f32x16_t& sc, uint32_t (&w)[8], float& part) __attribute__((always_inline)) {
+            const float m_item = t_max_with_other_half(t_max16(sc));
+            const float m_new = t_vmax(m_run, m_item);
+            const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * cc);  // m_run = -inf -> 0
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int tt = 0; tt < DT; tt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc_o[tt][i] *= alpha;
+            const float mc = m_use * cc;
+            // a valid row that has seen no key yet keeps taking this path (and gets P = 0 from it: exp2(-inf - 0))
+            neg_mc = (m_new == neg_inf()) ? (valid ? __uint_as_float(0x7f800000u) : 0.0f) : -mc;
+            exp_plain(sc, -mc, w, part);
+        };
+        // An item whose three phases run one after the other (head dims above 128): S, the softmax step, P.V
+        auto step_simple = [&](int it, int k0, const uint16_t* kp, const uint16_t* vp) __attribute__((always_inline)) {
+            if (BIAS) bias_fetch(k0, bv_a);
+#pragma unroll
+            for (int i = 0; i < 16; i++) s_a[i] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++)
+                s_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)(kp + 16 * ks), qreg[ks], s_a, 0, 0, 0);
+            mask_item(it, k0, s_a, bv_a);
+            uint32_t w[8];
+            float part;
+            exp_plain(s_a, neg_mc, w, part);
+            if (__builtin_expect(__any(!(part <= kTileTrigSum)), 0)) raise_max_and_redo(s_a, w, part);
+            l_run += part;
+            p_a[0] = __builtin_bit_cast(bf16x8_t, u32x4_t{w[0], w[1], w[2], w[3]});
+            p_a[1] = __builtin_bit_cast(bf16x8_t, u32x4_t{w[4], w[5], w[6], w[7]});
+            drain(vp);
+        };
+
+        // One step of the pipeline: item j (keys k0 .., item `it` of its tile) gets its softmax step; K rows of item
+        // j + 1 are at kp, V rows of item j - 1 at vp.
+        //
+        // The softmax step takes no row max in the steady state: P is formed against the running max as it stands (a
+        // stale max scales a row's P, O and l by one common factor, harmless until it overflows), and the lane's share
+        // of the row sum, which is needed anyway, bounds every P of the lane.  Only when a share passes kTileTrigSum, or
+        // is not a number, or a valid row has no max yet (neg_mc = +inf), does the wave take the item max, rescale O and
+        // l and form P again from the scores, which are still in their registers.
+        //
+        // The vector work is laid out in six groups (arguments, exponentials, sums and conversions, for either half of
+        // the scores), the step's matrix instructions are dealt to the groups in order, S and P.V alternating (a chain
+        // on one accumulator waits for itself), and an operand is read from LDS one or two groups ahead of its instruction.
+        // The fences between the groups name the vector values and the B operands of the matrix instructions on
+        // either side, which is what keeps each matrix instruction inside its group.
+        auto step = [&](int it, int k0, const uint16_t* kp, const uint16_t* vp, f32x16_t& s_cur, f32x16_t& s_next,
+                        bf16x8_t (&p_prev)[2], bf16x8_t (&p_new)[2], f32x4_t (&bv_cur)[4],
+                        f32x4_t (&bv_next)[4]) __attribute__((always_inline)) {
+            if (BIAS) bias_fetch(k0 + 32, bv_next);
+            mask_item(it, k0, s_cur, bv_cur);
+#pragma unroll
+            for (int i = 0; i < 16; i++) s_next[i] = 0.0f;
+            u32x4_t ops[NM];
+            auto group_of = [](int m) __attribute__((always_inline)) { return NM >= 6 ? m * 6 / NM : (m * 6 + NM - 1) / NM; };
+            auto fetch_group = [&](int gq) __attribute__((always_inline)) {
+#pragma unroll
+                for (int m = 0; m < NM; m++)
+                    if (group_of(m) == gq) ops[m] = load_op(m, kp, vp);
+            };
+            auto fence_b = [&](int gq) __attribute__((always_inline)) {  // the B operands of the matrix instructions of group gq
+#pragma unroll
+                for (int m = 0; m < NM; m++) {
+                    if (group_of(m) != gq) continue;
+                    if (m & 1) pin_b(p_prev[(m >> 1) / DT]);
+                    else pin_b(qreg[m >> 1]);
+                }
+            };
+            auto multiply_group = [&](int gq) __attribute__((always_inline)) {
+#pragma unroll
+                for (int m = 0; m < NM; m++) {
+                    if (group_of(m) != gq) continue;
+                    const bf16x8_t a_op = __builtin_bit_cast(bf16x8_t, ops[m]);
+                    if ((m & 1) == 0) {
+                        s_next = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op, qreg[m >> 1], s_next, 0, 0, 0);
+                    } else {
+                        const int i = m >> 1, u = i / DT, dt = i - u * DT;
+                        acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op, p_prev[u], acc_o[dt], 0, 0, 0);
+                    }
+                }
+            };
+            float t[8];
+            uint32_t w[8];
+            float part0 = 0.0f, part1 = 0.0f;
+            constexpr int LOOK = DP <= 64 ? 2 : 1;  // groups between an operand's LDS read and its matrix instruction
+            fetch_group(0);
+            if (LOOK > 1) fetch_group(1);
+            fence_b(0);
+#pragma unroll
+            for (int gq = 0; gq < 6; gq++) {
+                if (gq + LOOK < 6) fetch_group(gq + LOOK);
+                multiply_group(gq);
+                const int half = gq / 3;
+                if (gq % 3 == 0) {
+#pragma unroll
+                    for (int i = 0; i < 8; i++) t[i] = __builtin_fmaf(s_cur[8 * half + i], cc, neg_mc);
+                } else if (gq % 3 == 1) {
+#pragma unroll
+                    for (int i = 0; i < 8; i++) t[i] = __builtin_amdgcn_exp2f(t[i]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; i += 2) {
+                        part0 += t[i];
+                        part1 += t[i + 1];
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++) w[4 * half + e] = t_cvt_pk_bf16(t[2 * e], t[2 * e + 1]);
+                }
+                // the fence behind group gq
+#pragma unroll
+                for (int i = 0; i < 8; i++) pin_f(t[i]);
+                if (gq % 3 == 2) {
+                    pin_f(part0);
+                    pin_f(part1);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) pin_u(w[4 * half + e]);
+                }
+                fence_b(gq);
+                if (gq + 1 < 6) fence_b(gq + 1);
+            }
+            float part = part0 + part1;
+            if (__builtin_expect(__any(!(part <= kTileTrigSum)), 0)) raise_max_and_redo(s_cur, w, part);
+            l_run += part;
+            p_new[0] = __builtin_bit_cast(bf16x8_t, u32x4_t{w[0], w[1], w[2], w[3]});
+            p_new[1] = __builtin_bit_cast(bf16x8_t, u32x4_t{w[4], w[5], w[6], w[7]});
+        };
+        // a step whose results are moved back into the first of each pair
+        auto step_a = [&](int it, int k0, const uint16_t* kp, const uint16_t* vp) __attribute__((always_inline)) {
+            step(it, k0, kp, vp, s_a, s_b, p_a, p_b, bv_a, bv_b);
+            s_a = s_b;
+            p_a[0] = p_b[0];
+            p_a[1] = p_b[1];
+            if (BIAS) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) bv_a[j] = bv_b[j];
+            }
+        };
+        // slot j of the walk: a step while the wave has items left, then once the P.V of its last item
+        auto slot = [&](int j, int it, const uint16_t* kp, const uint16_t* vp) __attribute__((always_inline)) {
+            if (j < n_it) step_a(it, 32 * j, kp, vp);
+            else if (j == n_it && n_it > 0) drain(vp);
+        };
+
+        // tile t: the step of its first item, the barrier, K(t+2) and V(t+1) parked from sets KSET and VSET (which
+        // are refilled with K(t+2+PF) and V(t+1+PF)), then the steps of its other items
+        auto park_next = [&](int t, auto kset_c, auto vset_c) __attribute__((always_inline)) {
+            constexpr int KSET = decltype(kset_c)::value;
             const int st = t & 1;
-            const int k0 = t * KT + 32 * NI * grp;  // first key of this wave's items
-            if (NI == 2 && !BIAS && DP <= 64 && k0 + 32 <= wave_lim_max) {
-                two_items(st, k0);
+            // (behind the last tiles these park and request copies of the last tile, which nobody reads)
+            park_k(kreg[KSET], st);
+            park_v(vset_c, st ^ 1);
+            issue_k(kreg[KSET], (t + 2 + PF) * KT);
+            issue_v(vset_c, (t + 1 + PF) * KT);
+        };
+        // the same for a tile of which the wave walks every item: straight-line code, the pairs swapped from step to step
+        auto walk_full = [&](int t, auto kset_c, auto vset_c) __attribute__((always_inline)) {
+            const int st = t & 1;
+            const uint16_t* const k_st = Ks + st * KT * LDK + k_off;
+            const uint16_t* const k_ot = Ks + (st ^ 1) * KT * LDK + k_off;
+            const uint16_t* const v_st = Vs + st * KT * LDV + v_off;
+            const uint16_t* const v_ot = Vs + (st ^ 1) * KT * LDV + v_off;
+            const int k0 = t * KT;
+            if (NI > 1) {
+                step(0, k0, k_st + 32 * LDK, t == 0 ? v_st : v_ot + 32 * (NI - 1) * LDV, s_a, s_b, p_a, p_b, bv_a, bv_b);
+                __syncthreads();
+                park_next(t, kset_c, vset_c);
+                step(1, k0 + 32, k_ot, v_st, s_b, s_a, p_b, p_a, bv_b, bv_a);
             } else {
+                step_a(0, k0, k_ot, t == 0 ? v_st : v_ot);
+                __syncthreads();
+                park_next(t, kset_c, vset_c);
+                __syncthreads();
+            }
+            keep_cur = keep_next;
+        };
+        auto walk_tile = [&](int t, auto kset_c, auto vset_c) __attribute__((always_inline)) {
+            const int st = t & 1;
+            const uint16_t* const k_st = Ks + st * KT * LDK + k_off;         // K(t)
+            const uint16_t* const k_ot = Ks + (st ^ 1) * KT * LDK + k_off;   // K(t+1)
+            const uint16_t* const v_st = Vs + st * KT * LDV + v_off;         // V(t)
+            const uint16_t* const v_ot = Vs + (st ^ 1) * KT * LDV + v_off;   // V(t-1)
+            // first item: the next item is item 1 of this tile (or item 0 of the next tile when a tile is one item);
+            // the previous item is the last of tile t - 1 (at t = 0 there is none: P is zero, and V(0) stands in)
+            slot(t * NI, 0, NI > 1 ? k_st + 32 * LDK : k_ot, t == 0 ? v_st : v_ot + 32 * (NI - 1) * LDV);
+            __syncthreads();
+            park_next(t, kset_c, vset_c);
+            if (NI > 1) {
+                slot(t * NI + 1, 1, k_ot, v_st);
+            } else {
+                __syncthreads();  // one item per tile: K(t+2) is read by the very next step
+            }
+            keep_cur = keep_next;
+        };
+        int t0 = 0;  // t0 % PF == 0 throughout: the set indices below are compile-time
+        if (!PIPE) {
+            static_assert(PIPE || PF == 1, "the unpipelined walk keeps one register set");
+            for (int t = 0; t < n_tiles; t++) {
+                const int st = t & 1;
 #pragma unroll
                 for (int it = 0; it < NI; it++)
-                    // else every row of this wave has all of these keys hidden (wave-uniform)
-                    if (k0 + 32 * it <= wave_lim_max) one_item(st, it, k0 + 32 * it);
+                    if (t * NI + it < n_it)
+                        step_simple(it, t * KT + 32 * it, Ks + st * KT * LDK + 32 * it * LDK + k_off, Vs + st * KT * LDV + 32 * it * LDV + v_off);
+                park_k(kreg[0], st ^ 1);
+                park_v(std::integral_constant<int, 0>{}, st ^ 1);
+                issue_k(kreg[0], (t + 2) * KT);
+                issue_v(std::integral_constant<int, 0>{}, (t + 2) * KT);
+                __syncthreads();
+                keep_cur = keep_next;
             }
-            // ---- the next tile: its registers have been in flight during the last PF tiles' work
-            if (t + 1 < n_tiles) {
-                park(set_c, st ^ 1);
-                if (t + 1 + PF < n_tiles) issue_loads(set_c, (t + 1 + PF) * KT);
-            }
-            __syncthreads();
-        };
-        for (int t0 = 0; t0 < n_tiles; t0 += PF) {  // t0 % PF == 0: the set indices below are compile-time
-            walk_tile(t0, std::integral_constant<int, 1 % PF>{});
-            if (PF >= 2 && t0 + 1 < n_tiles) walk_tile(t0 + 1, std::integral_constant<int, 2 % PF>{});
-            if (PF >= 3 && t0 + 2 < n_tiles) walk_tile(t0 + 2, std::integral_constant<int, 3 % PF>{});
+            t0 = n_tiles;
         }
-
-        // ---- the two key halves of a row meet: group 1 leaves its (O, m, l) in LDS, group 0 folds it into its own
-        // with the online-softmax monoid (crates/rustorch-attention/src/online_softmax.rs:105-131, extended with O).
-        // Slot i of a region is 64 lanes x 16 bytes: lane-contiguous, so reads and writes are free of bank conflicts.
-        if (NG == 2) {
-            f32x4_t* region = (f32x4_t*)(lds + wq * Cfg::REGION);
-            if (grp == 1) {
-#pragma unroll
-                for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        region[(4 * dt + j) * 64 + lane] =
-                            f32x4_t{acc_o[dt][4 * j], acc_o[dt][4 * j + 1], acc_o[dt][4 * j + 2], acc_o[dt][4 * j + 3]};
-                region[4 * DT * 64 + lane] = f32x4_t{m_run, l_run, 0.0f, 0.0f};
-            }
-            __syncthreads();
-            if (grp == 1) return;
-            const f32x4_t ml = region[4 * DT * 64 + lane];
-            const float m_new = t_vmax(m_run, ml[0]);
-            const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
-            const float a0 = __builtin_amdgcn_exp2f((m_run - m_use) * cc);  // an empty side (m = -inf) weighs 0
-            const float a1 = __builtin_amdgcn_exp2f((ml[0] - m_use) * cc);
-            l_run = l_run * a0 + ml[1] * a1;
-            m_run = m_new;
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const f32x4_t o1 = region[(4 * dt + j) * 64 + lane];
-#pragma unroll
-                    for (int e = 0; e < 4; e++) acc_o[dt][4 * j + e] = acc_o[dt][4 * j + e] * a0 + o1[e] * a1;
-                }
+        for (const int t_full = n_it / NI; PIPE && t0 + PF <= t_full; t0 += PF) {
+            walk_full(t0, std::integral_constant<int, 2 % PF>{}, std::integral_constant<int, 1 % PF>{});
+            if (PF >= 2) walk_full(t0 + 1, std::integral_constant<int, 3 % PF>{}, std::integral_constant<int, 2 % PF>{});
+            if (PF >= 3) walk_full(t0 + 2, std::integral_constant<int, 4 % PF>{}, std::integral_constant<int, 3 % PF>{});
         }
-    } else if (grp == 1) {
-        return;  // a tile of padded rows: the first group writes the fill value
+        for (; t0 < n_tiles; t0 += PF) {
+            walk_tile(t0, std::integral_constant<int, 2 % PF>{}, std::integral_constant<int, 1 % PF>{});
+            if (PF >= 2 && t0 + 1 < n_tiles) walk_tile(t0 + 1, std::integral_constant<int, 3 % PF>{}, std::integral_constant<int, 2 % PF>{});
+            if (PF >= 3 && t0 + 2 < n_tiles) walk_tile(t0 + 2, std::integral_constant<int, 4 % PF>{}, std::integral_constant<int, 3 % PF>{});
+        }
+        // a wave that walked every item of the workgroup still owes the last P.V
+        if (PIPE && n_it == n_tiles * NI && n_it > 0)
+            drain(Vs + ((n_tiles - 1) & 1) * KT * LDV + v_off + 32 * (NI - 1) * LDV);
+        __syncthreads();  // the output rows are staged over the tiles
     }
 
     // ---- output: acc_o[dt][4j + e] = O^T[d = 32dt + 8j + 4hh + e][row col of the wave].  A lane holds 8-byte pieces of
@@ -554,19 +709,20 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, TileCfg<DP>::OCC) void flash_
     }
 }
 
-template <int DP, int MODE, bool BIAS>
+template <int DP, int MODE, bool BIAS, bool PACKED>
 hipError_t launch_one(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
-    hipLaunchKernelGGL((flash_tile_bf16_kernel<DP, MODE, BIAS>), grid, dim3(TileCfg<DP>::THREADS), 0, stream, p);
+    hipLaunchKernelGGL((flash_tile_bf16_kernel<DP, MODE, BIAS, PACKED>), grid, dim3(TileCfg<DP>::THREADS), 0, stream, p);
     return hipGetLastError();
 }
 
 template <int DP>
 hipError_t launch_dp(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
-    if (p.bias) return launch_one<DP, kMaskNone, true>(stream, p, grid);
+    if (p.pack > 1) return launch_one<DP, kMaskCausal, false, true>(stream, p, grid);
+    if (p.bias) return launch_one<DP, kMaskNone, true, false>(stream, p, grid);
     switch (p.mask) {
-        case kMaskNone: return launch_one<DP, kMaskNone, false>(stream, p, grid);
-        case kMaskCausal: return launch_one<DP, kMaskCausal, false>(stream, p, grid);
-        case kMaskPadding: return launch_one<DP, kMaskPadding, false>(stream, p, grid);
+        case kMaskNone: return launch_one<DP, kMaskNone, false, false>(stream, p, grid);
+        case kMaskCausal: return launch_one<DP, kMaskCausal, false, false>(stream, p, grid);
+        case kMaskPadding: return launch_one<DP, kMaskPadding, false, false>(stream, p, grid);
         default: return hipErrorInvalidValue;
     }
 }
@@ -575,15 +731,18 @@ hipError_t launch_dp(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
 
 bool flash_tile_bf16_supported(int dim) { return dim > 0 && dim <= 256 && dim % 8 == 0; }
 
-hipError_t launch_flash_tile_bf16(hipStream_t stream, const FlashTileParams& p) {
+hipError_t launch_flash_tile_bf16(hipStream_t stream, const FlashTileParams& params) {
+    FlashTileParams p = params;
     if (p.batch == 0 || p.heads == 0 || p.seq_q == 0) return hipSuccess;
     if (!flash_tile_bf16_supported(p.dim) || p.pack < 1) return hipErrorInvalidValue;
     if (p.bias && p.mask != kMaskNone) return hipErrorInvalidValue;
+    if (p.pack > 1 && (p.bias || p.mask != kMaskCausal)) return hipErrorInvalidValue;  // packed rows: the chunked decode only
     const long long rows = (long long)p.seq_q * p.pack;
     const long long n_qtiles = (rows + TROWS - 1) / TROWS;
-    const long long units = (long long)p.batch * (p.pack > 1 ? p.kv_heads : p.heads);
-    if (n_qtiles * units > 0x7fffffffll) return hipErrorInvalidValue;
-    dim3 grid((unsigned)(n_qtiles * units));
+    const long long heads_u = p.pack > 1 ? p.kv_heads : p.heads;
+    if (p.batch > 65535 || n_qtiles > 65535 || heads_u > 65535 || p.group < 1) return hipErrorInvalidValue;  // grid limits
+    p.group_magic = p.group > 1 ? (uint32_t)(0x100000000ull / (unsigned long long)p.group) + 1u : 0u;
+    dim3 grid((unsigned)heads_u, (unsigned)p.batch, (unsigned)n_qtiles);
     if (p.dim <= 32) return launch_dp<32>(stream, p, grid);
     if (p.dim <= 64) return launch_dp<64>(stream, p, grid);
     if (p.dim <= 96) return launch_dp<96>(stream, p, grid);

@@ -107,6 +107,7 @@ struct FlashTileParams {
     long long bias_bh_stride; // elements between the biases of consecutive (batch, head) pairs; 0 = one for all
     int bias_vec4;            // bias rows may be read 16 bytes at a time (base and seq_kv * 4 bytes both 16-byte aligned)
     int batch, heads, kv_heads, group;
+    uint32_t group_magic;     // set by the launcher: 2^32 / group + 1 (0 when group is 1), for head / group by a multiply
     // 1: a tile's rows are positions of one head.  group: rows run over (position, head of the GQA group), row
     // r = position * group + head-in-group, so that all heads of a kv head share one pass over its keys.
     int pack;
