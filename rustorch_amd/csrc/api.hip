@@ -676,7 +676,8 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
     if (shape->dim > 256 || shape->dim % 8 != 0)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 256, shape->dim,
                     "bf16 flash kernels cover head dims up to 256 that are a multiple of 8");
-    if ((shape->seq + 127) / 128 * shape->batch * shape->heads > 0x7fffffffull)
+    // the tile kernel's grid is (heads, batch, query tiles of 128 rows), each dimension below 2^16
+    if (shape->heads > 65535 || shape->batch > 65535 || (shape->seq + 127) / 128 > 65535)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
     // the persistent kernel needs a job (256 query rows of one head) for every CU and gains on the tile kernel as the
     // rows get longer; a padded batch is a set of jobs of very different lengths, which the tile kernel's
@@ -952,7 +953,7 @@ RT_API int rt_mha_forward_masked_bf16_dev(void* stream, const void* q, const voi
     if (!rt::flash_tile_bf16_supported((int)std::min<size_t>(head_dim, 1 << 20)))
         return fail(err, RT_ERR_UNSUPPORTED, -1, 256, head_dim, "bf16 kernels cover head dims up to 256 that are a multiple of 8");
     if (heads > 65535 || batch > 65535 || t_q > 0x7fffffffull || t_kv > 0x7fffffffull || embed > 0x7fffffffull ||
-        (t_q + 127) / 128 * batch * heads > 0x7fffffffull)
+        (t_q + 127) / 128 > 65535)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
     if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0 || ((uintptr_t)mask & 3) != 0)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 16, 0, "bf16 kernels need 16-byte aligned tensors");
@@ -1183,7 +1184,8 @@ RT_API int rt_gqa_decode_chunk_bf16(void* stream, const void* q, const void* k_c
     if ((((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)out) & 15) != 0)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 16, 0, "bf16 kernels need 16-byte aligned tensors");
     const int group = n_heads / n_kv;
-    if ((int64_t)seq_new * group > 0x7fffffffll) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    if (((int64_t)seq_new * group + 127) / 128 > 65535 || batch > 65535 || n_kv > 65535)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
     rc = ensure_device(err);
     if (rc) return rc;
     rt::FlashTileParams t{};

@@ -146,11 +146,60 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     // the end of a tile see more keys than those at its start: the assignment rotates from workgroup to workgroup
     // so that no SIMD collects the long rows of every tile.
     const int wq = (wave + hx + b + (int)blockIdx.z) & 3;
+    const int D = p.dim;
+
+    const uint16_t* __restrict__ Kg = p.k + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+    const uint16_t* __restrict__ Vg = p.v + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+
+    // ---- tile movement: chunk c = tid + TTHREADS n of a tile is (row c / CH, 16-byte chunk c % CH).  A tile
+    // travels global -> registers -> LDS.  LDS holds two stages of each matrix; PF register sets per matrix hold
+    // the tiles behind them, so that a load has PF tile-times to arrive.
+    u32x4_t kreg[PF][NL], vreg[PF][NL];
+    uint32_t keep_raw[PF];
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+        keep_raw[i] = 1;
+#pragma unroll
+        for (int n = 0; n < NL; n++) kreg[i][n] = vreg[i][n] = u32x4_t{0u, 0u, 0u, 0u};  // (only read when there are no keys at all)
+    }
+    // per-thread constants of the movement (hoisted: the loop then spends a handful of instructions per tile on it)
+    int ld_row[NL];       // row of the tile this thread moves
+    uint32_t ld_col[NL];  // element offset inside a row; the same in K and V
+    uint32_t st_k[NL], st_v[NL];  // byte offsets of the chunk in an LDS stage
+    bool ld_on[NL];
+#pragma unroll
+    for (int n = 0; n < NL; n++) {
+        const int c = tid + TTHREADS * n;
+        const int row = c / CH, ch = c - row * CH;
+        ld_row[n] = row;
+        st_k[n] = (uint32_t)((row * LDK + 8 * ch) * 2);
+        st_v[n] = (uint32_t)((2 * KT * LDK + row * LDV + 8 * ch) * 2);
+        ld_on[n] = 8 * ch < D;
+        ld_col[n] = ld_on[n] ? (uint32_t)(8 * ch) : 0u;  // a chunk past the head dim is requested (from column 0) but never parked
+    }
+    // Tile 0 (K and V) and K of tile 1 are requested before the sequence lengths are even read (those are a
+    // dependent load away): their rows are clamped to the tensor only, and the rows of V(0) past the last key are
+    // zeroed once the length is known (the matching rows of K are masked in the score tile whatever they hold).
+    // A workgroup that turns out to have no keys to walk leaves the requests unused.
+    const uint32_t kv_pitch = (uint32_t)p.lkv.row_pitch;
+    u32x4_t k1[NL];
+#pragma unroll
+    for (int n = 0; n < NL; n++) k1[n] = u32x4_t{0u, 0u, 0u, 0u};
+    if (p.seq_kv > 0) {  // (no keys at all: there is no row to read, and no tile will be walked)
+        const int last_row = p.seq_kv - 1;
+#pragma unroll
+        for (int n = 0; n < NL; n++) {
+            const size_t e0 = (size_t)(uint32_t)min(ld_row[n], last_row) * kv_pitch + ld_col[n];
+            kreg[0][n] = *(const u32x4_t*)(Kg + e0);
+            vreg[0][n] = *(const u32x4_t*)(Vg + e0);
+            if (PIPE) k1[n] = *(const u32x4_t*)(Kg + (size_t)(uint32_t)min(KT + ld_row[n], last_row) * kv_pitch + ld_col[n]);
+        }
+        if (MODE == kMaskPadding) keep_raw[0] = p.keep[min(lane & (KT - 1), last_row)];
+    }
 
     const int n_q = p.q_lens ? min(max(p.q_lens[b], 0), p.seq_q) : p.seq_q;          // valid query positions
     const int n_keys = p.kv_lens ? min(max(p.kv_lens[b], 0), p.seq_kv) : p.seq_kv;  // keys that exist
     const int off = n_keys - n_q;  // causal: the last valid query sees every key
-    const int D = p.dim;
 
     // keys the workgroup walks
     int kv_end = n_keys;
@@ -174,35 +223,6 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     const float cc = BIAS ? kLog2e : p.scale_log2e;  // exp2 argument per unit of score
 
     if (n_tiles > 0) {
-        const uint16_t* __restrict__ Kg = p.k + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
-        const uint16_t* __restrict__ Vg = p.v + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
-
-        // ---- tile movement: chunk c = tid + TTHREADS n of a tile is (row c / CH, 16-byte chunk c % CH).  A tile
-        // travels global -> registers -> LDS.  LDS holds two stages of each matrix; PF register sets per matrix hold
-        // the tiles behind them, so that a load has PF tile-times to arrive.
-        u32x4_t kreg[PF][NL], vreg[PF][NL];
-        uint32_t keep_raw[PF];
-#pragma unroll
-        for (int i = 0; i < PF; i++) {
-            keep_raw[i] = 1;
-#pragma unroll
-            for (int n = 0; n < NL; n++) kreg[i][n] = vreg[i][n] = u32x4_t{0u, 0u, 0u, 0u};
-        }
-        // per-thread constants of the movement (hoisted: the loop then spends a handful of instructions per tile on it)
-        int ld_row[NL];       // row of the tile this thread moves
-        uint32_t ld_col[NL];  // element offset inside a row; the same in K and V
-        uint32_t st_k[NL], st_v[NL];  // byte offsets of the chunk in an LDS stage
-        bool ld_on[NL];
-#pragma unroll
-        for (int n = 0; n < NL; n++) {
-            const int c = tid + TTHREADS * n;
-            const int row = c / CH, ch = c - row * CH;
-            ld_row[n] = row;
-            st_k[n] = (uint32_t)((row * LDK + 8 * ch) * 2);
-            st_v[n] = (uint32_t)((2 * KT * LDK + row * LDV + 8 * ch) * 2);
-            ld_on[n] = 8 * ch < D;
-            ld_col[n] = ld_on[n] ? (uint32_t)(8 * ch) : 0u;  // a chunk past the head dim is requested (from column 0) but never parked
-        }
         static_assert(CHUNKS % TTHREADS == 0, "every thread moves NL chunks of every tile");
         // Every request below is unconditional -- a tile index past the last tile is clamped to it, a chunk past the
         // head dim reads column 0 -- and only the LDS write is predicated.  With no branch around a load the compiler
@@ -213,7 +233,6 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             __syncthreads();
         }
         const int last_kv0 = (n_tiles - 1) * KT;
-        const uint32_t kv_pitch = (uint32_t)p.lkv.row_pitch;
         // rows past the end re-read the last key; they are masked in the score tile
         auto chunk_at = [&](int n, int kv0) __attribute__((always_inline)) { return (size_t)(uint32_t)min(kv0 + ld_row[n], n_keys - 1) * kv_pitch + ld_col[n]; };
         auto issue_k = [&](u32x4_t (&dst)[NL], int kv0) __attribute__((always_inline)) {
@@ -247,13 +266,13 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             if (MODE == kMaskPadding) keep_next = __ballot(keep_raw[SET] != 0);
         };
 
-        // tiles 0 (K and V) and 1 (K) are requested before anything else of the set-up: their latency covers it
-        u32x4_t k1[NL];
+        // tile 0's early requests: V rows past the last key become zero, keep bytes past it count as kept
+        if (n_keys < KT) {
 #pragma unroll
-        for (int n = 0; n < NL; n++) k1[n] = u32x4_t{0u, 0u, 0u, 0u};
-        issue_k(kreg[0], 0);
-        issue_v(std::integral_constant<int, 0>{}, 0);
-        if (PIPE) issue_k(k1, KT);
+            for (int n = 0; n < NL; n++)
+                if (ld_row[n] >= n_keys) vreg[0][n] = u32x4_t{0u, 0u, 0u, 0u};
+            if (MODE == kMaskPadding && (lane & (KT - 1)) >= n_keys) keep_raw[0] = 1u;
+        }
 
         // ---- this lane's query row
         const int r = q0 + 32 * wq + col;
