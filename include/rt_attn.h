@@ -301,6 +301,14 @@ int rt_gqa_decode_online_bf16(void *stream, const void *q, const void *k_cache, 
                               int32_t n_heads, int32_t n_kv, int32_t kv_len, int32_t head_dim, int32_t max_seq,
                               rt_err_detail *err);
 
+/* LlmKernels::gqa_decode_naive_bf16 -- llm_kernels.rs:461-545 (kernel), :990-1042 (launcher): the reference's first
+ * decode kernel, the same function of the same arguments as gqa_decode_online_bf16 (softmax(q.K^T * scale).V over the
+ * first kv_len cache rows, kv head = h*n_kv/n_heads) computed in three passes over a score buffer instead of one pass
+ * with a running max.  Here both names run the same kernels and give the same bits. */
+int rt_gqa_decode_naive_bf16(void *stream, const void *q, const void *k_cache, const void *v_cache, void *out,
+                             int32_t n_heads, int32_t n_kv, int32_t kv_len, int32_t head_dim, int32_t max_seq,
+                             rt_err_detail *err);
+
 /* The batched, ragged form of the same call: q/out [batch,n_heads,head_dim], caches
  * [batch,n_kv,max_seq,head_dim], kv_lens device int32[batch] (sequence b reads [..kv_lens[b]]).
  * Split-K over the context with a second-pass (m, l, o) merge; `workspace` (device, at least

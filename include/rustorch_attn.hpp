@@ -600,6 +600,13 @@ struct LlmKernels {
         detail::check_gqa(
             rt_gqa_decode_online_bf16(stream, q, k_cache, v_cache, out, n_heads, n_kv, kv_len, head_dim, max_seq, &e), e);
     }
+    // llm_kernels.rs:990-1042: the three-pass launcher of the same function
+    static void gqa_decode_naive_bf16(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out,
+                                      int32_t n_heads, int32_t n_kv, int32_t kv_len, int32_t head_dim, int32_t max_seq) {
+        rt_err_detail e;
+        detail::check_gqa(
+            rt_gqa_decode_naive_bf16(stream, q, k_cache, v_cache, out, n_heads, n_kv, kv_len, head_dim, max_seq, &e), e);
+    }
     static size_t gqa_decode_workspace_bytes(int32_t batch, int32_t n_heads, int32_t n_kv, int32_t head_dim,
                                              int32_t max_seq) {
         return rt_gqa_decode_workspace_bytes(batch, n_heads, n_kv, head_dim, max_seq);

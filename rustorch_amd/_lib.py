@@ -19,7 +19,7 @@ SYMBOLS = (
     "rt_flash_forward_stats_f32_dev", "rt_flash_backward_saved_f32_dev",
     "rt_flash_forward_f32_dev", "rt_flash_forward_bf16_dev", "rt_flash_forward_varlen_bf16_dev",
     "rt_mha_flash_forward_f32", "rt_mha_forward_masked_f32", "rt_mha_forward_masked_f32_dev", "rt_mha_forward_masked_bf16_dev", "rt_gqa_decode_chunk_bf16", "rt_flash_forward_bnhd_f32_dev", "rt_flash_forward_bnhd_bf16_dev",
-    "rt_kv_append_bf16", "rt_kv_cache_append_dev", "rt_qk_norm_rope_kv_append_bf16", "rt_gqa_decode_online_bf16", "rt_gqa_decode_batched_bf16",
+    "rt_kv_append_bf16", "rt_kv_cache_append_dev", "rt_qk_norm_rope_kv_append_bf16", "rt_gqa_decode_online_bf16", "rt_gqa_decode_naive_bf16", "rt_gqa_decode_batched_bf16",
     "rt_gqa_decode_workspace_bytes", "rt_gqa_decode_batched_bf16_noalloc",
     "rt_buf_alloc", "rt_buf_free", "rt_buf_zero", "rt_memcpy_h2d", "rt_memcpy_d2h", "rt_stream_synchronize",
     "rt_stream_create", "rt_stream_destroy",
@@ -104,6 +104,7 @@ def lib():
     L.rt_qk_norm_rope_kv_append_bf16.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, vp, vp, C.c_float, vp, vp, i32, i32,
                                                  i32, i32, i32, i32, i32, errp]
     L.rt_gqa_decode_online_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, errp]
+    L.rt_gqa_decode_naive_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, errp]
     L.rt_gqa_decode_batched_bf16.argtypes = [vp, vp, vp, vp, vp, i32p, i32, i32, i32, i32, i32, vp, sz, errp]
     L.rt_gqa_decode_batched_bf16_noalloc.argtypes = [vp, vp, vp, vp, vp, i32p, i32, i32, i32, i32, i32, errp]
     L.rt_gqa_decode_workspace_bytes.argtypes = [i32, i32, i32, i32, i32]

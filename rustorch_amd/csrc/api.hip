@@ -1163,6 +1163,12 @@ RT_API int rt_gqa_decode_online_bf16(void* stream, const void* q, const void* k_
     return RT_OK;
 }
 
+RT_API int rt_gqa_decode_naive_bf16(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out,
+                                    int32_t n_heads, int32_t n_kv, int32_t kv_len, int32_t head_dim, int32_t max_seq,
+                                    rt_err_detail* err) {
+    return rt_gqa_decode_online_bf16(stream, q, k_cache, v_cache, out, n_heads, n_kv, kv_len, head_dim, max_seq, err);
+}
+
 // Several new positions per sequence against the cache, causally masked: the bf16 form of gqa_decode_batched_f32
 // (crates/rustorch-metal/src/kernels.rs:14432-14516), batched over sequences with their own context lengths.
 RT_API int rt_gqa_decode_chunk_bf16(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out,

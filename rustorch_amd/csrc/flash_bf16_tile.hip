@@ -115,9 +115,9 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     constexpr int PF = Cfg::PF;        // register sets of tiles in flight behind the two LDS stages
     static_assert(2 * DT == KS, "one P.V matrix instruction per score matrix instruction");
     // Head dims above 128 do not have the registers for two score tiles and their operands in flight (O alone is 128
-    // registers), nor does head dim 128 with a bias (two items' bias values): there an item runs its three phases
-    // one after the other, and K is parked with V.
-    constexpr bool PIPE = DP <= 128 && !(BIAS && DP == 128);
+    // registers), nor does head dim 128 with a bias (two items' bias values) or with a key-padding mask: there an
+    // item runs its three phases one after the other, and K is parked with V.
+    constexpr bool PIPE = DP <= 128 && !((BIAS || MODE == kMaskPadding) && DP == 128);
 
     __shared__ __attribute__((aligned(16))) unsigned char lds[Cfg::LDS_BYTES];
     uint16_t* const Ks = (uint16_t*)lds;                      // [2][KT * LDK]

@@ -54,6 +54,14 @@ class LlmKernels:
                                                     C.byref(err)), err)
 
     @staticmethod
+    def gqa_decode_naive_bf16(stream, q, k_cache, v_cache, out, n_heads, n_kv, kv_len, head_dim, max_seq):
+        """llm_kernels.rs:990-1042: the reference's three-pass decode launcher; same function, same kernels here."""
+        err = L.RtErr()
+        raise_for(L.lib().rt_gqa_decode_naive_bf16(stream, dev_ptr(q), dev_ptr(k_cache), dev_ptr(v_cache),
+                                                   dev_ptr(out), n_heads, n_kv, kv_len, head_dim, max_seq,
+                                                   C.byref(err)), err)
+
+    @staticmethod
     def gqa_decode_workspace_bytes(batch, n_heads, n_kv, head_dim, max_seq) -> int:
         return L.lib().rt_gqa_decode_workspace_bytes(batch, n_heads, n_kv, head_dim, max_seq)
 

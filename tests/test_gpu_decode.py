@@ -29,6 +29,37 @@ def test_kv_append_bf16_matches_oracle(oracle):
         K.kv_append_bf16(None, dk, dv, dk, dv, max_seq, n_kv, d, max_seq)
 
 
+@pytest.mark.parametrize("hq,hkv,d,max_seq,kv_len", [(8, 2, 32, 320, 77), (32, 8, 128, 600, 600), (8, 2, 64, 10, 0)])
+def test_gqa_decode_naive_bf16_is_the_same_function(oracle, hq, hkv, d, max_seq, kv_len):
+    """llm_kernels.rs:461-545, :990-1042: the reference's three-pass decode kernel computes what the online one does
+    (max, then exp and sum, then the weighted sum of V).  Checked against a float64 three-pass softmax written out
+    here, and bit for bit against the online entry, whose kernels it runs."""
+    qb, qf = bf16_round(seeded_normal((hq, d), 11))
+    kb, kf = bf16_round(seeded_normal((hkv, max_seq, d), 12))
+    vb, vf = bf16_round(seeded_normal((hkv, max_seq, d), 13))
+    outs = []
+    for call in (K.gqa_decode_naive_bf16, K.gqa_decode_online_bf16):
+        dout = ra.HipStorage(hq * d * 2)
+        dout.upload(np.full(hq * d, 0x7B7B, dtype=np.uint16))
+        call(None, dev(qb), dev(kb), dev(vb), dout, hq, hkv, kv_len, d, max_seq)
+        ra.synchronize()
+        outs.append(dout.download(np.uint16))
+    assert np.array_equal(outs[0], outs[1])
+    got = oracle.bf16_to_f32(outs[0]).reshape(hq, d)
+    q64 = qf.reshape(hq, d).astype(np.float64)
+    k64 = kf.reshape(hkv, max_seq, d).astype(np.float64)
+    v64 = vf.reshape(hkv, max_seq, d).astype(np.float64)
+    for h in range(hq):
+        kvh = h * hkv // hq
+        if kv_len == 0:
+            assert np.all(got[h] == 0.0)
+            continue
+        sc = k64[kvh, :kv_len] @ q64[h] / np.sqrt(np.float64(np.float32(d)))  # pass 1
+        w = np.exp(sc - sc.max())                                               # pass 2
+        want = (w / w.sum()) @ v64[kvh, :kv_len]                                # pass 3
+        assert max_abs(got[h], want) <= TOL
+
+
 @pytest.mark.parametrize("hq,hkv,d,max_seq,kv_len", [(8, 2, 32, 320, 1), (8, 2, 32, 320, 77), (32, 8, 128, 600, 600),
                                                      (6, 3, 96, 50, 49), (4, 4, 256, 40, 40), (8, 2, 64, 10, 0),
                                                      (16, 2, 256, 4096, 4096), (16, 2, 256, 100, 64), (8, 8, 256, 300, 257)])
