@@ -373,11 +373,11 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
                 for (int i = 0; i < 16; i++) sc[i] = __builtin_fmaf(sc[i], p.scale, bv[i >> 2][i & 3]);
             }
             if (k0 + 31 > wave_lim_min) {
+                // key k0 + 8 (i / 4) + 4 hh + i % 4 is hidden when it lies past lim: one subtraction per item, then a
+                // comparison with a constant per score
+                const int room = lim - k0 - 4 * hh;
 #pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const int kr = k0 + 8 * (i >> 2) + 4 * hh + (i & 3);
-                    sc[i] = (kr > lim) ? neg_inf() : sc[i];
-                }
+                for (int i = 0; i < 16; i++) sc[i] = (8 * (i >> 2) + (i & 3) > room) ? neg_inf() : sc[i];
             }
             if (MODE == kMaskPadding) {
                 const uint32_t keep_word = (uint32_t)(keep_cur >> (32 * it));
@@ -423,6 +423,18 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++)
                     s_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)(Ks + k_off + 16 * ks), qreg[ks], s_a, 0, 0, 0);
+                // The running max starts at the max of item 0, taken here, so that the first step already runs the
+                // fast path (without it the step would form P twice and rescale an O that is still zero).  The masks
+                // are applied first; the step applies them again, which changes nothing.  (Not with a bias: adding it
+                // is part of the mask step and must happen once.)
+                if (!BIAS) {
+                    mask_item(0, 0, s_a, bv_a);
+                    const float m0 = t_max_with_other_half(t_max16(s_a));
+                    if (m0 > neg_inf()) {  // (false for -inf and for NaN: such a row waits for the slow path)
+                        m_run = m0;
+                        neg_mc = -m0 * cc;
+                    }
+                }
             }
         }
 
@@ -692,6 +704,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     uint16_t* const obuf = (uint16_t*)(lds + wq * Cfg::REGION);
     const float fill = p.zero_padded_rows ? 0.0f : quiet_nan();
     if (n_tiles > 0) {
+        const bool plain = __all(good && valid);  // the common wave: one multiplication per element
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
@@ -699,8 +712,11 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
                 float o[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    float x = good ? acc_o[dt][4 * j + e] * inv_l : quiet_nan();
-                    if (!valid) x = fill;
+                    float x = acc_o[dt][4 * j + e] * inv_l;
+                    if (!plain) {
+                        x = good ? x : quiet_nan();
+                        if (!valid) x = fill;
+                    }
                     o[e] = x;
                 }
                 *(u32x2_t*)(obuf + col * LDK + 32 * dt + 8 * j + 4 * hh) =
