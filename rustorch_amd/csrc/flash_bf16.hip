@@ -29,9 +29,8 @@
 //   S(k): P(k) = exp2(..), row sums, conversion to bf16, overflow check: vector work only.
 //
 // Waves 0-3 run C(k) while waves 4-7 run S(k-1), then they swap.  The alternation is not enforced cluster
-// by cluster: the matrix pipe is the shared resource, a wave in its matrix cluster runs at raised priority
-// (waves 0-3 above waves 4-7, which settles the tie at the start of a job), and a wave whose partner holds
-// the pipe gets the gaps.  The workgroup meets at two barriers per step only, the two the LDS tile needs:
+// by cluster: the matrix pipe is the shared resource, a wave in its matrix cluster runs at raised priority,
+// and a wave whose partner holds the pipe gets the gaps.  The workgroup meets at two barriers per step only, the two the LDS tile needs:
 // "the next tile has landed" before its first read (the matrix cluster of item 3) and "this tile has been
 // read" before the requests that overwrite it (item 0 of the next step).  Waves 0-3 pass them behind their
 // softmax clusters of items 2 and 3, waves 4-7 behind their matrix clusters of the same items, which also
@@ -527,10 +526,9 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         // ---- C: the products, and right after each the read that refills its operand for the next C.
         // Score and P.V instructions alternate: a score instruction accumulates onto the one before it,
         // and back-to-back dependent matrix instructions would wait for each other.
-        // the multiplying wave goes first (its next instruction frees the matrix pipe); when both waves of a SIMD
-        // multiply, waves 0-3 win and waves 4-7 fill the gaps
-        if (kLockstep || grp == 0) __builtin_amdgcn_s_setprio(3);
-        else __builtin_amdgcn_s_setprio(2);
+        // the multiplying wave goes first: its next instruction frees the matrix pipe.  (Both groups at the same
+        // priority: with waves 0-3 above waves 4-7 a launch took 1.5 % longer, with no priority at all 3.7 %.)
+        __builtin_amdgcn_s_setprio(3);
         lds_operands_ready();
         __builtin_amdgcn_sched_barrier(0);  // no matrix instruction may be moved ahead of that wait
         zero_s();
