@@ -499,7 +499,7 @@ def main():
                **tm.settle(),
                "saved_forward": {"kernel_ms_mean": tm_saved.mean_ms, "tflops": flops_b / (tm_saved.mean_ms * 1e-3) / 1e12,
                                  "note": "rt_flash_backward_saved_f32_dev: O and the row statistic come from the forward "
-                                         "pass instead of being recomputed (delta + dK/dV + dQ)"},
+                                         "pass instead of being recomputed (dQ, which also forms delta, then dK/dV)"},
                "config": {"workload": "f32 unmasked attention backward (dQ, dK, dV from Q, K, V, dO), B=1 H=8 N=2048 D=64, "
                                       "U(-1,1) inputs (seed 78), tensors resident in HBM",
                           "flop_convention": "10*B*H*N*N*D: the five N x N x D products of the backward; the step also "
@@ -508,8 +508,8 @@ def main():
                "roofline": {"bound": "mfma", "achieved": flops_b / (tm.mean_ms * 1e-3) / 1e12, "peak": PEAK_F32_TFLOPS,
                             "unit": "TFLOP/s", "frac": flops_b / (tm.mean_ms * 1e-3) / 1e12 / PEAK_F32_TFLOPS,
                             "traffic": profile_traffic("flash_bwd_f32_b1_h8_n2048_d64.md", "backward_step"),
-                            "kernels": "flash_fwd_f32_splitk_kernel<2> + flash_bwd_delta_kernel + flash_bwd_f32_dkdv_kernel<2> "
-                                       "+ flash_bwd_f32_dq_kernel<2> (one event pair around the timed steps)"}}
+                            "kernels": "flash_fwd_f32_splitk_kernel<2> + flash_bwd_f32_dq_kernel<2> (with the delta prologue) "
+                                       "+ flash_bwd_f32_dkdv_kernel<2> (one event pair around the timed steps)"}}
         if not args.no_cpu:
             n_slab = Bb * Hb  # the reference's backward is a single-threaded loop; the whole workload is a second or two
             slab = Nb * Db

@@ -4,10 +4,11 @@
 // The reference rebuilds the full seq x seq matrices P, dP and dS per (batch, head).  Here nothing of that
 // size exists: the forward kernel is run once more to leave O and the row statistic L_i = m_i + ln(l_i), and
 //
-//   delta_i = sum_j P_ij dP_ij = dO_i . O_i                                   (flash_bwd_delta_kernel)
+//   delta_i = sum_j P_ij dP_ij = dO_i . O_i                                   (prologue of flash_bwd_f32_dq_kernel)
 //   P_ij    = exp(scale * Q_i.K_j - L_i),   dP_ij = dO_i . V_j,   dS_ij = P_ij (dP_ij - delta_i)
-//   dV_j = sum_i P_ij dO_i,   dK_j = scale * sum_i dS_ij Q_i                  (flash_bwd_f32_dkdv_kernel)
 //   dQ_i = scale * sum_j dS_ij K_j                                            (flash_bwd_f32_dq_kernel)
+//   dV_j = sum_i P_ij dO_i,   dK_j = scale * sum_i dS_ij Q_i                  (flash_bwd_f32_dkdv_kernel, launched second:
+//                                                                              it reads the delta the dQ kernel left)
 //
 // are recomputed 32 x 32 tile by tile on the f32 matrix cores (v_mfma_f32_32x32x2_f32).  Each output row is owned
 // by exactly one workgroup, so there are no atomics and the result does not depend on scheduling.
@@ -145,19 +146,6 @@ __device__ __forceinline__ void owner_of_block(int& bh, int& tile) {
         bh = (r / nt) * 8 + xcd;
         tile = r % nt;
     }
-}
-
-// one wave per row: delta[row] = sum_d dO[row][d] * O[row][d]
-__global__ __launch_bounds__(256) void flash_bwd_delta_kernel(const float* __restrict__ o, const float* __restrict__ d_out,
-                                                              float* __restrict__ delta, long long rows, int D) {
-    const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63;
-    if (row >= rows) return;
-    float acc = 0.0f;
-    for (int d = lane; d < D; d += kWave) acc += d_out[row * D + d] * o[row * D + d];
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-    if (lane == 0) delta[row] = acc;
 }
 
 template <int DT>  // DT = ceil(dim / 32); the head dim is zero-padded to DPAD = 32 * DT in LDS
@@ -315,9 +303,23 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dq_kerne
     float* Kt = lds + wave * 2 * TILE;
     float* Vt = Kt + TILE;
 
-    // the owner rows Q[q0 + col], dO[q0 + col] as B operands
-    stage_tile<DPAD, LD>(Kt, Qg, q0, N, D, lane, vec);
-    stage_tile<DPAD, LD>(Vt, dOg, q0, N, D, lane, vec);
+    // the owner rows Q[q0 + col], dO[q0 + col] as B operands; the O rows follow them through the tile Q was staged in
+    const bool q_ok = q0 + col < N;
+    // a row beyond seq carries the statistic +inf: all its weights come out of exp2 as exact zeros
+    float lse_q = q_ok ? p.lse[bh * (size_t)N + q0 + col] : -neg_inf();
+    const float* __restrict__ Og = p.o + base;
+    TileRegs<DPAD> r_o;
+    if (vec) {
+        TileRegs<DPAD> r_q, r_do;
+        load_tile_regs<DPAD>(r_q, Qg, q0, N, D, lane);
+        load_tile_regs<DPAD>(r_do, dOg, q0, N, D, lane);
+        store_tile_regs<DPAD, LD>(Kt, r_q, lane);
+        store_tile_regs<DPAD, LD>(Vt, r_do, lane);
+        load_tile_regs<DPAD>(r_o, Og, q0, N, D, lane);  // travels while the operand registers are filled
+    } else {
+        stage_tile<DPAD, LD>(Kt, Qg, q0, N, D, lane, false);
+        stage_tile<DPAD, LD>(Vt, dOg, q0, N, D, lane, false);
+    }
     float qreg[DPAD / 2], oreg[DPAD / 2];
 #pragma unroll
     for (int j = 0; j < DPAD / 8; j++) {
@@ -329,11 +331,21 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dq_kerne
             oreg[4 * j + i] = c[i];
         }
     }
-    const bool q_ok = q0 + col < N;
-    // a row beyond seq carries the statistic +inf: all its weights come out of exp2 as exact zeros
-    float lse_q = q_ok ? p.lse[bh * (size_t)N + q0 + col] : -neg_inf();
-    float delta_q = q_ok ? p.delta[bh * (size_t)N + q0 + col] : 0.0f;
-    // have the two loads land here: a wait for them inside the loop would also wait for the tile prefetched there
+    // delta of the owner rows, dO_i . O_i: a lane adds up the half of row `col` it holds of dO, the other half sits
+    // in lane + 32.  Every wave of the workgroup needs all 32 values and computes them itself; wave 0 leaves them in
+    // memory for the dK/dV kernel.  (Rows beyond seq and columns beyond dim are staged as zeros.)
+    if (vec) store_tile_regs<DPAD, LD>(Kt, r_o, lane);
+    else stage_tile<DPAD, LD>(Kt, Og, q0, N, D, lane, false);
+    float delta_q = 0.0f;
+#pragma unroll
+    for (int j = 0; j < DPAD / 8; j++) {
+        const f32x4_t a = *(const f32x4_t*)(Kt + col * LD + 8 * j + 4 * hh);
+#pragma unroll
+        for (int i = 0; i < 4; i++) delta_q = __builtin_fmaf(a[i], oreg[4 * j + i], delta_q);
+    }
+    delta_q += __shfl_xor(delta_q, 32, 64);
+    if (wave == 0 && hh == 0 && q_ok) p.delta[bh * (size_t)N + q0 + col] = delta_q;
+    // have the statistic land here: a wait for it inside the loop would also wait for the tile prefetched there
     asm volatile("" : "+v"(lse_q), "+v"(delta_q));
 
     f32x16_t acc_dq[DT];
@@ -441,13 +453,8 @@ hipError_t launch_flash_bwd_f32_saved(hipStream_t stream, const FlashBwdF32Param
                                       float* delta) {
     if (p_in.batch == 0 || p_in.heads == 0 || p_in.seq == 0 || p_in.dim == 0) return hipSuccess;
     if (p_in.dim > 128) return hipErrorInvalidValue;
-    const size_t rows = (size_t)p_in.batch * p_in.heads * p_in.seq;
-    hipLaunchKernelGGL(flash_bwd_delta_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, o, p_in.d_out, delta,
-                       (long long)rows, p_in.dim);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
-
     FlashBwdF32Params p = p_in;
+    p.o = o;
     p.lse = lse;
     p.delta = delta;
     auto aligned = [](const void* ptr) { return (uintptr_t)ptr % 16 == 0; };
@@ -457,20 +464,20 @@ hipError_t launch_flash_bwd_f32_saved(hipStream_t stream, const FlashBwdF32Param
     const int dt = (p.dim + 31) / 32;
     switch (dt) {
         case 1:
-            hipLaunchKernelGGL(flash_bwd_f32_dkdv_kernel<1>, grid, block, 0, stream, p);
             hipLaunchKernelGGL(flash_bwd_f32_dq_kernel<1>, grid, block, 0, stream, p);
+            hipLaunchKernelGGL(flash_bwd_f32_dkdv_kernel<1>, grid, block, 0, stream, p);
             break;
         case 2:
-            hipLaunchKernelGGL(flash_bwd_f32_dkdv_kernel<2>, grid, block, 0, stream, p);
             hipLaunchKernelGGL(flash_bwd_f32_dq_kernel<2>, grid, block, 0, stream, p);
+            hipLaunchKernelGGL(flash_bwd_f32_dkdv_kernel<2>, grid, block, 0, stream, p);
             break;
         case 3:
-            hipLaunchKernelGGL(flash_bwd_f32_dkdv_kernel<3>, grid, block, 0, stream, p);
             hipLaunchKernelGGL(flash_bwd_f32_dq_kernel<3>, grid, block, 0, stream, p);
+            hipLaunchKernelGGL(flash_bwd_f32_dkdv_kernel<3>, grid, block, 0, stream, p);
             break;
         case 4:
-            hipLaunchKernelGGL(flash_bwd_f32_dkdv_kernel<4>, grid, block, 0, stream, p);
             hipLaunchKernelGGL(flash_bwd_f32_dq_kernel<4>, grid, block, 0, stream, p);
+            hipLaunchKernelGGL(flash_bwd_f32_dkdv_kernel<4>, grid, block, 0, stream, p);
             break;
         default: return hipErrorInvalidValue;
     }

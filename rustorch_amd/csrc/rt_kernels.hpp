@@ -60,16 +60,17 @@ struct FlashBwdF32Params {
     int batch, heads, seq, dim;
     float scale;
     // filled by the launcher
+    const float* o;
     const float* lse;
-    const float* delta;
+    float* delta;  // written by the dQ kernel (its owner rows), read by the dK/dV kernel that runs after it
     int vec;
 };
 // Floats of scratch launch_flash_bwd_f32 needs (O, the row statistic and delta).
 size_t flash_bwd_f32_workspace_floats(int batch, int heads, int seq, int dim);
-// dim <= 128.  Runs the forward kernel, then delta, dK/dV and dQ on `stream`.
+// dim <= 128.  Runs the forward kernel, then dQ (which also leaves delta) and dK/dV on `stream`.
 hipError_t launch_flash_bwd_f32(hipStream_t stream, const FlashBwdF32Params& p, float* workspace, int n_cus);
 // The same from a saved forward: `o` [B,H,N,D] and `lse` [B,H,N] as launch_flash_f32 leaves them (FlashF32Params::lse);
-// `delta` is B*H*N floats of scratch.  Runs delta, dK/dV and dQ.
+// `delta` is B*H*N floats of scratch.  Runs dQ (which also leaves delta), then dK/dV.
 hipError_t launch_flash_bwd_f32_saved(hipStream_t stream, const FlashBwdF32Params& p, const float* o, const float* lse,
                                       float* delta);
 
