@@ -529,3 +529,47 @@ def mha_forward_masked(q, k, v, batch, t_q, t_kv, heads, head_dim, attn_mask=Non
 
 def max_threads() -> int:
     return lib().ro_max_threads()
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Comparison rule of the bf16 parity checks (no reference arithmetic here: a rule about two result arrays)
+BF16_MAX_ABS = 2e-2    # the absolute bar
+BF16_REL_FRO = 1e-2    # the scale-aware bar beside it, per block of rows
+
+
+def rel_fro_blocks(got, want, dim, slab_rows=None, block_rows=256, min_elems=512):
+    """Largest relative Frobenius error ``||got - want||_F / ||want||_F`` over blocks of ``block_rows`` consecutive
+    rows of ``dim`` elements, blocks never crossing a slab of ``slab_rows`` rows (one (batch, head) pair; default:
+    the whole array is one slab).  The reference's own equivalence test carries a Frobenius criterion beside the
+    max-abs one (crates/rustorch-attention/tests/equivalence.rs:79-112: ``frob < tol * sqrt(n)``); this is its
+    scale-aware form, local in the rows: late rows of a long causal prefill average thousands of V rows and are
+    small (std 1/sqrt(N)), so an absolute bar alone cannot see a dropped key tile there, the relative one does.
+    Elements that are NaN in ``want`` are left out (NaN patterns are compared exactly elsewhere); a block whose
+    ``want`` is all zero must be reproduced exactly (the result is inf otherwise).  Blocks of fewer than
+    ``min_elems`` elements are too small for a norm ratio to mean anything: the array is then taken as one block.
+    Decode outputs are compared per (sequence, head) row: ``block_rows=1, min_elems=64``."""
+    got = np.asarray(got, dtype=np.float64).reshape(-1, dim)
+    want = np.asarray(want, dtype=np.float64).reshape(-1, dim)
+    assert got.shape == want.shape
+    rows = want.shape[0]
+    if rows == 0:
+        return 0.0
+    slab_rows = slab_rows or rows
+    assert rows % slab_rows == 0
+    nan = np.isnan(want)
+    with np.errstate(invalid="ignore"):
+        diff = np.where(nan | (got == want), 0.0, got - want)  # equal infinities agree
+    diff2 = (np.nan_to_num(diff, nan=np.inf, posinf=np.inf, neginf=np.inf) ** 2).sum(axis=1)
+    ref2 = np.where(nan | np.isinf(want), 0.0, want ** 2).sum(axis=1)
+    blk = min(block_rows, slab_rows)
+    if blk * dim < min_elems:
+        num, den = np.array([diff2.sum()]), np.array([ref2.sum()])
+    else:
+        n_blk = -(-slab_rows // blk)
+        pad = n_blk * blk - slab_rows
+        d2 = np.pad(diff2.reshape(-1, slab_rows), ((0, 0), (0, pad))).reshape(-1, n_blk, blk)
+        r2 = np.pad(ref2.reshape(-1, slab_rows), ((0, 0), (0, pad))).reshape(-1, n_blk, blk)
+        num, den = d2.sum(axis=2).ravel(), r2.sum(axis=2).ravel()
+    with np.errstate(divide="ignore", invalid="ignore"):
+        rel = np.where(den > 0, np.sqrt(num / den), np.where(num > 0, np.inf, 0.0))
+    return float(rel.max())

@@ -94,22 +94,17 @@ __device__ __forceinline__ float sum_with_other_half(float x) {
     auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
-// max of the 16 scores a lane holds: eight three-input maxima in one block of assembly (separate
-// statements would each be fenced by a wait state the hardware does not need between vector instructions)
+// Max of the 16 scores a lane holds, as three chains of three-input maxima.  Written with the compiler's own max and
+// not as inline assembly: the scores are results of matrix instructions, and a vector instruction that reads a
+// matrix result needs wait states that only the compiler's hazard pass inserts (it does not look inside assembly).
+// Runs on the slow path only.
+__device__ __forceinline__ float max3(float a, float b, float c) { return __builtin_fmaxf(__builtin_fmaxf(a, b), c); }
 __device__ __forceinline__ float max16(const f32x16_t& s) {
-    float t0, t1, t2;
-    asm("v_max3_f32 %0, %3, %4, %5\n\t"
-        "v_max3_f32 %1, %6, %7, %8\n\t"
-        "v_max3_f32 %2, %9, %10, %11\n\t"
-        "v_max3_f32 %0, %0, %12, %13\n\t"
-        "v_max3_f32 %1, %1, %14, %15\n\t"
-        "v_max3_f32 %2, %2, %16, %17\n\t"
-        "v_max3_f32 %0, %0, %1, %2\n\t"
-        "v_max_f32 %0, %0, %18"
-        : "=&v"(t0), "=&v"(t1), "=&v"(t2)
-        : "v"(s[0]), "v"(s[1]), "v"(s[2]), "v"(s[3]), "v"(s[4]), "v"(s[5]), "v"(s[6]), "v"(s[7]), "v"(s[8]),
-          "v"(s[9]), "v"(s[10]), "v"(s[11]), "v"(s[12]), "v"(s[13]), "v"(s[14]), "v"(s[15]));
-    return t0;
+    float t0 = max3(s[0], s[1], s[2]), t1 = max3(s[3], s[4], s[5]), t2 = max3(s[6], s[7], s[8]);
+    t0 = max3(t0, s[9], s[10]);
+    t1 = max3(t1, s[11], s[12]);
+    t2 = max3(t2, s[13], s[14]);
+    return __builtin_fmaxf(max3(t0, t1, t2), s[15]);
 }
 // 16 bytes per lane from global memory straight into LDS: lane l lands at LDS byte address
 // lds_block + 16*l (lds_block is wave-uniform and goes through M0).  Issued as inline assembly so that the compiler's counter

@@ -37,6 +37,21 @@ def assert_close_nan(got, want, tol, label=""):
         assert d <= tol, f"{label}: max-abs {d:.3e} > {tol:.1e}"
 
 
+def assert_bf16_parity(got, want, dim, slab_rows=None, label="", block_rows=256, min_elems=512):
+    """The bar of every bf16 comparison with the oracle: NaN positions exact, max-abs <= 2e-2, and per block of 256
+    rows of a (batch, head) slab a relative Frobenius error <= 1e-2 (a kernel that loses a 32-key item of a long
+    row stays under the absolute bar and fails this one).  `slab_rows`: rows per (batch, head) pair; None takes the
+    array as one slab.  Decode outputs: one block per (sequence, head) row, see assert_decode_parity."""
+    assert_close_nan(got, want, oracle.BF16_MAX_ABS, label)
+    rel = oracle.rel_fro_blocks(got, want, dim, slab_rows, block_rows, min_elems)
+    assert rel <= oracle.BF16_REL_FRO, f"{label}: relative Frobenius error {rel:.3e} > {oracle.BF16_REL_FRO:.0e}"
+
+
+def assert_decode_parity(got, want, dim, label=""):
+    """Decode outputs [.., heads, dim]: the bf16 bar with one block per (sequence, head) row."""
+    assert_bf16_parity(got, want, dim, None, label, block_rows=1, min_elems=64)
+
+
 def flash_bf16(shape, q_bits, k_bits, v_bits, mask=None, n_kv_heads=0):
     """Run the bf16 device entry point on host bit-pattern arrays; returns f32 values of the bf16 output."""
     dq, dk, dv = dev(q_bits), dev(k_bits), dev(v_bits)

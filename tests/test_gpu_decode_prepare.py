@@ -5,6 +5,7 @@ import numpy as np
 import pytest
 
 import rustorch_amd as ra
+from _gpu import assert_decode_parity
 
 pytestmark = pytest.mark.gpu
 
@@ -140,4 +141,4 @@ def test_prepare_then_decode_matches_cpu_decode_step(oracle):
     want_q = oracle.decode_prepare_bf16(q, k, v, want_kc, want_vc, positions, qg, kg, 1e-6, oro, b_, hq, hkv, d, lmax)
     want = oracle.gqa_decode_batched_bf16(want_q, want_kc, want_vc, positions + 1, b_, hq, hkv, d, lmax)
     got = oracle.bf16_to_f32(dout.download(np.uint16))
-    assert np.abs(got - want).max() <= 2e-2
+    assert_decode_parity(got, want, d)

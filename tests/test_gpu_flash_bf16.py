@@ -1,11 +1,12 @@
 """GPU parity of the bf16 prefill kernels through the C ABI (rt_flash_forward_bf16_dev,
 rt_flash_forward_varlen_bf16_dev) against the CPU oracle run in f32 on the same bf16-rounded
-inputs.  Bar: max-abs <= 2e-2; NaN and zero-row patterns exact."""
+inputs.  Bar: max-abs <= 2e-2 and, per block of 256 query rows of a (b,h) slab, relative Frobenius error <= 1e-2;
+NaN and zero-row patterns exact."""
 import numpy as np
 import pytest
 
 import rustorch_amd as ra
-from _gpu import assert_close_nan, bf16_round, dev, flash_bf16, max_abs
+from _gpu import assert_bf16_parity, bf16_round, dev, flash_bf16, max_abs
 from _util import seeded_normal
 
 pytestmark = pytest.mark.gpu
@@ -45,7 +46,7 @@ def test_flash_bf16_matches_oracle(oracle, force_kernel, n, kernel, d):
     for mask, om in ((ra.Mask.none(), None), (ra.Mask.causal(), "causal"), (ra.Mask.padding(keep), ("padding", keep))):
         got = flash_bf16(shape, qb, kb, vb, mask)
         want = oracle.flash_forward_masked(oracle.AttentionShape(b, h, n, d), qf, kf, vf, om)
-        assert_close_nan(got, want, TOL, f"n={n} d={d} mask={mask.kind} kernel={kernel}")
+        assert_bf16_parity(got, want, d, n, f"n={n} d={d} mask={mask.kind} kernel={kernel}")
 
 
 @pytest.mark.parametrize("d", [64, 128])
@@ -61,7 +62,7 @@ def test_both_prefill_kernels_agree(oracle, force_kernel, n, d):
     for kernel in ("persistent", "tile"):
         force_kernel(kernel)
         outs[kernel] = flash_bf16(shape, qb, kb, vb, ra.Mask.causal())
-        assert_close_nan(outs[kernel], want, TOL, kernel)
+        assert_bf16_parity(outs[kernel], want, d, n, kernel)
     assert max_abs(outs["persistent"], outs["tile"]) <= TOL
 
 
@@ -88,7 +89,7 @@ def test_row_max_that_keeps_rising_along_the_keys(oracle, force_kernel, kernel, 
         got = flash_bf16(shape, qb, kb, vb, mask)
         want = oracle.flash_forward_masked(oracle.AttentionShape(b, h, n, d), qf, kf, vf, om)
         assert np.isfinite(want).all()
-        assert_close_nan(got, want, TOL, f"kernel={kernel} d={d} mask={mask.kind}")
+        assert_bf16_parity(got, want, d, n, f"kernel={kernel} d={d} mask={mask.kind}")
 
 
 def test_flash_bf16_closed_forms():
@@ -117,7 +118,7 @@ def test_flash_bf16_masks_nan_rules(oracle, force_kernel, kernel):
                  np.r_[np.zeros(63, bool), np.ones(n - 63, bool)], np.r_[np.ones(64, bool), np.zeros(n - 64, bool)]):
         got = flash_bf16(shape, qb, kb, vb, ra.Mask.padding(keep))
         want = oracle.flash_forward_masked(osh, qf, kf, vf, ("padding", keep))
-        assert_close_nan(got, want, TOL)
+        assert_bf16_parity(got, want, d, n)
     # NaN in a query row poisons that row only; NaN in a key row poisons the rows that see it
     qn = qf.copy()
     qn[5 * d + 3] = np.nan
@@ -126,7 +127,7 @@ def test_flash_bf16_masks_nan_rules(oracle, force_kernel, kernel):
     for mask, om in ((ra.Mask.causal(), "causal"), (ra.Mask.none(), None)):
         got = flash_bf16(shape, oracle.f32_to_bf16(qn), oracle.f32_to_bf16(kn), vb, mask)
         want = oracle.flash_forward_masked(osh, qn, kn, vf, om)
-        assert_close_nan(got, want, TOL)
+        assert_bf16_parity(got, want, d, n)
 
 
 @pytest.mark.parametrize("kernel", ["persistent", "tile"])
@@ -141,7 +142,7 @@ def test_flash_bf16_gqa_head_mapping(oracle, force_kernel, kernel, hq, hkv):
     kr = np.repeat(kf.reshape(b, hkv, n, d), g, axis=1)
     vr = np.repeat(vf.reshape(b, hkv, n, d), g, axis=1)
     want = oracle.flash_forward_masked(oracle.AttentionShape(b, hq, n, d), qf, kr, vr, "causal")
-    assert_close_nan(got, want, TOL)
+    assert_bf16_parity(got, want, d, n)
 
 
 def run_varlen(shape, qb, kb, vb, lens, zero=True):
@@ -166,7 +167,7 @@ def test_varlen_small(oracle, force_kernel, kernel, d):
     for zero in (True, False):
         got = run_varlen(shape, qb, kb, vb, lens, zero)
         want = oracle.varlen_causal_forward(qf, kf, vf, lens, b, h, n, d, zero_padded_rows=zero)
-        assert_close_nan(got, want, TOL)
+        assert_bf16_parity(got, want, d, n)
         if zero:
             g = got.reshape(b, h, n, d)
             for i, L in enumerate(lens):
@@ -183,7 +184,7 @@ def test_config_padded_batch_b16_h16_n1024_d64(oracle, force_kernel, kernel):
     (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d), (21, 22, 23))
     got = run_varlen(ra.AttentionShape.new(b, h, n, d), qb, kb, vb, lens)
     want = oracle.varlen_causal_forward(qf, kf, vf, lens, b, h, n, d)
-    assert_close_nan(got, want, TOL, f"lens={lens.tolist()}")
+    assert_bf16_parity(got, want, d, n, f"lens={lens.tolist()}")
     g = got.reshape(b, h, n, d)
     for i, L in enumerate(lens):
         assert (g[i, :, L:] == 0.0).all()
@@ -206,6 +207,7 @@ def test_config_prefill_b4_h32_n4096_d128(oracle):
         want = oracle.flash_forward_masked(oracle.AttentionShape(1, 1, n, d), q4[bi, hi], k4[bi, hi], v4[bi, hi],
                                            "causal").reshape(n, d)
         worst = max(worst, max_abs(got[bi, hi], want))
+        assert_bf16_parity(got[bi, hi], want, d, n, f"slab ({bi},{hi})")
     assert worst <= TOL, worst
     # rows are convex combinations of V rows
     assert (got.max(axis=2) <= v4.max(axis=2) + 1e-2).all() and (got.min(axis=2) >= v4.min(axis=2) - 1e-2).all()
@@ -227,12 +229,18 @@ def test_config_long_context_b1_h32_n16384_d128(oracle):
         m = 2048
         want = oracle.flash_forward_masked(oracle.AttentionShape(1, 1, m, d), q4[hi, :m], k4[hi, :m], v4[hi, :m],
                                            "causal").reshape(m, d)
-        assert max_abs(got[hi, :m], want) <= TOL
+        assert_bf16_parity(got[hi, :m], want, d, m, f"head {hi}, first {m} rows")
     rng = np.random.default_rng(5)
     for hi in (3, 31):
-        for i in [n - 1, n - 64, n - 65] + rng.integers(2048, n, size=5).tolist():
+        # whole 256-row blocks late in the sequence, each row through the single-row function (a key item lost
+        # there moves the block's relative error to ~0.1 and its max-abs by less than the absolute bar)
+        for r0 in (n - 256, 9 * 1024 + 512):
+            want = np.stack([oracle.gqa_forward_f32(q4[hi, i], k4[hi, :i + 1], v4[hi, :i + 1], 1, 1, 1, 1, i + 1, d)
+                             for i in range(r0, r0 + 256)])
+            assert_bf16_parity(got[hi, r0:r0 + 256], want, d, 256, f"head {hi}, rows {r0}..{r0 + 255}")
+        for i in rng.integers(2048, n, size=5).tolist():
             want = oracle.gqa_forward_f32(q4[hi, i], k4[hi, :i + 1], v4[hi, :i + 1], 1, 1, 1, 1, i + 1, d)
-            assert max_abs(got[hi, i], want) <= TOL, (hi, i)
+            assert_bf16_parity(got[hi, i], want, d, 1, f"head {hi}, row {i}")
 
 
 @pytest.mark.parametrize("d", [257, 264, 100, 4])
@@ -312,4 +320,4 @@ def test_padding_mask_longer_than_the_persistent_kernel_holds(oracle):
     q2 = qf.reshape(n, d)
     for i in (0, 1, 499, 500, 39999, 40000, 65535, 65536, 65999):
         want = oracle.gqa_forward_f32(q2[i], k2, v2, 1, 1, 1, 1, k2.shape[0], d)
-        assert max_abs(got[i], want) <= TOL, i
+        assert_bf16_parity(got[i], want, d, 1, f"row {i}")

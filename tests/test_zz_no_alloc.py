@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import rustorch_amd as ra
-from _gpu import bf16_round, dev, max_abs
+from _gpu import assert_decode_parity, bf16_round, dev
 from _util import seeded_normal
 
 pytestmark = pytest.mark.gpu
@@ -42,7 +42,7 @@ def test_noalloc_decode_equals_the_workspace_entry_on_two_calls_in_a_row(oracle)
     for b, hq, hkv, d, max_seq, lens, seed in cases:
         with_ws, static, want = both(oracle, b, hq, hkv, d, max_seq, lens, seed)
         assert np.array_equal(with_ws, static), (b, hq, hkv, d)
-        assert max_abs(oracle.bf16_to_f32(static), want) <= 2e-2
+        assert_decode_parity(oracle.bf16_to_f32(static), want, d)
 
 
 def test_noalloc_decode_limits():
