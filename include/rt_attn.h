@@ -188,11 +188,17 @@ int rt_flash_forward_f32_dev(void *stream, const rt_attention_shape *shape, uint
  * reference's forward takes any dim != 0, cpu_forward.rs:142-169; other dims return RT_ERR_UNSUPPORTED here and
  * are served by the f32 entries); tensors 16-byte aligned.  Two MFMA kernels stand behind it: a persistent
  * 8-wave kernel for dim 64 / 128 on unpadded batches of at least 512 rows per sequence and 256 jobs of 256 rows,
- * and a 4-wave tile kernel for everything else (short or few sequences, padded batches, other dims).  RT_ATTN_BF16_PREFILL=tile or =persistent in the environment forces one
- * of them where both apply. */
+ * and a 4-wave tile kernel for everything else (short or few sequences, padded batches, other dims).
+ * rt_debug_force_bf16_prefill_kernel forces one of them where both apply. */
 int rt_flash_forward_bf16_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const void *q,
                               const void *k, const void *v, int mask_kind, const uint8_t *keep, void *out,
                               rt_err_detail *err);
+
+/* No counterpart in the reference: a switch for measurements and tests.  which = 0 lets the library choose between
+ * its two bf16 prefill kernels (the default), 1 forces the tile kernel, 2 the persistent kernel where it applies
+ * (head dim 64 / 128, no per-sequence lengths).  Process-wide; until it is called the value is taken, once, from
+ * RT_ATTN_BF16_PREFILL=tile|persistent in the environment.  Returns RT_ERR_UNSUPPORTED for another value. */
+int rt_debug_force_bf16_prefill_kernel(int which);
 
 /* The same two calls on tensors laid out [batch, seq, heads, dim] (k/v: [batch, seq, n_kv_heads, dim]),
  * the layout rustorch_nn::MultiHeadAttention holds its projections in: the kernels walk the rows with a
@@ -291,10 +297,14 @@ int rt_qk_norm_rope_kv_append_bf16(void *stream, void *q, const void *k_in, cons
  * [n_heads,head_dim] bf16, caches [n_kv,max_seq,head_dim] bf16 of which [..kv_len] is read;
  * kv head = h*n_kv/n_heads; f32 accumulation, output rounded once.  Runs the split-K kernels of the batched entry on
  * a batch of one (head_dim 64, 128 or 256, at most 16 query heads per kv head; other shapes take a one-workgroup-per-head
- * kernel).  The reference's signature has no workspace: the partials go to a buffer the library keeps per
- * (device, stream), allocated by the first call on a stream (so that call must not be under stream capture; later
- * calls allocate nothing unless max_seq grows; a grown buffer replaces the old one, which is kept until
- * rt_stream_destroy / rt_shutdown, so concurrent callers never see freed memory).  q and the caches should be
+ * kernel).  The reference's signature has no workspace and its launcher allocates nothing (llm_kernels.rs:915-958):
+ * the partials go to a slot of a fixed 32 MiB block of device memory inside the library (8 slots of 4 MiB; a
+ * (device, stream) pair takes a free slot on its first call and keeps it until rt_stream_destroy / rt_shutdown, so
+ * calls on different streams never share scratch), and the call allocates nothing: it may be the first call on a
+ * stream and may be recorded into a HIP graph.  Only a ninth concurrent stream, or a shape whose partials do not fit a
+ * slot (more than ~250 kv heads at 16 query heads each and head_dim 256), falls back to a buffer the library allocates
+ * per (device, stream) on that stream's first call (then not under capture; a grown buffer replaces the old one,
+ * which is kept until rt_stream_destroy / rt_shutdown).  q and the caches should be
  * 16-byte aligned: the split-K kernels move 16 bytes per lane, and tensors that are not aligned take the
  * one-workgroup-per-head kernel instead (same results, slower). */
 int rt_gqa_decode_online_bf16(void *stream, const void *q, const void *k_cache, const void *v_cache, void *out,
@@ -365,6 +375,12 @@ int rt_buf_free(void *ptr, rt_err_detail *err);
  * fill kernel (safe to record into a HIP graph).  The reference's caches start as vec![0.0; n]
  * (crates/rustorch-nn/src/kv_cache.rs:63-66). */
 int rt_buf_zero(void *ptr, size_t bytes, void *stream, rt_err_detail *err);
+/* No counterpart in the reference (its decode loop keeps the position on the host, crates/rustorch-llm/src/
+ * cuda_backend.rs:516-556): adds `delta` to each of the `n` int32 values at device address `ptr`, asynchronously on
+ * `stream`.  A decode loop recorded into a HIP graph keeps its positions and context lengths on the device (the
+ * `positions` of rt_qk_norm_rope_kv_append_bf16, the `kv_lens` of the batched decode entries) and advances them
+ * with this call at the end of every token. */
+int rt_i32_add_dev(void *stream, int32_t *ptr, size_t n, int32_t delta, rt_err_detail *err);
 int rt_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream, rt_err_detail *err);
 int rt_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream, rt_err_detail *err);
 int rt_stream_synchronize(void *stream, rt_err_detail *err);

@@ -8,6 +8,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <vector>
@@ -215,6 +216,49 @@ void release_stream_ws(StreamWs& w) {
     w.retired.clear();
 }
 
+// Scratch that needs no allocation: the library's second fixed block is cut into rt::kStreamSlots slots, and a
+// (device, stream) pair is given one the first time it asks (host bookkeeping only: nothing is allocated, so the
+// call may be the first one under stream capture).  A stream keeps its slot until rt_stream_destroy / rt_shutdown;
+// when all slots are taken the caller falls back to stream_workspace.
+struct SlotTable {
+    hipStream_t owner[rt::kStreamSlots] = {};
+    bool used[rt::kStreamSlots] = {};
+};
+std::map<int, SlotTable> g_slots;  // per device; guarded by g_ws_mutex
+
+// The slot of `stream` on the current device (taking a free one if it has none yet): its scratch and size, or
+// *ptr = nullptr when no slot is free.
+int stream_slot_scratch(hipStream_t stream, float** ptr, size_t* bytes, rt_err_detail* err) {
+    *ptr = nullptr;
+    *bytes = 0;
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev), "hipGetDevice");
+    int slot = -1;
+    {
+        std::lock_guard<std::mutex> lock(g_ws_mutex);
+        SlotTable& t = g_slots[dev];
+        for (int i = 0; i < rt::kStreamSlots && slot < 0; i++)
+            if (t.used[i] && t.owner[i] == stream) slot = i;
+        for (int i = 0; i < rt::kStreamSlots && slot < 0; i++)
+            if (!t.used[i]) {
+                t.used[i] = true;
+                t.owner[i] = stream;
+                slot = i;
+            }
+    }
+    if (slot < 0) return RT_OK;
+    HIP_TRY(rt::stream_static_scratch(slot, ptr, bytes), "hipGetSymbolAddress(stream scratch)");
+    return RT_OK;
+}
+
+// the caller holds g_ws_mutex
+void release_stream_slot(int dev, hipStream_t stream) {
+    auto it = g_slots.find(dev);
+    if (it == g_slots.end()) return;
+    for (int i = 0; i < rt::kStreamSlots; i++)
+        if (it->second.used[i] && it->second.owner[i] == stream) it->second.used[i] = false;
+}
+
 struct DevPtr {  // a device address inside a Stage's block
     void* p = nullptr;
 };
@@ -349,6 +393,7 @@ RT_API int rt_init(int device, rt_err_detail* err) {
     float* scratch = nullptr;
     size_t scratch_bytes = 0;
     HIP_TRY(rt::decode_static_scratch(&scratch, &scratch_bytes), "hipGetSymbolAddress(static scratch)");
+    HIP_TRY(rt::stream_static_scratch(0, &scratch, &scratch_bytes), "hipGetSymbolAddress(stream scratch)");
     return RT_OK;
 }
 
@@ -655,12 +700,26 @@ RT_API int rt_flash_forward_f32_dev(void* stream, const rt_attention_shape* shap
 // on unpadded batches with at least 512 rows per sequence and a job for every CU, and the 4-wave tile kernel
 // everything else.
 enum class PrefillKernel { kAuto, kTile, kPersistent };
-static PrefillKernel prefill_kernel_override() {
-    const char* e = getenv("RT_ATTN_BF16_PREFILL");
+// A debug switch for measurements and tests, not part of the reference's surface: rt_debug_force_bf16_prefill_kernel
+// sets it; until that is called, the value is what RT_ATTN_BF16_PREFILL=tile|persistent held when the library made its
+// first bf16 prefill call (read once: a later change of the environment does not change which kernel a caller gets).
+static PrefillKernel parse_prefill_kernel(const char* e) {
     if (!e) return PrefillKernel::kAuto;
     if (strcmp(e, "tile") == 0) return PrefillKernel::kTile;
     if (strcmp(e, "persistent") == 0) return PrefillKernel::kPersistent;
     return PrefillKernel::kAuto;
+}
+static std::atomic<int> g_prefill_forced{-1};  // -1: not set through the API
+static PrefillKernel prefill_kernel_override() {
+    const int f = g_prefill_forced.load(std::memory_order_relaxed);
+    if (f >= 0) return (PrefillKernel)f;
+    static const PrefillKernel once = parse_prefill_kernel(getenv("RT_ATTN_BF16_PREFILL"));
+    return once;
+}
+RT_API int rt_debug_force_bf16_prefill_kernel(int which) {
+    if (which < 0 || which > 2) return RT_ERR_UNSUPPORTED;
+    g_prefill_forced.store(which, std::memory_order_relaxed);
+    return RT_OK;
 }
 
 static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads, const void* q,
@@ -679,12 +738,18 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
     // the tile kernel's grid is (heads, batch, query tiles of 128 rows), each dimension below 2^16
     if (shape->heads > 65535 || shape->batch > 65535 || (shape->seq + 127) / 128 > 65535)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 16, 0, "bf16 flash kernels need 16-byte aligned tensors");
+    if (!q || !k || !v || !out || (mask == rt::kMaskPadding && !keep) || (mask == rt::kMaskVarlenCausal && !seq_lens))
+        return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    rc = ensure_device(err);
+    if (rc) return rc;
     // the persistent kernel needs a job (256 query rows of one head) for every CU and gains on the tile kernel as the
     // rows get longer; a padded batch is a set of jobs of very different lengths, which the tile kernel's
     // dispatcher-balanced workgroups handle better
     const bool persistent_dim = shape->dim == 64 || shape->dim == 128;
     const uint64_t jobs256 = (shape->seq + 255) / 256 * shape->batch * shape->heads;
-    bool persistent = persistent_dim && shape->seq >= 512 && jobs256 >= 256 && mask != rt::kMaskVarlenCausal;
+    bool persistent = persistent_dim && shape->seq >= 512 && jobs256 >= (uint64_t)g_num_cus && mask != rt::kMaskVarlenCausal;
     const PrefillKernel forced = prefill_kernel_override();
     if (forced == PrefillKernel::kTile) persistent = false;
     if (forced == PrefillKernel::kPersistent && persistent_dim) persistent = true;
@@ -693,12 +758,6 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
         const uint64_t pitch_b = (bnhd ? shape->heads : 1) * shape->dim * 2;
         if (shape->seq * pitch_b >= (1ull << 32)) persistent = false;
     }
-    if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0)
-        return fail(err, RT_ERR_UNSUPPORTED, -1, 16, 0, "bf16 flash kernels need 16-byte aligned tensors");
-    if (!q || !k || !v || !out || (mask == rt::kMaskPadding && !keep) || (mask == rt::kMaskVarlenCausal && !seq_lens))
-        return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
-    rc = ensure_device(err);
-    if (rc) return rc;
     const int dim = (int)shape->dim;
     rt::TensorLayout lq, lkv;
     if (bnhd) {
@@ -1116,12 +1175,35 @@ RT_API int rt_gqa_decode_online_bf16(void* stream, const void* q, const void* k_
     // element-wise kernel below
     const bool aligned = ((((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0);
     if (aligned && rt::decode_split_supported(n_heads, n_kv, head_dim)) {
-        // the split-K kernels of the batched entry, on a batch of one; their partials go to a buffer the library keeps
-        // per stream (the reference's signature has no workspace argument)
-        float* ws = nullptr;
-        rc = stream_workspace((hipStream_t)stream, rt::decode_split_workspace_bytes(1, n_heads, head_dim, max_seq), &ws, err);
-        if (rc) return rc;
+        // the split-K kernels of the batched entry, on a batch of one.  The reference's signature has no workspace
+        // argument: the partials go to this stream's slot of the library's fixed scratch block (nothing is allocated,
+        // so the call can be captured into a graph), in the compact slot numbering; only when no slot is free, or the
+        // slot cannot hold a useful number of partials, to a buffer the library allocates per stream
         rt::DecodeSplitParams sp{};
+        sp.span_min = rt::decode_split_span_min(1);
+        // no more one-wave workgroups than there are spans of the minimum length (short contexts)
+        const long long steps = (long long)n_kv * ((kv_len + 31) / 32);
+        const long long spans = (steps + sp.span_min - 1) / sp.span_min;
+        sp.n_waves = (int)std::min<long long>(g_decode_waves, std::max<long long>(spans, 1));
+        float* ws = nullptr;
+        size_t slot_bytes = 0;
+        rc = stream_slot_scratch((hipStream_t)stream, &ws, &slot_bytes, err);
+        if (rc) return rc;
+        if (ws) {
+            // compact numbering: (waves + n_kv) * group partials of head_dim + 2 floats
+            const size_t per_wave = (size_t)(n_heads / n_kv) * ((size_t)head_dim + 2) * sizeof(float);
+            const long long fit = (long long)(slot_bytes / per_wave) - n_kv;
+            if (fit >= std::min<long long>(sp.n_waves, 256)) {
+                sp.n_waves = (int)std::min<long long>(sp.n_waves, fit);
+                sp.compact = 1;
+            } else {
+                ws = nullptr;
+            }
+        }
+        if (!ws) {
+            rc = stream_workspace((hipStream_t)stream, rt::decode_split_workspace_bytes(1, n_heads, head_dim, max_seq), &ws, err);
+            if (rc) return rc;
+        }
         sp.q = (const uint16_t*)q;
         sp.k_cache = (const uint16_t*)k_cache;
         sp.v_cache = (const uint16_t*)v_cache;
@@ -1135,11 +1217,6 @@ RT_API int rt_gqa_decode_online_bf16(void* stream, const void* q, const void* k_
         sp.dim = head_dim;
         sp.max_seq = max_seq;
         sp.n_part = rt::decode_split_parts(1, max_seq);
-        sp.span_min = rt::decode_split_span_min(1);
-        // no more one-wave workgroups than there are spans of the minimum length (short contexts)
-        const long long steps = (long long)n_kv * ((kv_len + 31) / 32);
-        const long long spans = (steps + sp.span_min - 1) / sp.span_min;
-        sp.n_waves = (int)std::min<long long>(g_decode_waves, std::max<long long>(spans, 1));
         sp.scale_log2e = (1.0f / sqrtf((float)head_dim)) * rt::kLog2eHost;
         HIP_TRY(rt::launch_decode_split((hipStream_t)stream, sp), "decode_split launch");
         return RT_OK;
@@ -1384,6 +1461,25 @@ RT_API int rt_buf_zero(void* ptr, size_t bytes, void* stream, rt_err_detail* err
     return RT_OK;
 }
 
+namespace {
+__global__ __launch_bounds__(256) void i32_add_kernel(int32_t* p, size_t n, int32_t delta) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] += delta;
+}
+}  // namespace
+
+RT_API int rt_i32_add_dev(void* stream, int32_t* ptr, size_t n, int32_t delta, rt_err_detail* err) {
+    clear_err(err);
+    if (n == 0) return RT_OK;
+    if (!ptr) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    if (((uintptr_t)ptr & 3) || n > ((size_t)1 << 30)) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, (uint64_t)n, "int32 add works on up to 2^30 aligned values");
+    int rc = ensure_device(err);
+    if (rc) return rc;
+    hipLaunchKernelGGL(i32_add_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, ptr, n, delta);
+    HIP_TRY(hipGetLastError(), "i32_add launch");
+    return RT_OK;
+}
+
 RT_API int rt_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream, rt_err_detail* err) {
     clear_err(err);
     if (bytes == 0) return RT_OK;
@@ -1432,6 +1528,7 @@ RT_API int rt_stream_destroy(void* stream, rt_err_detail* err) {
                 release_stream_ws(it->second);
                 g_ws.erase(it);
             }
+            release_stream_slot(dev, (hipStream_t)stream);
         }
     }
     HIP_TRY(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy");
@@ -1449,6 +1546,7 @@ RT_API int rt_shutdown(rt_err_detail* err) {
             release_stream_ws(kv.second);
         }
         g_ws.clear();
+        g_slots.clear();
     }
     {
         std::lock_guard<std::mutex> lock(g_pinned_mutex);

@@ -613,6 +613,36 @@ hipError_t decode_static_scratch(float** ptr, size_t* bytes) {
     return hipSuccess;
 }
 
+// ---- scratch slots for entry points whose reference signature has no workspace ----------------------------------
+// A second fixed block, cut into kStreamSlots slots of kStreamSlotBytes: the host side hands a slot to a stream the
+// first time an entry point needs scratch on it (no allocation, so such a call can be the first one under stream
+// capture), and calls on different streams never share a slot.  As above, the array's name is only a handle for
+// hipGetSymbolAddress.
+static __device__ __align__(256) unsigned char stream_scratch[(size_t)kStreamSlots * kStreamSlotBytes];
+
+namespace {
+void* g_stream_scratch_ptr[kMaxDevices] = {};
+}  // namespace
+
+hipError_t stream_static_scratch(int slot, float** ptr, size_t* bytes) {
+    if (slot < 0 || slot >= kStreamSlots) return hipErrorInvalidValue;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_stream_scratch_ptr[dev]) {
+        void* addr = nullptr;
+        e = hipGetSymbolAddress(&addr, HIP_SYMBOL(stream_scratch));
+        if (e != hipSuccess) return e;
+        if (!addr) return hipErrorInvalidSymbol;
+        g_stream_scratch_ptr[dev] = addr;
+    }
+    *ptr = (float*)((unsigned char*)g_stream_scratch_ptr[dev] + (size_t)slot * kStreamSlotBytes);
+    *bytes = kStreamSlotBytes;
+    return hipSuccess;
+}
+
 hipError_t launch_decode_split(hipStream_t stream, const DecodeSplitParams& p) {
     if (p.batch == 0 || p.heads == 0) return hipSuccess;
     if (p.n_waves <= 0 || p.span_min <= 0) return hipErrorInvalidValue;

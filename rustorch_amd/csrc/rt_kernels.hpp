@@ -173,6 +173,12 @@ size_t decode_split_compact_bytes(int batch, int heads, int kv_heads, int dim, i
 // held until the process ends).  Looks its address up once per device (the device must be current) and returns it
 // with its size.
 hipError_t decode_static_scratch(float** ptr, size_t* bytes);
+// A second fixed block, cut into slots: scratch for the entry points whose reference signature has no workspace
+// argument.  The host side hands one slot to each (device, stream) that needs one, so calls on different streams
+// never share scratch.  Returns the address of a slot on the current device and its size.
+constexpr int kStreamSlots = 8;
+constexpr size_t kStreamSlotBytes = (size_t)4 << 20;
+hipError_t stream_static_scratch(int slot, float** ptr, size_t* bytes);
 hipError_t launch_decode_split(hipStream_t stream, const DecodeSplitParams& p);
 
 // KVLayerCache::append on device buffers of 2- or 4-byte elements: [batch_heads, seq_added, head_dim] into

@@ -111,14 +111,28 @@ def shutdown():
     raise_for(L.lib().rt_shutdown(C.byref(err)), err)
 
 
+def i32_add_dev(buf, n: int, delta: int, stream=None):
+    """Adds `delta` to the `n` int32 values of a device buffer, asynchronously on `stream` (positions and context
+    lengths of a decode loop that lives in a HIP graph)."""
+    err = L.RtErr()
+    raise_for(L.lib().rt_i32_add_dev(stream, dev_ptr(buf), n, delta, C.byref(err)), err)
+
+
+def debug_force_bf16_prefill_kernel(name: str = "auto"):
+    """Measurement / test switch: "auto", "tile" or "persistent" for the bf16 prefill entries."""
+    rc = L.lib().rt_debug_force_bf16_prefill_kernel({"auto": 0, "tile": 1, "persistent": 2}[name])
+    if rc:
+        raise ValueError(name)
+
+
 def dev_ptr(x) -> int:
     """Raw device address of a HipStorage, a torch tensor on the GPU, or an int."""
     if x is None:
         return None
     if isinstance(x, HipStorage):
         return x.ptr
-    if isinstance(x, int):
-        return x
+    if isinstance(x, (int, np.integer)):
+        return int(x)
     if hasattr(x, "data_ptr"):
         assert x.is_cuda and x.is_contiguous(), "device entry points take contiguous GPU tensors"
         return x.data_ptr()

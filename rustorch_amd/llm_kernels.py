@@ -94,7 +94,7 @@ class LlmKernels:
         [B,Hkv,max_seq,D] already holding the new positions; `kv_lens` a device int32[B] buffer of key counts that
         include the new positions, or an int used for every sequence."""
         err = L.RtErr()
-        if isinstance(kv_lens, (int,)):
+        if isinstance(kv_lens, (int, np.integer)):
             lens_ptr, kv_len = None, int(kv_lens)
         else:
             lens_ptr, kv_len = dev_ptr(kv_lens), 0

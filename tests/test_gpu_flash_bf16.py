@@ -20,17 +20,16 @@ def inputs(shape_q, shape_kv, seeds=(1, 2, 3), q_mul=1.0):
     return bf16_round(q), bf16_round(k), bf16_round(v)
 
 
-# (kernel forced through RT_ATTN_BF16_PREFILL, head dim): the persistent 8-wave kernel covers 64 and 128, the
+# (kernel forced through rt_debug_force_bf16_prefill_kernel, head dim): the persistent 8-wave kernel covers 64 and 128, the
 # 4-wave tile kernel every multiple of 8 up to 256 (zero-padded to 32 / 64 / 96 / 128 / 256 in LDS)
 KERNEL_DIMS = [("persistent", 64), ("persistent", 128), ("tile", 32), ("tile", 64), ("tile", 80), ("tile", 96),
                ("tile", 128), ("tile", 8), ("tile", 200), ("tile", 256)]
 
 
 @pytest.fixture
-def force_kernel(monkeypatch):
-    def force(name):
-        monkeypatch.setenv("RT_ATTN_BF16_PREFILL", name)
-    return force
+def force_kernel():
+    yield ra.debug_force_bf16_prefill_kernel
+    ra.debug_force_bf16_prefill_kernel("auto")
 
 
 @pytest.mark.parametrize("kernel,d", KERNEL_DIMS)

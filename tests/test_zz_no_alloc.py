@@ -1,6 +1,8 @@
 """rt_gqa_decode_batched_bf16_noalloc (the decode entry that allocates nothing: its split-K partials live in a fixed
 block of device memory inside the library) against rt_gqa_decode_batched_bf16 with a caller workspace, through the
 C ABI.  Same kernels, same arithmetic: the outputs must be equal bit for bit, and within 2e-2 of the CPU oracle."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -10,6 +12,16 @@ from _util import seeded_normal
 
 pytestmark = pytest.mark.gpu
 K = ra.LlmKernels()
+
+
+_hip = C.CDLL("libamdhip64.so")
+_hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+
+
+def device_free_bytes():
+    free, total = C.c_size_t(), C.c_size_t()
+    assert _hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
 
 
 def both(oracle, b, hq, hkv, d, max_seq, lens, seed):
@@ -26,7 +38,9 @@ def both(oracle, b, hq, hkv, d, max_seq, lens, seed):
         if entry == "ws":
             K.gqa_decode_batched_bf16(None, dq, dk, dv, dout, dl, b, hq, hkv, d, max_seq, ws, ws.byte_len)
         else:
+            free_before = device_free_bytes()
             K.gqa_decode_batched_bf16_noalloc(None, dq, dk, dv, dout, dl, b, hq, hkv, d, max_seq)
+            assert device_free_bytes() == free_before, "the no-allocation entry changed the free device memory"
         ra.synchronize()
         outs.append(dout.download(np.uint16))
     want = oracle.gqa_decode_batched_bf16(qb, kb, vb, lens, b, hq, hkv, d, max_seq)
@@ -38,7 +52,10 @@ def test_noalloc_decode_equals_the_workspace_entry_on_two_calls_in_a_row(oracle)
     # a large ragged batch first, then a smaller one: the second call finds the first call's partials in the block
     cases = [(12, 32, 8, 128, 2100, [2100, 1, 511, 512, 513, 0, 1025, 77, 2048, 1500, 33, 900], 11),
              (3, 8, 2, 64, 300, [300, 17, 129], 21),
-             (2, 16, 4, 256, 200, [200, 64], 31)]
+             (2, 16, 4, 256, 200, [200, 64], 31),
+             # one sequence: spans of two steps, ~125 partials per head, the merge that folds them four ways in parallel
+             (1, 32, 8, 128, 8192, [8001], 41),
+             (1, 8, 2, 64, 100, [33], 51)]
     for b, hq, hkv, d, max_seq, lens, seed in cases:
         with_ws, static, want = both(oracle, b, hq, hkv, d, max_seq, lens, seed)
         assert np.array_equal(with_ws, static), (b, hq, hkv, d)
