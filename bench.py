@@ -423,6 +423,55 @@ def main():
                                    "GB/s": (2 * Hkv * kv_len * Dd * 2 + 2 * Hq * Dd * 2) / (t1.mean_ms * 1e-3) / 1e9}
         decode["single_sequence"] = dict(single, note="rt_gqa_decode_online_bf16, 32 q / 8 kv heads, D=128: two launches "
                                                       "per call, issued back to back from the host")
+        # several new positions of ONE sequence against its long cache, each causal to itself (the reference's
+        # gqa_decode_batched_f32 call shape): the keys are cut into spans, a second kernel folds the partials.  Every
+        # call reads another sequence's slab of the rotated caches (192 slabs of 34 MB), so none finds its keys in
+        # the last-level cache.
+        chunk = {}
+        slab_bytes = Hkv * Lmax * Dd * 2
+        for s_new in (4, 16):
+            q_c = oracle.f32_to_bf16(np.random.default_rng(90 + s_new).standard_normal(s_new * Hq * Dd, dtype=np.float32))
+            d_qc = ra.HipStorage.from_numpy(q_c)
+            d_oc = ra.HipStorage(s_new * Hq * Dd * 2)
+
+            def launch_chunk(i, d_qc=d_qc, d_oc=d_oc, s_new=s_new):
+                k_, v_ = sets[(i // Bd) % n_sets]
+                off = (i % Bd) * slab_bytes
+                K.gqa_decode_chunk_bf16(stream, d_qc, k_.ptr + off, v_.ptr + off, d_oc, Lmax, 1, s_new, Hq, Hkv, Dd, Lmax)
+
+            tc = time_steps(hip, stream, launch_chunk, args.steps, args.warmup)
+            bytes_c = float(2 * Hkv * Lmax * Dd * 2 + 2 * s_new * Hq * Dd * 2)
+            leg_c = {"us_per_call": tc.mean_ms * 1e3, **spread(tc.per), **tc.settle(), "algorithmic_bytes": bytes_c,
+                     "roofline": {"bound": "hbm", "achieved": bytes_c / (tc.mean_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                                  "unit": "GB/s", "frac": bytes_c / (tc.mean_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                  "traffic": profile_traffic("chunk_decode_b1_hq32_hkv8_d128_ctx8192.md", f"chunk_{s_new}"),
+                                  "kernels": "flash_tile_bf16_kernel<128, causal, packed, split> + flash_split_merge_kernel "
+                                             "(one event pair around the timed calls)"}}
+            if not args.no_cpu:
+                K.gqa_decode_chunk_bf16(stream, d_qc, sets[0][0], sets[0][1], d_oc, Lmax, 1, s_new, Hq, Hkv, Dd, Lmax)
+                hip.sync()
+                got_c = oracle.bf16_to_f32(d_oc.download(np.uint16))
+                n_slab = Hkv * Lmax * Dd
+                t0 = time.perf_counter()
+                want_c = oracle.gqa_decode_chunk_bf16(q_c, kc[:n_slab], vc[:n_slab], [Lmax], 1, s_new, Hq, Hkv, Dd, Lmax,
+                                                      threads=threads)
+                cpu_c = time.perf_counter() - t0
+                err_c = float(np.abs(got_c - want_c).max())
+                rel_c = oracle.rel_fro_blocks(got_c, want_c, Dd, block_rows=1, min_elems=64)
+                leg_c["parity_max_abs"], leg_c["parity_rel_fro"] = err_c, rel_c
+                leg_c["cpu_baseline"] = {"value": bytes_c / cpu_c / 1e9, "unit": "GB/s", "cores": min(threads, Hq),
+                                         "kind": "port",
+                                         "sample": f"one call ({cpu_c * 1e3:.0f} ms): the shader's four phases per (position, "
+                                                   f"head), one task per head; K and V are read once per query head and "
+                                                   f"position there, once per kv head in the byte count"}
+                if not (err_c <= oracle.BF16_MAX_ABS and rel_c <= oracle.BF16_REL_FRO):
+                    print(f"PARITY FAILURE: chunk decode seq_new={s_new} max-abs {err_c}, relative {rel_c}", file=sys.stderr)
+                    sys.exit(1)
+            chunk[str(s_new)] = leg_c
+        decode["chunk_decode"] = dict(chunk, config={"workload": "bf16 chunked causal decode of one sequence: batch 1, 32 q / 8 kv "
+                                                                 "heads, D=128, seq_new new positions (4, 16) over a cache "
+                                                                 "that holds 8192 keys with them (pos_base = 8192 - seq_new), "
+                                                                 "rt_gqa_decode_chunk_bf16 with a host length"})
         if not args.no_cpu:
             got = oracle.bf16_to_f32(d_o.download(np.uint16))
             t0 = time.perf_counter()

@@ -298,11 +298,11 @@ int rt_qk_norm_rope_kv_append_bf16(void *stream, void *q, const void *k_in, cons
  * kv head = h*n_kv/n_heads; f32 accumulation, output rounded once.  Runs the split-K kernels of the batched entry on
  * a batch of one (head_dim 64, 128 or 256, at most 16 query heads per kv head; other shapes take a one-workgroup-per-head
  * kernel).  The reference's signature has no workspace and its launcher allocates nothing (llm_kernels.rs:915-958):
- * the partials go to a slot of a fixed 32 MiB block of device memory inside the library (8 slots of 4 MiB; a
+ * the partials go to a slot of a fixed 64 MiB block of device memory inside the library (8 slots of 8 MiB; a
  * (device, stream) pair takes a free slot on its first call and keeps it until rt_stream_destroy / rt_shutdown, so
  * calls on different streams never share scratch), and the call allocates nothing: it may be the first call on a
  * stream and may be recorded into a HIP graph.  Only a ninth concurrent stream, or a shape whose partials do not fit a
- * slot (more than ~250 kv heads at 16 query heads each and head_dim 256), falls back to a buffer the library allocates
+ * slot (more than ~500 kv heads at 16 query heads each and head_dim 256), falls back to a buffer the library allocates
  * per (device, stream) on that stream's first call (then not under capture; a grown buffer replaces the old one,
  * which is kept until rt_stream_destroy / rt_shutdown).  q and the caches should be
  * 16-byte aligned: the split-K kernels move 16 bytes per lane, and tensors that are not aligned take the
@@ -343,8 +343,13 @@ int rt_gqa_decode_batched_bf16(void *stream, const void *q, const void *k_cache,
  * the cache INCLUDING the new ones, or NULL: every sequence has `kv_len`.  Position s of sequence b sees keys
  * [0, kv_lens[b] - seq_new + s]: pos_base of the reference is kv_lens[b] - seq_new.  batch = 1, kv_lens = NULL,
  * kv_len = pos_base + B is the reference call; seq_new = 1 is rt_gqa_decode_batched_bf16.  kv head = h / (n_heads /
- * n_kv).  A position that sees no key (kv_lens[b] < seq_new - s) gives a NaN row.  head_dim up to 256, a multiple of 8;
- * tensors 16-byte aligned; no workspace.  Asynchronous on `stream`. */
+ * n_kv).  A position that sees no key (kv_lens[b] < seq_new - s) gives a row of +0.0, as the batched entry does for
+ * kv_lens[b] == 0 (the shader's loops run zero times and leave acc = 0.0); kv_lens[b] above max_seq counts as
+ * max_seq.  head_dim up to 256, a multiple of 8; tensors 16-byte aligned.  When the batch has fewer (sequence, kv
+ * head, 128-row tile) units than the GPU has CUs and the cache is at least four key tiles long -- one sequence over
+ * a long cache, the reference's call -- the keys are cut into spans, each span's (o, m, l) partials go to the
+ * stream's slot of the library's fixed scratch block (see rt_gqa_decode_online_bf16: no allocation) and a second
+ * kernel folds them.  Asynchronous on `stream`. */
 int rt_gqa_decode_chunk_bf16(void *stream, const void *q, const void *k_cache, const void *v_cache, void *out,
                              const int32_t *kv_lens, int32_t kv_len, int32_t batch, int32_t seq_new, int32_t n_heads,
                              int32_t n_kv, int32_t head_dim, int32_t max_seq, rt_err_detail *err);

@@ -641,8 +641,10 @@ RO_EXPORT void ro_gqa_decode_batched_bf16(const uint16_t *q, const uint16_t *k_c
  * shader).  Phases as in the shader: scores = dot * inv_sqrt_d; max; e = exp(score - max); sum; weights =
  * e * (1 / sum); out[d] = sum_p weights[p] * v[p][d] in ascending p.  q/out [B,seq_new,Hq,D] (position-major, the
  * shader's q + b * n_heads * head_dim + q_h * head_dim), caches [B,Hkv,max_seq,D]; kv head = q_h / (Hq / Hkv).
- * bf16 bit patterns in, f32 out.  A position with no visible key (kv_lens[b] - seq_new + s < 0) has an empty
- * softmax: the shader would divide 0 by 0; the row is NaN here. */
+ * bf16 bit patterns in, f32 out.  A position with no visible key (kv_lens[b] - seq_new + s < 0; cannot happen in
+ * the reference, whose kv_len is at least 1) runs every loop of the shader zero times: inv_sum = 1/0 is formed but
+ * never multiplied into anything, and phase D writes acc = 0.0 -- a row of zeros, the same outcome as
+ * decode_attn_row's and the CUDA kernel's for an empty context (gqa.rs:260-261, llm_kernels.rs:456). */
 RO_EXPORT void ro_gqa_decode_chunk_bf16(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache,
                                         const int32_t *kv_lens, float *out, int batch, int seq_new, int n_heads,
                                         int n_kv, int head_dim, int max_seq, int threads) {
@@ -663,7 +665,7 @@ RO_EXPORT void ro_gqa_decode_chunk_bf16(const uint16_t *q, const uint16_t *k_cac
             long kv_len = pos_base + s + 1;
             if (kv_len > max_seq) kv_len = max_seq;
             if (kv_len <= 0) {
-                for (size_t d = 0; d < D; d++) op[d] = NAN;
+                for (size_t d = 0; d < D; d++) op[d] = 0.0f;
                 continue;
             }
             float max_score = -INFINITY;

@@ -101,8 +101,16 @@ struct TileCfg {
 // matrix pipe and the vector pipe busy at once instead of running the three phases of an item back to back.
 // K therefore sits in LDS one tile ahead of V: during tile t the waves read K(t+1) and V(t-1), and after the
 // tile's one barrier (behind the step of its first item) K(t+2) and V(t+1) are parked over K(t) and V(t-1).
-template <int DP, int MODE, bool BIAS, bool PACKED>
+//
+// SPLIT (packed rows only): the keys of a (sequence, kv head) are cut into p.n_splits spans of whole tiles, a
+// workgroup walks one span and leaves the unnormalised O, the running max and the row sum of its rows as a partial
+// (o, m, l); flash_split_merge_kernel folds the partials with the online-softmax monoid
+// (crates/rustorch-attention/src/online_softmax.rs:105-131 extended with o) -- the split over the context of the
+// decode kernels, for a chunk of new positions over one long cache, whose few query tiles would otherwise keep a
+// handful of CUs busy.
+template <int DP, int MODE, bool BIAS, bool PACKED, bool SPLIT = false>
 __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : TileCfg<DP>::OCC) void flash_tile_bf16_kernel(FlashTileParams p) {
+    static_assert(!SPLIT || (PACKED && !BIAS && MODE == kMaskCausal), "the split over the keys serves the chunked decode");
     using Cfg = TileCfg<DP>;
     constexpr int KT = Cfg::KT, LDK = Cfg::LDK, LDV = Cfg::LDV, NI = Cfg::NI, TTHREADS = Cfg::THREADS;
     constexpr int KS = DP / 16;        // contraction steps of the score product
@@ -137,7 +145,9 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     const int G = PACKED ? p.pack : 1;  // heads per packed row block (1: rows are positions of one head)
     const int rows_total = p.seq_q * G;
     const int hx = blockIdx.x, b = blockIdx.y;
-    const int qtile = (int)gridDim.z - 1 - (int)blockIdx.z;
+    const int zz = (int)gridDim.z - 1 - (int)blockIdx.z;
+    const int qtile = SPLIT ? zz / p.n_splits : zz;
+    const int split = SPLIT ? zz - qtile * p.n_splits : 0;
     const int q0 = qtile * TROWS;
     // kv head: hx itself when rows are packed, else hx / group (group_magic = 2^32 / group + 1, exact below 2^16 heads)
     const int kvh = (PACKED || p.group_magic == 0) ? hx : (int)__umulhi((uint32_t)hx, p.group_magic);
@@ -150,6 +160,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
 
     const uint16_t* __restrict__ Kg = p.k + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
     const uint16_t* __restrict__ Vg = p.v + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+    (void)split;
 
     // ---- tile movement: chunk c = tid + TTHREADS n of a tile is (row c / CH, 16-byte chunk c % CH).  A tile
     // travels global -> registers -> LDS.  LDS holds two stages of each matrix; PF register sets per matrix hold
@@ -185,7 +196,8 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     u32x4_t k1[NL];
 #pragma unroll
     for (int n = 0; n < NL; n++) k1[n] = u32x4_t{0u, 0u, 0u, 0u};
-    if (p.seq_kv > 0) {  // (no keys at all: there is no row to read, and no tile will be walked)
+    // (A span of the keys starts where the sequence's own length puts it: those requests wait for the lengths.)
+    if (!SPLIT && p.seq_kv > 0) {  // (no keys at all: there is no row to read, and no tile will be walked)
         const int last_row = p.seq_kv - 1;
 #pragma unroll
         for (int n = 0; n < NL; n++) {
@@ -198,8 +210,8 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     }
 
     const int n_q = p.q_lens ? min(max(p.q_lens[b], 0), p.seq_q) : p.seq_q;          // valid query positions
-    const int n_keys = p.kv_lens ? min(max(p.kv_lens[b], 0), p.seq_kv) : p.seq_kv;  // keys that exist
-    const int off = n_keys - n_q;  // causal: the last valid query sees every key
+    int n_keys = p.kv_lens ? min(max(p.kv_lens[b], 0), p.seq_kv) : p.seq_kv;  // keys that exist
+    int off = n_keys - n_q;  // causal: the last valid query sees every key
 
     // keys the workgroup walks
     int kv_end = n_keys;
@@ -210,7 +222,32 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         if (s_first >= n_q) kv_end = 0;  // a tile of padded query rows only
         kv_end = max(kv_end, 0);
     }
-    const int n_tiles = (kv_end + KT - 1) / KT;
+    int n_tiles = (kv_end + KT - 1) / KT;
+    if (SPLIT) {
+        // this workgroup's span of the walk: tiles [t_begin, t_end).  From here on keys are counted from the span's
+        // first key: the tensors' base, the key count, the causal offset and the end of the walk all move by it, and
+        // the walk below is that of a sequence whose keys are the span's (a row whose last visible key lies before the
+        // span gets a negative limit: every score masked, an empty partial).
+        const int per = (n_tiles + p.n_splits - 1) / p.n_splits;
+        const int t_begin = split * per, t_end = min(n_tiles, t_begin + per);
+        const int key0 = t_begin * KT;
+        n_tiles = max(t_end - t_begin, 0);
+        kv_end = min(kv_end, t_end * KT) - key0;
+        n_keys = min(n_keys, t_end * KT) - key0;
+        off -= key0;
+        Kg += (size_t)key0 * (size_t)p.lkv.row_pitch;
+        Vg += (size_t)key0 * (size_t)p.lkv.row_pitch;
+        if (n_tiles > 0) {  // the requests the unsplit kernel makes before it knows the lengths
+            const int last_row = n_keys - 1;
+#pragma unroll
+            for (int n = 0; n < NL; n++) {
+                const size_t e0 = (size_t)(uint32_t)min(ld_row[n], last_row) * kv_pitch + ld_col[n];
+                kreg[0][n] = *(const u32x4_t*)(Kg + e0);
+                vreg[0][n] = *(const u32x4_t*)(Vg + e0);
+                if (PIPE) k1[n] = *(const u32x4_t*)(Kg + (size_t)(uint32_t)min(KT + ld_row[n], last_row) * kv_pitch + ld_col[n]);
+            }
+        }
+    }
 
     f32x16_t acc_o[DT];
 #pragma unroll
@@ -699,8 +736,34 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     // barrier, and the region's previous content was read by this wave alone) and streams them out as whole rows,
     // 16 bytes per lane.
     const float l = t_sum_with_other_half(l_run);
+    if constexpr (SPLIT) {
+        // the partial of this span: O as accumulated (relative to the running max as it stands), that max in the exp2
+        // domain, the row sum.  A workgroup without tiles, or a row that saw no key of the span, leaves (0, -inf, 0).
+        const int r = q0 + 32 * wq + col;
+        if (r < rows_total) {
+            const size_t slot = (((size_t)b * p.kv_heads + kvh) * (size_t)rows_total + (size_t)r) * (size_t)p.n_splits + (size_t)split;
+            float* const po = p.part_o + slot * (size_t)D;
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int d0 = 32 * dt + 8 * j + 4 * hh;
+                    if (d0 < D)
+                        *(f32x4_t*)(po + d0) = f32x4_t{acc_o[dt][4 * j], acc_o[dt][4 * j + 1], acc_o[dt][4 * j + 2], acc_o[dt][4 * j + 3]};
+                }
+            if (hh == 0) {
+                p.part_ml[2 * slot] = m_run * cc;
+                p.part_ml[2 * slot + 1] = l;
+            }
+        }
+        return;
+    }
     const bool good = (l > 0.0f) && (l < __uint_as_float(0x7f800000u)) && !poison;
     const float inv_l = 1.0f / l;
+    // Packed rows are positions of a chunked decode: one that sees no key at all is a row of zeros, as the reference's
+    // decode kernels leave it (crates/rustorch-metal/src/kernels.rs:14504-14514: every loop runs zero times), not the
+    // NaN row of flash_forward's l > 0 test.  l == 0 exactly when no key was weighed (a visible key gives P >= 1).
+    const float bad = (PACKED && l == 0.0f) ? 0.0f : quiet_nan();
     uint16_t* const obuf = (uint16_t*)(lds + wq * Cfg::REGION);
     const float fill = p.zero_padded_rows ? 0.0f : quiet_nan();
     if (n_tiles > 0) {
@@ -714,7 +777,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
                 for (int e = 0; e < 4; e++) {
                     float x = acc_o[dt][4 * j + e] * inv_l;
                     if (!plain) {
-                        x = good ? x : quiet_nan();
+                        x = good ? x : bad;
                         if (!valid) x = fill;
                     }
                     o[e] = x;
@@ -732,8 +795,9 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         const int rr = q0 + 32 * wq + row;
         const int sp = G > 1 ? rr / G : rr;
         const int gg = rr - sp * G;
-        // no key tile walked: padded rows get the fill value, valid rows (which then see no key at all) NaN
-        const uint32_t f2 = sp < n_q ? 0x7fc07fc0u : fill2;
+        // no key tile walked: padded rows get the fill value, valid rows (which then see no key at all) NaN -- zeros
+        // when the rows are positions of a chunked decode
+        const uint32_t f2 = sp < n_q ? (PACKED ? 0u : 0x7fc07fc0u) : fill2;
         u32x4_t val = {f2, f2, f2, f2};
         if (n_tiles > 0) val = *(const u32x4_t*)(obuf + row * LDK + 8 * ch);
         if (rr < rows_total && 8 * ch < D) {
@@ -744,14 +808,76 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     }
 }
 
-template <int DP, int MODE, bool BIAS, bool PACKED>
+// Folds the partials the SPLIT kernel leaves: thread (row, d) walks the row's n_splits partials (o[d], m, l), weighs each
+// by 2^(m - max m) and writes o / l as bf16 where the unsplit kernel would have written the row.  No partial with a
+// key (every m is -inf): the position sees no key at all, a row of zeros.
+__global__ __launch_bounds__(256) void flash_split_merge_kernel(FlashTileParams p) {
+    const int D = p.dim, G = p.pack;
+    const size_t rows_total = (size_t)p.seq_q * G;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t row_all = idx / (size_t)D;
+    const int d = (int)(idx - row_all * (size_t)D);
+    if (row_all >= (size_t)p.batch * p.kv_heads * rows_total) return;
+    const size_t r = row_all % rows_total, bk = row_all / rows_total;
+    const int kvh = (int)(bk % (size_t)p.kv_heads), b = (int)(bk / (size_t)p.kv_heads);
+    const float* ml = p.part_ml + 2 * row_all * (size_t)p.n_splits;
+    const float* po = p.part_o + row_all * (size_t)p.n_splits * (size_t)D + d;
+    // One pass, eight partials at a time: the loads of a group are independent of each other (a dependent load per
+    // partial would cost a memory latency each), and the running (m, acc, l) is rescaled once per group.
+    constexpr int kGroup = 8;
+    float m_all = neg_inf(), acc = 0.0f, l_all = 0.0f;
+    bool nan_m = false;
+    for (int k0 = 0; k0 < p.n_splits; k0 += kGroup) {
+        float mv[kGroup], lv[kGroup], ov[kGroup];
+#pragma unroll
+        for (int j = 0; j < kGroup; j++) {
+            const int k = min(k0 + j, p.n_splits - 1);  // repeats of the last partial get weight 0 below
+            mv[j] = ml[2 * k];
+            lv[j] = ml[2 * k + 1];
+            ov[j] = po[(size_t)k * D];
+        }
+        float m_new = m_all;
+#pragma unroll
+        for (int j = 0; j < kGroup; j++) {
+            m_new = fmaxf(m_new, mv[j]);
+            nan_m |= (mv[j] != mv[j]);
+        }
+        const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+        const float rescale = (m_all == neg_inf()) ? 0.0f : __builtin_amdgcn_exp2f(m_all - m_use);
+        acc *= rescale;
+        l_all *= rescale;
+#pragma unroll
+        for (int j = 0; j < kGroup; j++) {
+            // an empty partial (m = -inf) is the identity
+            const float w = (k0 + j < p.n_splits && mv[j] != neg_inf()) ? __builtin_amdgcn_exp2f(mv[j] - m_use) : 0.0f;
+            acc += ov[j] * w;
+            l_all += lv[j] * w;
+        }
+        m_all = m_new;
+    }
+    float x = acc / l_all;
+    if (m_all == neg_inf() && !nan_m) x = 0.0f;
+    const size_t s_pos = r / (size_t)G;
+    const int g = (int)(r - s_pos * (size_t)G);
+    p.out[(size_t)b * p.lo.batch_stride + (size_t)(kvh * G + g) * p.lo.head_stride + s_pos * (size_t)p.lo.row_pitch + d] =
+        f32_to_bf16_bits(x);
+}
+
+template <int DP, int MODE, bool BIAS, bool PACKED, bool SPLIT = false>
 hipError_t launch_one(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
-    hipLaunchKernelGGL((flash_tile_bf16_kernel<DP, MODE, BIAS, PACKED>), grid, dim3(TileCfg<DP>::THREADS), 0, stream, p);
+    hipLaunchKernelGGL((flash_tile_bf16_kernel<DP, MODE, BIAS, PACKED, SPLIT>), grid, dim3(TileCfg<DP>::THREADS), 0, stream, p);
     return hipGetLastError();
 }
 
 template <int DP>
 hipError_t launch_dp(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
+    if (p.n_splits > 1) {  // (rows packed over a group of one head are rows of that head)
+        hipError_t e = launch_one<DP, kMaskCausal, false, true, true>(stream, p, grid);
+        if (e != hipSuccess) return e;
+        const size_t total = (size_t)p.batch * p.kv_heads * (size_t)p.seq_q * p.pack * (size_t)p.dim;
+        hipLaunchKernelGGL(flash_split_merge_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p);
+        return hipGetLastError();
+    }
     if (p.pack > 1) return launch_one<DP, kMaskCausal, false, true>(stream, p, grid);
     if (p.bias) return launch_one<DP, kMaskNone, true, false>(stream, p, grid);
     switch (p.mask) {
@@ -765,6 +891,7 @@ hipError_t launch_dp(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
 }  // namespace
 
 bool flash_tile_bf16_supported(int dim) { return dim > 0 && dim <= 256 && dim % 8 == 0; }
+int flash_tile_bf16_key_tile(int dim) { return dim <= 128 ? 64 : 32; }
 
 hipError_t launch_flash_tile_bf16(hipStream_t stream, const FlashTileParams& params) {
     FlashTileParams p = params;
@@ -775,9 +902,12 @@ hipError_t launch_flash_tile_bf16(hipStream_t stream, const FlashTileParams& par
     const long long rows = (long long)p.seq_q * p.pack;
     const long long n_qtiles = (rows + TROWS - 1) / TROWS;
     const long long heads_u = p.pack > 1 ? p.kv_heads : p.heads;
-    if (p.batch > 65535 || n_qtiles > 65535 || heads_u > 65535 || p.group < 1) return hipErrorInvalidValue;  // grid limits
+    if (p.n_splits < 1) p.n_splits = 1;
+    if (p.n_splits > 1 && (p.pack != p.group || p.bias || p.mask != kMaskCausal || !p.part_o || !p.part_ml))
+        return hipErrorInvalidValue;  // the chunked decode only
+    if (p.batch > 65535 || n_qtiles * p.n_splits > 65535 || heads_u > 65535 || p.group < 1) return hipErrorInvalidValue;  // grid limits
     p.group_magic = p.group > 1 ? (uint32_t)(0x100000000ull / (unsigned long long)p.group) + 1u : 0u;
-    dim3 grid((unsigned)heads_u, (unsigned)p.batch, (unsigned)n_qtiles);
+    dim3 grid((unsigned)heads_u, (unsigned)p.batch, (unsigned)(n_qtiles * p.n_splits));
     if (p.dim <= 32) return launch_dp<32>(stream, p, grid);
     if (p.dim <= 64) return launch_dp<64>(stream, p, grid);
     if (p.dim <= 96) return launch_dp<96>(stream, p, grid);

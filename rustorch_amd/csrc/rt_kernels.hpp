@@ -119,8 +119,17 @@ struct FlashTileParams {
     float scale_log2e;     // (1/sqrt(dim)) * log2(e)
     float scale;           // 1/sqrt(dim)
     TensorLayout lq, lkv, lo;
+    // Split over the keys (packed rows only; zero-initialise to leave it off): n_splits > 1 cuts every (sequence, kv
+    // head)'s walk into that many spans of whole tiles; each leaves a partial per packed row in part_o
+    // ([batch, kv_heads, seq_q * pack, n_splits, dim] f32) and part_ml (the same index, (m, l) pairs), and a second
+    // kernel folds them into `out`.
+    int n_splits;
+    float* part_o;
+    float* part_ml;
 };
 bool flash_tile_bf16_supported(int dim);
+// keys per LDS tile of the tile kernel at head dim `dim` (the unit the split over the keys is cut in)
+int flash_tile_bf16_key_tile(int dim);
 hipError_t launch_flash_tile_bf16(hipStream_t stream, const FlashTileParams& p);
 
 // Unmasked attention of every query row over all keys; generic in dim (<= 512), head
@@ -177,7 +186,7 @@ hipError_t decode_static_scratch(float** ptr, size_t* bytes);
 // argument.  The host side hands one slot to each (device, stream) that needs one, so calls on different streams
 // never share scratch.  Returns the address of a slot on the current device and its size.
 constexpr int kStreamSlots = 8;
-constexpr size_t kStreamSlotBytes = (size_t)4 << 20;
+constexpr size_t kStreamSlotBytes = (size_t)8 << 20;
 hipError_t stream_static_scratch(int slot, float** ptr, size_t* bytes);
 hipError_t launch_decode_split(hipStream_t stream, const DecodeSplitParams& p);
 

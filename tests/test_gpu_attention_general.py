@@ -113,15 +113,31 @@ def run_chunk(oracle, b, s, hq, hkv, d, max_seq, lens, seed=0, scalar_len=False)
     (2, 130, 4, 1, 64, 500, [500, 131]),      # more rows than one tile holds
     (2, 3, 4, 4, 80, 64, [64, 3]),
     (1, 1, 32, 8, 128, 2100, [2100]),
+    # one long cache and few new positions (the reference's own call shape): the keys are cut into spans whose
+    # partials a second kernel folds
+    (1, 16, 32, 8, 128, 8192, [8192]),
+    (1, 4, 32, 8, 128, 8192, [8191]),
+    (2, 7, 8, 2, 64, 3000, [3000, 700]),      # spans of a sequence much shorter than the cache: most of them empty
+    (1, 33, 16, 2, 256, 2000, [1999]),
+    (1, 40, 4, 1, 96, 1000, [1000]),          # two query tiles, each with its spans
+    (3, 5, 8, 2, 128, 1500, [1500, 3, 0]),    # a sequence shorter than the chunk, and an empty one
 ])
 def test_chunk_decode_matches_oracle(oracle, b, s, hq, hkv, d, max_seq, lens):
     run_chunk(oracle, b, s, hq, hkv, d, max_seq, lens)
 
 
+@pytest.mark.parametrize("s", [4, 16])
+def test_chunk_decode_of_one_long_sequence_with_a_host_length(oracle, s):
+    """batch 1, kv_lens = NULL and kv_len = pos_base + B: the reference call (kernels.rs:14522-14570) at 8192 keys."""
+    run_chunk(oracle, 1, s, 32, 8, 128, 8192, [8192], seed=s, scalar_len=True)
+    run_chunk(oracle, 1, s, 32, 8, 128, 8192, [5000], seed=s + 1, scalar_len=True)
+
+
 def test_chunk_of_one_is_the_batched_decode(oracle):
-    """seq_new = 1: the same numbers as rt_gqa_decode_batched_bf16 (within the bar; the kernels differ)."""
-    b, hq, hkv, d, max_seq = 3, 32, 8, 128, 700
-    lens = [700, 1, 513]
+    """seq_new = 1: the same numbers as rt_gqa_decode_batched_bf16 (within the bar; the kernels differ), a sequence
+    without keys included: both leave a row of zeros for it."""
+    b, hq, hkv, d, max_seq = 4, 32, 8, 128, 700
+    lens = [700, 1, 513, 0]
     got, (qb, kb, vb) = run_chunk(oracle, b, 1, hq, hkv, d, max_seq, lens)
     want = oracle.gqa_decode_batched_bf16(qb, kb, vb, lens, b, hq, hkv, d, max_seq)
     assert_bf16_parity(got, want, d, None)
@@ -130,7 +146,9 @@ def test_chunk_of_one_is_the_batched_decode(oracle):
     dq, dk, dv, dl = dev(qb), dev(kb), dev(vb), dev(np.asarray(lens, np.int32))
     K.gqa_decode_batched_bf16(None, dq, dk, dv, dout, dl, b, hq, hkv, d, max_seq, ws, ws.byte_len)
     ra.synchronize()
-    assert_bf16_parity(got, oracle.bf16_to_f32(dout.download(np.uint16)), d, None)
+    batched = oracle.bf16_to_f32(dout.download(np.uint16))
+    assert_bf16_parity(got, batched, d, None)
+    assert not got.reshape(b, -1)[3].any() and not batched.reshape(b, -1)[3].any()
 
 
 def test_chunk_from_position_zero_is_causal_prefill(oracle):
@@ -155,7 +173,11 @@ def test_chunk_decode_errors_and_rows_without_keys(oracle):
     with pytest.raises(ra.DeviceError) as ei:
         K.gqa_decode_chunk_bf16(None, z, z, z, z, 8, 1, 4, 8, 2, 20, 16)
     assert ei.value.status == 21
-    # a sequence whose cache is shorter than the chunk: its first positions see no key and come out NaN
+    # a sequence whose cache is shorter than the chunk: its first positions see no key and come out as rows of zeros
     got, _ = run_chunk(oracle, 2, 4, 4, 2, 64, 32, [2, 32])
     g = got.reshape(2, 4, 4, 64)
-    assert np.isnan(g[0, :2]).all() and np.isfinite(g[0, 2:]).all() and np.isfinite(g[1]).all()
+    assert not g[0, :2].any() and g[0, 2:].any(axis=-1).all() and np.isfinite(g).all()
+    with pytest.raises(TypeError):
+        K.gqa_decode_chunk_bf16(None, z, z, z, z, 3.5, 1, 4, 8, 2, 64, 16)
+    K.gqa_decode_chunk_bf16(None, z, z, z, z, np.int32(16), 1, 4, 8, 2, 64, 16)  # a numpy integer is a length, not an address
+    ra.synchronize()

@@ -352,7 +352,14 @@ def test_chunk_from_position_zero_is_causal_attention(oracle):
     assert np.abs(got - want.reshape(b, hq, s, d).transpose(0, 2, 1, 3)).max() <= 1e-5
 
 
-def test_chunk_position_without_keys_is_nan(oracle):
+def test_chunk_position_without_keys_is_a_row_of_zeros(oracle):
+    """The shader's loops over an empty key range leave acc = 0.0 (kernels.rs:14504-14514); the same rule as the
+    single-position decode with kv_len == 0."""
     q, k, v = _chunk_inputs(oracle, 1, 3, 2, 1, 8, 10, 1)
     got = oracle.gqa_decode_chunk_bf16(q, k, v, [1], 1, 3, 2, 1, 8, 10).reshape(3, 2, 8)
-    assert np.isnan(got[:2]).all() and np.isfinite(got[2]).all()
+    assert (got[:2] == 0.0).all() and np.isfinite(got[2]).all() and got[2].any()
+    # seq_new = 1 with an empty cache: what gqa_decode_batched_bf16 gives for kv_len == 0
+    q, k, v = _chunk_inputs(oracle, 2, 1, 4, 2, 8, 10, 2)
+    got = oracle.gqa_decode_chunk_bf16(q, k, v, [0, 7], 2, 1, 4, 2, 8, 10)
+    want = oracle.gqa_decode_batched_bf16(q, k, v, [0, 7], 2, 4, 2, 8, 10)
+    assert np.abs(got - want).max() <= 1e-6 and not got.reshape(2, -1)[0].any()
