@@ -79,7 +79,9 @@ class Hip:
     """The few HIP runtime calls the timing needs (stream + events), straight from libamdhip64."""
 
     def __init__(self):
-        self.lib = C.CDLL("libamdhip64.so")
+        from rustorch_amd import _lib
+
+        self.lib = _lib.hip_runtime()
         for name, args in (("hipStreamCreate", [C.POINTER(C.c_void_p)]), ("hipEventCreate", [C.POINTER(C.c_void_p)]),
                            ("hipEventRecord", [C.c_void_p, C.c_void_p]), ("hipEventSynchronize", [C.c_void_p]),
                            ("hipEventElapsedTime", [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]),

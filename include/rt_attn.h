@@ -100,6 +100,11 @@ int rt_init(int device, rt_err_detail *err);
 int rt_shutdown(rt_err_detail *err);
 const char *rt_version(void);
 const char *rt_status_name(int status);
+/* No counterpart in the reference: the path of the HIP runtime library this library is bound to (dladdr of one of its
+ * entry points), "" if it cannot be told.  A host that creates streams, events or graphs of its own for the `stream`
+ * arguments below must create them in this runtime; a process can hold a second copy of the runtime (PyTorch wheels
+ * ship one) and dlopen("libamdhip64.so") may hand back that one. */
+const char *rt_hip_runtime_path(void);
 
 /* ---- prefill, host slices ------------------------------------------------------------------- */
 

@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "librt_attn_hip.so")
 
 # every symbol include/rt_attn.h declares
 SYMBOLS = (
-    "rt_init", "rt_shutdown", "rt_version", "rt_status_name",
+    "rt_init", "rt_shutdown", "rt_version", "rt_status_name", "rt_hip_runtime_path",
     "rt_flash_forward_f32", "rt_flash_forward_masked_f32", "rt_gqa_forward_f32", "rt_gqa_forward_f32_dev",
     "rt_flash_backward_f32", "rt_flash_backward_f32_dev", "rt_flash_backward_workspace_bytes",
     "rt_flash_forward_stats_f32_dev", "rt_flash_backward_saved_f32_dev",
@@ -77,6 +77,7 @@ def lib():
     i32, u64 = C.c_int32, C.c_uint64
     L.rt_init.argtypes = [C.c_int, errp]
     L.rt_version.restype = C.c_char_p
+    L.rt_hip_runtime_path.restype = C.c_char_p
     L.rt_status_name.argtypes = [C.c_int]
     L.rt_status_name.restype = C.c_char_p
     L.rt_flash_forward_f32.argtypes = [shp, fp, sz, fp, sz, fp, sz, fp, sz, errp]
@@ -124,6 +125,14 @@ def lib():
     L.rt_debug_force_bf16_prefill_kernel.argtypes = [C.c_int]
     _lib = L
     return L
+
+
+def hip_runtime():
+    """The HIP runtime librt_attn_hip.so is bound to, as a ctypes handle (loaded by the path the library reports for
+    it): a caller that wants streams, events or graphs of its own must talk to that runtime instance.  A process
+    that has imported PyTorch holds a second copy of the runtime, and `CDLL("libamdhip64.so")` may return that one."""
+    path = lib().rt_hip_runtime_path().decode()
+    return C.CDLL(path if path else "libamdhip64.so")
 
 
 def status_name(code: int) -> str:

@@ -1,6 +1,7 @@
 // C ABI of librt_attn_hip.so (declared in include/rt_attn.h): argument checks in the
 // reference's order, device selection, host staging for the slice entry points, kernel dispatch.
 // There is no CPU path in this library.
+#include <dlfcn.h>
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdio.h>
@@ -361,6 +362,15 @@ private:
 }  // namespace
 
 RT_API const char* rt_version(void) { return "rt_attn_hip 0.1 (gfx950)"; }
+
+// The file the HIP runtime this library is bound to was loaded from.  A host that wants streams, events or graphs of
+// its own must talk to the same runtime instance; a process can hold a second copy (PyTorch wheels ship one), and a
+// dlopen by bare name may return that one, whose calls do not know this library's streams.
+RT_API const char* rt_hip_runtime_path(void) {
+    Dl_info info;
+    if (dladdr((void*)&hipGetDeviceCount, &info) && info.dli_fname) return info.dli_fname;
+    return "";
+}
 
 RT_API const char* rt_status_name(int status) {
     switch (status) {

@@ -334,7 +334,10 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         // items this wave walks: the ones that hold a key some row of it sees (a prefix of the workgroup's items)
         const int n_it = wave_lim_max < 0 ? 0 : min(n_tiles * NI, (wave_lim_max >> 5) + 1);
 
-        const size_t q_off = (size_t)b * p.lq.batch_stride + (size_t)(h0 + g) * p.lq.head_stride + (size_t)s_pos * p.lq.row_pitch;
+        // (the query row is read without a test: a row past the tensor reads the tensor's last row)
+        const int r_q = min(r, rows_total - 1);
+        const int s_q = G > 1 ? r_q / G : r_q;
+        const size_t q_off = (size_t)b * p.lq.batch_stride + (size_t)(h0 + (r_q - s_q * G)) * p.lq.head_stride + (size_t)s_q * p.lq.row_pitch;
 
         // Mask::Padding hiding the reference's whole first key tile: every row NaN (the tiled recurrence of
         // cpu_forward.rs:268-425 takes exp(-inf - (-inf)) on that tile and never recovers)
@@ -349,9 +352,18 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         bf16x8_t qreg[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-            u32x4_t z = {0u, 0u, 0u, 0u};
+            // Unconditional loads (a row past the tensor is read from the tensor's last row, a chunk past the head dim
+            // from its last chunk): a load under a per-lane test costs a branch of its own.  A row that does not exist
+            // has every score masked and is not written, so what it holds does not matter; the columns past the head
+            // dim must be zero.
             const int d0 = 16 * ks + 8 * hh;
-            if (exists && d0 < D) z = *(const u32x4_t*)(p.q + q_off + d0);
+            u32x4_t z = {0u, 0u, 0u, 0u};
+            if constexpr (DP <= 128) {
+                z = *(const u32x4_t*)(p.q + q_off + min(d0, D - 8));
+                if (D < DP && d0 >= D) z = u32x4_t{0u, 0u, 0u, 0u};
+            } else {  // (head dim 256 has no register to spare for the clamped addresses)
+                if (exists && d0 < D) z = *(const u32x4_t*)(p.q + q_off + d0);
+            }
             qreg[ks] = __builtin_bit_cast(bf16x8_t, z);
         }
 
@@ -759,7 +771,8 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         return;
     }
     const bool good = (l > 0.0f) && (l < __uint_as_float(0x7f800000u)) && !poison;
-    const float inv_l = 1.0f / l;
+    // the hardware reciprocal (1 ulp) instead of the division's dozen instructions: the output is rounded to bf16
+    const float inv_l = __builtin_amdgcn_rcpf(l);
     // Packed rows are positions of a chunked decode: one that sees no key at all is a row of zeros, as the reference's
     // decode kernels leave it (crates/rustorch-metal/src/kernels.rs:14504-14514: every loop runs zero times), not the
     // NaN row of flash_forward's l > 0 test.  l == 0 exactly when no key was weighed (a visible key gives P >= 1).
@@ -767,43 +780,73 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     uint16_t* const obuf = (uint16_t*)(lds + wq * Cfg::REGION);
     const float fill = p.zero_padded_rows ? 0.0f : quiet_nan();
     if (n_tiles > 0) {
-        const bool plain = __all(good && valid);  // the common wave: one multiplication per element
+        uint16_t* const orow = obuf + col * LDK + 4 * hh;
+        if (__all(good && valid)) {
+            // the common wave: one multiplication per element (a branch of its own: as a select inside one loop the
+            // compiler kept three selects per element for every wave)
 #pragma unroll
-        for (int dt = 0; dt < DT; dt++)
+            for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                float o[4];
+                for (int j = 0; j < 4; j++)
+                    *(u32x2_t*)(orow + 32 * dt + 8 * j) =
+                        u32x2_t{t_cvt_pk_bf16(acc_o[dt][4 * j] * inv_l, acc_o[dt][4 * j + 1] * inv_l),
+                                t_cvt_pk_bf16(acc_o[dt][4 * j + 2] * inv_l, acc_o[dt][4 * j + 3] * inv_l)};
+        } else {
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    float x = acc_o[dt][4 * j + e] * inv_l;
-                    if (!plain) {
-                        x = good ? x : bad;
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    float o[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        float x = good ? acc_o[dt][4 * j + e] * inv_l : bad;
                         if (!valid) x = fill;
+                        o[e] = x;
                     }
-                    o[e] = x;
+                    *(u32x2_t*)(orow + 32 * dt + 8 * j) = u32x2_t{t_cvt_pk_bf16(o[0], o[1]), t_cvt_pk_bf16(o[2], o[3])};
                 }
-                *(u32x2_t*)(obuf + col * LDK + 32 * dt + 8 * j + 4 * hh) =
-                    u32x2_t{t_cvt_pk_bf16(o[0], o[1]), t_cvt_pk_bf16(o[2], o[3])};
-            }
+        }
     }
     // (the same wave wrote and now reads: no barrier needed, the LDS queue is in order)
     const uint32_t fill2 = t_cvt_pk_bf16(fill, fill);
+    if constexpr (!PACKED && 64 % CH == 0 && DP <= 128) {
+        // rows of one head, and a wave's store instruction covers whole rows: lane l moves chunk l % CH of the rows
+        // l / CH, l / CH + 64 / CH, ... -- one address, then a constant step
+        constexpr int RS = 64 / CH;  // rows per store instruction
+        const int row0 = (int)((unsigned)lane / (unsigned)CH), ch = (int)((unsigned)lane % (unsigned)CH);
+        const int rr0 = q0 + 32 * wq + row0;
+        uint16_t* dst = p.out + (size_t)b * p.lo.batch_stride + (size_t)h0 * p.lo.head_stride + (size_t)rr0 * p.lo.row_pitch + 8 * ch;
+        const size_t step = (size_t)RS * (size_t)p.lo.row_pitch;
+        const uint16_t* src = obuf + row0 * LDK + 8 * ch;
+        const bool col_ok = 8 * ch < D;
 #pragma unroll
-    for (int n = 0; n < CH / 2; n++) {
-        const int cidx = lane + 64 * n;
-        const int row = cidx / CH, ch = cidx - row * CH;
-        const int rr = q0 + 32 * wq + row;
-        const int sp = G > 1 ? rr / G : rr;
-        const int gg = rr - sp * G;
-        // no key tile walked: padded rows get the fill value, valid rows (which then see no key at all) NaN -- zeros
-        // when the rows are positions of a chunked decode
-        const uint32_t f2 = sp < n_q ? (PACKED ? 0u : 0x7fc07fc0u) : fill2;
-        u32x4_t val = {f2, f2, f2, f2};
-        if (n_tiles > 0) val = *(const u32x4_t*)(obuf + row * LDK + 8 * ch);
-        if (rr < rows_total && 8 * ch < D) {
-            uint16_t* dst = p.out + (size_t)b * p.lo.batch_stride + (size_t)(h0 + gg) * p.lo.head_stride +
-                            (size_t)sp * p.lo.row_pitch + 8 * ch;
-            *(u32x4_t*)dst = val;
+        for (int n = 0; n < CH / 2; n++) {
+            const int rr = rr0 + RS * n;
+            // no key tile walked: padded rows get the fill value, valid rows (which then see no key at all) NaN
+            const uint32_t f2 = rr < n_q ? 0x7fc07fc0u : fill2;
+            u32x4_t val = {f2, f2, f2, f2};
+            if (n_tiles > 0) val = *(const u32x4_t*)(src + RS * n * LDK);
+            if (rr < rows_total && col_ok) *(u32x4_t*)dst = val;
+            dst += step;
+        }
+    } else {
+#pragma unroll
+        for (int n = 0; n < CH / 2; n++) {
+            const int cidx = lane + 64 * n;
+            const int row = cidx / CH, ch = cidx - row * CH;
+            const int rr = q0 + 32 * wq + row;
+            const int sp = G > 1 ? rr / G : rr;
+            const int gg = rr - sp * G;
+            // no key tile walked: padded rows get the fill value, valid rows (which then see no key at all) NaN -- zeros
+            // when the rows are positions of a chunked decode
+            const uint32_t f2 = sp < n_q ? (PACKED ? 0u : 0x7fc07fc0u) : fill2;
+            u32x4_t val = {f2, f2, f2, f2};
+            if (n_tiles > 0) val = *(const u32x4_t*)(obuf + row * LDK + 8 * ch);
+            if (rr < rows_total && 8 * ch < D) {
+                uint16_t* dst = p.out + (size_t)b * p.lo.batch_stride + (size_t)(h0 + gg) * p.lo.head_stride +
+                                (size_t)sp * p.lo.row_pitch + 8 * ch;
+                *(u32x4_t*)dst = val;
+            }
         }
     }
 }

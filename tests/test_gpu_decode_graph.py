@@ -14,6 +14,7 @@ import numpy as np
 import pytest
 
 import rustorch_amd as ra
+from rustorch_amd import _lib
 from _gpu import assert_decode_parity
 
 pytestmark = pytest.mark.gpu
@@ -24,7 +25,7 @@ NODE_TYPE_MEMSET = 2  # hipGraphNodeTypeMemset
 
 class Hip:
     def __init__(self):
-        self.lib = C.CDLL("libamdhip64.so")
+        self.lib = _lib.hip_runtime()
         vp = C.c_void_p
         self.lib.hipStreamBeginCapture.argtypes = [vp, C.c_int]
         self.lib.hipStreamEndCapture.argtypes = [vp, C.POINTER(vp)]

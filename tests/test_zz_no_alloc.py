@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 import rustorch_amd as ra
+from rustorch_amd import _lib
 from _gpu import assert_decode_parity, bf16_round, dev
 from _util import seeded_normal
 
@@ -14,7 +15,7 @@ pytestmark = pytest.mark.gpu
 K = ra.LlmKernels()
 
 
-_hip = C.CDLL("libamdhip64.so")
+_hip = _lib.hip_runtime()
 _hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
 
 
