@@ -661,9 +661,9 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
 
         // tile t: the step of its first item, the barrier, K(t+2) and V(t+1) parked from sets KSET and VSET (which
         // are refilled with K(t+2+PF) and V(t+1+PF)), then the steps of its other items
-        auto park_next = [&](int t, auto kset_c, auto vset_c) __attribute__((always_inline)) {
+        auto park_next = [&](int t, auto kset_c, auto vset_c, auto st_c) __attribute__((always_inline)) {
             constexpr int KSET = decltype(kset_c)::value;
-            const int st = t & 1;
+            const int st = st_c;  // t & 1, as a constant where the caller knows it
             // (behind the last tiles these park and request copies of the last tile, which nobody reads)
             park_k(kreg[KSET], st);
             park_v(vset_c, st ^ 1);
@@ -671,22 +671,26 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             issue_v(vset_c, (t + 1 + PF) * KT);
         };
         // the same for a tile of which the wave walks every item: straight-line code, the pairs swapped from step to step
-        auto walk_full = [&](int t, auto kset_c, auto vset_c) __attribute__((always_inline)) {
-            const int st = t & 1;
+        // `st_c` is t & 1, as an integer or as a compile-time constant: with the stage known at compile time every LDS
+        // address of the tile is the lane's base plus an immediate, and `later` (t > 0 known) drops the choice of the
+        // first tile's stand-in for V(-1)
+        auto walk_full = [&](int t, auto kset_c, auto vset_c, auto st_c, auto later_c) __attribute__((always_inline)) {
+            const int st = st_c;
+            constexpr bool kLater = decltype(later_c)::value;
             const uint16_t* const k_st = Ks + st * KT * LDK + k_off;
             const uint16_t* const k_ot = Ks + (st ^ 1) * KT * LDK + k_off;
             const uint16_t* const v_st = Vs + st * KT * LDV + v_off;
             const uint16_t* const v_ot = Vs + (st ^ 1) * KT * LDV + v_off;
             const int k0 = t * KT;
             if (NI > 1) {
-                step(0, k0, k_st + 32 * LDK, t == 0 ? v_st : v_ot + 32 * (NI - 1) * LDV, s_a, s_b, p_a, p_b, bv_a, bv_b);
+                step(0, k0, k_st + 32 * LDK, (!kLater && t == 0) ? v_st : v_ot + 32 * (NI - 1) * LDV, s_a, s_b, p_a, p_b, bv_a, bv_b);
                 __syncthreads();
-                park_next(t, kset_c, vset_c);
+                park_next(t, kset_c, vset_c, st_c);
                 step(1, k0 + 32, k_ot, v_st, s_b, s_a, p_b, p_a, bv_b, bv_a);
             } else {
-                step_a(0, k0, k_ot, t == 0 ? v_st : v_ot);
+                step_a(0, k0, k_ot, (!kLater && t == 0) ? v_st : v_ot);
                 __syncthreads();
-                park_next(t, kset_c, vset_c);
+                park_next(t, kset_c, vset_c, st_c);
                 __syncthreads();
             }
             keep_cur = keep_next;
@@ -701,7 +705,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             // the previous item is the last of tile t - 1 (at t = 0 there is none: P is zero, and V(0) stands in)
             slot(t * NI, 0, NI > 1 ? k_st + 32 * LDK : k_ot, t == 0 ? v_st : v_ot + 32 * (NI - 1) * LDV);
             __syncthreads();
-            park_next(t, kset_c, vset_c);
+            park_next(t, kset_c, vset_c, st);
             if (NI > 1) {
                 slot(t * NI + 1, 1, k_ot, v_st);
             } else {
@@ -727,10 +731,32 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             }
             t0 = n_tiles;
         }
-        for (const int t_full = n_it / NI; PIPE && t0 + PF <= t_full; t0 += PF) {
-            walk_full(t0, std::integral_constant<int, 2 % PF>{}, std::integral_constant<int, 1 % PF>{});
-            if (PF >= 2) walk_full(t0 + 1, std::integral_constant<int, 3 % PF>{}, std::integral_constant<int, 2 % PF>{});
-            if (PF >= 3) walk_full(t0 + 2, std::integral_constant<int, 4 % PF>{}, std::integral_constant<int, 3 % PF>{});
+        const int t_full = PIPE ? n_it / NI : 0;
+        if constexpr (PF == 1 && DP == 64 && !BIAS && MODE != kMaskPadding) {
+            // (head dim 64 only: the wider kernels and the ones with a bias or a padding mask have no register to spare for
+            // the second copy of the tile's code)
+            // one register set: tile 0 on its own, then the tiles in pairs (odd, even) whose LDS stages are compile-time
+            // constants, then what is left of the tiles the wave walks in full
+            using IC0 = std::integral_constant<int, 0>;
+            using IC1 = std::integral_constant<int, 1>;
+            if (PIPE && t0 < t_full) {
+                walk_full(0, IC0{}, IC0{}, IC0{}, std::false_type{});
+                t0 = 1;
+            }
+            for (; PIPE && t0 + 2 <= t_full; t0 += 2) {
+                walk_full(t0, IC0{}, IC0{}, IC1{}, std::true_type{});
+                walk_full(t0 + 1, IC0{}, IC0{}, IC0{}, std::true_type{});
+            }
+            if (PIPE && t0 < t_full) {
+                walk_full(t0, IC0{}, IC0{}, t0 & 1, std::true_type{});
+                t0++;
+            }
+        } else {
+            for (; PIPE && t0 + PF <= t_full; t0 += PF) {
+                walk_full(t0, std::integral_constant<int, 2 % PF>{}, std::integral_constant<int, 1 % PF>{}, t0 & 1, std::false_type{});
+                if (PF >= 2) walk_full(t0 + 1, std::integral_constant<int, 3 % PF>{}, std::integral_constant<int, 2 % PF>{}, (t0 + 1) & 1, std::false_type{});
+                if (PF >= 3) walk_full(t0 + 2, std::integral_constant<int, 4 % PF>{}, std::integral_constant<int, 3 % PF>{}, (t0 + 2) & 1, std::false_type{});
+            }
         }
         for (; t0 < n_tiles; t0 += PF) {
             walk_tile(t0, std::integral_constant<int, 2 % PF>{}, std::integral_constant<int, 1 % PF>{});
