@@ -142,7 +142,41 @@ int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n
                      const float* k, const float* v, int mask_kind, const uint8_t* keep, float* out,
                      rt_err_detail* err, bool bnhd = false, const float* bias = nullptr, long long bias_bh_stride = 0,
                      float* lse = nullptr, uint64_t seq_kv = 0) {
-    if (s->dim > 256) return fail(err, RT_ERR_UNSUPPORTED, -1, 256, s->dim, "f32 flash kernels cover dim <= 256");
+    if (s->dim > 512) return fail(err, RT_ERR_UNSUPPORTED, -1, 512, s->dim, "f32 flash kernels cover dim <= 512");
+    if (s->dim > 256) {
+        // beyond the tiled kernels: one workgroup per query row (any speed), with flash_forward's masks and row rules
+        if (s->seq > 0x7fffffffull || seq_kv > 0x7fffffffull) return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+        rt::AttnRowsParams r{};
+        r.q = q;
+        r.k = k;
+        r.v = v;
+        r.out = out;
+        r.batch = (int)s->batch;
+        r.heads = (int)s->heads;
+        r.kv_heads = (int)n_kv_heads;
+        r.seq_q = (int)s->seq;
+        r.kv_len = r.kv_stride = (int)(seq_kv ? seq_kv : s->seq);
+        r.dim = (int)s->dim;
+        r.head_map = 0;
+        r.scale = 1.0f / sqrtf((float)s->dim);
+        r.bias = bias;
+        r.bias_bh_stride = bias_bh_stride;
+        r.use_layout = 1;
+        if (bnhd) {
+            r.lq = r.lo = rt::layout_bnhd((long long)s->heads, (long long)s->seq, r.dim);
+            r.lkv = rt::layout_bnhd((long long)n_kv_heads, (long long)r.kv_len, r.dim);
+        } else {
+            r.lq = r.lo = rt::layout_bhnd((long long)s->heads, (long long)s->seq, r.dim);
+            r.lkv = rt::layout_bhnd((long long)n_kv_heads, (long long)r.kv_len, r.dim);
+        }
+        r.mask = mask_kind;
+        r.keep = keep;
+        r.ref_bc = (int)(s->bc == 0 ? 1 : (s->bc > 0x7fffffffull ? 0x7fffffff : s->bc));
+        r.flash_rows = 1;
+        r.lse = lse;
+        HIP_TRY(rt::launch_attn_rows_f32(stream, r), "attn_rows_f32 launch");
+        return RT_OK;
+    }
     rt::FlashF32Params p{};
     p.bias = bias;
     p.bias_bh_stride = bias_bh_stride;
@@ -556,7 +590,7 @@ namespace {
 int flash_bwd_device(hipStream_t stream, const rt_attention_shape* s, const float* q, const float* k, const float* v,
                      const float* d_out, float* dq, float* dk, float* dv, float* workspace, rt_err_detail* err,
                      const float* saved_out = nullptr, const float* saved_lse = nullptr) {
-    if (s->dim > 128) return fail(err, RT_ERR_UNSUPPORTED, -1, 128, s->dim, "f32 backward kernels cover dim <= 128");
+    if (s->dim > 512) return fail(err, RT_ERR_UNSUPPORTED, -1, 512, s->dim, "f32 backward kernels cover dim <= 512");
     rt::FlashBwdF32Params p{};
     p.q = q;
     p.k = k;
@@ -570,10 +604,20 @@ int flash_bwd_device(hipStream_t stream, const rt_attention_shape* s, const floa
     p.seq = (int)s->seq;
     p.dim = (int)s->dim;
     p.scale = 1.0f / sqrtf((float)s->dim);
-    if (saved_out)
+    if (saved_out) {
         HIP_TRY(rt::launch_flash_bwd_f32_saved(stream, p, saved_out, saved_lse, workspace), "flash_bwd_f32 launch");
-    else
+    } else if (s->dim > 256) {
+        // the recomputed forward of a head dim the tiled forward kernels do not cover: O and the row statistic from
+        // the one-workgroup-per-row kernel, then the backward from them
+        const size_t rows = (size_t)(s->batch * s->heads * s->seq);
+        float* o = workspace;
+        float* lse_ws = workspace + rows * s->dim;
+        int rc = flash_f32_device(stream, s, s->heads, q, k, v, RT_MASK_NONE, nullptr, o, err, false, nullptr, 0, lse_ws);
+        if (rc) return rc;
+        HIP_TRY(rt::launch_flash_bwd_f32_saved(stream, p, o, lse_ws, lse_ws + rows), "flash_bwd_f32 launch");
+    } else {
         HIP_TRY(rt::launch_flash_bwd_f32(stream, p, workspace, g_num_cus), "flash_bwd_f32 launch");
+    }
     return RT_OK;
 }
 
@@ -742,18 +786,49 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
     if (shape->seq == 0 || shape->batch == 0 || shape->heads == 0) return RT_OK;
     int rc = check_flash_dims(shape, n_kv_heads, err);
     if (rc) return rc;
-    if (shape->dim > 256 || shape->dim % 8 != 0)
-        return fail(err, RT_ERR_UNSUPPORTED, -1, 256, shape->dim,
-                    "bf16 flash kernels cover head dims up to 256 that are a multiple of 8");
+    if (shape->dim > 512)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 512, shape->dim, "bf16 flash kernels cover head dims up to 512");
     // the tile kernel's grid is (heads, batch, query tiles of 128 rows), each dimension below 2^16
     if (shape->heads > 65535 || shape->batch > 65535 || (shape->seq + 127) / 128 > 65535)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
-    if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0)
-        return fail(err, RT_ERR_UNSUPPORTED, -1, 16, 0, "bf16 flash kernels need 16-byte aligned tensors");
     if (!q || !k || !v || !out || (mask == rt::kMaskPadding && !keep) || (mask == rt::kMaskVarlenCausal && !seq_lens))
         return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
     rc = ensure_device(err);
     if (rc) return rc;
+    // The matrix-core kernels move 16 bytes at a time: head dims up to 256 that are a multiple of 8, tensors 16-byte
+    // aligned.  Everything else (the reference takes any dim != 0, cpu_forward.rs:142-169) goes to the
+    // one-workgroup-per-row kernel: same masks, same row rules, any speed.
+    if (shape->dim > 256 || shape->dim % 8 != 0 || (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0) {
+        rt::AttnRowsParams r{};
+        r.q = q;
+        r.k = k;
+        r.v = v;
+        r.out = out;
+        r.kv_lens = mask == rt::kMaskVarlenCausal ? seq_lens : nullptr;
+        r.q_lens = r.kv_lens;
+        r.batch = (int)shape->batch;
+        r.heads = (int)shape->heads;
+        r.kv_heads = (int)n_kv_heads;
+        r.seq_q = r.kv_len = r.kv_stride = (int)shape->seq;
+        r.dim = (int)shape->dim;
+        r.head_map = 0;
+        r.scale = 1.0f / sqrtf((float)shape->dim);
+        r.use_layout = 1;
+        if (bnhd) {
+            r.lq = r.lo = rt::layout_bnhd((long long)shape->heads, (long long)shape->seq, r.dim);
+            r.lkv = rt::layout_bnhd((long long)n_kv_heads, (long long)shape->seq, r.dim);
+        } else {
+            r.lq = r.lo = rt::layout_bhnd((long long)shape->heads, (long long)shape->seq, r.dim);
+            r.lkv = rt::layout_bhnd((long long)n_kv_heads, (long long)shape->seq, r.dim);
+        }
+        r.mask = mask == rt::kMaskVarlenCausal ? rt::kMaskCausal : mask;
+        r.keep = keep;
+        r.ref_bc = (int)(shape->bc == 0 ? 1 : (shape->bc > 0x7fffffffull ? 0x7fffffff : shape->bc));
+        r.flash_rows = 1;
+        r.zero_padded_rows = zero_padded_rows;
+        HIP_TRY(rt::launch_attn_rows_bf16((hipStream_t)stream, r), "attn_rows_bf16 launch");
+        return RT_OK;
+    }
     // the persistent kernel needs a job (256 query rows of one head) for every CU and gains on the tile kernel as the
     // rows get longer; a padded batch is a set of jobs of very different lengths, which the tile kernel's
     // dispatcher-balanced workgroups handle better
@@ -1019,15 +1094,36 @@ RT_API int rt_mha_forward_masked_bf16_dev(void* stream, const void* q, const voi
         return fail(err, RT_ERR_WRONG_INPUT_LEN, RT_WHICH_MASK, one_mask, mask_len, "mask length");
     if (q_expected == 0) return RT_OK;
     if (!q || !out || (kv_expected && (!k || !v))) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
-    if (!rt::flash_tile_bf16_supported((int)std::min<size_t>(head_dim, 1 << 20)))
-        return fail(err, RT_ERR_UNSUPPORTED, -1, 256, head_dim, "bf16 kernels cover head dims up to 256 that are a multiple of 8");
+    if (head_dim > 512) return fail(err, RT_ERR_UNSUPPORTED, -1, 512, head_dim, "bf16 kernels cover head dims up to 512");
     if (heads > 65535 || batch > 65535 || t_q > 0x7fffffffull || t_kv > 0x7fffffffull || embed > 0x7fffffffull ||
         (t_q + 127) / 128 > 65535)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
-    if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0 || ((uintptr_t)mask & 3) != 0)
-        return fail(err, RT_ERR_UNSUPPORTED, -1, 16, 0, "bf16 kernels need 16-byte aligned tensors");
+    if (((uintptr_t)mask & 3) != 0) return fail(err, RT_ERR_UNSUPPORTED, -1, 4, 0, "the mask must be 4-byte aligned");
     int rc = ensure_device(err);
     if (rc) return rc;
+    if (!rt::flash_tile_bf16_supported((int)head_dim) || (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0) {
+        // head dims and alignments the matrix-core kernel does not cover: one workgroup per query row, any speed
+        if (t_kv == 0) return rt_buf_zero(out, q_expected * 2, stream, err);
+        rt::AttnRowsParams r{};
+        r.q = q;
+        r.k = k;
+        r.v = v;
+        r.out = out;
+        r.batch = (int)batch;
+        r.heads = r.kv_heads = (int)heads;
+        r.seq_q = (int)t_q;
+        r.kv_len = r.kv_stride = (int)t_kv;
+        r.dim = (int)head_dim;
+        r.head_map = 0;
+        r.scale = 1.0f / sqrtf((float)head_dim);
+        r.bias = mask_len ? mask : nullptr;
+        r.bias_bh_stride = (mask_len == all_masks && all_masks != one_mask) ? (long long)one_mask : 0;
+        r.use_layout = 1;
+        r.lq = r.lo = rt::layout_bnhd((long long)heads, (long long)t_q, (int)head_dim);
+        r.lkv = rt::layout_bnhd((long long)heads, (long long)t_kv, (int)head_dim);
+        HIP_TRY(rt::launch_attn_rows_bf16((hipStream_t)stream, r), "attn_rows_bf16 launch");
+        return RT_OK;
+    }
     rt::FlashTileParams t{};
     t.q = (const uint16_t*)q;
     t.k = (const uint16_t*)k;

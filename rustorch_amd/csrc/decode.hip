@@ -79,6 +79,28 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(AttnRowsParams p) {
     const float* __restrict__ bias_row =
         p.bias ? p.bias + ((size_t)b * p.heads + h) * (size_t)p.bias_bh_stride + (size_t)qi * (size_t)kv_len : nullptr;
 
+    // rows past a sequence's valid queries: the fill value, nothing else
+    const int n_q = p.q_lens ? min(max(p.q_lens[b], 0), p.seq_q) : p.seq_q;
+    if (qi >= n_q) {
+        const float fill = p.zero_padded_rows ? 0.0f : quiet_nan();
+        for (int d = threadIdx.x; d < D; d += 256) store_elem(O, d, fill);
+        if (p.lse && threadIdx.x == 0) p.lse[((size_t)b * p.heads + h) * p.seq_q + qi] = fill;
+        return;
+    }
+    // last key this row sees; under the causal mask the last valid query sees every key
+    int lim = kv_len - 1;
+    if (p.mask == kMaskCausal) lim = min(lim, qi + (kv_len - n_q));
+    const uint8_t* __restrict__ keep = p.mask == kMaskPadding ? p.keep : nullptr;
+    // Mask::Padding that hides the reference's whole first key tile: every row NaN (cpu_forward.rs:268-425 takes
+    // exp(-inf - (-inf)) on that tile and never recovers)
+    bool poison = false;
+    if (keep) {
+        const int lead = min(p.ref_bc, kv_len);
+        bool any = false;
+        for (int j = lane; j < lead; j += 64) any |= (keep[j] != 0);
+        poison = !__any(any);
+    }
+
     float qv[kMaxDJ], o[kMaxDJ];
 #pragma unroll
     for (int j = 0; j < kMaxDJ; j++) {
@@ -87,7 +109,8 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(AttnRowsParams p) {
         o[j] = 0.0f;
     }
     float m = neg_inf(), l = 0.0f;
-    for (int t = wave; t < kv_len; t += 4) {
+    for (int t = wave; t <= lim; t += 4) {
+        if (keep && keep[t] == 0) continue;  // (wave-uniform)
         float part = 0.0f;
 #pragma unroll
         for (int j = 0; j < kMaxDJ; j++) {
@@ -130,6 +153,8 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(AttnRowsParams p) {
         }
         // kv_len == 0: nothing accumulated; the reference writes zeros (gqa.rs:261, no key to add)
         float inv = kv_len > 0 ? 1.0f / l_all : 0.0f;
+        // flash_forward's rows: out = O * (1 / l) when l > 0 and finite, NaN otherwise (cpu_forward.rs:405-421)
+        const bool bad = p.flash_rows && (!(l_all > 0.0f) || !(l_all < __uint_as_float(0x7f800000u)) || poison);
 #pragma unroll
         for (int j = 0; j < kMaxDJ; j++) {
             int d = lane + 64 * j;
@@ -137,9 +162,10 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(AttnRowsParams p) {
                 float acc = 0.0f;
 #pragma unroll
                 for (int w = 0; w < 4; w++) acc += so[w][d] * cw[w];
-                store_elem(O, d, acc * inv);
+                store_elem(O, d, bad ? quiet_nan() : acc * inv);
             }
         }
+        if (p.lse && lane == 0) p.lse[((size_t)b * p.heads + h) * p.seq_q + qi] = bad ? quiet_nan() : m_all + logf(l_all);
     }
 }
 

@@ -413,6 +413,115 @@ __global__ __launch_bounds__(256, (DT <= 2 ? 2 : 1)) void flash_bwd_f32_dq_kerne
     reduce_store<DPAD, LD, 2 * TILE>(lds, 0, p.dq + base, q0, N, D, tid, vec);
 }
 
+// ---- any head dim up to 512: one workgroup per row, any speed ------------------------------------------------------
+// The gradients of cpu_backward.rs:46-185 for the head dims the tiled kernels above do not hold in registers.  The dQ
+// kernel owns a query row i (and leaves delta_i = dO_i . O_i for the second kernel), the dK/dV kernel a key row j;
+// each of the four waves takes every fourth row of the other side, forms s = q_i . k_j and dP = dO_i . v_j with the
+// lanes strided over the head dim, P = exp(s * scale - L_i), dS = P (dP - delta_i) scale, and adds its products
+// into per-lane sums that are folded through LDS at the end.  No atomics: every output row has one owner.
+constexpr int kGenDJ = 8;  // 64 lanes x 8 = head dims up to 512
+
+__device__ __forceinline__ float gen_wave_sum(float x) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off, 64);
+    return x;
+}
+
+__global__ __launch_bounds__(256) void flash_bwd_rows_dq_kernel(FlashBwdF32Params p) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int N = p.seq, D = p.dim;
+    const size_t slab = ((size_t)b * p.heads + h) * (size_t)N;
+    const float* qi = p.q + (slab + i) * D;
+    const float* doi = p.d_out + (slab + i) * D;
+    const float* oi = p.o + (slab + i) * D;
+    float qv[kGenDJ], dov[kGenDJ], acc[kGenDJ];
+    float dsum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kGenDJ; j++) {
+        const int d = lane + 64 * j;
+        qv[j] = d < D ? qi[d] : 0.0f;
+        dov[j] = d < D ? doi[d] : 0.0f;
+        acc[j] = 0.0f;
+        if (d < D) dsum += dov[j] * oi[d];
+    }
+    const float delta = gen_wave_sum(dsum);
+    const float L = p.lse[slab + i];
+    if (threadIdx.x == 0) p.delta[slab + i] = delta;
+    for (int t = wave; t < N; t += 4) {
+        const float* kt = p.k + (slab + t) * D;
+        const float* vt = p.v + (slab + t) * D;
+        float ps = 0.0f, pd = 0.0f;
+        float kk[kGenDJ];
+#pragma unroll
+        for (int j = 0; j < kGenDJ; j++) {
+            const int d = lane + 64 * j;
+            kk[j] = d < D ? kt[d] : 0.0f;
+            ps += qv[j] * kk[j];
+            if (d < D) pd += dov[j] * vt[d];
+        }
+        const float sc = gen_wave_sum(ps) * p.scale, dP = gen_wave_sum(pd);
+        const float ds = expf(sc - L) * (dP - delta) * p.scale;
+#pragma unroll
+        for (int j = 0; j < kGenDJ; j++) acc[j] += ds * kk[j];
+    }
+    __shared__ float part[4][64 * kGenDJ];
+#pragma unroll
+    for (int j = 0; j < kGenDJ; j++) part[wave][lane + 64 * j] = acc[j];
+    __syncthreads();
+    for (int d = threadIdx.x; d < D; d += 256) p.dq[(slab + i) * D + d] = (part[0][d] + part[1][d]) + (part[2][d] + part[3][d]);
+}
+
+__global__ __launch_bounds__(256) void flash_bwd_rows_dkdv_kernel(FlashBwdF32Params p) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int N = p.seq, D = p.dim;
+    const size_t slab = ((size_t)b * p.heads + h) * (size_t)N;
+    const float* kt = p.k + (slab + t) * D;
+    const float* vt = p.v + (slab + t) * D;
+    float kv[kGenDJ], vv[kGenDJ], acc_k[kGenDJ], acc_v[kGenDJ];
+#pragma unroll
+    for (int j = 0; j < kGenDJ; j++) {
+        const int d = lane + 64 * j;
+        kv[j] = d < D ? kt[d] : 0.0f;
+        vv[j] = d < D ? vt[d] : 0.0f;
+        acc_k[j] = acc_v[j] = 0.0f;
+    }
+    for (int i = wave; i < N; i += 4) {
+        const float* qi = p.q + (slab + i) * D;
+        const float* doi = p.d_out + (slab + i) * D;
+        float ps = 0.0f, pd = 0.0f;
+        float qq[kGenDJ], dd[kGenDJ];
+#pragma unroll
+        for (int j = 0; j < kGenDJ; j++) {
+            const int d = lane + 64 * j;
+            qq[j] = d < D ? qi[d] : 0.0f;
+            dd[j] = d < D ? doi[d] : 0.0f;
+            ps += qq[j] * kv[j];
+            pd += dd[j] * vv[j];
+        }
+        const float sc = gen_wave_sum(ps) * p.scale, dP = gen_wave_sum(pd);
+        const float pij = expf(sc - p.lse[slab + i]);
+        const float ds = pij * (dP - p.delta[slab + i]) * p.scale;
+#pragma unroll
+        for (int j = 0; j < kGenDJ; j++) {
+            acc_k[j] += ds * qq[j];
+            acc_v[j] += pij * dd[j];
+        }
+    }
+    __shared__ float part_k[4][64 * kGenDJ], part_v[4][64 * kGenDJ];
+#pragma unroll
+    for (int j = 0; j < kGenDJ; j++) {
+        part_k[wave][lane + 64 * j] = acc_k[j];
+        part_v[wave][lane + 64 * j] = acc_v[j];
+    }
+    __syncthreads();
+    for (int d = threadIdx.x; d < D; d += 256) {
+        p.dk[(slab + t) * D + d] = (part_k[0][d] + part_k[1][d]) + (part_k[2][d] + part_k[3][d]);
+        p.dv[(slab + t) * D + d] = (part_v[0][d] + part_v[1][d]) + (part_v[2][d] + part_v[3][d]);
+    }
+}
+
 }  // namespace
 
 size_t flash_bwd_f32_workspace_floats(int batch, int heads, int seq, int dim) {
@@ -421,7 +530,7 @@ size_t flash_bwd_f32_workspace_floats(int batch, int heads, int seq, int dim) {
 
 hipError_t launch_flash_bwd_f32(hipStream_t stream, const FlashBwdF32Params& p_in, float* workspace, int n_cus) {
     if (p_in.batch == 0 || p_in.heads == 0 || p_in.seq == 0 || p_in.dim == 0) return hipSuccess;
-    if (p_in.dim > 128) return hipErrorInvalidValue;
+    if (p_in.dim > 256) return hipErrorInvalidValue;  // (the tiled forward stops there; the caller brings O and the statistic)
     const size_t rows = (size_t)p_in.batch * p_in.heads * p_in.seq;
     float* o = workspace;
     float* lse = workspace + rows * p_in.dim;
@@ -452,11 +561,18 @@ hipError_t launch_flash_bwd_f32(hipStream_t stream, const FlashBwdF32Params& p_i
 hipError_t launch_flash_bwd_f32_saved(hipStream_t stream, const FlashBwdF32Params& p_in, const float* o, const float* lse,
                                       float* delta) {
     if (p_in.batch == 0 || p_in.heads == 0 || p_in.seq == 0 || p_in.dim == 0) return hipSuccess;
-    if (p_in.dim > 128) return hipErrorInvalidValue;
+    if (p_in.dim > 64 * kGenDJ) return hipErrorInvalidValue;
     FlashBwdF32Params p = p_in;
     p.o = o;
     p.lse = lse;
     p.delta = delta;
+    if (p.dim > 128) {  // beyond the registers of the tiled kernels: a workgroup per row
+        if (p.heads > 65535 || p.batch > 65535) return hipErrorInvalidValue;
+        dim3 grid_rows(p.seq, p.heads, p.batch);
+        hipLaunchKernelGGL(flash_bwd_rows_dq_kernel, grid_rows, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL(flash_bwd_rows_dkdv_kernel, grid_rows, dim3(256), 0, stream, p);
+        return hipGetLastError();
+    }
     auto aligned = [](const void* ptr) { return (uintptr_t)ptr % 16 == 0; };
     p.vec = (p.dim % 4 == 0) && aligned(p.q) && aligned(p.k) && aligned(p.v) && aligned(p.d_out) && aligned(p.dq) &&
             aligned(p.dk) && aligned(p.dv);

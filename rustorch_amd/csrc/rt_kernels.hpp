@@ -149,6 +149,16 @@ struct AttnRowsParams {
     long long bias_bh_stride;  // elements between the biases of consecutive (batch, head) pairs; 0 = one bias for all
     int use_layout;            // != 0: q/out and k/v are addressed through the layouts below instead of [B,H,S,D]
     TensorLayout lq, lkv, lo;
+    // the masks and row rules of flash_forward_masked (crates/rustorch-attention/src/cpu_forward.rs:193-425), for the
+    // head dims the tiled kernels do not cover (zero-initialise to leave them off: plain attention over kv_len keys,
+    // a row without keys is a row of zeros as in the decode kernels)
+    int mask;                  // kMaskNone, kMaskCausal (key t visible to query i iff t <= i + (keys - valid queries)), kMaskPadding
+    const uint8_t* keep;       // kMaskPadding: device, kv_len bytes
+    int ref_bc;                // kMaskPadding: the reference's key-tile size (a wholly hidden first tile makes every row NaN)
+    int flash_rows;            // != 0: a row that sees no key, or whose sum is not finite, is NaN (the l > 0 && finite test)
+    const int32_t* q_lens;     // optional device int32[batch]: valid query rows; rows past them get the fill value
+    int zero_padded_rows;      // the fill value: +0.0 (else NaN)
+    float* lse;                // optional f32 [batch, heads, seq_q]: m + ln(l) of every row (f32 tensors only)
 };
 hipError_t launch_attn_rows_f32(hipStream_t stream, const AttnRowsParams& p);
 hipError_t launch_attn_rows_bf16(hipStream_t stream, const AttnRowsParams& p);

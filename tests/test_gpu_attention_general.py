@@ -32,7 +32,7 @@ def run_masked(oracle, b, tq, tkv, h, d, mask, seed=0):
 
 
 @pytest.mark.parametrize("b,t,h,d", [(1, 1, 1, 8), (2, 5, 3, 8), (2, 128, 4, 64), (1, 70, 2, 96), (1, 33, 1, 136),
-                                     (2, 257, 2, 32), (1, 130, 2, 256), (1, 200, 3, 80)])
+                                     (2, 257, 2, 32), (1, 130, 2, 256), (1, 200, 3, 80), (2, 40, 2, 20), (1, 65, 2, 300)])
 @pytest.mark.parametrize("kind", ["none", "causal", "window", "bool", "per_head"])
 def test_self_attention_with_masks(oracle, b, t, h, d, kind):
     rng = np.random.default_rng(7)
@@ -79,8 +79,8 @@ def test_masked_rows_and_edge_cases(oracle):
 
 def test_masked_bf16_errors():
     z = ra.HipStorage(1 << 16)
-    with pytest.raises(ra.DeviceError) as ei:  # head dim not a multiple of 8
-        ra.mha_forward_masked_bf16_dev(z, z, z, z, 1, 4, 4, 2, 20)
+    with pytest.raises(ra.DeviceError) as ei:  # head dim above 512
+        ra.mha_forward_masked_bf16_dev(z, z, z, z, 1, 4, 4, 2, 520)
     assert ei.value.status == 21
     with pytest.raises(ra.WrongInputLen):  # mask of the wrong size
         ra.mha_forward_masked_bf16_dev(z, z, z, z, 1, 4, 4, 2, 16, z, 15)

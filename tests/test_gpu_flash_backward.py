@@ -59,7 +59,9 @@ def test_shape_mismatch_and_empty_seq():
 # ---- parity with the oracle -----------------------------------------------------------------------------------
 
 SHAPES = [(1, 1, 4, 4), (1, 1, 1, 16), (2, 3, 17, 8), (1, 2, 64, 32), (1, 1, 33, 5), (1, 1, 130, 64), (2, 2, 100, 128),
-          (1, 2, 257, 96), (1, 1, 300, 100), (3, 1, 31, 33), (1, 4, 512, 64), (1, 1, 129, 1), (1, 1, 96, 127)]
+          (1, 2, 257, 96), (1, 1, 300, 100), (3, 1, 31, 33), (1, 4, 512, 64), (1, 1, 129, 1), (1, 1, 96, 127),
+          # above the tiled kernels' registers: a workgroup per row (the reference has no limit, cpu_backward.rs:46-185)
+          (1, 2, 70, 129), (2, 1, 33, 200), (1, 1, 130, 256), (1, 1, 65, 257), (1, 2, 40, 320), (1, 1, 17, 512)]
 
 
 @pytest.mark.parametrize("bhnd", SHAPES)
@@ -81,6 +83,14 @@ def test_backward_matches_oracle_on_normal_inputs(oracle):
     for name, g, w in zip(("dq", "dk", "dv"), got, want):
         # standard-normal scores reach +-10: gradients of a few units, errors scale with them
         assert max_abs(g, w) <= 1e-5 * max(1.0, float(np.abs(w).max())) * 4, name
+
+
+def test_backward_head_dim_above_512_is_refused():
+    shape = ra.AttentionShape.new(1, 1, 4, 513)
+    z = np.zeros(shape.buffer_len(), np.float32)
+    with pytest.raises(ra.DeviceError) as ei:
+        ra.flash_backward(shape, z, z, z, z)
+    assert ei.value.status == 21 and ei.value.expected == 512
 
 
 def test_outputs_are_overwritten(oracle):

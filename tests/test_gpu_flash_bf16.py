@@ -242,14 +242,34 @@ def test_config_long_context_b1_h32_n16384_d128(oracle):
             assert_bf16_parity(got[hi, i], want, d, 1, f"head {hi}, row {i}")
 
 
-@pytest.mark.parametrize("d", [257, 264, 100, 4])
-def test_unsupported_dim_is_an_error(d):
-    """Head dims above 256, or not a multiple of 8 (rows would not be 16-byte aligned), are refused."""
-    shape = ra.AttentionShape.new(1, 1, 8, d)
-    z = dev(np.zeros(8 * d, dtype=np.uint16))
+@pytest.mark.parametrize("d", [4, 100, 257, 264, 320, 12])
+@pytest.mark.parametrize("n", [1, 33, 130])
+def test_head_dims_outside_the_matrix_core_kernels(oracle, n, d):
+    """Head dims above 256, or not a multiple of 8 (rows are then not 16-byte aligned): a workgroup per query row, the
+    same masks and row rules (the reference takes any dim != 0, cpu_forward.rs:142-169)."""
+    b, h = 2, 3
+    (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d), (n, n + 1, n + 2))
+    shape = ra.AttentionShape.new(b, h, n, d)
+    keep = np.random.default_rng(n).random(n) < 0.7
+    keep[0] = True
+    for mask, om in ((ra.Mask.none(), None), (ra.Mask.causal(), "causal"), (ra.Mask.padding(keep), ("padding", keep)),
+                     (ra.Mask.padding(np.zeros(n, bool)), ("padding", np.zeros(n, bool)))):
+        got = flash_bf16(shape, qb, kb, vb, mask)
+        want = oracle.flash_forward_masked(oracle.AttentionShape(b, h, n, d), qf, kf, vf, om)
+        assert_bf16_parity(got, want, d, n, f"n={n} d={d} mask={mask.kind}")
+    lens = [n, n // 2]
+    for zero in (True, False):
+        got = run_varlen(shape, qb, kb, vb, lens, zero)
+        want = oracle.varlen_causal_forward(qf, kf, vf, lens, b, h, n, d, zero_padded_rows=zero)
+        assert_bf16_parity(got, want, d, n, f"varlen n={n} d={d}")
+
+
+def test_head_dim_above_512_is_an_error():
+    shape = ra.AttentionShape.new(1, 1, 8, 520)
+    z = dev(np.zeros(8 * 520, dtype=np.uint16))
     with pytest.raises(ra.DeviceError) as ei:
         ra.flash_forward_bf16_dev(shape, z, z, z, z)
-    assert ei.value.status == 21
+    assert ei.value.status == 21 and ei.value.expected == 512
 
 
 @pytest.mark.parametrize("kernel", ["persistent", "tile"])

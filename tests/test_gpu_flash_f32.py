@@ -61,12 +61,27 @@ def test_flash_head_dims_above_128(oracle, bhnd):
         assert_close_nan(got, want, TOL, f"{bhnd} mask={mask.kind}")
 
 
-def test_flash_head_dim_above_256_is_refused():
-    shape = ra.AttentionShape.new(1, 1, 4, 257)
+@pytest.mark.parametrize("bhnd", [(1, 2, 70, 257), (2, 1, 33, 320), (1, 1, 130, 512), (1, 2, 5, 300)])
+def test_flash_head_dims_above_256(oracle, bhnd):
+    """The reference takes any dim != 0 (cpu_forward.rs:142-169): above the tiled kernels a workgroup per query row
+    serves the same masks and row rules, fully masked rows and the leading-masked-tile rule included."""
+    shape = ra.AttentionShape.new(*bhnd)
+    q, k, v = buffers(shape.buffer_len(), 2.0)
+    n = bhnd[2]
+    keep = np.arange(n) % 3 != 1
+    lead = np.r_[np.zeros(min(64, n), bool), np.ones(max(n - 64, 0), bool)]
+    for mask in (ra.Mask.none(), ra.Mask.causal(), ra.Mask.padding(keep), ra.Mask.padding(lead), ra.Mask.padding(np.zeros(n, bool))):
+        got = ra.flash_forward_masked(shape, q, k, v, mask)
+        want = oracle.flash_forward_masked(oracle.AttentionShape(*bhnd), q, k, v, omask(mask))
+        assert_close_nan(got, want, TOL, f"{bhnd} mask={mask.kind}")
+
+
+def test_flash_head_dim_above_512_is_refused():
+    shape = ra.AttentionShape.new(1, 1, 4, 513)
     z = np.zeros(shape.buffer_len(), np.float32)
     with pytest.raises(ra.DeviceError) as ei:
         ra.flash_forward(shape, z, z, z)
-    assert ei.value.status == 21
+    assert ei.value.status == 21 and ei.value.expected == 512
 
 
 def test_scaling_factor_is_one_over_sqrt_d():
