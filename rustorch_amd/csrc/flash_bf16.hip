@@ -271,10 +271,18 @@ __global__ __launch_bounds__(NTHREADS, 1) void flash_fwd_bf16_kernel(FlashBf16Pa
         }
         int r = kv0 + ld_row0 + NWAVES * RPI * n;
         asm volatile("" : "+v"(r));  // recompute per call: hoisted copies of these offsets only cost registers
+        const bool past_end = r >= n_keys;
         r = min(r, n_keys - 1);
         const uint32_t row_off = (uint32_t)r * kv_pitch_b;  // seq * row pitch stays below 4 GiB (checked by the caller)
         load_to_lds(Kg, row_off + ld_k0, kdst);
-        load_to_lds(Vg, row_off + ld_v0, kdst + 2 * TILE_B);
+        // V rows behind the last key are zeros: their weights are zero, and zero times a copy of a non-finite last
+        // row would be NaN.  An ordinary LDS write (lgkmcnt), complete before the barrier that publishes the tile:
+        // every cluster starts with lgkmcnt(0), and a job's first tile is published by __syncthreads.
+        if (past_end) {
+            *(u32x4_t*)(lds + (st * TILE_B + (wave + NWAVES * n) * 1024) + 2 * TILE_B + 16 * lane) = u32x4_t{0u, 0u, 0u, 0u};
+        } else {
+            load_to_lds(Vg, row_off + ld_v0, kdst + 2 * TILE_B);
+        }
     };
     auto load_tile = [&](int kv0, int st) {
 #pragma unroll

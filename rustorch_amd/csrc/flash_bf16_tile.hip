@@ -270,7 +270,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             __syncthreads();
         }
         const int last_kv0 = (n_tiles - 1) * KT;
-        // rows past the end re-read the last key; they are masked in the score tile
+        // rows past the end re-read the last key: masked in the score tile, and parked as zeros for V (see park_v)
         auto chunk_at = [&](int n, int kv0) __attribute__((always_inline)) { return (size_t)(uint32_t)min(kv0 + ld_row[n], n_keys - 1) * kv_pitch + ld_col[n]; };
         auto issue_k = [&](u32x4_t (&dst)[NL], int kv0) __attribute__((always_inline)) {
             kv0 = min(kv0, last_kv0);
@@ -295,21 +295,23 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
                 if (D == DP || ld_on[n]) *(u32x4_t*)(lds + st * (KT * LDK * 2) + st_k[n]) = src[n];
         };
         uint64_t keep_cur = ~0ull, keep_next = ~0ull;  // keep bits of the tile whose items are in their softmax step, and of the next
-        auto park_v = [&](auto set_c, int st) __attribute__((always_inline)) {
+        // `kv0` is the first key of the tile in the set.  In the tile that holds the last key the rows behind it become
+        // zero: their weights are zero, and zero times a copy of a non-finite last row would be NaN.
+        auto park_v = [&](auto set_c, int st, int kv0) __attribute__((always_inline)) {
             constexpr int SET = decltype(set_c)::value;
+            if (kv0 + KT > n_keys) {
+#pragma unroll
+                for (int n = 0; n < NL; n++)
+                    if (kv0 + ld_row[n] >= n_keys) vreg[SET][n] = u32x4_t{0u, 0u, 0u, 0u};
+            }
 #pragma unroll
             for (int n = 0; n < NL; n++)
                 if (D == DP || ld_on[n]) *(u32x4_t*)(lds + st * (KT * LDV * 2) + st_v[n]) = vreg[SET][n];
             if (MODE == kMaskPadding) keep_next = __ballot(keep_raw[SET] != 0);
         };
 
-        // tile 0's early requests: V rows past the last key become zero, keep bytes past it count as kept
-        if (n_keys < KT) {
-#pragma unroll
-            for (int n = 0; n < NL; n++)
-                if (ld_row[n] >= n_keys) vreg[0][n] = u32x4_t{0u, 0u, 0u, 0u};
-            if (MODE == kMaskPadding && (lane & (KT - 1)) >= n_keys) keep_raw[0] = 1u;
-        }
+        // tile 0's early requests: keep bytes past the last key count as kept
+        if (MODE == kMaskPadding && n_keys < KT && (lane & (KT - 1)) >= n_keys) keep_raw[0] = 1u;
 
         // ---- this lane's query row
         const int r = q0 + 32 * wq + col;
@@ -378,7 +380,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         // K(0), V(0) -> stage 0, K(1) -> stage 1; then the register sets take K(2) .. K(1 + PF) and V(1) .. V(PF)
         // (K(j) travels in set j % PF, and so does V(j))
         park_k(kreg[0], 0);
-        park_v(std::integral_constant<int, 0>{}, 0);
+        park_v(std::integral_constant<int, 0>{}, 0, 0);
         keep_cur = keep_next;
         if (PIPE) park_k(k1, 1);
         {
@@ -666,7 +668,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             const int st = st_c;  // t & 1, as a constant where the caller knows it
             // (behind the last tiles these park and request copies of the last tile, which nobody reads)
             park_k(kreg[KSET], st);
-            park_v(vset_c, st ^ 1);
+            park_v(vset_c, st ^ 1, (t + 1) * KT);
             issue_k(kreg[KSET], (t + 2 + PF) * KT);
             issue_v(vset_c, (t + 1 + PF) * KT);
         };
@@ -723,7 +725,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
                     if (t * NI + it < n_it)
                         step_simple(it, t * KT + 32 * it, Ks + st * KT * LDK + 32 * it * LDK + k_off, Vs + st * KT * LDV + 32 * it * LDV + v_off);
                 park_k(kreg[0], st ^ 1);
-                park_v(std::integral_constant<int, 0>{}, st ^ 1);
+                park_v(std::integral_constant<int, 0>{}, st ^ 1, (t + 1) * KT);
                 issue_k(kreg[0], (t + 2) * KT);
                 issue_v(std::integral_constant<int, 0>{}, (t + 2) * KT);
                 __syncthreads();

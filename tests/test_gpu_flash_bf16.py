@@ -305,6 +305,35 @@ def test_non_finite_v_row_at_a_causally_hidden_position(oracle, force_kernel, ke
     assert np.isfinite(got[..., :5]).all() and np.isfinite(want_ref[..., :5]).all()
 
 
+@pytest.mark.parametrize("kernel", ["persistent", "tile"])
+@pytest.mark.parametrize("mask", ["none", "padding"])
+@pytest.mark.parametrize("n,d", [(200, 128), (100, 128), (200, 64), (40, 64), (330, 96)])
+def test_infinite_last_v_row_with_a_ragged_last_key_tile(oracle, force_kernel, kernel, mask, n, d):
+    """+Inf in the last key's V row, sequence lengths that end inside a key tile.  Every row that weighs that key
+    gets +Inf in that column, as in the reference (cpu_forward.rs:268-425); the key slots behind the last key carry
+    weight zero and must not turn the column into NaN (0 * Inf), whichever tile the last key falls in."""
+    force_kernel(kernel)
+    b, h = 2, 2
+    (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d), (61, 62, 63))
+    vbad = vf.copy().reshape(b, h, n, d)
+    vbad[:, :, n - 1, 5] = np.inf
+    vbad = vbad.ravel()
+    shape, osh = ra.AttentionShape.new(b, h, n, d), oracle.AttentionShape(b, h, n, d)
+    if mask == "padding":
+        keep = np.ones(n, dtype=bool)
+        keep[3] = keep[n // 2] = False
+        want = oracle.flash_forward_masked(osh, qf, kf, vbad, ("padding", keep)).reshape(b, h, n, d)
+        got = flash_bf16(shape, qb, kb, oracle.f32_to_bf16(vbad), ra.Mask.padding(keep)).reshape(b, h, n, d)
+    else:
+        want = oracle.flash_forward_masked(osh, qf, kf, vbad, None).reshape(b, h, n, d)
+        got = flash_bf16(shape, qb, kb, oracle.f32_to_bf16(vbad)).reshape(b, h, n, d)
+    assert np.isposinf(want[..., 5]).all()
+    assert np.isposinf(got[..., 5]).all()
+    rest = np.ones(d, dtype=bool)
+    rest[5] = False
+    assert np.isfinite(got[..., rest]).all() and max_abs(got[..., rest], want[..., rest]) <= TOL
+
+
 @pytest.mark.parametrize("kernel,d", [("persistent", 64), ("persistent", 128), ("tile", 64), ("tile", 128), ("tile", 96)])
 def test_two_launches_give_the_same_bits(force_kernel, kernel, d):
     """No atomics, no order that depends on timing: the same inputs give the same output bits on every launch.
