@@ -183,18 +183,20 @@ int rt_flash_backward_saved_f32_dev(void *stream, const rt_attention_shape *shap
  * probabilities (exact zeros) into V, so a NaN or Inf in V row j makes EVERY query row NaN in that column
  * (0 * NaN; cpu_forward.rs:268-425 skips no tile).  The kernels skip key tiles that lie wholly past a query tile
  * and never read those rows: query rows i >= j are NaN as in the reference, rows i <= j - 256 are finite (the value
- * the reference gives with V row j zeroed), rows in between may be either.  Finite inputs are unaffected. */
+ * the reference gives with V row j zeroed), rows in between may be either.  Finite inputs are unaffected.
+ * rt_set_strict_non_finite_v(1) removes the divergence at the cost of one more pass over V. */
 int rt_flash_forward_f32_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const float *q,
                              const float *k, const float *v, int mask_kind, const uint8_t *keep, float *out,
                              rt_err_detail *err);
 
 /* The bf16 counterpart (bf16 in, f32 accumulate, bf16 out rounded once, to nearest even):
- * q/out [batch,heads,seq,dim], k/v [batch,n_kv_heads,seq,dim].  Any dim up to 256 that is a multiple of 8 (the
- * reference's forward takes any dim != 0, cpu_forward.rs:142-169; other dims return RT_ERR_UNSUPPORTED here and
- * are served by the f32 entries); tensors 16-byte aligned.  Two MFMA kernels stand behind it: a persistent
- * 8-wave kernel for dim 64 / 128 on unpadded batches of at least 512 rows per sequence and 256 jobs of 256 rows,
- * and a 4-wave tile kernel for everything else (short or few sequences, padded batches, other dims).
- * rt_debug_force_bf16_prefill_kernel forces one of them where both apply. */
+ * q/out [batch,heads,seq,dim], k/v [batch,n_kv_heads,seq,dim].  Any dim up to 512 (the reference's forward takes
+ * any dim != 0, cpu_forward.rs:142-169; above 512: RT_ERR_UNSUPPORTED with expected = 512).  Two MFMA kernels serve
+ * dims up to 256 that are a multiple of 8 on 16-byte aligned tensors: a persistent 8-wave kernel for dim 64 / 128 on
+ * unpadded batches of at least 512 rows per sequence and one job of 256 rows per compute unit, and a 4-wave tile
+ * kernel for everything else (short or few sequences, padded batches, other dims);
+ * rt_debug_force_bf16_prefill_kernel forces one of them where both apply.  The remaining dims and alignments run on
+ * a one-workgroup-per-row kernel with the same masks and row rules (correct at any speed, not tuned). */
 int rt_flash_forward_bf16_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const void *q,
                               const void *k, const void *v, int mask_kind, const uint8_t *keep, void *out,
                               rt_err_detail *err);
@@ -204,6 +206,14 @@ int rt_flash_forward_bf16_dev(void *stream, const rt_attention_shape *shape, uin
  * (head dim 64 / 128, no per-sequence lengths).  Process-wide; until it is called the value is taken, once, from
  * RT_ATTN_BF16_PREFILL=tile|persistent in the environment.  Returns RT_ERR_UNSUPPORTED for another value. */
 int rt_debug_force_bf16_prefill_kernel(int which);
+
+/* No counterpart in the reference, whose CPU loop needs none: on != 0 makes every causal prefill entry (f32 and bf16,
+ * every layout, padded batches included) follow its kernel with a pass that reads V once and writes NaN into each
+ * (query row, column) for which a key the row does not see holds a NaN or Inf in that column of V -- the outcome of
+ * cpu_forward.rs:268-425, which multiplies the hidden zeros into every V tile.  Off by default: the pass costs a
+ * read of V (a few percent of a long prefill, more of a short one) and changes nothing for finite V.  Process-wide;
+ * returns the previous setting. */
+int rt_set_strict_non_finite_v(int on);
 
 /* The same two calls on tensors laid out [batch, seq, heads, dim] (k/v: [batch, seq, n_kv_heads, dim]),
  * the layout rustorch_nn::MultiHeadAttention holds its projections in: the kernels walk the rows with a

@@ -22,7 +22,7 @@ SYMBOLS = (
     "rt_kv_append_bf16", "rt_kv_cache_append_dev", "rt_qk_norm_rope_kv_append_bf16", "rt_gqa_decode_online_bf16", "rt_gqa_decode_naive_bf16", "rt_gqa_decode_batched_bf16",
     "rt_gqa_decode_workspace_bytes", "rt_gqa_decode_batched_bf16_noalloc",
     "rt_buf_alloc", "rt_buf_free", "rt_buf_zero", "rt_memcpy_h2d", "rt_memcpy_d2h", "rt_stream_synchronize",
-    "rt_stream_create", "rt_stream_destroy", "rt_i32_add_dev", "rt_debug_force_bf16_prefill_kernel",
+    "rt_stream_create", "rt_stream_destroy", "rt_i32_add_dev", "rt_debug_force_bf16_prefill_kernel", "rt_set_strict_non_finite_v",
 )
 
 RT_OK = 0
@@ -123,6 +123,8 @@ def lib():
     L.rt_stream_destroy.argtypes = [vp, errp]
     L.rt_i32_add_dev.argtypes = [vp, vp, sz, i32, errp]
     L.rt_debug_force_bf16_prefill_kernel.argtypes = [C.c_int]
+    L.rt_set_strict_non_finite_v.argtypes = [C.c_int]
+    L.rt_set_strict_non_finite_v.restype = C.c_int
     _lib = L
     return L
 

@@ -138,6 +138,35 @@ int check_flash_dims(const rt_attention_shape* s, uint64_t n_kv_heads, rt_err_de
 }
 
 // bnhd: tensors are [batch, seq, heads, dim] instead of [batch, heads, seq, dim]
+// rt_set_strict_non_finite_v: off by default
+std::atomic<int> g_strict_v{0};
+
+// After a causal forward, when the strict switch is on: the pass that gives query rows the reference's NaN for
+// non-finite V elements at keys they do not see (the forward kernels skip those key tiles).
+int strict_pass(hipStream_t stream, const rt_attention_shape* s, uint64_t n_kv_heads, const void* v, void* out,
+                const int32_t* seq_lens, int mask_kind, bool bnhd, bool bf16, rt_err_detail* err) {
+    if (mask_kind != rt::kMaskCausal && mask_kind != rt::kMaskVarlenCausal) return RT_OK;
+    if (!g_strict_v.load(std::memory_order_relaxed)) return RT_OK;
+    rt::StrictVParams p{};
+    p.v = v;
+    p.out = out;
+    p.seq_lens = seq_lens;
+    p.batch = (int)s->batch;
+    p.heads = (int)s->heads;
+    p.kv_heads = (int)n_kv_heads;
+    p.seq = (int)s->seq;
+    p.dim = (int)s->dim;
+    if (bnhd) {
+        p.lo = rt::layout_bnhd((long long)s->heads, (long long)s->seq, p.dim);
+        p.lkv = rt::layout_bnhd((long long)n_kv_heads, (long long)s->seq, p.dim);
+    } else {
+        p.lo = rt::layout_bhnd((long long)s->heads, (long long)s->seq, p.dim);
+        p.lkv = rt::layout_bhnd((long long)n_kv_heads, (long long)s->seq, p.dim);
+    }
+    HIP_TRY(rt::launch_strict_hidden_v(stream, p, bf16), "strict_hidden_v launch");
+    return RT_OK;
+}
+
 int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n_kv_heads, const float* q,
                      const float* k, const float* v, int mask_kind, const uint8_t* keep, float* out,
                      rt_err_detail* err, bool bnhd = false, const float* bias = nullptr, long long bias_bh_stride = 0,
@@ -175,7 +204,7 @@ int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n
         r.flash_rows = 1;
         r.lse = lse;
         HIP_TRY(rt::launch_attn_rows_f32(stream, r), "attn_rows_f32 launch");
-        return RT_OK;
+        return seq_kv ? RT_OK : strict_pass(stream, s, n_kv_heads, v, out, nullptr, mask_kind, bnhd, false, err);
     }
     rt::FlashF32Params p{};
     p.bias = bias;
@@ -206,7 +235,7 @@ int flash_f32_device(hipStream_t stream, const rt_attention_shape* s, uint64_t n
         p.lkv = rt::layout_bhnd((long long)n_kv_heads, kv_rows, p.dim);
     }
     HIP_TRY(rt::launch_flash_f32(stream, p), "flash_fwd_f32 launch");
-    return RT_OK;
+    return seq_kv ? RT_OK : strict_pass(stream, s, n_kv_heads, v, out, nullptr, mask_kind, bnhd, false, err);
 }
 
 // Scratch the library keeps for entry points whose reference signature has no workspace argument: one buffer per
@@ -776,6 +805,8 @@ RT_API int rt_debug_force_bf16_prefill_kernel(int which) {
     return RT_OK;
 }
 
+RT_API int rt_set_strict_non_finite_v(int on) { return g_strict_v.exchange(on ? 1 : 0); }
+
 static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads, const void* q,
                              const void* k, const void* v, int mask, const uint8_t* keep, const int32_t* seq_lens,
                              int zero_padded_rows, void* out, rt_err_detail* err, bool bnhd = false) {
@@ -827,7 +858,7 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
         r.flash_rows = 1;
         r.zero_padded_rows = zero_padded_rows;
         HIP_TRY(rt::launch_attn_rows_bf16((hipStream_t)stream, r), "attn_rows_bf16 launch");
-        return RT_OK;
+        return strict_pass((hipStream_t)stream, shape, n_kv_heads, v, out, seq_lens, mask, bnhd, true, err);
     }
     // the persistent kernel needs a job (256 query rows of one head) for every CU and gains on the tile kernel as the
     // rows get longer; a padded batch is a set of jobs of very different lengths, which the tile kernel's
@@ -879,7 +910,7 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
         t.lq = t.lo = lq;
         t.lkv = lkv;
         HIP_TRY(rt::launch_flash_tile_bf16((hipStream_t)stream, t), "flash_tile_bf16 launch");
-        return RT_OK;
+        return strict_pass((hipStream_t)stream, shape, n_kv_heads, v, out, seq_lens, mask, bnhd, true, err);
     }
     rt::FlashBf16Params p;
     p.q = (const uint16_t*)q;
@@ -902,7 +933,7 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
     p.lq = p.lo = lq;
     p.lkv = lkv;
     HIP_TRY(rt::launch_flash_bf16((hipStream_t)stream, p), "flash_fwd_bf16 launch");
-    return RT_OK;
+    return strict_pass((hipStream_t)stream, shape, n_kv_heads, v, out, seq_lens, mask, bnhd, true, err);
 }
 
 RT_API int rt_flash_forward_bf16_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,

@@ -692,6 +692,59 @@ hipError_t launch_attn_rows_bf16(hipStream_t stream, const AttnRowsParams& p) {
     return hipGetLastError();
 }
 
+// The reference's outcome for a non-finite V element under the causal mask (cpu_forward.rs:268-425 walks every key
+// tile and multiplies the hidden probabilities, exact zeros, into V: 0 * NaN and 0 * Inf are NaN).  The forward kernels
+// skip key tiles that no row of a query tile sees, so this pass, run after them on request, restores that outcome:
+// one workgroup per (batch, kv head) finds, per column, the last key whose V element is not finite, and writes NaN
+// into that column of every query row that does not see that key.  Rows that see it already hold what the reference
+// holds (the kernels multiply every key a row sees).  Reads V once; writes only where something was found.
+template <typename T>
+__global__ __launch_bounds__(256) void strict_hidden_v_kernel(StrictVParams p) {
+    const int kvh = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const int group = p.heads / p.kv_heads;
+    int n_keys = p.seq, n_q = p.seq;
+    if (p.seq_lens) n_keys = n_q = min(max(p.seq_lens[b], 0), p.seq);
+    __shared__ int last_bad[512];
+    for (int c = tid; c < p.dim; c += 256) last_bad[c] = -1;
+    __syncthreads();
+    const T* vb = (const T*)p.v + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+    // thread t looks at columns t % cw + k * cw of rows t / cw + k * (256 / cw): consecutive lanes, consecutive addresses
+    const int cw = p.dim >= 256 ? 256 : (p.dim >= 128 ? 128 : (p.dim >= 64 ? 64 : (p.dim >= 32 ? 32 : 16)));
+    const int rows_per_pass = 256 / cw;
+    for (int c = tid % cw; c < p.dim; c += cw) {
+        int mine = -1;
+        for (int j = tid / cw; j < n_keys; j += rows_per_pass) {
+            const T x = vb[(size_t)j * p.lkv.row_pitch + c];
+            bool bad;
+            if constexpr (sizeof(T) == 2) bad = (x & 0x7f80u) == 0x7f80u;
+            else bad = (__float_as_uint(x) & 0x7f800000u) == 0x7f800000u;
+            mine = bad ? j : mine;
+        }
+        if (mine >= 0) atomicMax(&last_bad[c], mine);
+    }
+    __syncthreads();
+    const int off = n_keys - n_q;  // query row i sees keys j <= i + off
+    for (int c = 0; c < p.dim; c++) {
+        const int hidden_rows = min(last_bad[c] - off, n_q);  // rows 0 .. hidden_rows-1 do not see that key
+        if (hidden_rows <= 0) continue;
+        for (int g = 0; g < group; g++) {
+            T* ob = (T*)p.out + (size_t)b * p.lo.batch_stride + (size_t)(kvh * group + g) * p.lo.head_stride + c;
+            for (int i = tid; i < hidden_rows; i += 256) {
+                if constexpr (sizeof(T) == 2) ob[(size_t)i * p.lo.row_pitch] = (T)0x7fc0u;
+                else ob[(size_t)i * p.lo.row_pitch] = __uint_as_float(0x7fc00000u);
+            }
+        }
+    }
+}
+
+hipError_t launch_strict_hidden_v(hipStream_t stream, const StrictVParams& p, bool bf16) {
+    if (p.batch == 0 || p.heads == 0 || p.seq == 0) return hipSuccess;
+    if (p.dim > 512 || p.kv_heads <= 0 || p.heads % p.kv_heads != 0 || p.kv_heads > 65535 || p.batch > 65535) return hipErrorInvalidValue;
+    if (bf16) hipLaunchKernelGGL(strict_hidden_v_kernel<uint16_t>, dim3(p.kv_heads, p.batch), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(strict_hidden_v_kernel<float>, dim3(p.kv_heads, p.batch), dim3(256), 0, stream, p);
+    return hipGetLastError();
+}
+
 hipError_t launch_kv_append_bf16(hipStream_t stream, uint16_t* k_cache, uint16_t* v_cache, const uint16_t* k_in,
                                  const uint16_t* v_in, int pos, int n_kv, int head_dim, int max_seq) {
     int n = n_kv * head_dim;

@@ -163,6 +163,18 @@ struct AttnRowsParams {
 hipError_t launch_attn_rows_f32(hipStream_t stream, const AttnRowsParams& p);
 hipError_t launch_attn_rows_bf16(hipStream_t stream, const AttnRowsParams& p);
 
+// The pass behind rt_set_strict_non_finite_v: NaN into every (query row, column) whose causally hidden keys hold a
+// non-finite V element in that column.  Tensors f32 or bf16 bits ([batch, heads | kv_heads, seq, dim] through the
+// layouts); head_map as in flash_forward (kv_h = h / (heads / kv_heads)); seq_lens optional (padded batches).
+struct StrictVParams {
+    const void* v;
+    void* out;
+    const int32_t* seq_lens;
+    int batch, heads, kv_heads, seq, dim;
+    TensorLayout lkv, lo;
+};
+hipError_t launch_strict_hidden_v(hipStream_t stream, const StrictVParams& p, bool bf16);
+
 struct DecodeSplitParams {
     const uint16_t* q;        // [batch, heads, dim]
     const uint16_t* k_cache;  // [batch, kv_heads, max_seq, dim]

@@ -125,6 +125,12 @@ def debug_force_bf16_prefill_kernel(name: str = "auto"):
         raise ValueError(name)
 
 
+def set_strict_non_finite_v(on: bool) -> bool:
+    """Causal prefill entries follow the reference for non-finite V at hidden keys (every row NaN in that column,
+    cpu_forward.rs:268-425) at the cost of one more pass over V.  Returns the previous setting."""
+    return bool(L.lib().rt_set_strict_non_finite_v(1 if on else 0))
+
+
 def dev_ptr(x) -> int:
     """Raw device address of a HipStorage, a torch tensor on the GPU, or an int."""
     if x is None:

@@ -210,6 +210,14 @@ def test_shutdown_without_a_device_is_a_no_op():
     ra.shutdown()
 
 
+def test_process_wide_switches_need_no_device():
+    lib = L.lib()
+    assert lib.rt_set_strict_non_finite_v(1) == 0 and lib.rt_set_strict_non_finite_v(0) == 1
+    assert lib.rt_set_strict_non_finite_v(0) == 0
+    assert lib.rt_debug_force_bf16_prefill_kernel(7) == L.RT_ERR_UNSUPPORTED
+    assert lib.rt_debug_force_bf16_prefill_kernel(0) == L.RT_OK
+
+
 def test_general_bf16_entries_argument_errors_before_any_device_use():
     """rt_mha_forward_masked_bf16_dev, rt_gqa_decode_chunk_bf16 and rt_gqa_decode_batched_bf16_noalloc refuse bad
     arguments in the host checks (the pointers below are never dereferenced)."""

@@ -173,6 +173,28 @@ def test_varlen_small(oracle, force_kernel, kernel, d):
                 assert (g[i, :, L:] == 0.0).all() and not np.signbit(g[i, :, L:]).any()
 
 
+def test_strict_mode_on_a_padded_batch(oracle, strict_v):
+    """The strict pass takes each sequence's own length: a non-finite V element inside a sequence reaches the rows
+    before its key, one in the padding behind a sequence reaches nothing."""
+    b, h, n, d = 3, 2, 400, 64
+    lens = [400, 130, 257]
+    (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d), (71, 72, 73))
+    v4 = vf.copy().reshape(b, h, n, d)
+    v4[0, 1, 399, 7] = np.inf
+    v4[1, 0, 129, 0] = np.nan
+    v4[1, 1, 131, 3] = np.nan   # behind the 130 keys of sequence 1
+    v4[2, 0, 5, 9] = -np.inf
+    shape = ra.AttentionShape.new(b, h, n, d)
+    strict_v(True)
+    got = run_varlen(shape, qb, kb, oracle.f32_to_bf16(v4.ravel()), lens, True).reshape(b, h, n, d)
+    want = oracle.varlen_causal_forward(qf, kf, v4.ravel(), lens, b, h, n, d, zero_padded_rows=True).reshape(b, h, n, d)
+    assert np.array_equal(np.isfinite(got), np.isfinite(want))
+    assert np.isnan(got[0, 1, :399, 7]).all() and np.isnan(got[1, 0, :129, 0]).all() and np.isnan(got[2, 0, :5, 9]).all()
+    assert np.isfinite(got[1, 1]).all() and (got[1, :, 130:] == 0.0).all()
+    fin = np.isfinite(want)
+    assert np.abs(got[fin] - want[fin]).max() <= TOL
+
+
 @pytest.mark.parametrize("kernel", ["auto", "persistent", "tile"])
 def test_config_padded_batch_b16_h16_n1024_d64(oracle, force_kernel, kernel):
     """The variable-length workload of the benchmark set: lengths uniform in [128, 1024] from a seed, key padding + causal,
@@ -270,6 +292,40 @@ def test_head_dim_above_512_is_an_error():
     with pytest.raises(ra.DeviceError) as ei:
         ra.flash_forward_bf16_dev(shape, z, z, z, z)
     assert ei.value.status == 21 and ei.value.expected == 512
+
+
+@pytest.fixture
+def strict_v():
+    yield ra.set_strict_non_finite_v
+    ra.set_strict_non_finite_v(False)
+
+
+@pytest.mark.parametrize("kernel,n,d,j", [("persistent", 1024, 128, 700), ("tile", 1024, 128, 700), ("tile", 777, 64, 500),
+                                          ("tile", 300, 100, 299)])
+@pytest.mark.parametrize("bad", [np.nan, -np.inf])
+def test_strict_mode_gives_the_reference_outcome_for_non_finite_v(oracle, force_kernel, strict_v, kernel, n, d, j, bad):
+    """With rt_set_strict_non_finite_v on, a non-finite V element at key j makes that column NaN in every row that
+    does not see key j, as the reference's walk over every key tile does (cpu_forward.rs:268-425); rows that see it
+    are non-finite as before, and every other column equals the oracle's."""
+    force_kernel(kernel)
+    assert strict_v(True) is False
+    b, hq, hkv = 2, 4, 2
+    (qb, qf), (kb, kf), (vb, vf) = inputs((b, hq, n, d), (b, hkv, n, d), (51, 52, 53))
+    vbad = vf.copy().reshape(b, hkv, n, d)
+    vbad[1, 0, j, 5] = bad
+    vbad[0, 1, j // 2, 2] = bad
+    vbad = vbad.ravel()
+    shape = ra.AttentionShape.new(b, hq, n, d)
+    got = flash_bf16(shape, qb, kb, oracle.f32_to_bf16(vbad), ra.Mask.causal(), n_kv_heads=hkv).reshape(b, hq, n, d)
+    g = hq // hkv
+    k4, v4 = kf.reshape(b, hkv, n, d), vbad.reshape(b, hkv, n, d)
+    want = oracle.flash_forward_masked(oracle.AttentionShape(b, hq, n, d), qf, np.repeat(k4, g, axis=1).ravel(),
+                                       np.repeat(v4, g, axis=1).ravel(), "causal").reshape(b, hq, n, d)
+    assert np.array_equal(np.isfinite(got), np.isfinite(want))
+    assert np.isnan(got[1, 0:g, :j, 5]).all() and np.isnan(got[0, g:2 * g, :j // 2, 2]).all()
+    fin = np.isfinite(want)
+    assert np.abs(got[fin] - want[fin]).max() <= TOL
+    assert strict_v(False) is True
 
 
 @pytest.mark.parametrize("kernel", ["persistent", "tile"])

@@ -310,6 +310,29 @@ def test_host_slice_calls_from_several_threads(oracle):
     assert not errors, errors[:3]
 
 
+@pytest.mark.parametrize("n,d,j", [(600, 64, 400), (300, 128, 290), (200, 320, 150)])
+@pytest.mark.parametrize("bad", [np.nan, -np.inf])
+def test_strict_mode_gives_the_reference_outcome_for_non_finite_v(oracle, n, d, j, bad):
+    """rt_set_strict_non_finite_v: the column of a non-finite V element is NaN in every row that does not see its
+    key, as in the reference (cpu_forward.rs:268-425); finite elements agree with the oracle as ever."""
+    b, h = 2, 2
+    q, k, v = (seeded_normal(b * h * n * d, s) for s in (61, 62, 63))
+    vbad = v.copy().reshape(b, h, n, d)
+    vbad[1, 0, j, 3] = bad
+    vbad[0, 1, n - 1, 0] = bad
+    shape, osh = ra.AttentionShape.new(b, h, n, d), oracle.AttentionShape(b, h, n, d)
+    want = oracle.flash_forward_masked(osh, q, k, vbad.ravel(), "causal").reshape(b, h, n, d)
+    assert ra.set_strict_non_finite_v(True) is False
+    try:
+        got = ra.flash_forward_masked(shape, q, k, vbad.ravel(), ra.Mask.causal()).reshape(b, h, n, d)
+    finally:
+        assert ra.set_strict_non_finite_v(False) is True
+    assert np.array_equal(np.isfinite(got), np.isfinite(want))
+    assert np.isnan(got[1, 0, :j, 3]).all() and np.isnan(got[0, 1, :n - 1, 0]).all()
+    fin = np.isfinite(want)
+    assert np.abs(got[fin] - want[fin]).max() <= TOL
+
+
 @pytest.mark.parametrize("bad", [np.nan, -np.inf])
 def test_non_finite_v_row_at_a_causally_hidden_position(oracle, bad):
     """A non-finite V row j under the causal mask.  The reference multiplies the hidden probabilities (exact zeros)
