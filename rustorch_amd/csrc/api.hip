@@ -829,7 +829,10 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
     // The matrix-core kernels move 16 bytes at a time: head dims up to 256 that are a multiple of 8, tensors 16-byte
     // aligned.  Everything else (the reference takes any dim != 0, cpu_forward.rs:142-169) goes to the
     // one-workgroup-per-row kernel: same masks, same row rules, any speed.
-    if (shape->dim > 256 || shape->dim % 8 != 0 || (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0) {
+    // (so does a K/V slab of 4 GiB or more per (batch, kv head): the tile kernel addresses it with 32-bit offsets)
+    const bool tile_addressable = rt::flash_tile_bf16_addressable((long long)shape->seq, (long long)((bnhd ? n_kv_heads : 1) * shape->dim));
+    if (shape->dim > 256 || shape->dim % 8 != 0 || (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0 ||
+        !tile_addressable) {
         rt::AttnRowsParams r{};
         r.q = q;
         r.k = k;
@@ -1132,7 +1135,8 @@ RT_API int rt_mha_forward_masked_bf16_dev(void* stream, const void* q, const voi
     if (((uintptr_t)mask & 3) != 0) return fail(err, RT_ERR_UNSUPPORTED, -1, 4, 0, "the mask must be 4-byte aligned");
     int rc = ensure_device(err);
     if (rc) return rc;
-    if (!rt::flash_tile_bf16_supported((int)head_dim) || (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0) {
+    if (!rt::flash_tile_bf16_supported((int)head_dim) || (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0 ||
+        !rt::flash_tile_bf16_addressable((long long)t_kv, (long long)(heads * head_dim))) {
         // head dims and alignments the matrix-core kernel does not cover: one workgroup per query row, any speed
         if (t_kv == 0) return rt_buf_zero(out, q_expected * 2, stream, err);
         rt::AttnRowsParams r{};
@@ -1403,6 +1407,8 @@ RT_API int rt_gqa_decode_chunk_bf16(void* stream, const void* q, const void* k_c
                     "bf16 kernels cover head dims up to 256 that are a multiple of 8");
     if ((((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)out) & 15) != 0)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 16, 0, "bf16 kernels need 16-byte aligned tensors");
+    if (!rt::flash_tile_bf16_addressable((long long)max_seq, (long long)head_dim))
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, (uint64_t)max_seq, "a cache slab of one (sequence, kv head) must stay below 4 GiB");
     const int group = n_heads / n_kv;
     if (((int64_t)seq_new * group + 127) / 128 > 65535 || batch > 65535 || n_kv > 65535)
         return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");

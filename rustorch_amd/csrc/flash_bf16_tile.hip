@@ -30,6 +30,7 @@ namespace rt {
 
 namespace {
 
+constexpr uint32_t kBufferFlags = 0x00020000u;  // dword 3 of a raw buffer descriptor: 32-bit data format, no swizzle
 constexpr int TROWS = 128;  // query rows per workgroup: four waves' worth, each wave 32
 constexpr float kTileTrigSum = 65536.0f;  // a lane's 16-key share of a row sum above this sends the wave to the slow path
 
@@ -146,21 +147,13 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     const int rows_total = p.seq_q * G;
     const int hx = blockIdx.x, b = blockIdx.y;
     const int zz = (int)gridDim.z - 1 - (int)blockIdx.z;
-    const int qtile = SPLIT ? zz / p.n_splits : zz;
-    const int split = SPLIT ? zz - qtile * p.n_splits : 0;
-    const int q0 = qtile * TROWS;
     // kv head: hx itself when rows are packed, else hx / group (group_magic = 2^32 / group + 1, exact below 2^16 heads)
     const int kvh = (PACKED || p.group_magic == 0) ? hx : (int)__umulhi((uint32_t)hx, p.group_magic);
     const int h0 = PACKED ? hx * G : hx;  // head of a row with g = 0
-    // which 32 query rows of the tile a wave owns.  Wave w runs on SIMD w % 4, and under a causal mask the rows at
-    // the end of a tile see more keys than those at its start: the assignment rotates from workgroup to workgroup
-    // so that no SIMD collects the long rows of every tile.
-    const int wq = (wave + hx + b + (int)blockIdx.z) & 3;
     const int D = p.dim;
 
     const uint16_t* __restrict__ Kg = p.k + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
     const uint16_t* __restrict__ Vg = p.v + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
-    (void)split;
 
     // ---- tile movement: chunk c = tid + TTHREADS n of a tile is (row c / CH, 16-byte chunk c % CH).  A tile
     // travels global -> registers -> LDS.  LDS holds two stages of each matrix; PF register sets per matrix hold
@@ -174,43 +167,56 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         for (int n = 0; n < NL; n++) kreg[i][n] = vreg[i][n] = u32x4_t{0u, 0u, 0u, 0u};  // (only read when there are no keys at all)
     }
     // per-thread constants of the movement (hoisted: the loop then spends a handful of instructions per tile on it)
-    int ld_row[NL];       // row of the tile this thread moves
-    uint32_t ld_col[NL];  // element offset inside a row; the same in K and V
+    uint32_t ld_off[NL];  // byte offset of the thread's chunk from the first byte of a tile; the same in K and V
     uint32_t st_k[NL], st_v[NL];  // byte offsets of the chunk in an LDS stage
     bool ld_on[NL];
+    const uint32_t kv_pitch = (uint32_t)p.lkv.row_pitch;
 #pragma unroll
     for (int n = 0; n < NL; n++) {
         const int c = tid + TTHREADS * n;
         const int row = c / CH, ch = c - row * CH;
-        ld_row[n] = row;
         st_k[n] = (uint32_t)((row * LDK + 8 * ch) * 2);
         st_v[n] = (uint32_t)((2 * KT * LDK + row * LDV + 8 * ch) * 2);
         ld_on[n] = 8 * ch < D;
-        ld_col[n] = ld_on[n] ? (uint32_t)(8 * ch) : 0u;  // a chunk past the head dim is requested (from column 0) but never parked
+        // a chunk past the head dim is requested (from column 0) but never parked
+        ld_off[n] = ((uint32_t)row * kv_pitch + (ld_on[n] ? (uint32_t)(8 * ch) : 0u)) * 2u;
     }
-    // Tile 0 (K and V) and K of tile 1 are requested before the sequence lengths are even read (those are a
-    // dependent load away): their rows are clamped to the tensor only, and the rows of V(0) past the last key are
-    // zeroed once the length is known (the matching rows of K are masked in the score tile whatever they hold).
-    // A workgroup that turns out to have no keys to walk leaves the requests unused.
-    const uint32_t kv_pitch = (uint32_t)p.lkv.row_pitch;
     u32x4_t k1[NL];
-#pragma unroll
-    for (int n = 0; n < NL; n++) k1[n] = u32x4_t{0u, 0u, 0u, 0u};
-    // (A span of the keys starts where the sequence's own length puts it: those requests wait for the lengths.)
-    if (!SPLIT && p.seq_kv > 0) {  // (no keys at all: there is no row to read, and no tile will be walked)
-        const int last_row = p.seq_kv - 1;
+    // Tile 0 (K and V) and K of tile 1 are requested before the sequence lengths have arrived (a dependent load
+    // away), through descriptors that end with the tensor's last row: the rows of V(0) past the last key are zeroed
+    // once the length is known, those of K are masked in the score tile whatever they hold.  (A span of the keys
+    // starts where the sequence's own length puts it: its requests wait for the lengths.)
+    const uint32_t tile_bytes_g = (uint32_t)KT * kv_pitch * 2u;  // from a tile's first row to the next tile's, in memory
+    if (!SPLIT) {
+        const uint32_t all_bytes = p.seq_kv > 0 ? ((uint32_t)(p.seq_kv - 1) * kv_pitch + (uint32_t)D) * 2u : 0u;
+        const __amdgpu_buffer_rsrc_t Kall = __builtin_amdgcn_make_buffer_rsrc((void*)Kg, 0, all_bytes, kBufferFlags);
+        const __amdgpu_buffer_rsrc_t Vall = __builtin_amdgcn_make_buffer_rsrc((void*)Vg, 0, all_bytes, kBufferFlags);
 #pragma unroll
         for (int n = 0; n < NL; n++) {
-            const size_t e0 = (size_t)(uint32_t)min(ld_row[n], last_row) * kv_pitch + ld_col[n];
-            kreg[0][n] = *(const u32x4_t*)(Kg + e0);
-            vreg[0][n] = *(const u32x4_t*)(Vg + e0);
-            if (PIPE) k1[n] = *(const u32x4_t*)(Kg + (size_t)(uint32_t)min(KT + ld_row[n], last_row) * kv_pitch + ld_col[n]);
+            kreg[0][n] = __builtin_amdgcn_raw_buffer_load_b128(Kall, ld_off[n], 0, 0);
+            vreg[0][n] = __builtin_amdgcn_raw_buffer_load_b128(Vall, ld_off[n], 0, 0);
+            k1[n] = PIPE ? __builtin_amdgcn_raw_buffer_load_b128(Kall, ld_off[n], tile_bytes_g, 0) : u32x4_t{0u, 0u, 0u, 0u};
         }
-        if (MODE == kMaskPadding) keep_raw[0] = p.keep[min(lane & (KT - 1), last_row)];
     }
 
-    const int n_q = p.q_lens ? min(max(p.q_lens[b], 0), p.seq_q) : p.seq_q;          // valid query positions
+    const int n_q = p.q_lens ? min(max(p.q_lens[b], 0), p.seq_q) : p.seq_q;  // valid query positions
     int n_keys = p.kv_lens ? min(max(p.kv_lens[b], 0), p.seq_kv) : p.seq_kv;  // keys that exist
+    int qtile = SPLIT ? zz / p.n_splits : zz;
+    const int split = SPLIT ? zz - qtile * p.n_splits : 0;
+    (void)split;
+    // A padded batch ranks each sequence's OWN query tiles, last (longest) first: rank 0 is the tile that holds the
+    // sequence's last valid row, and the tiles of padded rows only, which have nothing to walk, take the ranks behind
+    // the valid ones and so are dispatched last, into the gaps at the end, instead of holding the first slots.
+    if (!SPLIT && p.q_lens) {
+        const int n_qt = (n_q * G + TROWS - 1) / TROWS;  // tiles with valid rows
+        const int rank = (int)blockIdx.z;
+        qtile = rank < n_qt ? n_qt - 1 - rank : rank;
+    }
+    const int q0 = qtile * TROWS;
+    // which 32 query rows of the tile a wave owns.  Wave w runs on SIMD w % 4, and under a causal mask the rows at
+    // the end of a tile see more keys than those at its start: the assignment rotates from workgroup to workgroup
+    // so that no SIMD collects the long rows of every tile.
+    const int wq = (wave + hx + b + (int)blockIdx.z) & 3;
     int off = n_keys - n_q;  // causal: the last valid query sees every key
 
     // keys the workgroup walks
@@ -237,16 +243,43 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         off -= key0;
         Kg += (size_t)key0 * (size_t)p.lkv.row_pitch;
         Vg += (size_t)key0 * (size_t)p.lkv.row_pitch;
-        if (n_tiles > 0) {  // the requests the unsplit kernel makes before it knows the lengths
-            const int last_row = n_keys - 1;
-#pragma unroll
-            for (int n = 0; n < NL; n++) {
-                const size_t e0 = (size_t)(uint32_t)min(ld_row[n], last_row) * kv_pitch + ld_col[n];
-                kreg[0][n] = *(const u32x4_t*)(Kg + e0);
-                vreg[0][n] = *(const u32x4_t*)(Vg + e0);
-                if (PIPE) k1[n] = *(const u32x4_t*)(Kg + (size_t)(uint32_t)min(KT + ld_row[n], last_row) * kv_pitch + ld_col[n]);
-            }
+    }
+    // A tile of padded query rows only (a padded batch has many: every tile behind a sequence's last row) has nothing
+    // to load or walk: its rows get the fill value and the workgroup is done.
+    if (!SPLIT && !PACKED && q0 >= n_q) {
+        const uint32_t f2 = p.zero_padded_rows ? 0u : 0x7fc07fc0u;
+        const u32x4_t val = {f2, f2, f2, f2};
+        uint16_t* const ob = p.out + (size_t)b * p.lo.batch_stride + (size_t)h0 * p.lo.head_stride;
+        for (int c = tid; c < TROWS * CH; c += TTHREADS) {
+            const int row = c / CH, ch = c - row * CH;
+            if (q0 + row < rows_total && 8 * ch < D) *(u32x4_t*)(ob + (size_t)(q0 + row) * p.lo.row_pitch + 8 * ch) = val;
         }
+        return;
+    }
+    // K and V are read through buffer descriptors that end with the last key's row: a request for a row behind it
+    // returns zeros without touching memory.  Zero rows of V are what the walk needs there (their weights are zero,
+    // and zero times a copy of a non-finite row would be NaN); zero rows of K give score 0, masked like any score
+    // past the last key.  The lane's offset is a constant of the thread and the tile's offset a scalar, so a request
+    // costs no address arithmetic.  (Offsets are 32-bit: the launcher refuses slabs of 4 GiB and more.)
+    const uint32_t slab_bytes = n_keys > 0 ? ((uint32_t)(n_keys - 1) * kv_pitch + (uint32_t)D) * 2u : 0u;
+    const __amdgpu_buffer_rsrc_t Kbuf = __builtin_amdgcn_make_buffer_rsrc((void*)Kg, 0, slab_bytes, kBufferFlags);
+    const __amdgpu_buffer_rsrc_t Vbuf = __builtin_amdgcn_make_buffer_rsrc((void*)Vg, 0, slab_bytes, kBufferFlags);
+    if (SPLIT) {  // tile 0 (K and V) and K of tile 1 of the span
+#pragma unroll
+        for (int n = 0; n < NL; n++) {
+            kreg[0][n] = __builtin_amdgcn_raw_buffer_load_b128(Kbuf, ld_off[n], 0, 0);
+            vreg[0][n] = __builtin_amdgcn_raw_buffer_load_b128(Vbuf, ld_off[n], 0, 0);
+            k1[n] = PIPE ? __builtin_amdgcn_raw_buffer_load_b128(Kbuf, ld_off[n], tile_bytes_g, 0) : u32x4_t{0u, 0u, 0u, 0u};
+        }
+    } else if (n_keys < KT) {  // the early requests ended with the tensor, not with the sequence
+#pragma unroll
+        for (int n = 0; n < NL; n++)
+            if ((tid + TTHREADS * n) / CH >= n_keys) vreg[0][n] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+    if (MODE == kMaskPadding && n_keys > 0) {  // keep bytes past the last key count as kept: `lim` masks those keys
+        const int j = lane & (KT - 1);
+        const uint32_t kb = p.keep[min(j, n_keys - 1)];
+        keep_raw[0] = j < n_keys ? kb : 1u;
     }
 
     f32x16_t acc_o[DT];
@@ -270,18 +303,17 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             __syncthreads();
         }
         const int last_kv0 = (n_tiles - 1) * KT;
-        // rows past the end re-read the last key: masked in the score tile, and parked as zeros for V (see park_v)
-        auto chunk_at = [&](int n, int kv0) __attribute__((always_inline)) { return (size_t)(uint32_t)min(kv0 + ld_row[n], n_keys - 1) * kv_pitch + ld_col[n]; };
         auto issue_k = [&](u32x4_t (&dst)[NL], int kv0) __attribute__((always_inline)) {
-            kv0 = min(kv0, last_kv0);
+            const uint32_t tile_off = (uint32_t)min(kv0, last_kv0) * (kv_pitch * 2u);
 #pragma unroll
-            for (int n = 0; n < NL; n++) dst[n] = *(const u32x4_t*)(Kg + chunk_at(n, kv0));
+            for (int n = 0; n < NL; n++) dst[n] = __builtin_amdgcn_raw_buffer_load_b128(Kbuf, ld_off[n], tile_off, 0);
         };
         auto issue_v = [&](auto set_c, int kv0) __attribute__((always_inline)) {
             constexpr int SET = decltype(set_c)::value;
             kv0 = min(kv0, last_kv0);
+            const uint32_t tile_off = (uint32_t)kv0 * (kv_pitch * 2u);
 #pragma unroll
-            for (int n = 0; n < NL; n++) vreg[SET][n] = *(const u32x4_t*)(Vg + chunk_at(n, kv0));
+            for (int n = 0; n < NL; n++) vreg[SET][n] = __builtin_amdgcn_raw_buffer_load_b128(Vbuf, ld_off[n], tile_off, 0);
             // key-padding vector of the tile: one byte per lane, turned into bits with a ballot when the tile is parked
             if (MODE == kMaskPadding) {
                 const int j = kv0 + (lane & (KT - 1));
@@ -295,23 +327,13 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
                 if (D == DP || ld_on[n]) *(u32x4_t*)(lds + st * (KT * LDK * 2) + st_k[n]) = src[n];
         };
         uint64_t keep_cur = ~0ull, keep_next = ~0ull;  // keep bits of the tile whose items are in their softmax step, and of the next
-        // `kv0` is the first key of the tile in the set.  In the tile that holds the last key the rows behind it become
-        // zero: their weights are zero, and zero times a copy of a non-finite last row would be NaN.
-        auto park_v = [&](auto set_c, int st, int kv0) __attribute__((always_inline)) {
+        auto park_v = [&](auto set_c, int st) __attribute__((always_inline)) {
             constexpr int SET = decltype(set_c)::value;
-            if (kv0 + KT > n_keys) {
-#pragma unroll
-                for (int n = 0; n < NL; n++)
-                    if (kv0 + ld_row[n] >= n_keys) vreg[SET][n] = u32x4_t{0u, 0u, 0u, 0u};
-            }
 #pragma unroll
             for (int n = 0; n < NL; n++)
                 if (D == DP || ld_on[n]) *(u32x4_t*)(lds + st * (KT * LDV * 2) + st_v[n]) = vreg[SET][n];
             if (MODE == kMaskPadding) keep_next = __ballot(keep_raw[SET] != 0);
         };
-
-        // tile 0's early requests: keep bytes past the last key count as kept
-        if (MODE == kMaskPadding && n_keys < KT && (lane & (KT - 1)) >= n_keys) keep_raw[0] = 1u;
 
         // ---- this lane's query row
         const int r = q0 + 32 * wq + col;
@@ -380,7 +402,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         // K(0), V(0) -> stage 0, K(1) -> stage 1; then the register sets take K(2) .. K(1 + PF) and V(1) .. V(PF)
         // (K(j) travels in set j % PF, and so does V(j))
         park_k(kreg[0], 0);
-        park_v(std::integral_constant<int, 0>{}, 0, 0);
+        park_v(std::integral_constant<int, 0>{}, 0);
         keep_cur = keep_next;
         if (PIPE) park_k(k1, 1);
         {
@@ -668,7 +690,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             const int st = st_c;  // t & 1, as a constant where the caller knows it
             // (behind the last tiles these park and request copies of the last tile, which nobody reads)
             park_k(kreg[KSET], st);
-            park_v(vset_c, st ^ 1, (t + 1) * KT);
+            park_v(vset_c, st ^ 1);
             issue_k(kreg[KSET], (t + 2 + PF) * KT);
             issue_v(vset_c, (t + 1 + PF) * KT);
         };
@@ -725,7 +747,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
                     if (t * NI + it < n_it)
                         step_simple(it, t * KT + 32 * it, Ks + st * KT * LDK + 32 * it * LDK + k_off, Vs + st * KT * LDV + 32 * it * LDV + v_off);
                 park_k(kreg[0], st ^ 1);
-                park_v(std::integral_constant<int, 0>{}, st ^ 1, (t + 1) * KT);
+                park_v(std::integral_constant<int, 0>{}, st ^ 1);
                 issue_k(kreg[0], (t + 2) * KT);
                 issue_v(std::integral_constant<int, 0>{}, (t + 2) * KT);
                 __syncthreads();
@@ -963,12 +985,18 @@ hipError_t launch_dp(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
 
 bool flash_tile_bf16_supported(int dim) { return dim > 0 && dim <= 256 && dim % 8 == 0; }
 int flash_tile_bf16_key_tile(int dim) { return dim <= 128 ? 64 : 32; }
+// The kernel addresses the keys of one (batch, kv head) with 32-bit byte offsets (tile offset + lane offset, the
+// requests that run a few tiles past the last one included).
+bool flash_tile_bf16_addressable(long long seq_kv, long long row_pitch) {
+    return seq_kv >= 0 && row_pitch > 0 && (unsigned long long)(seq_kv + 512) * (unsigned long long)row_pitch * 2ull < (1ull << 32);
+}
 
 hipError_t launch_flash_tile_bf16(hipStream_t stream, const FlashTileParams& params) {
     FlashTileParams p = params;
     if (p.batch == 0 || p.heads == 0 || p.seq_q == 0) return hipSuccess;
     if (!flash_tile_bf16_supported(p.dim) || p.pack < 1) return hipErrorInvalidValue;
     if (p.bias && p.mask != kMaskNone) return hipErrorInvalidValue;
+    if (!flash_tile_bf16_addressable(p.seq_kv, p.lkv.row_pitch)) return hipErrorInvalidValue;
     if (p.pack > 1 && (p.bias || p.mask != kMaskCausal)) return hipErrorInvalidValue;  // packed rows: the chunked decode only
     const long long rows = (long long)p.seq_q * p.pack;
     const long long n_qtiles = (rows + TROWS - 1) / TROWS;

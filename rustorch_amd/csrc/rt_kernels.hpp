@@ -131,6 +131,7 @@ bool flash_tile_bf16_supported(int dim);
 // keys per LDS tile of the tile kernel at head dim `dim` (the unit the split over the keys is cut in)
 int flash_tile_bf16_key_tile(int dim);
 hipError_t launch_flash_tile_bf16(hipStream_t stream, const FlashTileParams& p);
+bool flash_tile_bf16_addressable(long long seq_kv, long long row_pitch);  // K/V slabs below 4 GiB (32-bit offsets)
 
 // Unmasked attention of every query row over all keys; generic in dim (<= 512), head
 // grouping, kv_len and query count.  T is float or uint16_t (bf16 bits).
