@@ -7,15 +7,16 @@ times the batched GQA decode workload (batch 64, 32 query / 8 kv heads, D=128, c
 uniform in [512, 8192], Lmax 8192) and reports it under "decode", and the f32 causal prefill of
 B=1, H=8, N=2048, D=64 (the reference's own CPU-runnable case) under "f32_prefill", and the f32
 backward on that shape under "f32_backward", the padded-batch prefill (B=16, H=16, D=64, lengths in [128, 1024])
-under "padded_prefill" and the long-context prefill (B=1, H=32, N=16384, D=128, Q scaled by 2) under
-"long_prefill".
+under "padded_prefill", the long-context prefill (B=1, H=32, N=16384, D=128, Q scaled by 2) under
+"long_prefill" and a long prefill at the other head dim of the matrix-core kernels (B=4, H=32, N=4096, D=64) under
+"d64_prefill".
 
 Every leg first runs a settle phase: launches of the leg's own step until SETTLE_MS of device time have passed
 (after an idle period the clocks first drop and then recover over some tens of milliseconds); the phase is
 reported as settle_ms / settle_launches and is followed by the counted warm-up (--warmup) and the timed region
 (--steps), which is the only part that enters value, ms_per_step and roofline.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only prefill|decode|f32|bwd|padded|long]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only prefill|decode|f32|bwd|padded|long|d64]
 
 Prints ONE JSON line.  `value` is prefill TFLOP/s with causal-counted FLOPs
 (4*B*H*D*N*(N+1)/2: skipped tiles are not credited); `roofline` prices it against the dense bf16
@@ -207,7 +208,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity sample")
-    ap.add_argument("--only", choices=["prefill", "decode", "f32", "bwd", "padded", "long"], default=None)
+    ap.add_argument("--only", choices=["prefill", "decode", "f32", "bwd", "padded", "long", "d64"], default=None)
     ap.add_argument("--no-ceiling", action="store_true",
                     help="skip the run of rustorch_amd/lib/mfma_sustained (what a loop of nothing but bf16 MFMA "
                          "sustains on this GPU, reported beside the data-sheet peak)")
@@ -308,6 +309,17 @@ def main():
                   "config": {"workload": "bf16 long-context causal prefill, B=1 H=32 N=16384 D=128, N(0,1) inputs with Q "
                                          "scaled by 2.0 before rounding (seed 55), f32 accumulation",
                              "flop_convention": "4*B*H*D*N*(N+1)/2 (causal-counted)"}}
+
+    # ------------------------------------------------------------------ long prefill at head dim 64
+    d64_p = None
+    if args.only in (None, "d64"):
+        Bd, Hd, Nd, Dd = 4, 32, 4096, 64
+        d64_p = causal_prefill(Bd, Hd, Nd, Dd, 64, 1.0, 32, "flash_fwd_bf16_kernel<64, causal>",
+                               profile_traffic("flash_fwd_bf16_b4_h32_n4096_d64.md", "flash_fwd_bf16_kernel<64,causal>"))
+        d64_p = {"metric": "prefill attn TFLOP/s", "value": d64_p.pop("tflops"), "unit": "TFLOP/s", **d64_p,
+                 "config": {"workload": "bf16 causal prefill at head dim 64, B=4 H=32 N=4096 D=64, N(0,1) inputs "
+                                        "(seed 64), f32 accumulation",
+                            "flop_convention": "4*B*H*D*N*(N+1)/2 (causal-counted)"}}
 
     # ------------------------------------------------------------------ padded-batch prefill (per-sequence lengths + causal)
     padded = None
@@ -596,8 +608,8 @@ def main():
     tail = dict(n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True, data="synthetic",
                 vs_baseline=None, scaling="weak")
     if prefill is None:  # --only <one of the other legs>: that leg is the line
-        leg, dtype = next((x, t) for x, t in ((decode, "bf16"), (long_p, "bf16"), (padded, "bf16"), (f32, "f32"),
-                                              (bwd, "f32")) if x is not None)
+        leg, dtype = next((x, t) for x, t in ((decode, "bf16"), (long_p, "bf16"), (padded, "bf16"), (d64_p, "bf16"),
+                                              (f32, "f32"), (bwd, "f32")) if x is not None)
         print(json.dumps(dict(leg, dtype=dtype, **tail)))
         return
     sustained = None if args.no_ceiling else sustained_mfma()
@@ -622,8 +634,8 @@ def main():
         out["cpu_baseline"] = prefill["cpu_baseline"]
         out["parity_max_abs"] = prefill["parity_max_abs"]
         out["parity_rel_fro"] = prefill["parity_rel_fro"]
-    for key, leg in (("decode", decode), ("padded_prefill", padded), ("long_prefill", long_p), ("f32_prefill", f32),
-                     ("f32_backward", bwd)):
+    for key, leg in (("decode", decode), ("padded_prefill", padded), ("long_prefill", long_p), ("d64_prefill", d64_p),
+                     ("f32_prefill", f32), ("f32_backward", bwd)):
         if leg is not None:
             out[key] = leg
     print(json.dumps(out))
