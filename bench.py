@@ -314,8 +314,8 @@ def main():
     d64_p = None
     if args.only in (None, "d64"):
         Bd, Hd, Nd, Dd = 4, 32, 4096, 64
-        d64_p = causal_prefill(Bd, Hd, Nd, Dd, 64, 1.0, 32, "flash_fwd_bf16_kernel<64, causal>",
-                               profile_traffic("flash_fwd_bf16_b4_h32_n4096_d64.md", "flash_fwd_bf16_kernel<64,causal>"))
+        d64_p = causal_prefill(Bd, Hd, Nd, Dd, 64, 1.0, 32, "flash_wide_bf16_kernel<causal>",
+                               profile_traffic("flash_wide_bf16_b4_h32_n4096_d64.md", "flash_wide_bf16_kernel<causal>"))
         d64_p = {"metric": "prefill attn TFLOP/s", "value": d64_p.pop("tflops"), "unit": "TFLOP/s", **d64_p,
                  "config": {"workload": "bf16 causal prefill at head dim 64, B=4 H=32 N=4096 D=64, N(0,1) inputs "
                                         "(seed 64), f32 accumulation",

@@ -191,10 +191,12 @@ int rt_flash_forward_f32_dev(void *stream, const rt_attention_shape *shape, uint
 
 /* The bf16 counterpart (bf16 in, f32 accumulate, bf16 out rounded once, to nearest even):
  * q/out [batch,heads,seq,dim], k/v [batch,n_kv_heads,seq,dim].  Any dim up to 512 (the reference's forward takes
- * any dim != 0, cpu_forward.rs:142-169; above 512: RT_ERR_UNSUPPORTED with expected = 512).  Two MFMA kernels serve
+ * any dim != 0, cpu_forward.rs:142-169; above 512: RT_ERR_UNSUPPORTED with expected = 512).  Three MFMA kernels serve
  * dims up to 256 that are a multiple of 8 on 16-byte aligned tensors: a persistent 8-wave kernel for dim 64 / 128 on
- * unpadded batches of at least 512 rows per sequence and one job of 256 rows per compute unit, and a 4-wave tile
- * kernel for everything else (short or few sequences, padded batches, other dims);
+ * unpadded batches of at least 512 rows per sequence and one job of 256 rows per compute unit, a 4-wave tile
+ * kernel for everything else (short or few sequences, padded batches, other dims), and a form of the tile kernel
+ * with 64 query rows per wave for dim 64 on unpadded sequences of at least 2048 rows with four 256-row jobs per
+ * compute unit;
  * rt_debug_force_bf16_prefill_kernel forces one of them where both apply.  The remaining dims and alignments run on
  * a one-workgroup-per-row kernel with the same masks and row rules (correct at any speed, not tuned). */
 int rt_flash_forward_bf16_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const void *q,
@@ -202,9 +204,10 @@ int rt_flash_forward_bf16_dev(void *stream, const rt_attention_shape *shape, uin
                               rt_err_detail *err);
 
 /* No counterpart in the reference: a switch for measurements and tests.  which = 0 lets the library choose between
- * its two bf16 prefill kernels (the default), 1 forces the tile kernel, 2 the persistent kernel where it applies
- * (head dim 64 / 128, no per-sequence lengths).  Process-wide; until it is called the value is taken, once, from
- * RT_ATTN_BF16_PREFILL=tile|persistent in the environment.  Returns RT_ERR_UNSUPPORTED for another value. */
+ * its bf16 prefill kernels (the default), 1 forces the tile kernel, 2 the persistent kernel where it applies (head
+ * dim 64 / 128, no per-sequence lengths), 3 the kernel with 64 query rows per wave where it applies (head dim 64,
+ * mask none or causal; elsewhere the tile kernel).  Process-wide; until it is called the value is taken, once, from
+ * RT_ATTN_BF16_PREFILL=tile|persistent|wide in the environment.  Returns RT_ERR_UNSUPPORTED for another value. */
 int rt_debug_force_bf16_prefill_kernel(int which);
 
 /* No counterpart in the reference, whose CPU loop needs none: on != 0 makes every causal prefill entry (f32 and bf16,

@@ -782,7 +782,7 @@ RT_API int rt_flash_forward_f32_dev(void* stream, const rt_attention_shape* shap
 // where both apply (for measurements and tests); otherwise the persistent 8-wave kernel takes head dims 64 and 128
 // on unpadded batches with at least 512 rows per sequence and a job for every CU, and the 4-wave tile kernel
 // everything else.
-enum class PrefillKernel { kAuto, kTile, kPersistent };
+enum class PrefillKernel { kAuto, kTile, kPersistent, kWide };
 // A debug switch for measurements and tests, not part of the reference's surface: rt_debug_force_bf16_prefill_kernel
 // sets it; until that is called, the value is what RT_ATTN_BF16_PREFILL=tile|persistent held when the library made its
 // first bf16 prefill call (read once: a later change of the environment does not change which kernel a caller gets).
@@ -790,6 +790,7 @@ static PrefillKernel parse_prefill_kernel(const char* e) {
     if (!e) return PrefillKernel::kAuto;
     if (strcmp(e, "tile") == 0) return PrefillKernel::kTile;
     if (strcmp(e, "persistent") == 0) return PrefillKernel::kPersistent;
+    if (strcmp(e, "wide") == 0) return PrefillKernel::kWide;
     return PrefillKernel::kAuto;
 }
 static std::atomic<int> g_prefill_forced{-1};  // -1: not set through the API
@@ -800,7 +801,7 @@ static PrefillKernel prefill_kernel_override() {
     return once;
 }
 RT_API int rt_debug_force_bf16_prefill_kernel(int which) {
-    if (which < 0 || which > 2) return RT_ERR_UNSUPPORTED;
+    if (which < 0 || which > 3) return RT_ERR_UNSUPPORTED;
     g_prefill_forced.store(which, std::memory_order_relaxed);
     return RT_OK;
 }
@@ -870,7 +871,12 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
     const uint64_t jobs256 = (shape->seq + 255) / 256 * shape->batch * shape->heads;
     bool persistent = persistent_dim && shape->seq >= 512 && jobs256 >= (uint64_t)g_num_cus && mask != rt::kMaskVarlenCausal;
     const PrefillKernel forced = prefill_kernel_override();
-    if (forced == PrefillKernel::kTile) persistent = false;
+    if (forced == PrefillKernel::kTile || forced == PrefillKernel::kWide) persistent = false;
+    // head dim 64 on long, unpadded sequences with work for every CU several times over: 64 query rows per wave
+    // (256-row workgroups, two per CU), measured 5-6 % ahead of both other kernels there and behind them on less work
+    const bool wide_auto = forced == PrefillKernel::kAuto && shape->dim == 64 && (mask == rt::kMaskNone || mask == rt::kMaskCausal) &&
+                           shape->seq >= 2048 && jobs256 >= 4ull * (uint64_t)g_num_cus;
+    if (wide_auto) persistent = false;
     if (forced == PrefillKernel::kPersistent && persistent_dim) persistent = true;
     if (mask == rt::kMaskPadding && shape->seq > (uint64_t)rt::kFlashBf16MaxPaddingKeys) persistent = false;
     if (persistent) {  // that kernel addresses the rows of one (batch, head) slab with 32-bit byte offsets
@@ -912,6 +918,10 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
         t.scale_log2e = scale * rt::kLog2eHost;
         t.lq = t.lo = lq;
         t.lkv = lkv;
+        if ((forced == PrefillKernel::kWide || wide_auto) && rt::flash_wide_bf16_supported(t)) {
+            HIP_TRY(rt::launch_flash_wide_bf16((hipStream_t)stream, t), "flash_wide_bf16 launch");
+            return strict_pass((hipStream_t)stream, shape, n_kv_heads, v, out, seq_lens, mask, bnhd, true, err);
+        }
         HIP_TRY(rt::launch_flash_tile_bf16((hipStream_t)stream, t), "flash_tile_bf16 launch");
         return strict_pass((hipStream_t)stream, shape, n_kv_heads, v, out, seq_lens, mask, bnhd, true, err);
     }

@@ -956,6 +956,469 @@ __global__ __launch_bounds__(256) void flash_split_merge_kernel(FlashTileParams 
         f32_to_bf16_bits(x);
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The same walk with 64 query rows per wave (two blocks of 32), head dim 64, masks none / causal, rows of one head.
+// At head dim 64 a 32-key item is only 8 matrix instructions per 32 rows: what paces the tile kernel there is the
+// movement of a key tile (LDS parking, the workgroup barrier per tile) and the operand reads, which are the same
+// whether a wave multiplies a fragment into one row block or two.  Here every K and V fragment read from LDS feeds
+// two matrix instructions, a tile in LDS serves 256 query rows between two barriers, and a workgroup's set-up is
+// spread over twice the rows.  Two workgroups share a CU (two O blocks, two score tiles and their operands).
+constexpr int WROWS = 256;  // query rows per workgroup: four waves of 64
+
+template <int MODE>
+__global__ __launch_bounds__(256, 2) void flash_wide_bf16_kernel(FlashTileParams p) {
+    constexpr int DP = 64, KT = 64, LDK = DP + 8, LDV = DP + 32, NI = KT / 32, KS = DP / 16, DT = DP / 32, CH = DP / 8;
+    constexpr int TTHREADS = 256, NL = KT * CH / TTHREADS, RB = 2;
+    constexpr bool kCausal = MODE == kMaskCausal;
+    constexpr int TILE_BYTES = 2 * KT * (LDK + LDV) * 2;  // two stages of K and V
+    constexpr int REGION = 64 * LDK * 2;                  // a wave's staged output rows
+    static_assert(4 * REGION <= TILE_BYTES, "the staged output rows fit over the tiles");
+    static_assert(NI == 2 && KS == 2 * DT, "two items per tile, one P.V instruction per score instruction");
+
+    __shared__ __attribute__((aligned(16))) unsigned char lds[TILE_BYTES];
+    uint16_t* const Ks = (uint16_t*)lds;                 // [2][KT * LDK]
+    uint16_t* const Vs = (uint16_t*)lds + 2 * KT * LDK;  // [2][KT * LDV]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 31, hh = lane >> 5;
+    const int rows_total = p.seq_q;
+    const int hx = blockIdx.x, b = blockIdx.y;
+    const int kvh = p.group_magic == 0 ? hx : (int)__umulhi((uint32_t)hx, p.group_magic);
+    const uint16_t* const Kg = p.k + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+    const uint16_t* const Vg = p.v + (size_t)b * p.lkv.batch_stride + (size_t)kvh * p.lkv.head_stride;
+
+    // ---- tile movement, as in the tile kernel: chunk c = tid + 256 n of a tile is (row c / CH, 16-byte chunk c % CH)
+    u32x4_t kreg[NL], vreg[NL], k1[NL];
+    uint32_t ld_off[NL], st_k[NL], st_v[NL];
+    const uint32_t kv_pitch = (uint32_t)p.lkv.row_pitch;
+#pragma unroll
+    for (int n = 0; n < NL; n++) {
+        const int c = tid + TTHREADS * n;
+        const int row = c / CH, ch = c - row * CH;
+        st_k[n] = (uint32_t)((row * LDK + 8 * ch) * 2);
+        st_v[n] = (uint32_t)((2 * KT * LDK + row * LDV + 8 * ch) * 2);
+        ld_off[n] = ((uint32_t)row * kv_pitch + (uint32_t)(8 * ch)) * 2u;
+    }
+    const uint32_t tile_bytes_g = (uint32_t)KT * kv_pitch * 2u;
+    {  // tile 0 (K and V) and K of tile 1, before the lengths have arrived: descriptors that end with the tensor
+        const uint32_t all_bytes = p.seq_kv > 0 ? ((uint32_t)(p.seq_kv - 1) * kv_pitch + (uint32_t)DP) * 2u : 0u;
+        const __amdgpu_buffer_rsrc_t Kall = __builtin_amdgcn_make_buffer_rsrc((void*)Kg, 0, all_bytes, kBufferFlags);
+        const __amdgpu_buffer_rsrc_t Vall = __builtin_amdgcn_make_buffer_rsrc((void*)Vg, 0, all_bytes, kBufferFlags);
+#pragma unroll
+        for (int n = 0; n < NL; n++) {
+            kreg[n] = __builtin_amdgcn_raw_buffer_load_b128(Kall, ld_off[n], 0, 0);
+            vreg[n] = __builtin_amdgcn_raw_buffer_load_b128(Vall, ld_off[n], 0, 0);
+            k1[n] = __builtin_amdgcn_raw_buffer_load_b128(Kall, ld_off[n], tile_bytes_g, 0);
+        }
+    }
+
+    const int n_q = p.q_lens ? min(max(p.q_lens[b], 0), p.seq_q) : p.seq_q;          // valid query positions
+    const int n_keys = p.kv_lens ? min(max(p.kv_lens[b], 0), p.seq_kv) : p.seq_kv;  // keys that exist
+    // rank of the query tile: the last one first; in a padded batch counted from the sequence's own last valid tile
+    int qtile = (int)gridDim.z - 1 - (int)blockIdx.z;
+    if (p.q_lens) {
+        const int n_qt = (n_q + WROWS - 1) / WROWS;
+        const int rank = (int)blockIdx.z;
+        qtile = rank < n_qt ? n_qt - 1 - rank : rank;
+    }
+    const int q0 = qtile * WROWS;
+    const int wq = (wave + hx + b + (int)blockIdx.z) & 3;  // which 64 rows of the tile: rotated, as in the tile kernel
+    const int r0 = q0 + 64 * wq;                           // the wave's first row
+    const int off = n_keys - n_q;                          // causal: the last valid query sees every key
+
+    int kv_end = n_keys;
+    if (kCausal) kv_end = min(n_keys, min(q0 + WROWS - 1, n_q - 1) + off + 1);
+    if (q0 >= n_q) kv_end = 0;
+    kv_end = max(kv_end, 0);
+    const int n_tiles = (kv_end + KT - 1) / KT;
+
+    const uint32_t fill2 = p.zero_padded_rows ? 0u : 0x7fc07fc0u;
+    if (q0 >= n_q) {  // padded rows only: the fill value, and done
+        const u32x4_t val = {fill2, fill2, fill2, fill2};
+        uint16_t* const ob = p.out + (size_t)b * p.lo.batch_stride + (size_t)hx * p.lo.head_stride;
+        for (int c = tid; c < WROWS * CH; c += TTHREADS) {
+            const int row = c / CH, ch = c - row * CH;
+            if (q0 + row < rows_total) *(u32x4_t*)(ob + (size_t)(q0 + row) * p.lo.row_pitch + 8 * ch) = val;
+        }
+        return;
+    }
+    // descriptors that end with the last key's row: rows behind it come back as zeros
+    const uint32_t slab_bytes = n_keys > 0 ? ((uint32_t)(n_keys - 1) * kv_pitch + (uint32_t)DP) * 2u : 0u;
+    const __amdgpu_buffer_rsrc_t Kbuf = __builtin_amdgcn_make_buffer_rsrc((void*)Kg, 0, slab_bytes, kBufferFlags);
+    const __amdgpu_buffer_rsrc_t Vbuf = __builtin_amdgcn_make_buffer_rsrc((void*)Vg, 0, slab_bytes, kBufferFlags);
+    if (n_keys < KT) {  // the early requests ended with the tensor, not with the sequence
+#pragma unroll
+        for (int n = 0; n < NL; n++)
+            if ((tid + TTHREADS * n) / CH >= n_keys) vreg[n] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+
+    f32x16_t acc_o[RB][DT];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+        for (int t = 0; t < DT; t++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc_o[rb][t][i] = 0.0f;
+    float m_run[RB], l_run[RB];
+    bool valid[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+        m_run[rb] = neg_inf();
+        l_run[rb] = 0.0f;
+        valid[rb] = false;
+    }
+    const float cc = p.scale_log2e;  // exp2 argument per unit of score
+
+    if (n_tiles > 0) {
+        const int last_kv0 = (n_tiles - 1) * KT;
+        auto issue_k = [&](int kv0) __attribute__((always_inline)) {
+            const uint32_t tile_off = (uint32_t)min(kv0, last_kv0) * (kv_pitch * 2u);
+#pragma unroll
+            for (int n = 0; n < NL; n++) kreg[n] = __builtin_amdgcn_raw_buffer_load_b128(Kbuf, ld_off[n], tile_off, 0);
+        };
+        auto issue_v = [&](int kv0) __attribute__((always_inline)) {
+            const uint32_t tile_off = (uint32_t)min(kv0, last_kv0) * (kv_pitch * 2u);
+#pragma unroll
+            for (int n = 0; n < NL; n++) vreg[n] = __builtin_amdgcn_raw_buffer_load_b128(Vbuf, ld_off[n], tile_off, 0);
+        };
+        auto park_k = [&](const u32x4_t (&src)[NL], int st) __attribute__((always_inline)) {
+#pragma unroll
+            for (int n = 0; n < NL; n++) *(u32x4_t*)(lds + st * (KT * LDK * 2) + st_k[n]) = src[n];
+        };
+        auto park_v = [&](int st) __attribute__((always_inline)) {
+#pragma unroll
+            for (int n = 0; n < NL; n++) *(u32x4_t*)(lds + st * (KT * LDV * 2) + st_v[n]) = vreg[n];
+        };
+
+        // ---- this lane's two query rows, and the wave's limits as scalars
+        int lim[RB], wave_lim_min[RB];
+        const int r_lim = min(rows_total, n_q);  // rows below it are valid
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+            const int r = r0 + 32 * rb + col;
+            valid[rb] = r < r_lim;
+            int l = n_keys - 1;  // last key this row sees
+            if (kCausal) l = min(l, r + off);
+            lim[rb] = valid[rb] ? l : -1;
+            const int r_first = r0 + 32 * rb, r_last = r_first + 31;
+            wave_lim_min[rb] = r_last < r_lim ? (kCausal ? min(n_keys - 1, r_first + off) : n_keys - 1) : -1;
+        }
+        const int r_top = min(r0 + 63, r_lim - 1);
+        const int wave_lim_max = r0 < r_lim ? (kCausal ? min(n_keys - 1, r_top + off) : n_keys - 1) : -1;
+        // items this wave walks: the ones that hold a key some row of it sees (a prefix of the workgroup's items)
+        const int n_it = wave_lim_max < 0 ? 0 : min(n_tiles * NI, (wave_lim_max >> 5) + 1);
+
+        // ---- Q as B operands: column q = lane % 32 of either row block, contraction slots 16 ks + 8 hh .. + 8
+        bf16x8_t qreg[RB][KS];
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+            const int r_q = min(r0 + 32 * rb + col, rows_total - 1);  // (a row past the tensor reads the last row: it is masked and not written)
+            const size_t q_off = (size_t)b * p.lq.batch_stride + (size_t)hx * p.lq.head_stride + (size_t)r_q * p.lq.row_pitch;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++)
+                qreg[rb][ks] = __builtin_bit_cast(bf16x8_t, *(const u32x4_t*)(p.q + q_off + 16 * ks + 8 * hh));
+        }
+        const int k_off = col * LDK + 8 * hh;
+        const int v_off = (((lane & 15) >> 2) + 4 * hh) * LDV + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+        // K(0), V(0) -> stage 0, K(1) -> stage 1; the register sets then take K(2) and V(1)
+        park_k(kreg, 0);
+        park_v(0);
+        park_k(k1, 1);
+        issue_k(2 * KT);
+        issue_v(KT);
+        __syncthreads();
+
+        auto mask_item = [&](int rb, int k0, f32x16_t& sc) __attribute__((always_inline)) {
+            if (k0 + 31 > wave_lim_min[rb]) {
+                const int room = lim[rb] - k0 - 4 * hh;  // key k0 + 8 (i / 4) + 4 hh + i % 4 is hidden when it lies past lim
+#pragma unroll
+                for (int i = 0; i < 16; i++) sc[i] = (8 * (i >> 2) + (i & 3) > room) ? neg_inf() : sc[i];
+            }
+        };
+        auto load_v = [&](int i, const uint16_t* vp) __attribute__((always_inline)) {
+            const int u = i / DT, dt = i - u * DT;
+            const u32x2_t lo = t_lds_read_tr16(vp + 16 * u * LDV + 32 * dt);
+            const u32x2_t hi = t_lds_read_tr16(vp + 16 * u * LDV + 32 * dt + 8 * LDV);
+            return u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+        };
+        auto pin_f = [](float& x) __attribute__((always_inline)) { asm volatile("" : "+v"(x)); };
+        auto pin_u = [](uint32_t& x) __attribute__((always_inline)) { asm volatile("" : "+v"(x)); };
+        auto pin_b = [](bf16x8_t& x) __attribute__((always_inline)) { asm volatile("" : "+v"(x)); };
+
+        float neg_mc[RB];  // -m_run * cc; +inf while a valid row has no max yet
+        f32x16_t s_a[RB];                 // S(j), made at the end of step j - 1
+        bf16x8_t p_a[RB][2], p_b[RB][2];  // P(j - 1) and P(j)
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+            neg_mc[rb] = valid[rb] ? __uint_as_float(0x7f800000u) : 0.0f;
+            p_a[rb][0] = p_a[rb][1] = p_b[rb][0] = p_b[rb][1] = __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u});
+#pragma unroll
+            for (int i = 0; i < 16; i++) s_a[rb][i] = 0.0f;
+        }
+        // S(0), and the running max started from it, so that the first step already runs the fast path
+        if (n_it > 0) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                const bf16x8_t kf = *(const bf16x8_t*)(Ks + k_off + 16 * ks);
+#pragma unroll
+                for (int rb = 0; rb < RB; rb++) s_a[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qreg[rb][ks], s_a[rb], 0, 0, 0);
+            }
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++) {
+                mask_item(rb, 0, s_a[rb]);  // (the step applies the mask again, which changes nothing)
+                const float m0 = t_max_with_other_half(t_max16(s_a[rb]));
+                if (m0 > neg_inf()) {  // (false for -inf and for NaN: such a row waits for the slow path)
+                    m_run[rb] = m0;
+                    neg_mc[rb] = -m0 * cc;
+                }
+            }
+        }
+
+        // O^T += V(j-1)^T . P(j-1)^T alone: behind the wave's last item
+        auto drain = [&](const uint16_t* vp) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < KS; i++) {
+                const int u = i / DT, dt = i - u * DT;
+                const bf16x8_t av = __builtin_bit_cast(bf16x8_t, load_v(i, vp));
+#pragma unroll
+                for (int rb = 0; rb < RB; rb++)
+                    acc_o[rb][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, p_a[rb][u], acc_o[rb][dt], 0, 0, 0);
+            }
+        };
+        auto exp_plain = [&](const f32x16_t& sc, float nmc, uint32_t (&w)[8], float& part) __attribute__((always_inline)) {
+            float part0 = 0.0f, part1 = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[2 * e], cc, nmc));
+                const float x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[2 * e + 1], cc, nmc));
+                part0 += x0;
+                part1 += x1;
+                w[e] = t_cvt_pk_bf16(x0, x1);
+            }
+            part = part0 + part1;
+        };
+        // the slow path of a softmax step: the item max, O and l rescaled to it, P again from the scores
+        auto raise_max_and_redo = [&](int rb, const f32x16_t& sc, uint32_t (&w)[8], float& part) __attribute__((always_inline)) {
+            const float m_item = t_max_with_other_half(t_max16(sc));
+            const float m_new = t_vmax(m_run[rb], m_item);
+            const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f((m_run[rb] - m_use) * cc);  // m_run = -inf -> 0
+            m_run[rb] = m_new;
+            l_run[rb] *= alpha;
+#pragma unroll
+            for (int tt = 0; tt < DT; tt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc_o[rb][tt][i] *= alpha;
+            const float mc = m_use * cc;
+            neg_mc[rb] = (m_new == neg_inf()) ? (valid[rb] ? __uint_as_float(0x7f800000u) : 0.0f) : -mc;
+            exp_plain(sc, -mc, w, part);
+        };
+
+        // One step: item j (keys k0 ..) gets its softmax step in both row blocks; K rows of item j + 1 are at kp, V rows
+        // of item j - 1 at vp.  The registers hold one score tile per row block (two workgroups per CU), so the row
+        // blocks are staggered: while block 0's P(j) is made its P.V instructions of item j - 1 run; while block 1's
+        // P(j) is made, block 1's P.V instructions and block 0's S(j+1) run (into the registers block 0's S(j) has
+        // just left); block 1's S(j+1) follows, and is still in flight when the next step starts on block 0.  Every V
+        // and K fragment is read from LDS once and feeds both row blocks.  No row max in the steady state (see the
+        // tile kernel).
+        auto step = [&](int k0, const uint16_t* kp, const uint16_t* vp, bf16x8_t (&p_prev)[RB][2],
+                        bf16x8_t (&p_new)[RB][2]) __attribute__((always_inline)) {
+            mask_item(0, k0, s_a[0]);
+            u32x4_t vop[KS], kop[KS];
+            constexpr int PER = 16 / KS;  // scores of a row block per group
+            const f32x16_t zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+            // the vector work of group g of row block rb: a quarter of P(j), fenced
+            auto quarter = [&](int rb, int g, float (&part)[2], uint32_t (&w)[8]) __attribute__((always_inline)) {
+                float t[PER];
+#pragma unroll
+                for (int i = 0; i < PER; i++) t[i] = __builtin_fmaf(s_a[rb][PER * g + i], cc, neg_mc[rb]);
+#pragma unroll
+                for (int i = 0; i < PER; i++) t[i] = __builtin_amdgcn_exp2f(t[i]);
+#pragma unroll
+                for (int i = 0; i < PER; i += 2) {
+                    part[0] += t[i];
+                    part[1] += t[i + 1];
+                    w[(PER * g + i) / 2] = t_cvt_pk_bf16(t[i], t[i + 1]);
+                }
+#pragma unroll
+                for (int i = 0; i < PER; i++) pin_f(t[i]);
+                pin_f(part[0]);
+                pin_f(part[1]);
+#pragma unroll
+                for (int i = 0; i < PER; i += 2) pin_u(w[(PER * g + i) / 2]);
+            };
+            auto finish = [&](int rb, float (&part)[2], uint32_t (&w)[8]) __attribute__((always_inline)) {
+                float pt = part[0] + part[1];
+                if (__builtin_expect(__any(!(pt <= kTileTrigSum)), 0)) raise_max_and_redo(rb, s_a[rb], w, pt);
+                l_run[rb] += pt;
+                p_new[rb][0] = __builtin_bit_cast(bf16x8_t, u32x4_t{w[0], w[1], w[2], w[3]});
+                p_new[rb][1] = __builtin_bit_cast(bf16x8_t, u32x4_t{w[4], w[5], w[6], w[7]});
+            };
+            // ---- row block 0: P(j), with its P.V of item j - 1
+            {
+                float part[2] = {0.0f, 0.0f};
+                uint32_t w[8];
+                vop[0] = load_v(0, vp);
+#pragma unroll
+                for (int g = 0; g < KS; g++) {
+                    if (g + 1 < KS) vop[g + 1] = load_v(g + 1, vp);
+                    const int u = g / DT, dt = g - u * DT;
+                    acc_o[0][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vop[g]), p_prev[0][u], acc_o[0][dt], 0, 0, 0);
+                    quarter(0, g, part, w);
+                    pin_b(p_prev[0][u]);
+                }
+                finish(0, part, w);
+            }
+            // ---- row block 1: P(j), with its P.V of item j - 1 and row block 0's S(j+1)
+            {
+                mask_item(1, k0, s_a[1]);
+                float part[2] = {0.0f, 0.0f};
+                uint32_t w[8];
+                kop[0] = *(const u32x4_t*)(kp);
+#pragma unroll
+                for (int g = 0; g < KS; g++) {
+                    if (g + 1 < KS) kop[g + 1] = *(const u32x4_t*)(kp + 16 * (g + 1));
+                    const int u = g / DT, dt = g - u * DT;
+                    acc_o[1][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vop[g]), p_prev[1][u], acc_o[1][dt], 0, 0, 0);
+                    s_a[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kop[g]), qreg[0][g], g == 0 ? zero16 : s_a[0], 0, 0, 0);
+                    quarter(1, g, part, w);
+                    pin_b(p_prev[1][u]);
+                    pin_b(qreg[0][g]);
+                }
+                finish(1, part, w);
+            }
+            // ---- row block 1's S(j+1)
+#pragma unroll
+            for (int g = 0; g < KS; g++)
+                s_a[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kop[g]), qreg[1][g], g == 0 ? zero16 : s_a[1], 0, 0, 0);
+        };
+        // a step whose results are moved back into the first of each pair
+        auto step_a = [&](int k0, const uint16_t* kp, const uint16_t* vp) __attribute__((always_inline)) {
+            step(k0, kp, vp, p_a, p_b);
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++) {
+                p_a[rb][0] = p_b[rb][0];
+                p_a[rb][1] = p_b[rb][1];
+            }
+        };
+        // slot j of the walk: a step while the wave has items left, then once the P.V of its last item
+        auto slot = [&](int j, const uint16_t* kp, const uint16_t* vp) __attribute__((always_inline)) {
+            if (j < n_it) step_a(32 * j, kp, vp);
+            else if (j == n_it && n_it > 0) drain(vp);
+        };
+        // behind the barrier of tile t: K(t+2) and V(t+1) parked over K(t) and V(t-1), K(t+3) and V(t+2) requested
+        auto park_next = [&](int t, int st) __attribute__((always_inline)) {
+            park_k(kreg, st);
+            park_v(st ^ 1);
+            issue_k((t + 3) * KT);
+            issue_v((t + 2) * KT);
+        };
+        // a tile of which the wave walks both items: straight-line code, the pairs swapped from step to step
+        auto walk_full = [&](int t, auto st_c, auto later_c) __attribute__((always_inline)) {
+            const int st = st_c;
+            constexpr bool kLater = decltype(later_c)::value;
+            const uint16_t* const k_st = Ks + st * KT * LDK + k_off;
+            const uint16_t* const k_ot = Ks + (st ^ 1) * KT * LDK + k_off;
+            const uint16_t* const v_st = Vs + st * KT * LDV + v_off;
+            const uint16_t* const v_ot = Vs + (st ^ 1) * KT * LDV + v_off;
+            const int k0 = t * KT;
+            step(k0, k_st + 32 * LDK, (!kLater && t == 0) ? v_st : v_ot + 32 * LDV, p_a, p_b);
+            __syncthreads();
+            park_next(t, st);
+            step(k0 + 32, k_ot, v_st, p_b, p_a);
+        };
+        auto walk_tile = [&](int t) __attribute__((always_inline)) {
+            const int st = t & 1;
+            const uint16_t* const k_st = Ks + st * KT * LDK + k_off;
+            const uint16_t* const k_ot = Ks + (st ^ 1) * KT * LDK + k_off;
+            const uint16_t* const v_st = Vs + st * KT * LDV + v_off;
+            const uint16_t* const v_ot = Vs + (st ^ 1) * KT * LDV + v_off;
+            slot(t * NI, k_st + 32 * LDK, t == 0 ? v_st : v_ot + 32 * LDV);
+            __syncthreads();
+            park_next(t, st);
+            slot(t * NI + 1, k_ot, v_st);
+        };
+        using IC0 = std::integral_constant<int, 0>;
+        using IC1 = std::integral_constant<int, 1>;
+        const int t_full = n_it / NI;
+        int t0 = 0;
+        if (t0 < t_full) {
+            walk_full(0, IC0{}, std::false_type{});
+            t0 = 1;
+        }
+        for (; t0 + 2 <= t_full; t0 += 2) {
+            walk_full(t0, IC1{}, std::true_type{});
+            walk_full(t0 + 1, IC0{}, std::true_type{});
+        }
+        if (t0 < t_full) {
+            walk_full(t0, t0 & 1, std::true_type{});
+            t0++;
+        }
+        for (; t0 < n_tiles; t0++) walk_tile(t0);
+        // a wave that walked every item of the workgroup still owes the last P.V
+        if (n_it == n_tiles * NI && n_it > 0) drain(Vs + ((n_tiles - 1) & 1) * KT * LDV + v_off + 32 * LDV);
+        __syncthreads();  // the output rows are staged over the tiles
+    }
+
+    // ---- output: the wave parks its 64 normalised rows in its own region of LDS and streams them out as whole rows
+    uint16_t* const obuf = (uint16_t*)(lds + wq * REGION);
+    const float fill = p.zero_padded_rows ? 0.0f : quiet_nan();
+    if (n_tiles > 0) {
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+            const float l = t_sum_with_other_half(l_run[rb]);
+            const bool good = (l > 0.0f) && (l < __uint_as_float(0x7f800000u));
+            const float inv_l = __builtin_amdgcn_rcpf(l);
+            uint16_t* const orow = obuf + (32 * rb + col) * LDK + 4 * hh;
+            if (__all(good && valid[rb])) {
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        *(u32x2_t*)(orow + 32 * dt + 8 * j) =
+                            u32x2_t{t_cvt_pk_bf16(acc_o[rb][dt][4 * j] * inv_l, acc_o[rb][dt][4 * j + 1] * inv_l),
+                                    t_cvt_pk_bf16(acc_o[rb][dt][4 * j + 2] * inv_l, acc_o[rb][dt][4 * j + 3] * inv_l)};
+            } else {
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        float o[4];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            float x = good ? acc_o[rb][dt][4 * j + e] * inv_l : quiet_nan();
+                            if (!valid[rb]) x = fill;
+                            o[e] = x;
+                        }
+                        *(u32x2_t*)(orow + 32 * dt + 8 * j) = u32x2_t{t_cvt_pk_bf16(o[0], o[1]), t_cvt_pk_bf16(o[2], o[3])};
+                    }
+            }
+        }
+    }
+    // (the same wave wrote and now reads: no barrier needed, the LDS queue is in order)
+    {
+        constexpr int RS = 64 / CH;  // rows per store instruction
+        const int row0 = lane / CH, ch = lane % CH;
+        const int rr0 = r0 + row0;
+        uint16_t* dst = p.out + (size_t)b * p.lo.batch_stride + (size_t)hx * p.lo.head_stride + (size_t)rr0 * p.lo.row_pitch + 8 * ch;
+        const size_t step_e = (size_t)RS * (size_t)p.lo.row_pitch;
+        const uint16_t* src = obuf + row0 * LDK + 8 * ch;
+#pragma unroll
+        for (int n = 0; n < 64 / RS; n++) {
+            const int rr = rr0 + RS * n;
+            // no key tile walked: padded rows get the fill value, valid rows (which then see no key at all) NaN
+            const uint32_t f2 = rr < n_q ? 0x7fc07fc0u : fill2;
+            u32x4_t val = {f2, f2, f2, f2};
+            if (n_tiles > 0) val = *(const u32x4_t*)(src + RS * n * LDK);
+            if (rr < rows_total) *(u32x4_t*)dst = val;
+            dst += step_e;
+        }
+    }
+}
+
 template <int DP, int MODE, bool BIAS, bool PACKED, bool SPLIT = false>
 hipError_t launch_one(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
     hipLaunchKernelGGL((flash_tile_bf16_kernel<DP, MODE, BIAS, PACKED, SPLIT>), grid, dim3(TileCfg<DP>::THREADS), 0, stream, p);
@@ -989,6 +1452,26 @@ int flash_tile_bf16_key_tile(int dim) { return dim <= 128 ? 64 : 32; }
 // requests that run a few tiles past the last one included).
 bool flash_tile_bf16_addressable(long long seq_kv, long long row_pitch) {
     return seq_kv >= 0 && row_pitch > 0 && (unsigned long long)(seq_kv + 512) * (unsigned long long)row_pitch * 2ull < (1ull << 32);
+}
+
+// 64 rows per wave: head dim 64 exactly, rows of one head, masks none / causal (with or without per-sequence lengths)
+bool flash_wide_bf16_supported(const FlashTileParams& p) {
+    return p.dim == 64 && p.pack <= 1 && !p.bias && p.n_splits <= 1 && (p.mask == kMaskNone || p.mask == kMaskCausal) &&
+           flash_tile_bf16_addressable(p.seq_kv, p.lkv.row_pitch);
+}
+
+hipError_t launch_flash_wide_bf16(hipStream_t stream, const FlashTileParams& params) {
+    FlashTileParams p = params;
+    if (p.batch == 0 || p.heads == 0 || p.seq_q == 0) return hipSuccess;
+    if (!flash_wide_bf16_supported(p) || p.group < 1) return hipErrorInvalidValue;
+    const long long n_qtiles = ((long long)p.seq_q + WROWS - 1) / WROWS;
+    if (p.batch > 65535 || n_qtiles > 65535 || p.heads > 65535) return hipErrorInvalidValue;  // grid limits
+    p.pack = 1;
+    p.group_magic = p.group > 1 ? (uint32_t)(0x100000000ull / (unsigned long long)p.group) + 1u : 0u;
+    dim3 grid((unsigned)p.heads, (unsigned)p.batch, (unsigned)n_qtiles);
+    if (p.mask == kMaskCausal) hipLaunchKernelGGL(flash_wide_bf16_kernel<kMaskCausal>, grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(flash_wide_bf16_kernel<kMaskNone>, grid, dim3(256), 0, stream, p);
+    return hipGetLastError();
 }
 
 hipError_t launch_flash_tile_bf16(hipStream_t stream, const FlashTileParams& params) {

@@ -132,6 +132,9 @@ bool flash_tile_bf16_supported(int dim);
 int flash_tile_bf16_key_tile(int dim);
 hipError_t launch_flash_tile_bf16(hipStream_t stream, const FlashTileParams& p);
 bool flash_tile_bf16_addressable(long long seq_kv, long long row_pitch);  // K/V slabs below 4 GiB (32-bit offsets)
+// the same walk with 64 query rows per wave: head dim 64, masks none / causal, rows of one head
+bool flash_wide_bf16_supported(const FlashTileParams& p);
+hipError_t launch_flash_wide_bf16(hipStream_t stream, const FlashTileParams& p);
 
 // Unmasked attention of every query row over all keys; generic in dim (<= 512), head
 // grouping, kv_len and query count.  T is float or uint16_t (bf16 bits).

@@ -120,7 +120,7 @@ def i32_add_dev(buf, n: int, delta: int, stream=None):
 
 def debug_force_bf16_prefill_kernel(name: str = "auto"):
     """Measurement / test switch: "auto", "tile" or "persistent" for the bf16 prefill entries."""
-    rc = L.lib().rt_debug_force_bf16_prefill_kernel({"auto": 0, "tile": 1, "persistent": 2}[name])
+    rc = L.lib().rt_debug_force_bf16_prefill_kernel({"auto": 0, "tile": 1, "persistent": 2, "wide": 3}[name])
     if rc:
         raise ValueError(name)
 

@@ -23,7 +23,7 @@ def inputs(shape_q, shape_kv, seeds=(1, 2, 3), q_mul=1.0):
 # (kernel forced through rt_debug_force_bf16_prefill_kernel, head dim): the persistent 8-wave kernel covers 64 and 128, the
 # 4-wave tile kernel every multiple of 8 up to 256 (zero-padded to 32 / 64 / 96 / 128 / 256 in LDS)
 KERNEL_DIMS = [("persistent", 64), ("persistent", 128), ("tile", 32), ("tile", 64), ("tile", 80), ("tile", 96),
-               ("tile", 128), ("tile", 8), ("tile", 200), ("tile", 256)]
+               ("tile", 128), ("tile", 8), ("tile", 200), ("tile", 256), ("wide", 64)]
 
 
 @pytest.fixture
@@ -65,7 +65,7 @@ def test_both_prefill_kernels_agree(oracle, force_kernel, n, d):
     assert max_abs(outs["persistent"], outs["tile"]) <= TOL
 
 
-@pytest.mark.parametrize("kernel,d", [("persistent", 64), ("persistent", 128), ("tile", 64), ("tile", 128)])
+@pytest.mark.parametrize("kernel,d", [("persistent", 64), ("persistent", 128), ("tile", 64), ("tile", 128), ("wide", 64)])
 def test_row_max_that_keeps_rising_along_the_keys(oracle, force_kernel, kernel, d):
     """Scores that grow with the key index: a ramp that lifts the row max by tens of units from one 32-key item to
     the next, one key hundreds of units above everything before it (an exponential taken against the old max
@@ -106,7 +106,31 @@ def test_flash_bf16_closed_forms():
     assert max_abs(out, cf) <= 2 ** -7 * 2.0  # weights sum to 1 up to P's bf16 rounding
 
 
-@pytest.mark.parametrize("kernel", ["persistent", "tile"])
+@pytest.mark.parametrize("mask", ["causal", "none"])
+def test_long_head_dim_64_takes_the_64_rows_per_wave_kernel_by_itself(oracle, mask):
+    """B=4, H=32, N=2048, D=64: 1024 workgroups of 256 rows, the shape class the library routes to the kernel with 64
+    query rows per wave when nothing is forced.  Every row of eight (batch, head) slabs against the oracle, and the
+    whole output against the tile kernel's (both round the same f32 sums to bf16)."""
+    b, h, n, d = 4, 32, 2048, 64
+    (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d), (91, 92, 93))
+    shape = ra.AttentionShape.new(b, h, n, d)
+    m = ra.Mask.causal() if mask == "causal" else ra.Mask.none()
+    ra.debug_force_bf16_prefill_kernel("auto")
+    got = flash_bf16(shape, qb, kb, vb, m).reshape(b * h, n, d)
+    try:
+        ra.debug_force_bf16_prefill_kernel("tile")
+        tile = flash_bf16(shape, qb, kb, vb, m).reshape(b * h, n, d)
+    finally:
+        ra.debug_force_bf16_prefill_kernel("auto")
+    assert max_abs(got, tile) <= 2 ** -7 * 4.0  # a bf16 ulp or two of values below 4
+    q3, k3, v3 = (x.reshape(b * h, n * d) for x in (qf, kf, vf))
+    for slab in (0, 1, 31, 64, 77, 100, 126, 127):
+        want = oracle.flash_forward_masked(oracle.AttentionShape(1, 1, n, d), q3[slab], k3[slab], v3[slab],
+                                           "causal" if mask == "causal" else None).reshape(n, d)
+        assert_bf16_parity(got[slab], want, d, n, f"slab {slab}")
+
+
+@pytest.mark.parametrize("kernel", ["persistent", "tile", "wide"])
 def test_flash_bf16_masks_nan_rules(oracle, force_kernel, kernel):
     force_kernel(kernel)
     b, h, n, d = 1, 2, 150, 64
@@ -129,12 +153,12 @@ def test_flash_bf16_masks_nan_rules(oracle, force_kernel, kernel):
         assert_bf16_parity(got, want, d, n)
 
 
-@pytest.mark.parametrize("kernel", ["persistent", "tile"])
+@pytest.mark.parametrize("kernel,d", [("persistent", 128), ("tile", 128), ("wide", 64)])
 @pytest.mark.parametrize("hq,hkv", [(8, 2), (4, 1), (6, 6)])
-def test_flash_bf16_gqa_head_mapping(oracle, force_kernel, kernel, hq, hkv):
+def test_flash_bf16_gqa_head_mapping(oracle, force_kernel, kernel, d, hq, hkv):
     """kv head = h / (Hq/Hkv): equals the oracle on explicitly replicated K/V (gqa.rs:151-177)."""
     force_kernel(kernel)
-    b, n, d = 2, 130, 128
+    b, n = 2, 130
     (qb, qf), (kb, kf), (vb, vf) = inputs((b, hq, n, d), (b, hkv, n, d))
     got = flash_bf16(ra.AttentionShape.new(b, hq, n, d), qb, kb, vb, ra.Mask.causal(), n_kv_heads=hkv)
     g = hq // hkv
@@ -156,7 +180,7 @@ def run_varlen(shape, qb, kb, vb, lens, zero=True):
     return attn_oracle.bf16_to_f32(dout.download(np.uint16, n_out))
 
 
-@pytest.mark.parametrize("kernel,d", [("persistent", 64), ("tile", 64), ("tile", 96), ("persistent", 128)])
+@pytest.mark.parametrize("kernel,d", [("persistent", 64), ("tile", 64), ("tile", 96), ("persistent", 128), ("wide", 64)])
 def test_varlen_small(oracle, force_kernel, kernel, d):
     force_kernel(kernel)
     b, h, n = 4, 2, 200
@@ -195,7 +219,7 @@ def test_strict_mode_on_a_padded_batch(oracle, strict_v):
     assert np.abs(got[fin] - want[fin]).max() <= TOL
 
 
-@pytest.mark.parametrize("kernel", ["auto", "persistent", "tile"])
+@pytest.mark.parametrize("kernel", ["auto", "persistent", "tile", "wide"])
 def test_config_padded_batch_b16_h16_n1024_d64(oracle, force_kernel, kernel):
     """The variable-length workload of the benchmark set: lengths uniform in [128, 1024] from a seed, key padding + causal,
     padded query rows exactly 0."""
@@ -301,7 +325,7 @@ def strict_v():
 
 
 @pytest.mark.parametrize("kernel,n,d,j", [("persistent", 1024, 128, 700), ("tile", 1024, 128, 700), ("tile", 777, 64, 500),
-                                          ("tile", 300, 100, 299)])
+                                          ("tile", 300, 100, 299), ("wide", 777, 64, 500)])
 @pytest.mark.parametrize("bad", [np.nan, -np.inf])
 def test_strict_mode_gives_the_reference_outcome_for_non_finite_v(oracle, force_kernel, strict_v, kernel, n, d, j, bad):
     """With rt_set_strict_non_finite_v on, a non-finite V element at key j makes that column NaN in every row that
@@ -361,7 +385,7 @@ def test_non_finite_v_row_at_a_causally_hidden_position(oracle, force_kernel, ke
     assert np.isfinite(got[..., :5]).all() and np.isfinite(want_ref[..., :5]).all()
 
 
-@pytest.mark.parametrize("kernel", ["persistent", "tile"])
+@pytest.mark.parametrize("kernel", ["persistent", "tile", "wide"])
 @pytest.mark.parametrize("mask", ["none", "padding"])
 @pytest.mark.parametrize("n,d", [(200, 128), (100, 128), (200, 64), (40, 64), (330, 96)])
 def test_infinite_last_v_row_with_a_ragged_last_key_tile(oracle, force_kernel, kernel, mask, n, d):
@@ -390,7 +414,8 @@ def test_infinite_last_v_row_with_a_ragged_last_key_tile(oracle, force_kernel, k
     assert np.isfinite(got[..., rest]).all() and max_abs(got[..., rest], want[..., rest]) <= TOL
 
 
-@pytest.mark.parametrize("kernel,d", [("persistent", 64), ("persistent", 128), ("tile", 64), ("tile", 128), ("tile", 96)])
+@pytest.mark.parametrize("kernel,d", [("persistent", 64), ("persistent", 128), ("tile", 64), ("tile", 128), ("tile", 96),
+                                      ("wide", 64)])
 def test_two_launches_give_the_same_bits(force_kernel, kernel, d):
     """No atomics, no order that depends on timing: the same inputs give the same output bits on every launch.
     (A vector instruction that reads a matrix result too early, for one, shows up here as last-bit differences.)"""

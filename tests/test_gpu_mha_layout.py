@@ -47,9 +47,19 @@ def test_mha_flash_forward_f32_errors_follow_flash_forward():
     ra.mha_flash_forward_f32(z[:0], z[:0], z[:0], 2, 0, 3, 4, out=out)
 
 
+@pytest.mark.parametrize("kernel", ["auto", "wide"])
 @pytest.mark.parametrize("mask_name", ["none", "causal", "padding"])
-@pytest.mark.parametrize("b,n,h,hkv,d", [(2, 200, 4, 4, 64), (1, 513, 6, 2, 128), (2, 64, 8, 1, 128)])
-def test_flash_bnhd_bf16_matches_oracle(oracle, b, n, h, hkv, d, mask_name):
+@pytest.mark.parametrize("b,n,h,hkv,d", [(2, 200, 4, 4, 64), (1, 513, 6, 2, 128), (2, 64, 8, 1, 128), (1, 700, 8, 2, 64)])
+def test_flash_bnhd_bf16_matches_oracle(oracle, b, n, h, hkv, d, mask_name, kernel):
+    """(kernel "wide": the 64-rows-per-wave kernel where it applies, head dim 64 without a padding mask; else as "auto")"""
+    ra.debug_force_bf16_prefill_kernel(kernel)
+    try:
+        _bnhd_bf16_case(oracle, b, n, h, hkv, d, mask_name)
+    finally:
+        ra.debug_force_bf16_prefill_kernel("auto")
+
+
+def _bnhd_bf16_case(oracle, b, n, h, hkv, d, mask_name):
     (qb, qf) = bf16_round(seeded_normal((b, n, h, d), 21).ravel())
     (kb, kf) = bf16_round(seeded_normal((b, n, hkv, d), 22).ravel())
     (vb, vf) = bf16_round(seeded_normal((b, n, hkv, d), 23).ravel())
