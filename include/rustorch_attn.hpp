@@ -640,7 +640,18 @@ struct LlmKernels {
                                                    n_heads, n_kv, head_dim, max_seq, &e),
                           e);
     }
+    // No counterpart in the reference: adds `delta` to n int32 values on the device, on `stream` -- the positions and
+    // context lengths of a decode loop recorded into a HIP graph advance inside the graph.
+    static void i32_add_dev(void* stream, int32_t* values, size_t n, int32_t delta) {
+        rt_err_detail e;
+        detail::check_gqa(rt_i32_add_dev(stream, values, n, delta, &e), e);
+    }
 };
+
+// Process-wide: causal prefill entries follow their kernel with a pass that gives rows the reference's NaN for
+// non-finite V elements at keys they do not see (cpu_forward.rs:268-425 multiplies the hidden zeros into every V tile).
+// Returns the previous setting.
+inline bool set_strict_non_finite_v(bool on) { return rt_set_strict_non_finite_v(on ? 1 : 0) != 0; }
 
 }  // namespace rustorch_attn
 

@@ -76,6 +76,11 @@ static std::vector<float> naive(const AttentionShape& s, const std::vector<float
 }
 
 static void test_errors() {
+    {   // the strict switch needs no device and returns the previous setting
+        CHECK(set_strict_non_finite_v(true) == false);
+        CHECK(set_strict_non_finite_v(false) == true);
+        CHECK(set_strict_non_finite_v(false) == false);
+    }
     {   // ZeroDim comes first (cpu_forward.rs:142-169)
         std::vector<float> e, out;
         AttentionError err(AttentionError::Kind::ZeroDim, "", 0, 0, "");
