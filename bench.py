@@ -486,6 +486,58 @@ def main():
                                                                  "heads, D=128, seq_new new positions (4, 16) over a cache "
                                                                  "that holds 8192 keys with them (pos_base = 8192 - seq_new), "
                                                                  "rt_gqa_decode_chunk_bf16 with a host length"})
+        # ---- the step ahead of decode attention (q/k RMSNorm + RoPE + cache append, one launch): a decode step of
+        # the batch, and a prompt of the headline shape
+        prep = {}
+        rope_p = ra.RoPE(Dd, Lmax)
+        rope_p.device_tables()
+        d_g = ra.HipStorage.from_numpy(np.ones(Dd, dtype=np.float32) + 0.01 * np.arange(Dd, dtype=np.float32) / Dd)
+        for name, (pb, pseq) in (("decode_step", (Bd, 1)), ("prompt", (4, 4096))):
+            rng_r = np.random.default_rng(4242 + pseq)
+            pq = oracle.f32_to_bf16(rng_r.standard_normal(pb * Hq * pseq * Dd, dtype=np.float32))
+            pk, pv = (oracle.f32_to_bf16(rng_r.standard_normal(pb * Hkv * pseq * Dd, dtype=np.float32)) for _ in range(2))
+            d_pq, d_pk, d_pv = (ra.HipStorage.from_numpy(x) for x in (pq, pk, pv))
+            k_, v_ = sets[0]  # (pb sequences of the first cache set: positions 0 .. pseq - 1 are overwritten)
+            launch_p = lambda i: K.qk_norm_rope_kv_append_bf16(stream, d_pq, d_pk, d_pv, k_, v_, 0, rope_p, pb, Hq, Hkv, Dd,
+                                                               Lmax, q_gamma=d_g, k_gamma=d_g, seq=pseq)
+            tp = time_steps(hip, stream, launch_p, args.steps, args.warmup)
+            bytes_p = float(pb * pseq * Dd * 2 * (2 * Hq + 4 * Hkv))  # q in and out, k and v in, two cache rows out
+            leg_p = {"us_per_call": tp.mean_ms * 1e3, **spread(tp.per), **tp.settle(), "algorithmic_bytes": bytes_p,
+                     "roofline": {"bound": "hbm", "achieved": bytes_p / (tp.mean_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                                  "unit": "GB/s", "frac": bytes_p / (tp.mean_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                  "traffic": profile_traffic("prepare_hq32_hkv8_d128.md", name),
+                                  "kernel": "prompt_prepare_kernel<64, 128>" if pseq >= 32 else "decode_prepare_kernel"}}
+            if not args.no_cpu:
+                # q is rewritten in place: a fresh copy of the inputs, one call, every bit against the oracle
+                d_pq.upload(pq)
+                launch_p(0)
+                hip.sync()
+                kc_w = np.zeros(pb * Hkv * pseq * Dd, dtype=np.uint16)  # the oracle's cache holds the new rows only
+                vc_w = np.zeros_like(kc_w)
+                oro_p = oracle.RoPE(Dd, Lmax)
+                oro_p.cos, oro_p.sin = rope_p.cos.copy(), rope_p.sin.copy()
+                g_host = d_g.download(np.float32)
+                t0 = time.perf_counter()
+                want_q = oracle.decode_prepare_bf16(pq, pk, pv, kc_w, vc_w, np.zeros(pb, dtype=np.int32), g_host, g_host, 1e-6,
+                                                    oro_p, pb, Hq, Hkv, Dd, pseq, seq=pseq)
+                cpu_p = time.perf_counter() - t0
+                got_q = d_pq.download(np.uint16)
+                got_kc = k_.download(np.uint16, pb * Hkv * Lmax * Dd).reshape(pb * Hkv, Lmax, Dd)[:, :pseq]
+                got_vc = v_.download(np.uint16, pb * Hkv * Lmax * Dd).reshape(pb * Hkv, Lmax, Dd)[:, :pseq]
+                same = (np.array_equal(got_q, want_q) and np.array_equal(got_kc, kc_w.reshape(pb * Hkv, pseq, Dd))
+                        and np.array_equal(got_vc, vc_w.reshape(pb * Hkv, pseq, Dd)))
+                leg_p["parity_bit_exact"] = bool(same)
+                leg_p["cpu_baseline"] = {"value": bytes_p / cpu_p / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                                         "sample": f"the whole call once ({cpu_p * 1e3:.0f} ms), single-threaded loops as in "
+                                                   f"the reference's decode_step"}
+                if not same:
+                    print(f"PARITY FAILURE: prepare ({name}) differs from the oracle's bits", file=sys.stderr)
+                    sys.exit(1)
+            prep[name] = leg_p
+            del d_pq, d_pk, d_pv
+        decode["prepare"] = dict(prep, config={"workload": "rt_qk_norm_rope_kv_append_bf16, 32 q / 8 kv heads, D=128, both "
+                                                           "gammas: decode_step = batch 64, one new token each; prompt = "
+                                                           "batch 4, 4096 new tokens each at position 0"})
         if not args.no_cpu:
             got = oracle.bf16_to_f32(d_o.download(np.uint16))
             t0 = time.perf_counter()

@@ -53,13 +53,19 @@ def test_matches_oracle_bit_for_bit(oracle, norms, b_, hq, hkv, d, lmax):
     _run(oracle, rope, oro, q, k, v, kc, vc, qg, kg, positions, b_, hq, hkv, d, lmax, 1e-6)
 
 
-@pytest.mark.parametrize("b_,hq,hkv,d,lmax,seq", [(2, 3, 1, 16, 24, 5), (2, 8, 2, 128, 700, 300), (1, 4, 4, 64, 64, 64)])
-def test_several_new_tokens_match_oracle_bit_for_bit(oracle, b_, hq, hkv, d, lmax, seq):
-    """A prompt: [batch, heads, seq, head_dim] inputs, token s at position p + s and cache row p + s."""
+@pytest.mark.parametrize("norms", [(True, True), (False, False), (True, False)])
+@pytest.mark.parametrize("b_,hq,hkv,d,lmax,seq", [(2, 3, 1, 16, 24, 5), (2, 8, 2, 128, 700, 300), (1, 4, 4, 64, 64, 64),
+                                                  (2, 4, 2, 256, 400, 257), (1, 2, 1, 96, 1100, 1024), (2, 2, 2, 72, 80, 40),
+                                                  (1, 6, 2, 32, 40, 33), (3, 2, 1, 128, 31, 31)])
+def test_several_new_tokens_match_oracle_bit_for_bit(oracle, b_, hq, hkv, d, lmax, seq, norms):
+    """A prompt: [batch, heads, seq, head_dim] inputs, token s at position p + s and cache row p + s.  From 32 tokens
+    on, head dims that are a multiple of 16 up to 256 take the kernel that moves 64 consecutive tokens of a head
+    through LDS; the others (and head dim 72 here) the one-wave-per-row kernel: the same
+    bits either way."""
     rng = np.random.default_rng(300 + seq)
     positions = rng.integers(0, lmax - seq + 1, size=b_).astype(np.int32)
     positions[-1] = lmax - seq
-    rope, oro, q, k, v, kc, vc, qg, kg = _case(oracle, rng, b_, hq, hkv, d, lmax, positions, (True, True), seq=seq)
+    rope, oro, q, k, v, kc, vc, qg, kg = _case(oracle, rng, b_, hq, hkv, d, lmax, positions, norms, seq=seq)
     _run(oracle, rope, oro, q, k, v, kc, vc, qg, kg, positions, b_, hq, hkv, d, lmax, 1e-6, seq=seq)
 
 
