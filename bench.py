@@ -8,15 +8,16 @@ uniform in [512, 8192], Lmax 8192) and reports it under "decode", and the f32 ca
 B=1, H=8, N=2048, D=64 (the reference's own CPU-runnable case) under "f32_prefill", and the f32
 backward on that shape under "f32_backward", the padded-batch prefill (B=16, H=16, D=64, lengths in [128, 1024])
 under "padded_prefill", the long-context prefill (B=1, H=32, N=16384, D=128, Q scaled by 2) under
-"long_prefill" and a long prefill at the other head dim of the matrix-core kernels (B=4, H=32, N=4096, D=64) under
-"d64_prefill".
+"long_prefill", a long prefill at the other head dim of the matrix-core kernels (B=4, H=32, N=4096, D=64) under
+"d64_prefill", and under "other_shapes" the tile kernel at head dims 32, 96 and 256 (B=4, H=32, N=2048, causal) and
+the bf16 masked self-attention of MultiHeadAttention (B=4, T=1024, H=16, hd=64, a sliding-window mask as an f32 bias).
 
 Every leg first runs a settle phase: launches of the leg's own step until SETTLE_MS of device time have passed
 (after an idle period the clocks first drop and then recover over some tens of milliseconds); the phase is
 reported as settle_ms / settle_launches and is followed by the counted warm-up (--warmup) and the timed region
 (--steps), which is the only part that enters value, ms_per_step and roofline.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only prefill|decode|f32|bwd|padded|long|d64]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only prefill|decode|f32|bwd|padded|long|d64|shapes]
 
 Prints ONE JSON line.  `value` is prefill TFLOP/s with causal-counted FLOPs
 (4*B*H*D*N*(N+1)/2: skipped tiles are not credited); `roofline` prices it against the dense bf16
@@ -208,7 +209,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity sample")
-    ap.add_argument("--only", choices=["prefill", "decode", "f32", "bwd", "padded", "long", "d64"], default=None)
+    ap.add_argument("--only", choices=["prefill", "decode", "f32", "bwd", "padded", "long", "d64", "shapes"], default=None)
     ap.add_argument("--no-ceiling", action="store_true",
                     help="skip the run of rustorch_amd/lib/mfma_sustained (what a loop of nothing but bf16 MFMA "
                          "sustains on this GPU, reported beside the data-sheet peak)")
@@ -320,6 +321,48 @@ def main():
                  "config": {"workload": "bf16 causal prefill at head dim 64, B=4 H=32 N=4096 D=64, N(0,1) inputs "
                                         "(seed 64), f32 accumulation",
                             "flop_convention": "4*B*H*D*N*(N+1)/2 (causal-counted)"}}
+
+    # ------------------------------------------------------------------ shapes no BASELINE config names: timed for the record
+    shapes = None
+    if args.only in (None, "shapes"):
+        shapes = {}
+        for Ds in (32, 96, 256):
+            leg_s = causal_prefill(4, 32, 2048, Ds, 300 + Ds, 1.0, 8, f"flash_tile_bf16_kernel<{Ds}, causal>", None)
+            leg_s["value"] = leg_s.pop("tflops")
+            leg_s["unit"] = "TFLOP/s"
+            shapes[f"causal_prefill_b4_h32_n2048_d{Ds}"] = leg_s
+        # masked self-attention on bf16 [B,T,H*hd] activations with an additive f32 mask [T,T] (a sliding window of 256)
+        Bm, Tm, Hm, Dm, win = 4, 1024, 16, 64, 256
+        rng_m = np.random.default_rng(909)
+        n_m = Bm * Tm * Hm * Dm
+        qm, km, vm = (oracle.f32_to_bf16(rng_m.standard_normal(n_m, dtype=np.float32)) for _ in range(3))
+        ii, jj = np.arange(Tm)[:, None], np.arange(Tm)[None, :]
+        bias_m = np.where((jj <= ii) & (jj > ii - win), 0.0, -1.0e4).astype(np.float32)
+        d_qm, d_km, d_vm, d_bm = (ra.HipStorage.from_numpy(x) for x in (qm, km, vm, bias_m.ravel()))
+        d_om = ra.HipStorage(n_m * 2)
+        tmm = time_steps(hip, stream, lambda i: ra.mha_forward_masked_bf16_dev(d_qm, d_km, d_vm, d_om, Bm, Tm, Tm, Hm, Dm,
+                                                                               attn_mask=d_bm, mask_len=Tm * Tm,
+                                                                               stream=stream), args.steps, args.warmup)
+        flops_m = 4.0 * Bm * Hm * Dm * float(Tm) * Tm  # every (query, key) pair is scored: the mask is a bias
+        ach_m = flops_m / (tmm.mean_ms * 1e-3) / 1e12
+        leg_m = {"value": ach_m, "unit": "TFLOP/s", "us_per_call": tmm.mean_ms * 1e3, **spread(tmm.per), **tmm.settle(),
+                 "roofline": {"bound": "mfma", "achieved": ach_m, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                              "frac": ach_m / PEAK_BF16_TFLOPS, "traffic": None,
+                              "kernel": "flash_tile_bf16_kernel<64, none, bias>"},
+                 "config": {"workload": "bf16 masked self-attention, B=4 T=1024 H=16 hd=64 on [B,T,H*hd] tensors, additive f32 "
+                                        "mask [T,T] (causal sliding window of 256 keys, -1e4 elsewhere)",
+                            "flop_convention": "4*B*H*T*T*hd (the mask is a bias: every pair is scored)"}}
+        if not args.no_cpu:
+            got_m = oracle.bf16_to_f32(d_om.download(np.uint16)).reshape(Bm, Tm, Hm * Dm)
+            want_m = oracle.mha_forward_masked(oracle.bf16_to_f32(qm), oracle.bf16_to_f32(km), oracle.bf16_to_f32(vm), Bm, Tm,
+                                               Tm, Hm, Dm, attn_mask=bias_m).reshape(Bm, Tm, Hm * Dm)
+            leg_m["parity_max_abs"] = float(np.abs(got_m - want_m).max())
+            leg_m["parity_rel_fro"] = float(np.linalg.norm(got_m - want_m) / np.linalg.norm(want_m))
+            if not (leg_m["parity_max_abs"] <= oracle.BF16_MAX_ABS and leg_m["parity_rel_fro"] <= oracle.BF16_REL_FRO):
+                print(f"PARITY FAILURE: masked MHA bf16 {leg_m['parity_max_abs']} {leg_m['parity_rel_fro']}", file=sys.stderr)
+                sys.exit(1)
+        shapes["mha_masked_bf16_b4_t1024_h16_hd64"] = leg_m
+        del d_qm, d_km, d_vm, d_bm, d_om
 
     # ------------------------------------------------------------------ padded-batch prefill (per-sequence lengths + causal)
     padded = None
@@ -661,7 +704,7 @@ def main():
                 vs_baseline=None, scaling="weak")
     if prefill is None:  # --only <one of the other legs>: that leg is the line
         leg, dtype = next((x, t) for x, t in ((decode, "bf16"), (long_p, "bf16"), (padded, "bf16"), (d64_p, "bf16"),
-                                              (f32, "f32"), (bwd, "f32")) if x is not None)
+                                              (shapes, "bf16"), (f32, "f32"), (bwd, "f32")) if x is not None)
         print(json.dumps(dict(leg, dtype=dtype, **tail)))
         return
     sustained = None if args.no_ceiling else sustained_mfma()
@@ -687,7 +730,7 @@ def main():
         out["parity_max_abs"] = prefill["parity_max_abs"]
         out["parity_rel_fro"] = prefill["parity_rel_fro"]
     for key, leg in (("decode", decode), ("padded_prefill", padded), ("long_prefill", long_p), ("d64_prefill", d64_p),
-                     ("f32_prefill", f32), ("f32_backward", bwd)):
+                     ("other_shapes", shapes), ("f32_prefill", f32), ("f32_backward", bwd)):
         if leg is not None:
             out[key] = leg
     print(json.dumps(out))
