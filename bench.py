@@ -10,7 +10,8 @@ backward on that shape under "f32_backward", the padded-batch prefill (B=16, H=1
 under "padded_prefill", the long-context prefill (B=1, H=32, N=16384, D=128, Q scaled by 2) under
 "long_prefill", a long prefill at the other head dim of the matrix-core kernels (B=4, H=32, N=4096, D=64) under
 "d64_prefill", and under "other_shapes" the tile kernel at head dims 32, 96 and 256 (B=4, H=32, N=2048, causal) and
-the bf16 masked self-attention of MultiHeadAttention (B=4, T=1024, H=16, hd=64, a sliding-window mask as an f32 bias).
+the bf16 masked self-attention of MultiHeadAttention (B=4, T=1024, H=16, hd=64, a sliding-window mask as an f32 bias)
+and the sliding-window entry that needs no mask tensor (B=4, T=4096, H=16, hd=64, window 256).
 
 Every leg first runs a settle phase: launches of the leg's own step until SETTLE_MS of device time have passed
 (after an idle period the clocks first drop and then recover over some tens of milliseconds); the phase is
@@ -363,6 +364,39 @@ def main():
                 sys.exit(1)
         shapes["mha_masked_bf16_b4_t1024_h16_hd64"] = leg_m
         del d_qm, d_km, d_vm, d_bm, d_om
+        # the same kind of mask without the tensor: causal sliding window of 256 keys over T = 4096
+        Bw, Tw, Hw, Dw, win_w = 4, 4096, 16, 64, 256
+        rng_w = np.random.default_rng(910)
+        n_w = Bw * Tw * Hw * Dw
+        qw_, kw_, vw_ = (oracle.f32_to_bf16(rng_w.standard_normal(n_w, dtype=np.float32)) for _ in range(3))
+        d_qw, d_kw, d_vw = (ra.HipStorage.from_numpy(x) for x in (qw_, kw_, vw_))
+        d_ow = ra.HipStorage(n_w * 2)
+        shape_w = ra.AttentionShape.new(Bw, Hw, Tw, Dw)
+        tw = time_steps(hip, stream, lambda i: ra.flash_forward_window_bf16_dev(shape_w, d_qw, d_kw, d_vw, d_ow, win_w, bnhd=True,
+                                                                                stream=stream), args.steps, args.warmup)
+        pairs_w = float(sum(min(i + 1, win_w) for i in range(Tw)))
+        ach_w = 4.0 * Bw * Hw * Dw * pairs_w / (tw.mean_ms * 1e-3) / 1e12
+        leg_w = {"value": ach_w, "unit": "TFLOP/s", "us_per_call": tw.mean_ms * 1e3, **spread(tw.per), **tw.settle(),
+                 "roofline": {"bound": "mfma", "achieved": ach_w, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                              "frac": ach_w / PEAK_BF16_TFLOPS, "traffic": None,
+                              "kernel": "flash_tile_bf16_kernel<64, causal, window>"},
+                 "config": {"workload": "bf16 causal sliding-window self-attention, B=4 T=4096 H=16 hd=64 on [B,T,H*hd] tensors, "
+                                        "window 256, rt_flash_forward_window_bnhd_bf16_dev (no mask tensor)",
+                            "flop_convention": "4*B*H*hd*(visible pairs): sum over i of min(i + 1, window)"}}
+        if not args.no_cpu:
+            got_w = oracle.bf16_to_f32(d_ow.download(np.uint16)).reshape(Bw, Tw, Hw, Dw)
+            hb, hh_ = 1, 5
+            q1, k1, v1 = (oracle.bf16_to_f32(x).reshape(Bw, Tw, Hw, Dw)[hb, :, hh_] for x in (qw_, kw_, vw_))
+            want_w = oracle.mha_forward_masked(q1, k1, v1, 1, Tw, Tw, 1, Dw,
+                                               attn_mask=oracle.sliding_window_mask(Tw, win_w)).reshape(Tw, Dw)
+            leg_w["parity_max_abs"] = float(np.abs(got_w[hb, :, hh_] - want_w).max())
+            leg_w["parity_rel_fro"] = oracle.rel_fro_blocks(got_w[hb, :, hh_], want_w, Dw, Tw)
+            leg_w["parity_sample"] = "one (batch, head) slab against the composed path with sliding_window_mask as its bias"
+            if not (leg_w["parity_max_abs"] <= oracle.BF16_MAX_ABS and leg_w["parity_rel_fro"] <= oracle.BF16_REL_FRO):
+                print(f"PARITY FAILURE: window {leg_w['parity_max_abs']} {leg_w['parity_rel_fro']}", file=sys.stderr)
+                sys.exit(1)
+        shapes["window_bf16_b4_t4096_h16_hd64_w256"] = leg_w
+        del d_qw, d_kw, d_vw, d_ow
 
     # ------------------------------------------------------------------ padded-batch prefill (per-sequence lengths + causal)
     padded = None

@@ -203,6 +203,22 @@ int rt_flash_forward_bf16_dev(void *stream, const rt_attention_shape *shape, uin
                               const void *k, const void *v, int mask_kind, const uint8_t *keep, void *out,
                               rt_err_detail *err);
 
+/* Causal self-attention with a sliding window, on bf16 device tensors: position i sees keys j with j <= i and
+ * i - j < window -- what MultiHeadAttention computes with sliding_window_mask(seq, window) as its additive mask
+ * (crates/rustorch-nn/src/masks.rs:41-60, applied at crates/rustorch-nn/src/attention.rs:378-392), without the
+ * [seq, seq] f32 tensor (64 MB at seq = 4096, re-read per head) and without scoring the pairs it hides: a query tile
+ * walks window + 128 keys.  The reference adds -1e4 to the hidden scores where this entry leaves the keys out; the
+ * weights agree exactly (exp underflows to 0) as long as scaled scores stay far below 1e4 in magnitude.  window >= 1
+ * (0: RT_ERR_UNSUPPORTED, the reference asserts); window >= seq is the causal mask.  Tensors [batch, heads, seq, dim]
+ * (k, v: n_kv_heads; 0 = heads) or, for the _bnhd_ entry, [batch, seq, heads, dim]; head dims up to 256 that are a
+ * multiple of 8 and 16-byte aligned tensors (others: RT_ERR_UNSUPPORTED; rt_mha_forward_masked_bf16_dev with the
+ * mask tensor serves them). */
+int rt_flash_forward_window_bf16_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const void *q,
+                                     const void *k, const void *v, uint64_t window, void *out, rt_err_detail *err);
+int rt_flash_forward_window_bnhd_bf16_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads,
+                                          const void *q, const void *k, const void *v, uint64_t window, void *out,
+                                          rt_err_detail *err);
+
 /* No counterpart in the reference: a switch for measurements and tests.  which = 0 lets the library choose between
  * its bf16 prefill kernels (the default), 1 forces the tile kernel, 2 the persistent kernel where it applies (head
  * dim 64 / 128, no per-sequence lengths), 3 the kernel with 64 query rows per wave where it applies (head dim 64,

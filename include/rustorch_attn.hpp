@@ -449,6 +449,18 @@ inline void flash_forward_varlen_bf16_dev(const AttentionShape& shape, const voi
         e);
 }
 
+// Causal attention with a sliding window (key j visible to query i iff j <= i and i - j < window: sliding_window_mask,
+// crates/rustorch-nn/src/masks.rs:41-60) without the mask tensor; bnhd: [batch, seq, heads, dim] tensors.
+inline void flash_forward_window_bf16_dev(const AttentionShape& shape, const void* q, const void* k, const void* v,
+                                          void* out, size_t window, size_t n_kv_heads = 0, bool bnhd = false,
+                                          void* stream = nullptr) {
+    rt_attention_shape s = shape.c();
+    rt_err_detail e;
+    detail::check_attention(bnhd ? rt_flash_forward_window_bnhd_bf16_dev(stream, &s, n_kv_heads, q, k, v, window, out, &e)
+                                 : rt_flash_forward_window_bf16_dev(stream, &s, n_kv_heads, q, k, v, window, out, &e),
+                            e);
+}
+
 // ---- device-resident f32 backward (cpu_backward.rs:46-185; the saved-forward form of its header comment) ----------
 
 inline size_t flash_backward_workspace_bytes(const AttentionShape& shape) {

@@ -9,7 +9,7 @@ from .attention import (AttentionShape, Mask, flash_backward, flash_backward_f32
                         flash_forward_stats_f32_dev,
                         flash_backward_workspace_bytes, flash_forward, flash_forward_bf16_dev, flash_forward_bnhd_bf16_dev,
                         flash_forward_bnhd_f32_dev, flash_forward_f32_dev, flash_forward_masked,
-                        flash_forward_varlen_bf16_dev, mha_attention_f32, mha_attention_route, mha_flash_forward_f32, mha_forward_masked_bf16_dev, mha_forward_masked_f32_dev,
+                        flash_forward_varlen_bf16_dev, flash_forward_window_bf16_dev, mha_attention_f32, mha_attention_route, mha_flash_forward_f32, mha_forward_masked_bf16_dev, mha_forward_masked_f32_dev,
                         mha_forward_masked_f32)
 from .device import (HipStorage, Stream, debug_force_bf16_prefill_kernel, i32_add_dev, init, set_strict_non_finite_v,
                      shutdown, synchronize)

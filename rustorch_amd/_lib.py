@@ -23,6 +23,7 @@ SYMBOLS = (
     "rt_gqa_decode_workspace_bytes", "rt_gqa_decode_batched_bf16_noalloc",
     "rt_buf_alloc", "rt_buf_free", "rt_buf_zero", "rt_memcpy_h2d", "rt_memcpy_d2h", "rt_stream_synchronize",
     "rt_stream_create", "rt_stream_destroy", "rt_i32_add_dev", "rt_debug_force_bf16_prefill_kernel", "rt_set_strict_non_finite_v",
+    "rt_flash_forward_window_bf16_dev", "rt_flash_forward_window_bnhd_bf16_dev",
 )
 
 RT_OK = 0
@@ -100,6 +101,8 @@ def lib():
     L.rt_gqa_decode_chunk_bf16.argtypes = [vp, vp, vp, vp, vp, i32p, i32, i32, i32, i32, i32, i32, i32, errp]
     L.rt_flash_forward_bnhd_f32_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
     L.rt_flash_forward_bnhd_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, C.c_int, vp, vp, errp]
+    L.rt_flash_forward_window_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, u64, vp, errp]
+    L.rt_flash_forward_window_bnhd_bf16_dev.argtypes = [vp, shp, u64, vp, vp, vp, u64, vp, errp]
     L.rt_kv_append_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, errp]
     L.rt_kv_cache_append_dev.argtypes = [vp, vp, vp, vp, sz, vp, sz, sz, sz, sz, sz, sz, sz, sz, errp]
     L.rt_qk_norm_rope_kv_append_bf16.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, vp, vp, C.c_float, vp, vp, i32, i32,

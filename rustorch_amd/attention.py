@@ -172,6 +172,17 @@ def flash_forward_bf16_dev(shape, q, k, v, out, mask: Mask = None, keep_dev=None
     raise_for(rc, err)
 
 
+def flash_forward_window_bf16_dev(shape, q, k, v, out, window: int, n_kv_heads=0, bnhd=False, stream=None):
+    """Causal attention with a sliding window (position i sees keys j <= i with i - j < window: the mask of
+    rustorch_nn::masks::sliding_window_mask, crates/rustorch-nn/src/masks.rs:41-60, never materialised) on bf16 device
+    tensors [B,H,N,D], or [B,N,H,D] with `bnhd`.  Enqueues on `stream` and returns."""
+    err = L.RtErr()
+    s = shape._c()
+    fn = L.lib().rt_flash_forward_window_bnhd_bf16_dev if bnhd else L.lib().rt_flash_forward_window_bf16_dev
+    raise_for(fn(stream, C.byref(s), n_kv_heads, dev_ptr(q), dev_ptr(k), dev_ptr(v), int(window), dev_ptr(out),
+                 C.byref(err)), err)
+
+
 def flash_forward_varlen_bf16_dev(shape, q, k, v, seq_lens_dev, out, zero_padded_rows=True, n_kv_heads=0,
                                   stream=None):
     """Padded-batch causal prefill: per-sequence valid lengths (device int32[batch])."""

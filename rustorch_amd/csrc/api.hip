@@ -1197,6 +1197,70 @@ RT_API int rt_mha_forward_masked_bf16_dev(void* stream, const void* q, const voi
     return RT_OK;
 }
 
+// Causal attention with a sliding window on bf16 tensors, the mask itself never built: position i sees keys
+// (i - window, i].  bnhd: [batch, seq, heads, dim] tensors (MultiHeadAttention's), else [batch, heads, seq, dim].
+static int flash_window_bf16(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads, const void* q, const void* k,
+                             const void* v, uint64_t window, void* out, rt_err_detail* err, bool bnhd) {
+    clear_err(err);
+    if (!shape) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "shape is NULL");
+    if (shape->dim == 0) return fail(err, RT_ERR_ZERO_DIM, -1, 0, 0, "dim must be > 0");
+    if (window == 0) return fail(err, RT_ERR_UNSUPPORTED, -1, 1, 0, "window must be >= 1 (masks.rs:51)");
+    if (n_kv_heads == 0) n_kv_heads = shape->heads;
+    if (shape->seq == 0 || shape->batch == 0 || shape->heads == 0) return RT_OK;
+    int rc = check_flash_dims(shape, n_kv_heads, err);
+    if (rc) return rc;
+    if (shape->heads > 65535 || shape->batch > 65535 || (shape->seq + 127) / 128 > 65535)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, 0, "shape too large for the launch grid");
+    if (!q || !k || !v || !out) return fail(err, RT_ERR_NULL_POINTER, -1, 0, 0, "NULL buffer");
+    if (!rt::flash_tile_bf16_supported((int)shape->dim))
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 256, shape->dim,
+                    "the windowed kernel covers head dims up to 256 that are a multiple of 8 (others: the additive-mask entry)");
+    if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0)
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 16, 0, "bf16 kernels need 16-byte aligned tensors");
+    if (!rt::flash_tile_bf16_addressable((long long)shape->seq, (long long)((bnhd ? n_kv_heads : 1) * shape->dim)))
+        return fail(err, RT_ERR_UNSUPPORTED, -1, 0, shape->seq, "a K/V slab of one (batch, kv head) must stay below 4 GiB");
+    rc = ensure_device(err);
+    if (rc) return rc;
+    const int dim = (int)shape->dim;
+    rt::FlashTileParams t{};
+    t.q = (const uint16_t*)q;
+    t.k = (const uint16_t*)k;
+    t.v = (const uint16_t*)v;
+    t.out = (uint16_t*)out;
+    t.batch = (int)shape->batch;
+    t.heads = (int)shape->heads;
+    t.kv_heads = (int)n_kv_heads;
+    t.group = (int)(shape->heads / n_kv_heads);
+    t.pack = 1;
+    t.seq_q = t.seq_kv = (int)shape->seq;
+    t.dim = dim;
+    t.mask = rt::kMaskCausal;
+    t.ref_bc = 64;
+    t.scale = 1.0f / sqrtf((float)dim);
+    t.scale_log2e = t.scale * rt::kLog2eHost;
+    t.window = (int)(window > shape->seq ? shape->seq : window);  // a window of the whole sequence and more is the causal mask
+    if (bnhd) {
+        t.lq = t.lo = rt::layout_bnhd((long long)shape->heads, (long long)shape->seq, dim);
+        t.lkv = rt::layout_bnhd((long long)n_kv_heads, (long long)shape->seq, dim);
+    } else {
+        t.lq = t.lo = rt::layout_bhnd((long long)shape->heads, (long long)shape->seq, dim);
+        t.lkv = rt::layout_bhnd((long long)n_kv_heads, (long long)shape->seq, dim);
+    }
+    HIP_TRY(rt::launch_flash_tile_bf16((hipStream_t)stream, t), "flash_tile_bf16 (window) launch");
+    return RT_OK;
+}
+
+RT_API int rt_flash_forward_window_bf16_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads, const void* q,
+                                            const void* k, const void* v, uint64_t window, void* out, rt_err_detail* err) {
+    return flash_window_bf16(stream, shape, n_kv_heads, q, k, v, window, out, err, false);
+}
+
+RT_API int rt_flash_forward_window_bnhd_bf16_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,
+                                                 const void* q, const void* k, const void* v, uint64_t window, void* out,
+                                                 rt_err_detail* err) {
+    return flash_window_bf16(stream, shape, n_kv_heads, q, k, v, window, out, err, true);
+}
+
 RT_API int rt_flash_forward_varlen_bf16_dev(void* stream, const rt_attention_shape* shape, uint64_t n_kv_heads,
                                             const void* q, const void* k, const void* v, const int32_t* seq_lens,
                                             int zero_padded_rows, void* out, rt_err_detail* err) {

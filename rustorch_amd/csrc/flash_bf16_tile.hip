@@ -109,9 +109,16 @@ struct TileCfg {
 // (crates/rustorch-attention/src/online_softmax.rs:105-131 extended with o) -- the split over the context of the
 // decode kernels, for a chunk of new positions over one long cache, whose few query tiles would otherwise keep a
 // handful of CUs busy.
-template <int DP, int MODE, bool BIAS, bool PACKED, bool SPLIT = false>
+//
+// WIN (causal mask, rows of one head): a sliding window, query i sees keys (i + off - window, i + off] -- the
+// reference's sliding_window_mask (crates/rustorch-nn/src/masks.rs:41-60) without its [T, T] bias tensor.  The walk
+// starts at the tile that holds the first key the workgroup's first row sees (tensor base, key count and causal offset
+// moved by that many keys, as for a span of SPLIT), and an item that holds keys below some row's window is masked on
+// that side as well.
+template <int DP, int MODE, bool BIAS, bool PACKED, bool SPLIT = false, bool WIN = false>
 __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : TileCfg<DP>::OCC) void flash_tile_bf16_kernel(FlashTileParams p) {
     static_assert(!SPLIT || (PACKED && !BIAS && MODE == kMaskCausal), "the split over the keys serves the chunked decode");
+    static_assert(!WIN || (!PACKED && !BIAS && !SPLIT && MODE == kMaskCausal), "the window is a causal mask's");
     using Cfg = TileCfg<DP>;
     constexpr int KT = Cfg::KT, LDK = Cfg::LDK, LDV = Cfg::LDV, NI = Cfg::NI, TTHREADS = Cfg::THREADS;
     constexpr int KS = DP / 16;        // contraction steps of the score product
@@ -187,7 +194,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     // once the length is known, those of K are masked in the score tile whatever they hold.  (A span of the keys
     // starts where the sequence's own length puts it: its requests wait for the lengths.)
     const uint32_t tile_bytes_g = (uint32_t)KT * kv_pitch * 2u;  // from a tile's first row to the next tile's, in memory
-    if (!SPLIT) {
+    if (!SPLIT && !WIN) {
         const uint32_t all_bytes = p.seq_kv > 0 ? ((uint32_t)(p.seq_kv - 1) * kv_pitch + (uint32_t)D) * 2u : 0u;
         const __amdgpu_buffer_rsrc_t Kall = __builtin_amdgcn_make_buffer_rsrc((void*)Kg, 0, all_bytes, kBufferFlags);
         const __amdgpu_buffer_rsrc_t Vall = __builtin_amdgcn_make_buffer_rsrc((void*)Vg, 0, all_bytes, kBufferFlags);
@@ -244,6 +251,16 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         Kg += (size_t)key0 * (size_t)p.lkv.row_pitch;
         Vg += (size_t)key0 * (size_t)p.lkv.row_pitch;
     }
+    if (WIN) {
+        // the first key any row of the workgroup sees, rounded down to a tile: the walk starts there
+        const int key0 = (max(q0 + off - p.window + 1, 0) / KT) * KT;
+        n_tiles = max(n_tiles - key0 / KT, 0);
+        kv_end -= key0;
+        n_keys -= key0;
+        off -= key0;
+        Kg += (size_t)key0 * (size_t)p.lkv.row_pitch;
+        Vg += (size_t)key0 * (size_t)p.lkv.row_pitch;
+    }
     // A tile of padded query rows only (a padded batch has many: every tile behind a sequence's last row) has nothing
     // to load or walk: its rows get the fill value and the workgroup is done.
     if (!SPLIT && !PACKED && q0 >= n_q) {
@@ -264,7 +281,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     const uint32_t slab_bytes = n_keys > 0 ? ((uint32_t)(n_keys - 1) * kv_pitch + (uint32_t)D) * 2u : 0u;
     const __amdgpu_buffer_rsrc_t Kbuf = __builtin_amdgcn_make_buffer_rsrc((void*)Kg, 0, slab_bytes, kBufferFlags);
     const __amdgpu_buffer_rsrc_t Vbuf = __builtin_amdgcn_make_buffer_rsrc((void*)Vg, 0, slab_bytes, kBufferFlags);
-    if (SPLIT) {  // tile 0 (K and V) and K of tile 1 of the span
+    if (SPLIT || WIN) {  // tile 0 (K and V) and K of tile 1 of the span / of the window
 #pragma unroll
         for (int n = 0; n < NL; n++) {
             kreg[0][n] = __builtin_amdgcn_raw_buffer_load_b128(Kbuf, ld_off[n], 0, 0);
@@ -357,6 +374,9 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         }
         // items this wave walks: the ones that hold a key some row of it sees (a prefix of the workgroup's items)
         const int n_it = wave_lim_max < 0 ? 0 : min(n_tiles * NI, (wave_lim_max >> 5) + 1);
+        // a window: the first key this row sees, and the largest such key over the wave's rows (its last valid row's)
+        const int lo = WIN ? max(lim - p.window + 1, 0) : 0;
+        const int wave_lo_max = WIN ? max(wave_lim_max - p.window + 1, 0) : 0;
 
         // (the query row is read without a test: a row past the tensor reads the tensor's last row)
         const int r_q = min(r, rows_total - 1);
@@ -451,6 +471,11 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
                 const int room = lim - k0 - 4 * hh;
 #pragma unroll
                 for (int i = 0; i < 16; i++) sc[i] = (8 * (i >> 2) + (i & 3) > room) ? neg_inf() : sc[i];
+            }
+            if (WIN && k0 < wave_lo_max) {
+                const int room_lo = lo - k0 - 4 * hh;  // key k0 + 8 (i / 4) + 4 hh + i % 4 lies before the window when below lo
+#pragma unroll
+                for (int i = 0; i < 16; i++) sc[i] = (8 * (i >> 2) + (i & 3) < room_lo) ? neg_inf() : sc[i];
             }
             if (MODE == kMaskPadding) {
                 const uint32_t keep_word = (uint32_t)(keep_cur >> (32 * it));
@@ -1419,9 +1444,9 @@ __global__ __launch_bounds__(256, 2) void flash_wide_bf16_kernel(FlashTileParams
     }
 }
 
-template <int DP, int MODE, bool BIAS, bool PACKED, bool SPLIT = false>
+template <int DP, int MODE, bool BIAS, bool PACKED, bool SPLIT = false, bool WIN = false>
 hipError_t launch_one(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
-    hipLaunchKernelGGL((flash_tile_bf16_kernel<DP, MODE, BIAS, PACKED, SPLIT>), grid, dim3(TileCfg<DP>::THREADS), 0, stream, p);
+    hipLaunchKernelGGL((flash_tile_bf16_kernel<DP, MODE, BIAS, PACKED, SPLIT, WIN>), grid, dim3(TileCfg<DP>::THREADS), 0, stream, p);
     return hipGetLastError();
 }
 
@@ -1435,6 +1460,7 @@ hipError_t launch_dp(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
         return hipGetLastError();
     }
     if (p.pack > 1) return launch_one<DP, kMaskCausal, false, true>(stream, p, grid);
+    if (p.window > 0) return launch_one<DP, kMaskCausal, false, false, false, true>(stream, p, grid);
     if (p.bias) return launch_one<DP, kMaskNone, true, false>(stream, p, grid);
     switch (p.mask) {
         case kMaskNone: return launch_one<DP, kMaskNone, false, false>(stream, p, grid);
@@ -1481,6 +1507,7 @@ hipError_t launch_flash_tile_bf16(hipStream_t stream, const FlashTileParams& par
     if (p.bias && p.mask != kMaskNone) return hipErrorInvalidValue;
     if (!flash_tile_bf16_addressable(p.seq_kv, p.lkv.row_pitch)) return hipErrorInvalidValue;
     if (p.pack > 1 && (p.bias || p.mask != kMaskCausal)) return hipErrorInvalidValue;  // packed rows: the chunked decode only
+    if (p.window < 0 || (p.window > 0 && (p.pack > 1 || p.bias || p.mask != kMaskCausal || p.n_splits > 1))) return hipErrorInvalidValue;
     const long long rows = (long long)p.seq_q * p.pack;
     const long long n_qtiles = (rows + TROWS - 1) / TROWS;
     const long long heads_u = p.pack > 1 ? p.kv_heads : p.heads;

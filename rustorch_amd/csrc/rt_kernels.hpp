@@ -126,6 +126,9 @@ struct FlashTileParams {
     int n_splits;
     float* part_o;
     float* part_ml;
+    // Sliding window (causal mask only, unpacked rows, no bias; 0 = none): position i sees the `window` keys that end
+    // with key i + (keys - valid queries), as sliding_window_mask builds it (crates/rustorch-nn/src/masks.rs:41-60).
+    int window;
 };
 bool flash_tile_bf16_supported(int dim);
 // keys per LDS tile of the tile kernel at head dim `dim` (the unit the split over the keys is cut in)

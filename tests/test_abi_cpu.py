@@ -210,6 +210,24 @@ def test_shutdown_without_a_device_is_a_no_op():
     ra.shutdown()
 
 
+def test_window_entries_argument_errors_before_any_device_use():
+    lib = L.lib()
+    err = L.RtErr()
+    import ctypes as C
+    p = 0x1000
+    s = ra.AttentionShape.new(1, 2, 16, 64)._c()
+    for fn in (lib.rt_flash_forward_window_bf16_dev, lib.rt_flash_forward_window_bnhd_bf16_dev):
+        assert fn(None, C.byref(s), 0, p, p, p, 0, p, C.byref(err)) == L.RT_ERR_UNSUPPORTED and err.expected == 1
+        assert fn(None, C.byref(s), 3, p, p, p, 4, p, C.byref(err)) == L.RT_ERR_HEAD_COUNT_MISMATCH
+        assert fn(None, C.byref(s), 0, None, p, p, 4, p, C.byref(err)) == L.RT_ERR_NULL_POINTER
+        assert fn(None, C.byref(s), 0, p + 2, p, p, 4, p, C.byref(err)) == L.RT_ERR_UNSUPPORTED
+        s20 = ra.AttentionShape.new(1, 2, 16, 20)._c()
+        assert fn(None, C.byref(s20), 0, p, p, p, 4, p, C.byref(err)) == L.RT_ERR_UNSUPPORTED
+        s0 = ra.AttentionShape.new(1, 2, 16, 0)._c()
+        assert fn(None, C.byref(s0), 0, p, p, p, 4, p, C.byref(err)) == L.RT_ERR_ZERO_DIM
+        assert fn(None, C.byref(s), 0, p, p, p, 4, p, C.byref(err)) in (L.RT_ERR_NO_DEVICE, L.RT_OK)
+
+
 def test_process_wide_switches_need_no_device():
     lib = L.lib()
     assert lib.rt_set_strict_non_finite_v(1) == 0 and lib.rt_set_strict_non_finite_v(0) == 1
