@@ -323,7 +323,7 @@ def main():
                                         "(seed 64), f32 accumulation",
                             "flop_convention": "4*B*H*D*N*(N+1)/2 (causal-counted)"}}
 
-    # ------------------------------------------------------------------ shapes no BASELINE config names: timed for the record
+    # ------------------------------------------------------------------ shapes outside the five configurations the metric is quoted on: timed for the record
     shapes = None
     if args.only in (None, "shapes"):
         shapes = {}
