@@ -74,19 +74,21 @@ __global__ __launch_bounds__(64) void decode_prepare_kernel(DecodePrepareParams 
 
 // The same arithmetic for a prompt.  With many consecutive tokens per head the one-wave kernel above is bound by its
 // own redundancy (all 64 lanes of a wave take the same sum of squares, and a row is moved two bytes per lane): 308 us
-// for B=4, 32 + 8 heads, 4096 tokens, D=128 (1.3 TB/s; 80 us = 5.1 TB/s here).  A workgroup takes ROWS consecutive tokens of one
+// for B=4, 32 + 8 heads, 4096 tokens, D=128 (1.3 TB/s; 84 us = 4.8 TB/s here, 70 us when the cache rows are contiguous).  A workgroup takes ROWS consecutive tokens of one
 // (sequence, head) -- contiguous rows in q / k_in and in the cache -- through LDS: the rows arrive with 16-byte loads,
 // every thread takes the sum of squares of ONE row in index order (the reference's order, model.rs:862-885), and
 // the normalised, rotated rows leave with 16-byte stores.  Rows sit in LDS as bf16 with a pitch of D + 2 elements (an odd
 // number of 32-bit words: the 64 lanes that walk 64 rows in step hit 64 different banks).  D a multiple of 16, at most
-// DMAX; every pointer 16-byte aligned.
+// DMAX; every pointer 16-byte aligned.  Grid (token blocks, heads, batch), token blocks fastest: workgroups go round-robin
+// to the 8 XCDs in that order, so all heads of a token block run on one XCD and its cos / sin rows are fetched into one
+// L2, once (with the heads fastest every XCD fetched every table row: 76 MB more on the prompt above).
 template <int ROWS, int DMAX>
 __global__ __launch_bounds__(256) void prompt_prepare_kernel(DecodePrepareParams p) {
     __shared__ uint32_t rows_w[ROWS * (DMAX + 2) / 2];
     __shared__ float inv[ROWS];
     const int tid = threadIdx.x;
-    const int h = blockIdx.x, b = blockIdx.z;
-    const int sq0 = (int)blockIdx.y * ROWS;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int sq0 = (int)blockIdx.x * ROWS;
     const int D = p.head_dim, half = D / 2, S = p.seq;
     const int pitch_w = (D + 2) / 2;  // words per row in LDS
     const int CH = D / 8;             // 16-byte chunks per row
@@ -187,9 +189,9 @@ hipError_t launch_decode_prepare(hipStream_t stream, const DecodePrepareParams& 
                          aligned16(p.sin_table) && aligned16(p.q_gamma) && aligned16(p.k_gamma) && p.n_heads + p.n_kv <= 65535;
     if (wide_ok) {
         if (p.head_dim <= 128) {
-            hipLaunchKernelGGL((prompt_prepare_kernel<64, 128>), dim3(p.n_heads + p.n_kv, (p.seq + 63) / 64, p.batch), dim3(256), 0, stream, p);
+            hipLaunchKernelGGL((prompt_prepare_kernel<64, 128>), dim3((p.seq + 63) / 64, p.n_heads + p.n_kv, p.batch), dim3(256), 0, stream, p);
         } else {
-            hipLaunchKernelGGL((prompt_prepare_kernel<64, 256>), dim3(p.n_heads + p.n_kv, (p.seq + 63) / 64, p.batch), dim3(256), 0, stream, p);
+            hipLaunchKernelGGL((prompt_prepare_kernel<64, 256>), dim3((p.seq + 63) / 64, p.n_heads + p.n_kv, p.batch), dim3(256), 0, stream, p);
         }
         return hipGetLastError();
     }
