@@ -316,8 +316,16 @@ def main():
     d64_p = None
     if args.only in (None, "d64"):
         Bd, Hd, Nd, Dd = 4, 32, 4096, 64
-        d64_p = causal_prefill(Bd, Hd, Nd, Dd, 64, 1.0, 32, "flash_wide_bf16_kernel<causal>",
-                               profile_traffic("flash_wide_bf16_b4_h32_n4096_d64.md", "flash_wide_bf16_kernel<causal>"))
+        # (the library takes the tile kernel here; RT_ATTN_BF16_PREFILL=wide|persistent in the environment forces another,
+        # which the leg then names)
+        d64_kernel, d64_traffic = {
+            "wide": ("flash_wide_bf16_kernel<causal>",
+                     profile_traffic("flash_wide_bf16_b4_h32_n4096_d64.md", "flash_wide_bf16_kernel<causal>")),
+            "persistent": ("flash_fwd_bf16_kernel<64, causal>", None),
+        }.get(os.environ.get("RT_ATTN_BF16_PREFILL", ""),
+              ("flash_tile_bf16_kernel<64, causal, direct>",
+               profile_traffic("flash_tile_bf16_b4_h32_n4096_d64.md", "flash_tile_bf16_kernel<64,causal,direct>")))
+        d64_p = causal_prefill(Bd, Hd, Nd, Dd, 64, 1.0, 32, d64_kernel, d64_traffic)
         d64_p = {"metric": "prefill attn TFLOP/s", "value": d64_p.pop("tflops"), "unit": "TFLOP/s", **d64_p,
                  "config": {"workload": "bf16 causal prefill at head dim 64, B=4 H=32 N=4096 D=64, N(0,1) inputs "
                                         "(seed 64), f32 accumulation",
@@ -379,7 +387,7 @@ def main():
         leg_w = {"value": ach_w, "unit": "TFLOP/s", "us_per_call": tw.mean_ms * 1e3, **spread(tw.per), **tw.settle(),
                  "roofline": {"bound": "mfma", "achieved": ach_w, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                               "frac": ach_w / PEAK_BF16_TFLOPS, "traffic": None,
-                              "kernel": "flash_tile_bf16_kernel<64, causal, window>"},
+                              "kernel": "flash_tile_bf16_kernel<64, causal, window, direct>"},
                  "config": {"workload": "bf16 causal sliding-window self-attention, B=4 T=4096 H=16 hd=64 on [B,T,H*hd] tensors, "
                                         "window 256, rt_flash_forward_window_bnhd_bf16_dev (no mask tensor)",
                             "flop_convention": "4*B*H*hd*(visible pairs): sum over i of min(i + 1, window)"}}
@@ -427,7 +435,7 @@ def main():
                                "frac": achieved / PEAK_BF16_TFLOPS,
                                "traffic": profile_traffic("flash_tile_bf16_varlen_b16_h16_n1024_d64.md",
                                                           "flash_tile_bf16_kernel<64,causal>"),
-                               "kernel": "flash_tile_bf16_kernel<64, causal> (per-sequence lengths)",
+                               "kernel": "flash_tile_bf16_kernel<64, causal, direct> (per-sequence lengths)",
                                "kernel_ms_mean": tm.mean_ms}}
         if not args.no_cpu:
             # the oracle of a sequence is the reference's causal forward on the problem truncated to its length

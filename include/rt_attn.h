@@ -192,12 +192,12 @@ int rt_flash_forward_f32_dev(void *stream, const rt_attention_shape *shape, uint
 /* The bf16 counterpart (bf16 in, f32 accumulate, bf16 out rounded once, to nearest even):
  * q/out [batch,heads,seq,dim], k/v [batch,n_kv_heads,seq,dim].  Any dim up to 512 (the reference's forward takes
  * any dim != 0, cpu_forward.rs:142-169; above 512: RT_ERR_UNSUPPORTED with expected = 512).  Three MFMA kernels serve
- * dims up to 256 that are a multiple of 8 on 16-byte aligned tensors: a persistent 8-wave kernel for dim 64 / 128 on
- * unpadded batches of at least 512 rows per sequence and one job of 256 rows per compute unit, a 4-wave tile
- * kernel for everything else (short or few sequences, padded batches, other dims), and a form of the tile kernel
- * with 64 query rows per wave for dim 64 on unpadded sequences of at least 2048 rows with four 256-row jobs per
- * compute unit;
- * rt_debug_force_bf16_prefill_kernel forces one of them where both apply.  The remaining dims and alignments run on
+ * dims up to 256 that are a multiple of 8 on 16-byte aligned tensors: a persistent 8-wave kernel for dim 128 (and
+ * dim 64 under a key-padding mask) on unpadded batches of at least 512 rows per sequence and one job of 256 rows
+ * per compute unit, a 4-wave tile kernel for everything else (dim 64 with no mask or the causal one, short or few
+ * sequences, padded batches, other dims), and a form of the tile kernel with 64 query rows per wave for dim 64, which
+ * runs only when it is asked for;
+ * rt_debug_force_bf16_prefill_kernel forces one of them where it applies.  The remaining dims and alignments run on
  * a one-workgroup-per-row kernel with the same masks and row rules (correct at any speed, not tuned). */
 int rt_flash_forward_bf16_dev(void *stream, const rt_attention_shape *shape, uint64_t n_kv_heads, const void *q,
                               const void *k, const void *v, int mask_kind, const uint8_t *keep, void *out,

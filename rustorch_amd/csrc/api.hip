@@ -778,10 +778,10 @@ RT_API int rt_flash_forward_f32_dev(void* stream, const rt_attention_shape* shap
     return flash_f32_device((hipStream_t)stream, shape, n_kv_heads, q, k, v, mask_kind, keep, out, err);
 }
 
-// Which bf16 prefill kernel serves a call.  RT_ATTN_BF16_PREFILL=tile|persistent in the environment forces one
-// where both apply (for measurements and tests); otherwise the persistent 8-wave kernel takes head dims 64 and 128
-// on unpadded batches with at least 512 rows per sequence and a job for every CU, and the 4-wave tile kernel
-// everything else.
+// Which bf16 prefill kernel serves a call.  RT_ATTN_BF16_PREFILL=tile|persistent|wide in the environment forces one
+// where it applies (for measurements and tests); otherwise the persistent 8-wave kernel takes head dim 128 (and head
+// dim 64 under a key-padding mask) on unpadded batches with at least 512 rows per sequence and a job for every CU,
+// and the 4-wave tile kernel everything else.
 enum class PrefillKernel { kAuto, kTile, kPersistent, kWide };
 // A debug switch for measurements and tests, not part of the reference's surface: rt_debug_force_bf16_prefill_kernel
 // sets it; until that is called, the value is what RT_ATTN_BF16_PREFILL=tile|persistent held when the library made its
@@ -872,11 +872,10 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
     bool persistent = persistent_dim && shape->seq >= 512 && jobs256 >= (uint64_t)g_num_cus && mask != rt::kMaskVarlenCausal;
     const PrefillKernel forced = prefill_kernel_override();
     if (forced == PrefillKernel::kTile || forced == PrefillKernel::kWide) persistent = false;
-    // head dim 64 on long, unpadded sequences with work for every CU several times over: 64 query rows per wave
-    // (256-row workgroups, two per CU), measured 5-6 % ahead of both other kernels there and behind them on less work
-    const bool wide_auto = forced == PrefillKernel::kAuto && shape->dim == 64 && (mask == rt::kMaskNone || mask == rt::kMaskCausal) &&
-                           shape->seq >= 2048 && jobs256 >= 4ull * (uint64_t)g_num_cus;
-    if (wide_auto) persistent = false;
+    // head dim 64 exactly, no mask or the causal one: the tile kernel (whose K/V tiles go straight from memory to LDS
+    // at this head dim) measured ahead of the persistent kernel on every shape tried (N = 1024 .. 32768, 4-9 %) and
+    // level with the kernel of 64 query rows per wave, which therefore runs only when it is asked for
+    if (forced == PrefillKernel::kAuto && shape->dim == 64 && (mask == rt::kMaskNone || mask == rt::kMaskCausal)) persistent = false;
     if (forced == PrefillKernel::kPersistent && persistent_dim) persistent = true;
     if (mask == rt::kMaskPadding && shape->seq > (uint64_t)rt::kFlashBf16MaxPaddingKeys) persistent = false;
     if (persistent) {  // that kernel addresses the rows of one (batch, head) slab with 32-bit byte offsets
@@ -918,7 +917,7 @@ static int flash_bf16_common(void* stream, const rt_attention_shape* shape, uint
         t.scale_log2e = scale * rt::kLog2eHost;
         t.lq = t.lo = lq;
         t.lkv = lkv;
-        if ((forced == PrefillKernel::kWide || wide_auto) && rt::flash_wide_bf16_supported(t)) {
+        if (forced == PrefillKernel::kWide && rt::flash_wide_bf16_supported(t)) {
             HIP_TRY(rt::launch_flash_wide_bf16((hipStream_t)stream, t), "flash_wide_bf16 launch");
             return strict_pass((hipStream_t)stream, shape, n_kv_heads, v, out, seq_lens, mask, bnhd, true, err);
         }

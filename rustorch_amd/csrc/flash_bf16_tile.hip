@@ -86,7 +86,31 @@ struct TileCfg {
     static constexpr int TILE_BYTES = 2 * KT * (LDK + LDV) * 2;           // two stages of K and V
     static constexpr int REGION = 32 * LDK * 2;                           // a wave's staged output rows
     static constexpr int LDS_BYTES = TILE_BYTES > 4 * REGION ? TILE_BYTES : 4 * REGION;
+    // DIRECT: unpadded tiles (rows of DP * 2 bytes, 16-byte slots swizzled), filled by loads that go straight to LDS
+    static constexpr int STAGE_BYTES = KT * DP * 2;
+    static constexpr int LDS_BYTES_DIRECT = 4 * STAGE_BYTES > 4 * REGION ? 4 * STAGE_BYTES : 4 * REGION;
+    static constexpr int OCC_DIRECT = 3;
 };
+
+// 16 bytes per lane from a buffer straight into LDS: lane l lands at LDS byte address lds_block + 16 l (lds_block is
+// wave-uniform and goes through M0); a lane whose offset lies past the end of the descriptor lands zeros.  Issued as
+// inline assembly so that the compiler's counter bookkeeping does not make every later LDS read wait for it:
+// completion is awaited explicitly (s_waitcnt vmcnt(0) before the barrier that publishes the tile).  Loads the
+// compiler does not know of can only make its own vmcnt waits longer, never shorter: the counter retires in order.
+__device__ __forceinline__ void t_buffer_to_lds(const u32x4_t& rsrc, uint32_t lane_off, uint32_t tile_off, uint32_t lds_block) {
+    const uint32_t m = __builtin_amdgcn_readfirstlane(lds_block);
+    const uint32_t so = __builtin_amdgcn_readfirstlane(tile_off);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(m), "v"(lane_off), "s"(rsrc), "s"(so)
+                 : "memory");
+}
+// a raw buffer descriptor as four scalars: base, no stride, `bytes` addressable
+__device__ __forceinline__ u32x4_t t_make_rsrc(const void* base, uint32_t bytes) {
+    const uint64_t a = (uint64_t)(uintptr_t)base;
+    return u32x4_t{(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)a), (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu),
+                   (uint32_t)__builtin_amdgcn_readfirstlane(bytes), kBufferFlags};
+}
 
 // MODE: kMaskNone, kMaskCausal, kMaskPadding.  BIAS: an additive f32 score bias is applied (then MODE is kMaskNone).
 // PACKED: query rows run over (position, head of the GQA group) (then MODE is kMaskCausal and there is no bias).
@@ -115,10 +139,20 @@ struct TileCfg {
 // starts at the tile that holds the first key the workgroup's first row sees (tensor base, key count and causal offset
 // moved by that many keys, as for a span of SPLIT), and an item that holds keys below some row's window is masked on
 // that side as well.
-template <int DP, int MODE, bool BIAS, bool PACKED, bool SPLIT = false, bool WIN = false>
-__global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : TileCfg<DP>::OCC) void flash_tile_bf16_kernel(FlashTileParams p) {
+//
+// DIRECT (head dim 64 exactly, no bias, no key-padding vector): the tiles travel from memory straight into LDS
+// (buffer_load_dwordx4 ... lds) instead of through registers and LDS writes.  After a tile's barrier the waves request
+// K(t+2) and V(t+1) into the stages K(t) and V(t-1) have just left and wait for their own requests ahead of the next
+// tile's barrier.  LDS rows are unpadded (a landing block of 1 KB is contiguous) and their 16-byte slots are XORed
+// with bits of the row, as in flash_bf16.hip.  Same instructions on the same operands otherwise: the same bits.
+// Measured against the register path, interleaved in one process: 3-5 % on short or padded sequences (B=16 H=16
+// N=1024: 52.3 -> 49.3 us), 7-9 % on long ones (B=4 H=32 N=4096: 306 -> 283 us); three stages per matrix or four
+// workgroups per CU are no faster.
+template <int DP, int MODE, bool BIAS, bool PACKED, bool SPLIT = false, bool WIN = false, bool DIRECT = false>
+__global__ __launch_bounds__(TileCfg<DP>::THREADS, DIRECT ? TileCfg<DP>::OCC_DIRECT : ((BIAS && DP == 64) ? 2 : TileCfg<DP>::OCC)) void flash_tile_bf16_kernel(FlashTileParams p) {
     static_assert(!SPLIT || (PACKED && !BIAS && MODE == kMaskCausal), "the split over the keys serves the chunked decode");
     static_assert(!WIN || (!PACKED && !BIAS && !SPLIT && MODE == kMaskCausal), "the window is a causal mask's");
+    static_assert(!DIRECT || (DP == 64 && !BIAS && MODE != kMaskPadding), "tiles straight into LDS: head dim 64 exactly");
     using Cfg = TileCfg<DP>;
     constexpr int KT = Cfg::KT, LDK = Cfg::LDK, LDV = Cfg::LDV, NI = Cfg::NI, TTHREADS = Cfg::THREADS;
     constexpr int KS = DP / 16;        // contraction steps of the score product
@@ -135,9 +169,11 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     // item runs its three phases one after the other, and K is parked with V.
     constexpr bool PIPE = DP <= 128 && !((BIAS || MODE == kMaskPadding) && DP == 128);
 
-    __shared__ __attribute__((aligned(16))) unsigned char lds[Cfg::LDS_BYTES];
+    __shared__ alignas(DIRECT ? 1024 : 16) unsigned char lds[DIRECT ? Cfg::LDS_BYTES_DIRECT : Cfg::LDS_BYTES];
     uint16_t* const Ks = (uint16_t*)lds;                      // [2][KT * LDK]
     uint16_t* const Vs = (uint16_t*)lds + 2 * KT * LDK;       // [2][KT * LDV]
+    // DIRECT: [K stage 0][K stage 1][V stage 0][V stage 1], rows of ROWB bytes without padding
+    constexpr int ROWB = DP * 2, STAGE_B = Cfg::STAGE_BYTES;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -189,6 +225,22 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         ld_off[n] = ((uint32_t)row * kv_pitch + (ld_on[n] ? (uint32_t)(8 * ch) : 0u)) * 2u;
     }
     u32x4_t k1[NL];
+    // DIRECT: a wave's load instruction fills 1 KB of LDS (8 rows), lane l the 16 bytes at 16 l; instruction n of
+    // wave w fills block w + 4 n of a stage.  Bank conflicts are avoided by an XOR of the 16-byte slot index with bits
+    // of the row (K rows are read 16 at a time at one slot, V rows 4 at a time over 4 adjacent slots by the
+    // transposing reads), applied on the way in: the lane fetches the slot that belongs at its LDS position.
+    auto swz_k = [](int r) __attribute__((always_inline)) { return (r >> 1) & 7; };
+    auto swz_v = [](int r) __attribute__((always_inline)) { return 4 * ((r >> 1) & 1); };
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    const int dl_row = 8 * wave + (lane >> 3);  // row of the lane's chunk in instruction 0; instruction n: + 32 n (the swizzles do not see n)
+    const uint32_t dl_k = (uint32_t)dl_row * kv_pitch * 2u + (uint32_t)(((lane & 7) ^ swz_k(dl_row)) * 16);
+    const uint32_t dl_v = (uint32_t)dl_row * kv_pitch * 2u + (uint32_t)(((lane & 7) ^ swz_v(dl_row)) * 16);
+    // the tile whose first row lies tile_off bytes into the descriptor -> the stage at stage_off
+    auto dl_tile = [&](const u32x4_t& rs, uint32_t lane_off, uint32_t tile_off, uint32_t stage_off) __attribute__((always_inline)) {
+#pragma unroll
+        for (int n = 0; n < 2; n++)
+            t_buffer_to_lds(rs, lane_off, tile_off + (uint32_t)(32 * n) * kv_pitch * 2u, lds_base + stage_off + (uint32_t)((wave + 4 * n) * 1024));
+    };
     // Tile 0 (K and V) and K of tile 1 are requested before the sequence lengths have arrived (a dependent load
     // away), through descriptors that end with the tensor's last row: the rows of V(0) past the last key are zeroed
     // once the length is known, those of K are masked in the score tile whatever they hold.  (A span of the keys
@@ -196,13 +248,20 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     const uint32_t tile_bytes_g = (uint32_t)KT * kv_pitch * 2u;  // from a tile's first row to the next tile's, in memory
     if (!SPLIT && !WIN) {
         const uint32_t all_bytes = p.seq_kv > 0 ? ((uint32_t)(p.seq_kv - 1) * kv_pitch + (uint32_t)D) * 2u : 0u;
-        const __amdgpu_buffer_rsrc_t Kall = __builtin_amdgcn_make_buffer_rsrc((void*)Kg, 0, all_bytes, kBufferFlags);
-        const __amdgpu_buffer_rsrc_t Vall = __builtin_amdgcn_make_buffer_rsrc((void*)Vg, 0, all_bytes, kBufferFlags);
+        if constexpr (DIRECT) {
+            const u32x4_t Kall = t_make_rsrc(Kg, all_bytes), Vall = t_make_rsrc(Vg, all_bytes);
+            dl_tile(Kall, dl_k, 0u, 0u);
+            dl_tile(Vall, dl_v, 0u, 2u * STAGE_B);
+            dl_tile(Kall, dl_k, tile_bytes_g, STAGE_B);
+        } else {
+            const __amdgpu_buffer_rsrc_t Kall = __builtin_amdgcn_make_buffer_rsrc((void*)Kg, 0, all_bytes, kBufferFlags);
+            const __amdgpu_buffer_rsrc_t Vall = __builtin_amdgcn_make_buffer_rsrc((void*)Vg, 0, all_bytes, kBufferFlags);
 #pragma unroll
-        for (int n = 0; n < NL; n++) {
-            kreg[0][n] = __builtin_amdgcn_raw_buffer_load_b128(Kall, ld_off[n], 0, 0);
-            vreg[0][n] = __builtin_amdgcn_raw_buffer_load_b128(Vall, ld_off[n], 0, 0);
-            k1[n] = PIPE ? __builtin_amdgcn_raw_buffer_load_b128(Kall, ld_off[n], tile_bytes_g, 0) : u32x4_t{0u, 0u, 0u, 0u};
+            for (int n = 0; n < NL; n++) {
+                kreg[0][n] = __builtin_amdgcn_raw_buffer_load_b128(Kall, ld_off[n], 0, 0);
+                vreg[0][n] = __builtin_amdgcn_raw_buffer_load_b128(Vall, ld_off[n], 0, 0);
+                k1[n] = PIPE ? __builtin_amdgcn_raw_buffer_load_b128(Kall, ld_off[n], tile_bytes_g, 0) : u32x4_t{0u, 0u, 0u, 0u};
+            }
         }
     }
 
@@ -271,6 +330,8 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             const int row = c / CH, ch = c - row * CH;
             if (q0 + row < rows_total && 8 * ch < D) *(u32x4_t*)(ob + (size_t)(q0 + row) * p.lo.row_pitch + 8 * ch) = val;
         }
+        // (the early requests land in this workgroup's LDS: not to be left in flight when it is handed on)
+        if constexpr (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         return;
     }
     // K and V are read through buffer descriptors that end with the last key's row: a request for a row behind it
@@ -281,18 +342,24 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
     const uint32_t slab_bytes = n_keys > 0 ? ((uint32_t)(n_keys - 1) * kv_pitch + (uint32_t)D) * 2u : 0u;
     const __amdgpu_buffer_rsrc_t Kbuf = __builtin_amdgcn_make_buffer_rsrc((void*)Kg, 0, slab_bytes, kBufferFlags);
     const __amdgpu_buffer_rsrc_t Vbuf = __builtin_amdgcn_make_buffer_rsrc((void*)Vg, 0, slab_bytes, kBufferFlags);
-    if (SPLIT || WIN) {  // tile 0 (K and V) and K of tile 1 of the span / of the window
+    const u32x4_t Kd = t_make_rsrc(Kg, slab_bytes), Vd = t_make_rsrc(Vg, slab_bytes);  // (DIRECT: the same descriptors as scalars)
+    if (DIRECT && (SPLIT || WIN)) {
+        dl_tile(Kd, dl_k, 0u, 0u);
+        dl_tile(Vd, dl_v, 0u, 2u * STAGE_B);
+        dl_tile(Kd, dl_k, tile_bytes_g, STAGE_B);
+    } else if (SPLIT || WIN) {  // tile 0 (K and V) and K of tile 1 of the span / of the window
 #pragma unroll
         for (int n = 0; n < NL; n++) {
             kreg[0][n] = __builtin_amdgcn_raw_buffer_load_b128(Kbuf, ld_off[n], 0, 0);
             vreg[0][n] = __builtin_amdgcn_raw_buffer_load_b128(Vbuf, ld_off[n], 0, 0);
             k1[n] = PIPE ? __builtin_amdgcn_raw_buffer_load_b128(Kbuf, ld_off[n], tile_bytes_g, 0) : u32x4_t{0u, 0u, 0u, 0u};
         }
-    } else if (n_keys < KT) {  // the early requests ended with the tensor, not with the sequence
+    } else if (!DIRECT && n_keys < KT) {  // the early requests ended with the tensor, not with the sequence
 #pragma unroll
         for (int n = 0; n < NL; n++)
             if ((tid + TTHREADS * n) / CH >= n_keys) vreg[0][n] = u32x4_t{0u, 0u, 0u, 0u};
     }
+
     if (MODE == kMaskPadding && n_keys > 0) {  // keep bytes past the last key count as kept: `lim` masks those keys
         const int j = lane & (KT - 1);
         const uint32_t kb = p.keep[min(j, n_keys - 1)];
@@ -315,7 +382,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         // head dim reads column 0 -- and only the LDS write is predicated.  With no branch around a load the compiler
         // counts the loads in flight exactly and waits at a park for the oldest register set only; with one it
         // falls back to waiting for all of them, which empties the prefetch queue at every tile.
-        if (D < DP) {  // the columns that are never parked are zero in both stages
+        if (!DIRECT && D < DP) {  // the columns that are never parked are zero in both stages
             for (int i = tid; i < Cfg::TILE_BYTES / 16; i += TTHREADS) ((u32x4_t*)lds)[i] = u32x4_t{0u, 0u, 0u, 0u};
             __syncthreads();
         }
@@ -414,6 +481,25 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         // per-lane LDS offsets (elements): K operand row `col`, slots 8 hh; V operand row (j >> 2) + 4 hh, columns 16 g16 + 4 (j & 3)
         const int k_off = col * LDK + 8 * hh;
         const int v_off = (((lane & 15) >> 2) + 4 * hh) * LDV + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+        // DIRECT (byte offsets): the same operand rows and columns in the swizzled layout.  The swizzles only permute
+        // address bits that the operand index also occupies, so operand ks sits at k_base ^ 32 ks, operand dt at
+        // v_base ^ 64 dt.
+        uint32_t k_base = 0, v_base = 0;
+        if constexpr (DIRECT) {
+            const int j = lane & 15, g16 = (lane >> 4) & 1, vrow = (j >> 2) + 4 * hh, low = 2 * g16 + ((j & 3) >> 1);
+            k_base = (uint32_t)(col * ROWB + ((hh ^ swz_k(col)) * 16));
+            v_base = (uint32_t)(2 * STAGE_B + vrow * ROWB + ((low ^ swz_v(vrow)) * 16) + 8 * (j & 1));
+        }
+        // where the operands of item `item` of stage `st` start: with the lane's own offset (padded layout), or without
+        // it (DIRECT: load_op adds the lane's swizzled offset)
+        auto k_at = [&](int st, int item) __attribute__((always_inline)) -> const uint16_t* {
+            if constexpr (DIRECT) return (const uint16_t*)(lds + st * STAGE_B + item * 32 * ROWB);
+            else return Ks + st * KT * LDK + item * 32 * LDK + k_off;
+        };
+        auto v_at = [&](int st, int item) __attribute__((always_inline)) -> const uint16_t* {
+            if constexpr (DIRECT) return (const uint16_t*)(lds + st * STAGE_B + item * 32 * ROWB);
+            else return Vs + st * KT * LDV + item * 32 * LDV + v_off;
+        };
 
         // bias rows of this lane's query: f32 [seq_q, seq_kv] per (batch, head) or one for all
         const float* bias_row = nullptr;
@@ -421,6 +507,16 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
 
         // K(0), V(0) -> stage 0, K(1) -> stage 1; then the register sets take K(2) .. K(1 + PF) and V(1) .. V(PF)
         // (K(j) travels in set j % PF, and so does V(j))
+        if constexpr (DIRECT) {
+            // tile 0 and K(1) have landed (and the queries); V rows of tile 0 past the last key, requested before the
+            // lengths were known, are zeroed by the lane that fetched them
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (n_keys < KT) {
+#pragma unroll
+                for (int n = 0; n < 2; n++)
+                    if (dl_row + 32 * n >= n_keys) *(u32x4_t*)(lds + 2 * STAGE_B + (wave + 4 * n) * 1024 + 16 * lane) = u32x4_t{0u, 0u, 0u, 0u};
+            }
+        } else {
         park_k(kreg[0], 0);
         park_v(std::integral_constant<int, 0>{}, 0);
         keep_cur = keep_next;
@@ -436,6 +532,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             if (PF >= 2) prefetch(std::integral_constant<int, 1>{});
             if (PF >= 3) prefetch(std::integral_constant<int, 2>{});
             static_assert(PF <= 3, "prologue covers up to three sets");
+        }
         }
         __syncthreads();
 
@@ -492,6 +589,14 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         // operand m of a step: even m = K rows of the next item (A operand of score instruction m / 2), odd m = V of
         // the previous item (contraction slots 0-3 of a lane are keys 16u + 4hh + 0..3, slots 4-7 keys 16u + 8 + 4hh + 0..3)
         auto load_op = [&](int m, const uint16_t* kp, const uint16_t* vp) __attribute__((always_inline)) {
+            if constexpr (DIRECT) {
+                if ((m & 1) == 0) return *(const u32x4_t*)((const unsigned char*)kp + (k_base ^ (uint32_t)(32 * (m >> 1))));
+                const int i = m >> 1, u = i / DT, dt = i - u * DT;
+                const unsigned char* const vq = (const unsigned char*)vp + (v_base ^ (uint32_t)(64 * dt)) + 16 * u * ROWB;
+                const u32x2_t lo = t_lds_read_tr16((const uint16_t*)vq);
+                const u32x2_t hi = t_lds_read_tr16((const uint16_t*)(vq + 8 * ROWB));
+                return u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+            }
             if ((m & 1) == 0) return *(const u32x4_t*)(kp + 16 * (m >> 1));
             const int i = m >> 1, u = i / DT, dt = i - u * DT;
             const u32x2_t lo = t_lds_read_tr16(vp + 16 * u * LDV + 32 * dt);
@@ -520,7 +625,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             if (PIPE && n_it > 0) {
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++)
-                    s_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)(Ks + k_off + 16 * ks), qreg[ks], s_a, 0, 0, 0);
+                    s_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, load_op(2 * ks, k_at(0, 0), nullptr)), qreg[ks], s_a, 0, 0, 0);
                 // The running max starts at the max of item 0, taken here, so that the first step already runs the
                 // fast path (without it the step would form P twice and rescale an O that is still zero).  The masks
                 // are applied first; the step applies them again, which changes nothing.  (Not with a bias: adding it
@@ -713,11 +818,23 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         auto park_next = [&](int t, auto kset_c, auto vset_c, auto st_c) __attribute__((always_inline)) {
             constexpr int KSET = decltype(kset_c)::value;
             const int st = st_c;  // t & 1, as a constant where the caller knows it
-            // (behind the last tiles these park and request copies of the last tile, which nobody reads)
-            park_k(kreg[KSET], st);
-            park_v(vset_c, st ^ 1);
-            issue_k(kreg[KSET], (t + 2 + PF) * KT);
-            issue_v(vset_c, (t + 1 + PF) * KT);
+            if constexpr (DIRECT) {
+                // K(t+2) over K(t), V(t+1) over V(t-1): requested now that every wave is done with those, awaited
+                // (vmcnt) ahead of the next tile's barrier
+                if (t + 2 < n_tiles) dl_tile(Kd, dl_k, (uint32_t)(t + 2) * tile_bytes_g, (uint32_t)(st * STAGE_B));
+                if (t + 1 < n_tiles) dl_tile(Vd, dl_v, (uint32_t)(t + 1) * tile_bytes_g, (uint32_t)((2 + (st ^ 1)) * STAGE_B));
+            } else {
+                // (behind the last tiles these park and request copies of the last tile, which nobody reads)
+                park_k(kreg[KSET], st);
+                park_v(vset_c, st ^ 1);
+                issue_k(kreg[KSET], (t + 2 + PF) * KT);
+                issue_v(vset_c, (t + 1 + PF) * KT);
+            }
+        };
+        // what a wave does ahead of a tile's barrier: DIRECT waits for its own requests of a tile ago
+        auto meet = [&]() __attribute__((always_inline)) {
+            if constexpr (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
         };
         // the same for a tile of which the wave walks every item: straight-line code, the pairs swapped from step to step
         // `st_c` is t & 1, as an integer or as a compile-time constant: with the stage known at compile time every LDS
@@ -726,18 +843,14 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
         auto walk_full = [&](int t, auto kset_c, auto vset_c, auto st_c, auto later_c) __attribute__((always_inline)) {
             const int st = st_c;
             constexpr bool kLater = decltype(later_c)::value;
-            const uint16_t* const k_st = Ks + st * KT * LDK + k_off;
-            const uint16_t* const k_ot = Ks + (st ^ 1) * KT * LDK + k_off;
-            const uint16_t* const v_st = Vs + st * KT * LDV + v_off;
-            const uint16_t* const v_ot = Vs + (st ^ 1) * KT * LDV + v_off;
             const int k0 = t * KT;
             if (NI > 1) {
-                step(0, k0, k_st + 32 * LDK, (!kLater && t == 0) ? v_st : v_ot + 32 * (NI - 1) * LDV, s_a, s_b, p_a, p_b, bv_a, bv_b);
-                __syncthreads();
+                step(0, k0, k_at(st, 1), (!kLater && t == 0) ? v_at(st, 0) : v_at(st ^ 1, NI - 1), s_a, s_b, p_a, p_b, bv_a, bv_b);
+                meet();
                 park_next(t, kset_c, vset_c, st_c);
-                step(1, k0 + 32, k_ot, v_st, s_b, s_a, p_b, p_a, bv_b, bv_a);
+                step(1, k0 + 32, k_at(st ^ 1, 0), v_at(st, 0), s_b, s_a, p_b, p_a, bv_b, bv_a);
             } else {
-                step_a(0, k0, k_ot, (!kLater && t == 0) ? v_st : v_ot);
+                step_a(0, k0, k_at(st ^ 1, 0), (!kLater && t == 0) ? v_at(st, 0) : v_at(st ^ 1, 0));
                 __syncthreads();
                 park_next(t, kset_c, vset_c, st_c);
                 __syncthreads();
@@ -745,18 +858,14 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             keep_cur = keep_next;
         };
         auto walk_tile = [&](int t, auto kset_c, auto vset_c) __attribute__((always_inline)) {
-            const int st = t & 1;
-            const uint16_t* const k_st = Ks + st * KT * LDK + k_off;         // K(t)
-            const uint16_t* const k_ot = Ks + (st ^ 1) * KT * LDK + k_off;   // K(t+1)
-            const uint16_t* const v_st = Vs + st * KT * LDV + v_off;         // V(t)
-            const uint16_t* const v_ot = Vs + (st ^ 1) * KT * LDV + v_off;   // V(t-1)
+            const int st = t & 1;  // K(t) and V(t) sit in stage st, K(t+1) and V(t-1) in the other
             // first item: the next item is item 1 of this tile (or item 0 of the next tile when a tile is one item);
             // the previous item is the last of tile t - 1 (at t = 0 there is none: P is zero, and V(0) stands in)
-            slot(t * NI, 0, NI > 1 ? k_st + 32 * LDK : k_ot, t == 0 ? v_st : v_ot + 32 * (NI - 1) * LDV);
-            __syncthreads();
+            slot(t * NI, 0, NI > 1 ? k_at(st, 1) : k_at(st ^ 1, 0), t == 0 ? v_at(st, 0) : v_at(st ^ 1, NI - 1));
+            meet();
             park_next(t, kset_c, vset_c, st);
             if (NI > 1) {
-                slot(t * NI + 1, 1, k_ot, v_st);
+                slot(t * NI + 1, 1, k_at(st ^ 1, 0), v_at(st, 0));
             } else {
                 __syncthreads();  // one item per tile: K(t+2) is read by the very next step
             }
@@ -770,7 +879,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
 #pragma unroll
                 for (int it = 0; it < NI; it++)
                     if (t * NI + it < n_it)
-                        step_simple(it, t * KT + 32 * it, Ks + st * KT * LDK + 32 * it * LDK + k_off, Vs + st * KT * LDV + 32 * it * LDV + v_off);
+                        step_simple(it, t * KT + 32 * it, k_at(st, it), v_at(st, it));
                 park_k(kreg[0], st ^ 1);
                 park_v(std::integral_constant<int, 0>{}, st ^ 1);
                 issue_k(kreg[0], (t + 2) * KT);
@@ -813,10 +922,11 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, (BIAS && DP == 64) ? 2 : Tile
             if (PF >= 3 && t0 + 2 < n_tiles) walk_tile(t0 + 2, std::integral_constant<int, 4 % PF>{}, std::integral_constant<int, 3 % PF>{});
         }
         // a wave that walked every item of the workgroup still owes the last P.V
-        if (PIPE && n_it == n_tiles * NI && n_it > 0)
-            drain(Vs + ((n_tiles - 1) & 1) * KT * LDV + v_off + 32 * (NI - 1) * LDV);
+        if (PIPE && n_it == n_tiles * NI && n_it > 0) drain(v_at((n_tiles - 1) & 1, NI - 1));
         __syncthreads();  // the output rows are staged over the tiles
     }
+    // (a workgroup without tiles still has its early requests in flight: they land in its LDS)
+    if constexpr (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     // ---- output: acc_o[dt][4j + e] = O^T[d = 32dt + 8j + 4hh + e][row col of the wave].  A lane holds 8-byte pieces of
     // its row; the wave parks its 32 normalised rows in its own region of LDS (every wave is past the last
@@ -1444,24 +1554,31 @@ __global__ __launch_bounds__(256, 2) void flash_wide_bf16_kernel(FlashTileParams
     }
 }
 
-template <int DP, int MODE, bool BIAS, bool PACKED, bool SPLIT = false, bool WIN = false>
+template <int DP, int MODE, bool BIAS, bool PACKED, bool SPLIT = false, bool WIN = false, bool DIRECT = false>
 hipError_t launch_one(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
-    hipLaunchKernelGGL((flash_tile_bf16_kernel<DP, MODE, BIAS, PACKED, SPLIT, WIN>), grid, dim3(TileCfg<DP>::THREADS), 0, stream, p);
+    hipLaunchKernelGGL((flash_tile_bf16_kernel<DP, MODE, BIAS, PACKED, SPLIT, WIN, DIRECT>), grid, dim3(TileCfg<DP>::THREADS), 0, stream, p);
     return hipGetLastError();
 }
 
 template <int DP>
 hipError_t launch_dp(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
+    constexpr bool kDirect = DP == 64;  // head dim 64 exactly: the tiles go straight to LDS
+    const bool direct = kDirect && p.dim == 64;
     if (p.n_splits > 1) {  // (rows packed over a group of one head are rows of that head)
-        hipError_t e = launch_one<DP, kMaskCausal, false, true, true>(stream, p, grid);
+        hipError_t e = direct ? launch_one<DP, kMaskCausal, false, true, true, false, kDirect>(stream, p, grid)
+                              : launch_one<DP, kMaskCausal, false, true, true>(stream, p, grid);
         if (e != hipSuccess) return e;
         const size_t total = (size_t)p.batch * p.kv_heads * (size_t)p.seq_q * p.pack * (size_t)p.dim;
         hipLaunchKernelGGL(flash_split_merge_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p);
         return hipGetLastError();
     }
-    if (p.pack > 1) return launch_one<DP, kMaskCausal, false, true>(stream, p, grid);
-    if (p.window > 0) return launch_one<DP, kMaskCausal, false, false, false, true>(stream, p, grid);
+    if (p.pack > 1) return direct ? launch_one<DP, kMaskCausal, false, true, false, false, kDirect>(stream, p, grid)
+                                  : launch_one<DP, kMaskCausal, false, true>(stream, p, grid);
+    if (p.window > 0) return direct ? launch_one<DP, kMaskCausal, false, false, false, true, kDirect>(stream, p, grid)
+                                    : launch_one<DP, kMaskCausal, false, false, false, true>(stream, p, grid);
     if (p.bias) return launch_one<DP, kMaskNone, true, false>(stream, p, grid);
+    if (direct && !p.bias && p.mask == kMaskNone) return launch_one<DP, kMaskNone, false, false, false, false, kDirect>(stream, p, grid);
+    if (direct && !p.bias && p.mask == kMaskCausal) return launch_one<DP, kMaskCausal, false, false, false, false, kDirect>(stream, p, grid);
     switch (p.mask) {
         case kMaskNone: return launch_one<DP, kMaskNone, false, false>(stream, p, grid);
         case kMaskCausal: return launch_one<DP, kMaskCausal, false, false>(stream, p, grid);

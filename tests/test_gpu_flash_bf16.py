@@ -107,10 +107,10 @@ def test_flash_bf16_closed_forms():
 
 
 @pytest.mark.parametrize("mask", ["causal", "none"])
-def test_long_head_dim_64_takes_the_64_rows_per_wave_kernel_by_itself(oracle, mask):
-    """B=4, H=32, N=2048, D=64: 1024 workgroups of 256 rows, the shape class the library routes to the kernel with 64
-    query rows per wave when nothing is forced.  Every row of eight (batch, head) slabs against the oracle, and the
-    whole output against the tile kernel's (both round the same f32 sums to bf16)."""
+def test_long_head_dim_64_is_served_by_the_tile_kernel_and_the_64_rows_per_wave_kernel_agrees(oracle, mask):
+    """B=4, H=32, N=2048, D=64: with nothing forced the library takes the tile kernel here (the same bits as the
+    forced tile kernel); the kernel with 64 query rows per wave, which runs when asked for, rounds the same f32 sums.
+    Every row of eight (batch, head) slabs of either against the oracle."""
     b, h, n, d = 4, 32, 2048, 64
     (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d), (91, 92, 93))
     shape = ra.AttentionShape.new(b, h, n, d)
@@ -120,14 +120,18 @@ def test_long_head_dim_64_takes_the_64_rows_per_wave_kernel_by_itself(oracle, ma
     try:
         ra.debug_force_bf16_prefill_kernel("tile")
         tile = flash_bf16(shape, qb, kb, vb, m).reshape(b * h, n, d)
+        ra.debug_force_bf16_prefill_kernel("wide")
+        wide = flash_bf16(shape, qb, kb, vb, m).reshape(b * h, n, d)
     finally:
         ra.debug_force_bf16_prefill_kernel("auto")
-    assert max_abs(got, tile) <= 2 ** -7 * 4.0  # a bf16 ulp or two of values below 4
+    assert np.array_equal(got, tile, equal_nan=True)
+    assert max_abs(wide, tile) <= 2 ** -7 * 4.0  # a bf16 ulp or two of values below 4
     q3, k3, v3 = (x.reshape(b * h, n * d) for x in (qf, kf, vf))
     for slab in (0, 1, 31, 64, 77, 100, 126, 127):
         want = oracle.flash_forward_masked(oracle.AttentionShape(1, 1, n, d), q3[slab], k3[slab], v3[slab],
                                            "causal" if mask == "causal" else None).reshape(n, d)
         assert_bf16_parity(got[slab], want, d, n, f"slab {slab}")
+        assert_bf16_parity(wide[slab], want, d, n, f"slab {slab}, 64 rows per wave")
 
 
 @pytest.mark.parametrize("kernel", ["persistent", "tile", "wide"])
