@@ -201,6 +201,31 @@ def test_varlen_small(oracle, force_kernel, kernel, d):
                 assert (g[i, :, L:] == 0.0).all() and not np.signbit(g[i, :, L:]).any()
 
 
+@pytest.mark.parametrize("d", [32, 64, 128])
+def test_rows_behind_a_short_sequence_may_hold_anything(oracle, force_kernel, d):
+    """Sequences shorter than one key tile in a padded batch whose K and V rows behind each sequence's last key hold NaN
+    and infinities: the first key tile is requested before the lengths are known, so those rows do arrive in the
+    workgroup; nothing of them may reach a valid row (V rows behind the last key count as zeros, their scores are
+    masked), and the padded rows are zeros."""
+    force_kernel("tile")
+    b, h, n = 5, 2, 100
+    lens = [1, 5, 63, 64, 65]
+    (qb, qf), (kb, kf), (vb, vf) = inputs((b, h, n, d), (b, h, n, d), (81, 82, 83))
+    k4, v4 = kf.copy().reshape(b, h, n, d), vf.copy().reshape(b, h, n, d)
+    for i, L in enumerate(lens):
+        k4[i, :, L:] = np.nan
+        v4[i, :, L:] = np.inf
+        v4[i, :, L:, ::3] = np.nan
+    shape = ra.AttentionShape.new(b, h, n, d)
+    got = run_varlen(shape, qb, oracle.f32_to_bf16(k4.ravel()), oracle.f32_to_bf16(v4.ravel()), lens, True)
+    want = oracle.varlen_causal_forward(qf, kf, vf, lens, b, h, n, d, zero_padded_rows=True)
+    assert np.isfinite(got).all()
+    assert_bf16_parity(got, want, d, n)
+    g = got.reshape(b, h, n, d)
+    for i, L in enumerate(lens):
+        assert (g[i, :, L:] == 0.0).all()
+
+
 def test_strict_mode_on_a_padded_batch(oracle, strict_v):
     """The strict pass takes each sequence's own length: a non-finite V element inside a sequence reaches the rows
     before its key, one in the padding behind a sequence reaches nothing."""
