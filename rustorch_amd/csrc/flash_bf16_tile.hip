@@ -89,7 +89,7 @@ struct TileCfg {
     // DIRECT: unpadded tiles (rows of DP * 2 bytes, 16-byte slots swizzled), filled by loads that go straight to LDS
     static constexpr int STAGE_BYTES = KT * DP * 2;
     static constexpr int LDS_BYTES_DIRECT = 4 * STAGE_BYTES > 4 * REGION ? 4 * STAGE_BYTES : 4 * REGION;
-    static constexpr int OCC_DIRECT = 3;
+    static constexpr int OCC_DIRECT = DP <= 64 ? 3 : 2;
 };
 
 // 16 bytes per lane from a buffer straight into LDS: lane l lands at LDS byte address lds_block + 16 l (lds_block is
@@ -153,7 +153,7 @@ template <int DP, int MODE, bool BIAS, bool PACKED, bool SPLIT = false, bool WIN
 __global__ __launch_bounds__(TileCfg<DP>::THREADS, DIRECT ? TileCfg<DP>::OCC_DIRECT : ((BIAS && DP == 64) ? 2 : TileCfg<DP>::OCC)) void flash_tile_bf16_kernel(FlashTileParams p) {
     static_assert(!SPLIT || (PACKED && !BIAS && MODE == kMaskCausal), "the split over the keys serves the chunked decode");
     static_assert(!WIN || (!PACKED && !BIAS && !SPLIT && MODE == kMaskCausal), "the window is a causal mask's");
-    static_assert(!DIRECT || (DP == 64 && !BIAS && MODE != kMaskPadding), "tiles straight into LDS: head dim 64 exactly");
+    static_assert(!DIRECT || ((DP == 64 || DP == 128) && !BIAS && MODE != kMaskPadding), "tiles straight into LDS: head dim 64 or 128 exactly");
     using Cfg = TileCfg<DP>;
     constexpr int KT = Cfg::KT, LDK = Cfg::LDK, LDV = Cfg::LDV, NI = Cfg::NI, TTHREADS = Cfg::THREADS;
     constexpr int KS = DP / 16;        // contraction steps of the score product
@@ -226,21 +226,26 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, DIRECT ? TileCfg<DP>::OCC_DIR
         ld_off[n] = ((uint32_t)row * kv_pitch + (ld_on[n] ? (uint32_t)(8 * ch) : 0u)) * 2u;
     }
     u32x4_t k1[NL];
-    // DIRECT: a wave's load instruction fills 1 KB of LDS (8 rows), lane l the 16 bytes at 16 l; instruction n of
-    // wave w fills block w + 4 n of a stage.  Bank conflicts are avoided by an XOR of the 16-byte slot index with bits
-    // of the row (K rows are read 16 at a time at one slot, V rows 4 at a time over 4 adjacent slots by the
-    // transposing reads), applied on the way in: the lane fetches the slot that belongs at its LDS position.
-    auto swz_k = [](int r) __attribute__((always_inline)) { return (r >> 1) & 7; };
-    auto swz_v = [](int r) __attribute__((always_inline)) { return 4 * ((r >> 1) & 1); };
+    // DIRECT: a wave's load instruction fills 1 KB of LDS (RPI = 8 rows at head dim 64, 4 at 128), lane l the 16 bytes
+    // at 16 l; instruction n of wave w fills block w + 4 n of a stage.  Bank conflicts are avoided by an XOR of the
+    // 16-byte slot index with bits of the row (K rows are read 16 at a time at one slot, V rows 4 at a time over 4
+    // adjacent slots by the transposing reads), applied on the way in: the lane fetches the slot that belongs at its
+    // LDS position.
+    constexpr int SPR = DP / 8;                // 16-byte slots per row
+    constexpr int RPI = 64 / (SPR > 64 ? 64 : SPR);  // rows per load instruction of a wave
+    constexpr int NLD = KT / (4 * RPI);        // load instructions per wave, matrix and tile
+    auto swz_k = [](int r) __attribute__((always_inline)) { return DP == 128 ? (r & 15) : ((r >> 1) & 7); };
+    auto swz_v = [](int r) __attribute__((always_inline)) { return DP == 128 ? 4 * (r & 3) : 4 * ((r >> 1) & 1); };
+    static_assert(!DIRECT || (4 * RPI) % 16 == 0, "the row swizzles must not depend on the load index");
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
-    const int dl_row = 8 * wave + (lane >> 3);  // row of the lane's chunk in instruction 0; instruction n: + 32 n (the swizzles do not see n)
-    const uint32_t dl_k = (uint32_t)dl_row * kv_pitch * 2u + (uint32_t)(((lane & 7) ^ swz_k(dl_row)) * 16);
-    const uint32_t dl_v = (uint32_t)dl_row * kv_pitch * 2u + (uint32_t)(((lane & 7) ^ swz_v(dl_row)) * 16);
+    const int dl_row = RPI * wave + lane / SPR;  // row of the lane's chunk in instruction 0; instruction n: + 4 RPI n (the swizzles do not see n)
+    const uint32_t dl_k = (uint32_t)dl_row * kv_pitch * 2u + (uint32_t)(((lane % SPR) ^ swz_k(dl_row)) * 16);
+    const uint32_t dl_v = (uint32_t)dl_row * kv_pitch * 2u + (uint32_t)(((lane % SPR) ^ swz_v(dl_row)) * 16);
     // the tile whose first row lies tile_off bytes into the descriptor -> the stage at stage_off
     auto dl_tile = [&](const u32x4_t& rs, uint32_t lane_off, uint32_t tile_off, uint32_t stage_off) __attribute__((always_inline)) {
 #pragma unroll
-        for (int n = 0; n < 2; n++)
-            t_buffer_to_lds(rs, lane_off, tile_off + (uint32_t)(32 * n) * kv_pitch * 2u, lds_base + stage_off + (uint32_t)((wave + 4 * n) * 1024));
+        for (int n = 0; n < NLD; n++)
+            t_buffer_to_lds(rs, lane_off, tile_off + (uint32_t)(4 * RPI * n) * kv_pitch * 2u, lds_base + stage_off + (uint32_t)((wave + 4 * n) * 1024));
     };
     // Tile 0 (K and V) and K of tile 1 are requested before the sequence lengths have arrived (a dependent load
     // away), through descriptors that end with the tensor's last row: the rows of V(0) past the last key are zeroed
@@ -525,8 +530,8 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, DIRECT ? TileCfg<DP>::OCC_DIR
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             if (n_keys < KT) {
 #pragma unroll
-                for (int n = 0; n < 2; n++)
-                    if (dl_row + 32 * n >= n_keys) *(u32x4_t*)(lds + 2 * STAGE_B + (wave + 4 * n) * 1024 + 16 * lane) = u32x4_t{0u, 0u, 0u, 0u};
+                for (int n = 0; n < NLD; n++)
+                    if (dl_row + 4 * RPI * n >= n_keys) *(u32x4_t*)(lds + 2 * STAGE_B + (wave + 4 * n) * 1024 + 16 * lane) = u32x4_t{0u, 0u, 0u, 0u};
             }
         } else {
         park_k(kreg[0], 0);
@@ -902,7 +907,7 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, DIRECT ? TileCfg<DP>::OCC_DIR
             t0 = n_tiles;
         }
         const int t_full = PIPE ? n_it / NI : 0;
-        if constexpr (PF == 1 && DP == 64 && !BIAS && MODE != kMaskPadding) {
+        if constexpr (PF == 1 && (DP == 64 || (DIRECT && DP == 128)) && !BIAS && MODE != kMaskPadding) {
             // (head dim 64 only: the wider kernels and the ones with a bias or a padding mask have no register to spare for
             // the second copy of the tile's code)
             // one register set: tile 0 on its own, then the tiles in pairs (odd, even) whose LDS stages are compile-time
@@ -1574,8 +1579,8 @@ hipError_t launch_one(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
 
 template <int DP>
 hipError_t launch_dp(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
-    constexpr bool kDirect = DP == 64;  // head dim 64 exactly: the tiles go straight to LDS
-    const bool direct = kDirect && p.dim == 64;
+    constexpr bool kDirect = DP == 64 || DP == 128;  // head dim 64 or 128 exactly: the tiles go straight to LDS
+    const bool direct = kDirect && p.dim == DP;
     if (p.n_splits > 1) {  // (rows packed over a group of one head are rows of that head)
         hipError_t e = direct ? launch_one<DP, kMaskCausal, false, true, true, false, kDirect>(stream, p, grid)
                               : launch_one<DP, kMaskCausal, false, true, true>(stream, p, grid);
