@@ -544,7 +544,7 @@ def main():
                      "roofline": {"bound": "hbm", "achieved": bytes_c / (tc.mean_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                                   "unit": "GB/s", "frac": bytes_c / (tc.mean_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                                   "traffic": profile_traffic("chunk_decode_b1_hq32_hkv8_d128_ctx8192.md", f"chunk_{s_new}"),
-                                  "kernels": "flash_tile_bf16_kernel<128, causal, packed, split> + flash_split_merge_kernel "
+                                  "kernels": "flash_tile_bf16_kernel<128, causal, packed, split, direct> + flash_split_merge_kernel "
                                              "(one event pair around the timed calls)"}}
             if not args.no_cpu:
                 K.gqa_decode_chunk_bf16(stream, d_qc, sets[0][0], sets[0][1], d_oc, Lmax, 1, s_new, Hq, Hkv, Dd, Lmax)

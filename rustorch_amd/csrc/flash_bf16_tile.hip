@@ -141,14 +141,14 @@ __device__ __forceinline__ u32x4_t t_make_rsrc(const void* base, uint32_t bytes)
 // moved by that many keys, as for a span of SPLIT), and an item that holds keys below some row's window is masked on
 // that side as well.
 //
-// DIRECT (head dim 64 exactly, no bias, no key-padding vector): the tiles travel from memory straight into LDS
+// DIRECT (head dim 64 or 128 exactly, no bias, no key-padding vector): the tiles travel from memory straight into LDS
 // (buffer_load_dwordx4 ... lds) instead of through registers and LDS writes.  After a tile's barrier the waves request
 // K(t+2) and V(t+1) into the stages K(t) and V(t-1) have just left and wait for their own requests ahead of the next
 // tile's barrier.  LDS rows are unpadded (a landing block of 1 KB is contiguous) and their 16-byte slots are XORed
 // with bits of the row, as in flash_bf16.hip.  Same instructions on the same operands otherwise: the same bits.
 // Measured against the register path, interleaved in one process: 3-5 % on short or padded sequences (B=16 H=16
-// N=1024: 52.3 -> 49.3 us), 7-9 % on long ones (B=4 H=32 N=4096: 306 -> 283 us); three stages per matrix or four
-// workgroups per CU are no faster.
+// N=1024: 52.3 -> 49.3 us), 7-9 % on long ones (B=4 H=32 N=4096: 306 -> 283 us), 4-7 % at head dim 128; three stages
+// per matrix or four workgroups per CU (head dim 64) are no faster.
 template <int DP, int MODE, bool BIAS, bool PACKED, bool SPLIT = false, bool WIN = false, bool DIRECT = false>
 __global__ __launch_bounds__(TileCfg<DP>::THREADS, DIRECT ? TileCfg<DP>::OCC_DIRECT : ((BIAS && DP == 64) ? 2 : TileCfg<DP>::OCC)) void flash_tile_bf16_kernel(FlashTileParams p) {
     static_assert(!SPLIT || (PACKED && !BIAS && MODE == kMaskCausal), "the split over the keys serves the chunked decode");
