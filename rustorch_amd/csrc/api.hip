@@ -1498,6 +1498,7 @@ RT_API int rt_gqa_decode_chunk_bf16(void* stream, const void* q, const void* k_c
     t.kv_heads = n_kv;
     t.group = group;
     t.pack = group;  // rows of a tile run over (position, head of the group): one pass over a kv head's keys serves them all
+    t.decode_rows = 1;  // (also with one head per group: a position without keys is a row of zeros)
     t.seq_q = seq_new;
     t.seq_kv = kv_lens ? max_seq : kv_len;
     t.dim = head_dim;

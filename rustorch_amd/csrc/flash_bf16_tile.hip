@@ -1589,7 +1589,7 @@ hipError_t launch_dp(hipStream_t stream, const FlashTileParams& p, dim3 grid) {
         hipLaunchKernelGGL(flash_split_merge_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p);
         return hipGetLastError();
     }
-    if (p.pack > 1) return direct ? launch_one<DP, kMaskCausal, false, true, false, false, kDirect>(stream, p, grid)
+    if (p.pack > 1 || p.decode_rows) return direct ? launch_one<DP, kMaskCausal, false, true, false, false, kDirect>(stream, p, grid)
                                   : launch_one<DP, kMaskCausal, false, true>(stream, p, grid);
     if (p.window > 0) return direct ? launch_one<DP, kMaskCausal, false, false, false, true, kDirect>(stream, p, grid)
                                     : launch_one<DP, kMaskCausal, false, false, false, true>(stream, p, grid);
@@ -1640,11 +1640,11 @@ hipError_t launch_flash_tile_bf16(hipStream_t stream, const FlashTileParams& par
     if (!flash_tile_bf16_supported(p.dim) || p.pack < 1) return hipErrorInvalidValue;
     if (p.bias && p.mask != kMaskNone) return hipErrorInvalidValue;
     if (!flash_tile_bf16_addressable(p.seq_kv, p.lkv.row_pitch)) return hipErrorInvalidValue;
-    if (p.pack > 1 && (p.bias || p.mask != kMaskCausal)) return hipErrorInvalidValue;  // packed rows: the chunked decode only
-    if (p.window < 0 || (p.window > 0 && (p.pack > 1 || p.bias || p.mask != kMaskCausal || p.n_splits > 1))) return hipErrorInvalidValue;
+    if ((p.pack > 1 || p.decode_rows) && (p.bias || p.mask != kMaskCausal)) return hipErrorInvalidValue;  // packed rows: the chunked decode only
+    if (p.window < 0 || (p.window > 0 && (p.pack > 1 || p.decode_rows || p.bias || p.mask != kMaskCausal || p.n_splits > 1))) return hipErrorInvalidValue;
     const long long rows = (long long)p.seq_q * p.pack;
     const long long n_qtiles = (rows + TROWS - 1) / TROWS;
-    const long long heads_u = p.pack > 1 ? p.kv_heads : p.heads;
+    const long long heads_u = (p.pack > 1 || p.decode_rows) ? p.kv_heads : p.heads;
     if (p.n_splits < 1) p.n_splits = 1;
     if (p.n_splits > 1 && (p.pack != p.group || p.bias || p.mask != kMaskCausal || !p.part_o || !p.part_ml))
         return hipErrorInvalidValue;  // the chunked decode only

@@ -112,6 +112,10 @@ struct FlashTileParams {
     // 1: a tile's rows are positions of one head.  group: rows run over (position, head of the GQA group), row
     // r = position * group + head-in-group, so that all heads of a kv head share one pass over its keys.
     int pack;
+    // rows are positions of a chunked decode over a cache: a position that sees no key is a row of zeros (the
+    // reference's decode kernels leave it so), not the NaN row of flash_forward.  Implied by pack > 1; a group of one
+    // head sets it.
+    int decode_rows;
     int seq_q, seq_kv, dim;
     int mask;   // kMaskNone, kMaskCausal (key j visible to position i iff j <= i + (keys - valid queries)), kMaskPadding
     int ref_bc;

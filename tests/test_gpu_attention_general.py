@@ -121,6 +121,12 @@ def run_chunk(oracle, b, s, hq, hkv, d, max_seq, lens, seed=0, scalar_len=False)
     (1, 33, 16, 2, 256, 2000, [1999]),
     (1, 40, 4, 1, 96, 1000, [1000]),          # two query tiles, each with its spans
     (3, 5, 8, 2, 128, 1500, [1500, 3, 0]),    # a sequence shorter than the chunk, and an empty one
+    # one head per kv head (rows are not packed) and a cache too short for spans: positions without keys are rows of
+    # zeros here as well, not the NaN rows of flash_forward
+    (1, 8, 1, 1, 64, 64, [5]),
+    (1, 8, 1, 1, 128, 64, [0]),
+    (2, 8, 4, 4, 64, 64, [5, 64]),
+    (2, 6, 2, 2, 96, 100, [2, 100]),
 ])
 def test_chunk_decode_matches_oracle(oracle, b, s, hq, hkv, d, max_seq, lens):
     run_chunk(oracle, b, s, hq, hkv, d, max_seq, lens)
