@@ -169,3 +169,80 @@ def test_random_mha_and_gqa_cases_match_oracle(oracle, seed):
         out = np.zeros(b * h * tq * d, dtype=np.float32)
         ra.gqa_forward_f32(q, kk, vv, out, b, h, hkv, tq, tkv, d)
         _compare(f"gqa B{b} H{h}/{hkv} Sq{tq} Skv{tkv} D{d}", out, oracle.gqa_forward_f32(q, kk, vv, b, h, hkv, tq, tkv, d), 1e-5)
+
+
+def _window(oracle, rng):
+    """rt_flash_forward_window_bnhd_bf16_dev against MultiHeadAttention's masked path with sliding_window_mask."""
+    b = int(rng.integers(1, 3))
+    hkv = int(rng.choice([1, 2]))
+    g = int(rng.choice([1, 2, 4]))
+    h = hkv * g
+    n = int(rng.choice([1, 33, 64, 65, 127, 200, 257, 500, 900]))
+    d = int(rng.choice([32, 64, 96, 128]))
+    w = int(rng.choice([1, 2, 31, 64, 65, 100, 300, 2000]))
+    q, k, v = (_bf(oracle, rng.standard_normal(x)) for x in (b * n * h * d, b * n * hkv * d, b * n * hkv * d))
+    out = ra.HipStorage(b * n * h * d * 2)
+    dq, dk, dv = (ra.HipStorage.from_numpy(x) for x in (q, k, v))
+    ra.flash_forward_window_bf16_dev(ra.AttentionShape.new(b, h, n, d), dq, dk, dv, out, w, n_kv_heads=hkv, bnhd=True)
+    ra.synchronize()
+    got = oracle.bf16_to_f32(out.download(np.uint16))
+    kf = np.repeat(oracle.bf16_to_f32(k).reshape(b, n, hkv, d), g, axis=2).ravel()
+    vf = np.repeat(oracle.bf16_to_f32(v).reshape(b, n, hkv, d), g, axis=2).ravel()
+    want = oracle.mha_forward_masked(oracle.bf16_to_f32(q), kf, vf, b, n, n, h, d, attn_mask=oracle.sliding_window_mask(n, w))
+    _compare(f"window B{b} T{n} H{h}/{hkv} D{d} w{w}", got, np.asarray(want, dtype=np.float32).ravel(), oracle.BF16_MAX_ABS)
+
+
+def _chunk_decode(oracle, rng):
+    """rt_gqa_decode_chunk_bf16 on every grouping (one head per kv head included), caches short and long enough for
+    spans, sequences shorter than the chunk and empty ones."""
+    b = int(rng.integers(1, 4))
+    hkv = int(rng.choice([1, 2, 8]))
+    g = int(rng.choice([1, 2, 4]))
+    hq = hkv * g
+    d = int(rng.choice([64, 96, 128]))
+    max_seq = int(rng.choice([64, 300, 1100, 4000]))
+    s = int(rng.choice([1, 3, 8, 16, 40]))
+    lens = [int(rng.integers(0, max_seq + 1)) for _ in range(b)]
+    if rng.random() < 0.3:
+        lens[0] = int(rng.integers(0, s + 1))  # fewer keys than new positions
+    q, k, v = (_bf(oracle, rng.standard_normal(x)) for x in (b * s * hq * d, b * hkv * max_seq * d, b * hkv * max_seq * d))
+    out = ra.HipStorage(q.size * 2)
+    dq, dk, dv, dl = (ra.HipStorage.from_numpy(x) for x in (q, k, v, np.asarray(lens, dtype=np.int32)))
+    ra.LlmKernels().gqa_decode_chunk_bf16(None, dq, dk, dv, out, dl, b, s, hq, hkv, d, max_seq)
+    ra.synchronize()
+    got = oracle.bf16_to_f32(out.download(np.uint16))
+    want = oracle.gqa_decode_chunk_bf16(q, k, v, lens, b, s, hq, hkv, d, max_seq)
+    _compare(f"chunk B{b} S{s} H{hq}/{hkv} D{d} max{max_seq} lens={lens}", got, np.asarray(want, dtype=np.float32).ravel(),
+             oracle.BF16_MAX_ABS)
+
+
+def _masked_bf16(oracle, rng):
+    """rt_mha_forward_masked_bf16_dev: self and cross lengths, shared and per-head additive masks."""
+    b, h = int(rng.integers(1, 3)), int(rng.integers(1, 5))
+    tq = int(rng.choice([1, 7, 32, 33, 64, 100, 129, 257]))
+    tkv = tq if rng.random() < 0.4 else int(rng.choice([1, 3, 32, 65, 128, 200, 513]))
+    d = int(rng.choice([8, 16, 32, 40, 64, 96, 128, 256]))
+    q, k, v = (_bf(oracle, rng.standard_normal(x)) for x in (b * tq * h * d, b * tkv * h * d, b * tkv * h * d))
+    kind = int(rng.integers(0, 3))
+    mask = None
+    if kind == 1:
+        mask = np.where(rng.random((tq, tkv)) > 0.3, 0.0, -1.0e4).astype(np.float32)
+    elif kind == 2:
+        mask = rng.standard_normal((b * h, tq, tkv)).astype(np.float32)
+    out = ra.HipStorage(b * tq * h * d * 2)
+    dq, dk, dv = (ra.HipStorage.from_numpy(x) for x in (q, k, v))
+    dm = ra.HipStorage.from_numpy(mask.ravel()) if mask is not None else None
+    ra.mha_forward_masked_bf16_dev(dq, dk, dv, out, b, tq, tkv, h, d, attn_mask=dm, mask_len=0 if mask is None else mask.size)
+    ra.synchronize()
+    got = oracle.bf16_to_f32(out.download(np.uint16))
+    want = oracle.mha_forward_masked(oracle.bf16_to_f32(q), oracle.bf16_to_f32(k), oracle.bf16_to_f32(v), b, tq, tkv, h, d, mask)
+    _compare(f"masked bf16 B{b} Tq{tq} Tkv{tkv} H{h} D{d} mask{kind}", got, np.asarray(want, dtype=np.float32).ravel(),
+             oracle.BF16_MAX_ABS)
+
+
+@pytest.mark.parametrize("seed", [41, 42, 43])
+def test_random_window_chunk_and_masked_bf16_cases_match_oracle(oracle, seed):
+    rng = np.random.default_rng(seed)
+    cases = (_window, _chunk_decode, _masked_bf16)
+    for _ in range(60):
+        cases[int(rng.integers(0, len(cases)))](oracle, rng)
