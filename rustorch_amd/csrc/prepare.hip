@@ -74,7 +74,7 @@ __global__ __launch_bounds__(64) void decode_prepare_kernel(DecodePrepareParams 
 
 // The same arithmetic for a prompt.  With many consecutive tokens per head the one-wave kernel above is bound by its
 // own redundancy (all 64 lanes of a wave take the same sum of squares, and a row is moved two bytes per lane): 308 us
-// for B=4, 32 + 8 heads, 4096 tokens, D=128 (1.3 TB/s; 84 us = 4.8 TB/s here, 70 us when the cache rows are contiguous).  A workgroup takes ROWS consecutive tokens of one
+// for B=4, 32 + 8 heads, 4096 tokens, D=128 (1.3 TB/s; 84 us = 4.8 TB/s here).  A workgroup takes ROWS consecutive tokens of one
 // (sequence, head) -- contiguous rows in q / k_in and in the cache -- through LDS: the rows arrive with 16-byte loads,
 // every thread takes the sum of squares of ONE row in index order (the reference's order, model.rs:862-885), and
 // the normalised, rotated rows leave with 16-byte stores.  Rows sit in LDS as bf16 with a pitch of D + 2 elements (an odd
