@@ -534,22 +534,22 @@ __global__ __launch_bounds__(TileCfg<DP>::THREADS, DIRECT ? TileCfg<DP>::OCC_DIR
                     if (dl_row + 4 * RPI * n >= n_keys) *(u32x4_t*)(lds + 2 * STAGE_B + (wave + 4 * n) * 1024 + 16 * lane) = u32x4_t{0u, 0u, 0u, 0u};
             }
         } else {
-        park_k(kreg[0], 0);
-        park_v(std::integral_constant<int, 0>{}, 0);
-        keep_cur = keep_next;
-        if (PIPE) park_k(k1, 1);
-        {
-            auto prefetch = [&](auto i_c) __attribute__((always_inline)) {
-                constexpr int I = decltype(i_c)::value;  // 0 .. PF - 1
-                constexpr int KA = PIPE ? 2 : 1;         // K runs a tile ahead of V in the pipelined walk only
-                issue_k(kreg[(KA + I) % PF], (KA + I) * KT);
-                issue_v(std::integral_constant<int, (1 + I) % PF>{}, (1 + I) * KT);
-            };
-            prefetch(std::integral_constant<int, 0>{});
-            if (PF >= 2) prefetch(std::integral_constant<int, 1>{});
-            if (PF >= 3) prefetch(std::integral_constant<int, 2>{});
-            static_assert(PF <= 3, "prologue covers up to three sets");
-        }
+            park_k(kreg[0], 0);
+            park_v(std::integral_constant<int, 0>{}, 0);
+            keep_cur = keep_next;
+            if (PIPE) park_k(k1, 1);
+            {
+                auto prefetch = [&](auto i_c) __attribute__((always_inline)) {
+                    constexpr int I = decltype(i_c)::value;  // 0 .. PF - 1
+                    constexpr int KA = PIPE ? 2 : 1;         // K runs a tile ahead of V in the pipelined walk only
+                    issue_k(kreg[(KA + I) % PF], (KA + I) * KT);
+                    issue_v(std::integral_constant<int, (1 + I) % PF>{}, (1 + I) * KT);
+                };
+                prefetch(std::integral_constant<int, 0>{});
+                if (PF >= 2) prefetch(std::integral_constant<int, 1>{});
+                if (PF >= 3) prefetch(std::integral_constant<int, 2>{});
+                static_assert(PF <= 3, "prologue covers up to three sets");
+            }
         }
         __syncthreads();
 
